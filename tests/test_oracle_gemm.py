@@ -1,0 +1,130 @@
+"""Pins the GEMM-level functions of the CPU oracle against the fixtures the reference's portable
+code produced, against exact int64 numpy arithmetic, and through the identities the algebra fixes."""
+import numpy as np
+import pytest
+
+import oracle
+
+
+def wrap32(x):
+    return ((np.asarray(x, dtype=np.int64) + (1 << 31)) & 0xFFFFFFFF) - (1 << 31)
+
+
+def exact_t(A, B, ao, bo):
+    """sum_k (A+ao)(B+bo) in int64, wrapped to int32"""
+    return wrap32((A.astype(np.int64) + ao) @ (B.astype(np.int64) + bo)).astype(np.int32)
+
+
+def test_s32_fixture(golden):
+    g = golden("gemmlowp_s32.npz")
+    for n in range(int(g["count"])):
+        ao, bo = (int(x) for x in g["off%d" % n])
+        got = oracle.gemmlowp_s32(g["a%d" % n], g["b%d" % n], ao, bo)
+        np.testing.assert_array_equal(got, g["dst%d" % n])
+
+
+def test_s32_batched_fixture(golden):
+    g = golden("gemmlowp_batched.npz")
+    for n in range(int(g["count"])):
+        A, B = g["a%d" % n], g["b%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        for z in range(A.shape[0]):
+            got = oracle.gemmlowp_s32(A[z], B[z] if B.ndim == 3 else B, ao, bo)
+            np.testing.assert_array_equal(got, g["dst%d" % n][z])
+
+
+@pytest.mark.parametrize("a_dt,b_dt", [(np.uint8, np.uint8), (np.int8, np.int8), (np.uint8, np.int8),
+                                        (np.int8, np.uint8)])
+def test_s32_against_int64_matmul(a_dt, b_dt):
+    rng = np.random.default_rng(11)
+    for (M, N, K) in [(1, 1, 1), (5, 7, 300), (17, 9, 1000), (64, 48, 129)]:
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(np.iinfo(b_dt).min, np.iinfo(b_dt).max + 1, size=(K, N)).astype(b_dt)
+        for ao, bo in [(0, 0), (-128, 127), (3, 0), (0, -7), (2147480000, 5)]:
+            np.testing.assert_array_equal(oracle.gemmlowp_s32(A, B, ao, bo), exact_t(A, B, ao, bo))
+
+
+def test_flip_signedness_invariance():
+    """x ^ 0x80 on an operand with -/+128 on its offset leaves t unchanged
+    (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:153-190)."""
+    rng = np.random.default_rng(12)
+    A = rng.integers(0, 256, size=(9, 77), dtype=np.uint8)
+    B = rng.integers(0, 256, size=(77, 13), dtype=np.uint8)
+    want = oracle.gemmlowp_s32(A, B, -5, 9)
+    As = (A ^ 0x80).view(np.int8)
+    Bs = (B ^ 0x80).view(np.int8)
+    np.testing.assert_array_equal(oracle.gemmlowp_s32(As, B, -5 + 128, 9), want)
+    np.testing.assert_array_equal(oracle.gemmlowp_s32(As, Bs, -5 + 128, 9 + 128), want)
+
+
+def test_fused_fixedpoint_fixture(golden):
+    g = golden("gemmlowp_fused_fixedpoint.npz")
+    kinds = set()
+    for n in range(int(g["count"])):
+        ao, bo, roff, lo, hi, pc = (int(x) for x in g["p%d" % n])
+        dst = g["dst%d" % n]
+        got = oracle.gemmlowp_fixedpoint(g["a%d" % n], g["b%d" % n], g["bias%d" % n], ao, bo, g["mult%d" % n],
+                                         g["shift%d" % n], roff, lo, hi, dst.dtype)
+        np.testing.assert_array_equal(got, dst)
+        kinds.add((dst.dtype.name, pc, bool((g["shift%d" % n] < 0).any())))
+    # the fixture covers u8 / s8, per tensor / per channel, right and left shifts
+    assert ("uint8", 0, True) in kinds and ("int8", 1, True) in kinds and ("int8", 0, False) in kinds
+
+
+def test_output_stage_fixture(golden):
+    g = golden("output_stage.npz")
+    for n in range(int(g["count"])):
+        mult, shift, roff, lo, hi, with_bias = (int(x) for x in g["p%d" % n])
+        dst = g["dst%d" % n]
+        got = oracle.output_stage_fixedpoint(g["src%d" % n], g["bias%d" % n] if with_bias else None, [mult], [shift],
+                                             roff, lo, hi, dst.dtype)
+        np.testing.assert_array_equal(got, dst)
+
+
+def test_f32_fixture(golden):
+    """The reference's test oracle rounds once (float(t)*scale); the NEON order this oracle follows rounds
+    acc*scale and offsets*scale separately. Identical when offsets are zero, else equal to ~1 ulp of the
+    larger term."""
+    g = golden("gemmlowp_f32.npz")
+    scale = float(g["scale"])
+    for n in range(int(g["count"])):
+        ao, bo = (int(x) for x in g["off%d" % n])
+        A, B = g["a%d" % n], g["b%d" % n]
+        got = oracle.gemmlowp_f32(A, B, None, ao, bo, scale)
+        want = g["dst%d" % n]
+        if ao == 0 and bo == 0:
+            np.testing.assert_array_equal(got, want)
+        else:
+            acc = np.abs(A.astype(np.int64) @ B.astype(np.int64)).astype(np.float64) * scale
+            off = np.abs(exact_t(A, B, ao, bo).astype(np.float64) * scale - (A.astype(np.int64) @ B.astype(np.int64)) * scale)
+            tol = (acc + off + np.abs(want)) * 2.0 ** -23
+            assert (np.abs(got.astype(np.float64) - want) <= tol).all()
+
+
+def test_f32_bias_and_activation():
+    rng = np.random.default_rng(13)
+    A = rng.integers(-128, 128, size=(6, 40), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(40, 10), dtype=np.int8)
+    bias = rng.normal(0, 3, size=10).astype(np.float32)
+    scale = np.float32(0.02) * np.float32(0.005)
+    got = oracle.gemmlowp_f32(A, B, bias, 0, 0, float(scale), 0.0, 6.0)
+    acc = (A.astype(np.int32) @ B.astype(np.int32)).astype(np.float32)
+    want = np.clip(acc * scale + bias, np.float32(0), np.float32(6))
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.skipif(not oracle.ref_available(), reason="oracle/_ref not built (needs the reference checkout)")
+def test_fused_against_live_reference_config1_shape():
+    """BASELINE config 1 at full size (256^3, QASYMM8, both zero-point conventions) through the reference's code."""
+    rng = np.random.default_rng(1)
+    A = rng.integers(0, 256, size=(256, 256), dtype=np.uint8)
+    B = rng.integers(0, 256, size=(256, 256), dtype=np.uint8)
+    bias = rng.integers(-1000, 1001, size=256, dtype=np.int32)
+    for ao, bo in [(-128, -127), (128, 127)]:
+        t = oracle.ref_gemmlowp_core(A, B, ao, bo)
+        want = oracle.ref_quantize_down_fixedpoint(t, bias, [1518500250], [8], 10, 0, 255, np.uint8)
+        got = oracle.gemmlowp_fixedpoint(A, B, bias, ao, bo, [1518500250], [8], 10, 0, 255, np.uint8)
+        np.testing.assert_array_equal(got, want)
+        if ao < 0:
+            inside = ((want > 0) & (want < 255)).mean()
+            assert 0.2 < inside < 0.6  # a meaningful share of outputs is not clamped

@@ -1,0 +1,212 @@
+"""ctypes binding of include/mi355_gemmlowp.h for tests and bench.py. Accepts numpy arrays (host pointers) and
+torch CUDA tensors (device pointers) interchangeably; no computation happens here."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmi355gemmlowp.so")
+
+U8, S8, S32, F32 = 0, 1, 2, 3
+EPI_S32, EPI_FIXEDPOINT, EPI_F32 = 0, 1, 2
+PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
+
+EXPORTS = [
+    "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_run",
+    "mi355_gemmlowp_destroy", "mi355_gemmlowp_kernel_name", "mi355_output_stage_run", "mi355_conv_create",
+    "mi355_conv_prepare", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
+    "mi355_im2col_nhwc_run", "mi355_last_error", "mi355_device_info",
+]
+
+
+class Requant(C.Structure):
+    _fields_ = [("per_channel", C.c_int32), ("multiplier", C.c_int32), ("shift", C.c_int32),
+                ("result_offset", C.c_int32), ("min_bound", C.c_int32), ("max_bound", C.c_int32)]
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("batch", C.c_int32),
+                ("a_dtype", C.c_int32), ("b_dtype", C.c_int32), ("dst_dtype", C.c_int32), ("epilogue", C.c_int32),
+                ("lda", C.c_int64), ("ldb", C.c_int64), ("ldd", C.c_int64),
+                ("a_batch_stride", C.c_int64), ("b_batch_stride", C.c_int64), ("d_batch_stride", C.c_int64),
+                ("a_offset", C.c_int32), ("b_offset", C.c_int32), ("requant", Requant),
+                ("scale", C.c_float), ("act_min", C.c_float), ("act_max", C.c_float),
+                ("path", C.c_int32), ("reserved", C.c_int32)]
+
+
+class OutputStageDesc(C.Structure):
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("ld_src", C.c_int64), ("ld_dst", C.c_int64),
+                ("dst_dtype", C.c_int32), ("requant", Requant)]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("batch", "H", "W", "C", "OFM", "KH", "KW", "stride_x", "stride_y", "pad_left", "pad_top",
+                 "pad_right", "pad_bottom", "dilation_x", "dilation_y", "src_dtype", "weights_dtype", "dst_dtype",
+                 "src_offset", "weights_offset", "pad_value")] + [("requant", Requant), ("path", C.c_int32),
+                                                                  ("reserved", C.c_int32)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded shared library. Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m computelibrary_amd.build`" % LIB_PATH)
+        # A process may hold only one HIP runtime. PyTorch ships its own copy with the same soname as ROCm's, and
+        # whichever is loaded first serves both: load torch's first so device tensors and this library share it.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
+        l = C.CDLL(LIB_PATH)
+        vp, i32p, f32p = C.c_void_p, C.c_void_p, C.c_void_p
+        l.mi355_gemmlowp_create.argtypes = [C.POINTER(GemmDesc), C.POINTER(vp)]
+        l.mi355_gemmlowp_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
+        l.mi355_gemmlowp_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(Requant), C.c_float, vp]
+        l.mi355_gemmlowp_run.argtypes = [vp, vp, f32p, vp, vp]
+        l.mi355_gemmlowp_destroy.argtypes = [vp]
+        l.mi355_gemmlowp_destroy.restype = None
+        l.mi355_gemmlowp_kernel_name.argtypes = [vp]
+        l.mi355_gemmlowp_kernel_name.restype = C.c_char_p
+        l.mi355_output_stage_run.argtypes = [C.POINTER(OutputStageDesc), vp, i32p, vp, vp]
+        l.mi355_conv_create.argtypes = [C.POINTER(ConvDesc), C.POINTER(vp)]
+        l.mi355_conv_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
+        l.mi355_conv_run.argtypes = [vp, vp, vp, vp]
+        l.mi355_conv_out_dims.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+        l.mi355_conv_out_dims.restype = None
+        l.mi355_conv_destroy.argtypes = [vp]
+        l.mi355_conv_destroy.restype = None
+        l.mi355_conv_kernel_name.argtypes = [vp]
+        l.mi355_conv_kernel_name.restype = C.c_char_p
+        l.mi355_im2col_nhwc_run.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+        l.mi355_last_error.restype = C.c_char_p
+        l.mi355_device_info.argtypes = [C.c_char_p, C.c_size_t]
+        _lib = l
+    return _lib
+
+
+class Mi355Error(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise Mi355Error(lib().mi355_last_error().decode())
+
+
+def ptr(x):
+    """host pointer of a numpy array / device pointer of a torch tensor / None"""
+    if x is None:
+        return None
+    if isinstance(x, np.ndarray):
+        return x.ctypes.data
+    return x.data_ptr()
+
+
+def dtype_code(x):
+    name = str(x.dtype).replace("torch.", "")
+    return {"uint8": U8, "int8": S8, "int32": S32, "float32": F32}[name]
+
+
+def requant(mult=0, shift=0, offset=0, lo=-(1 << 31), hi=(1 << 31) - 1, per_channel=False):
+    return Requant(1 if per_channel else 0, int(mult), int(shift), int(offset), int(lo), int(hi))
+
+
+def device_info():
+    buf = C.create_string_buffer(64)
+    cus = lib().mi355_device_info(buf, 64)
+    return buf.value.decode(), cus
+
+
+class Gemm:
+    """create -> prepare -> run, for row-major contiguous (or explicitly strided) operands"""
+
+    def __init__(self, M, N, K, a_dtype, b_dtype, dst_dtype, epilogue, a_offset=0, b_offset=0, rq=None, scale=1.0,
+                 act_min=-np.inf, act_max=np.inf, batch=1, b_batched=False, lda=None, ldb=None, ldd=None,
+                 path=PATH_AUTO):
+        lda, ldb, ldd = lda or K, ldb or N, ldd or N
+        self.desc = GemmDesc(M, N, K, batch, a_dtype, b_dtype, dst_dtype, epilogue, lda, ldb, ldd, M * lda,
+                             K * ldb if b_batched else 0, M * ldd, a_offset, b_offset, rq or requant(), scale,
+                             act_min, act_max, path, 0)
+        self._h = C.c_void_p()
+        _check(lib().mi355_gemmlowp_create(C.byref(self.desc), C.byref(self._h)))
+
+    @property
+    def kernel_name(self):
+        return lib().mi355_gemmlowp_kernel_name(self._h).decode()
+
+    def prepare(self, B, bias=None, mult=None, shift=None, stream=None):
+        _check(lib().mi355_gemmlowp_prepare(self._h, ptr(B), ptr(bias), ptr(mult), ptr(shift), stream))
+
+    def update_quant(self, a_offset, b_offset, rq, scale=1.0, stream=None):
+        _check(lib().mi355_gemmlowp_update_quant(self._h, a_offset, b_offset, C.byref(rq) if rq else None, scale,
+                                                 stream))
+
+    def run(self, A, D, bias_f32=None, stream=None):
+        _check(lib().mi355_gemmlowp_run(self._h, ptr(A), ptr(bias_f32), ptr(D), stream))
+
+    def close(self):
+        if self._h:
+            lib().mi355_gemmlowp_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def output_stage(src, bias, dst, rq, stream=None, ld_src=None, ld_dst=None):
+    M, N = src.shape[0], src.shape[1]
+    d = OutputStageDesc(M, N, ld_src or N, ld_dst or N, dtype_code(dst), rq)
+    _check(lib().mi355_output_stage_run(C.byref(d), ptr(src), ptr(bias), ptr(dst), stream))
+
+
+def conv_desc(batch, H, W, Cc, OFM, KH, KW, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), src_dtype=S8,
+              weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0):
+    return ConvDesc(batch, H, W, Cc, OFM, KH, KW, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0],
+                    dilation[1], src_dtype, weights_dtype, dst_dtype, src_offset, weights_offset, pad_value,
+                    rq or requant(), path, 0)
+
+
+class Conv:
+    def __init__(self, desc):
+        self.desc = desc
+        self._h = C.c_void_p()
+        _check(lib().mi355_conv_create(C.byref(self.desc), C.byref(self._h)))
+
+    @property
+    def kernel_name(self):
+        return lib().mi355_conv_kernel_name(self._h).decode()
+
+    def out_dims(self):
+        oh, ow = C.c_int32(0), C.c_int32(0)
+        lib().mi355_conv_out_dims(C.byref(self.desc), C.byref(oh), C.byref(ow))
+        return oh.value, ow.value
+
+    def prepare(self, weights, bias=None, mult=None, shift=None, stream=None):
+        _check(lib().mi355_conv_prepare(self._h, ptr(weights), ptr(bias), ptr(mult), ptr(shift), stream))
+
+    def run(self, src, dst, stream=None):
+        _check(lib().mi355_conv_run(self._h, ptr(src), ptr(dst), stream))
+
+    def close(self):
+        if self._h:
+            lib().mi355_conv_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def im2col_nhwc(desc, src, dst, stream=None):
+    _check(lib().mi355_im2col_nhwc_run(C.byref(desc), ptr(src), ptr(dst), stream))

@@ -1,0 +1,774 @@
+// Implementation of the C ABI declared in include/mi355_gemmlowp.h: descriptor checks, kernel selection, device
+// workspace ownership, host <-> device staging, and the launches. No arithmetic lives here.
+#include "../../include/mi355_gemmlowp.h"
+#include "internal.hpp"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+
+using namespace mi355;
+
+namespace
+{
+thread_local std::string g_err;
+
+int fail(const char *fmt, ...)
+{
+    char    buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return 1;
+}
+
+#define HIP_TRY(expr)                                                                                  \
+    do                                                                                                 \
+    {                                                                                                  \
+        const hipError_t e_ = (hipError_t)(expr);                                                      \
+        if (e_ != hipSuccess)                                                                          \
+            return fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__);    \
+    } while (0)
+#define TRY(expr)            \
+    do                       \
+    {                        \
+        if ((expr) != 0)     \
+            return 1;        \
+    } while (0)
+
+bool is_device_ptr(const void *p)
+{
+    if (p == nullptr)
+        return false;
+    hipPointerAttribute_t attr;
+    const hipError_t      e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess)
+    {
+        (void)hipGetLastError(); // plain host memory: clear the sticky error
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+struct DevBuf
+{
+    void  *p   = nullptr;
+    size_t cap = 0;
+    int    ensure(size_t bytes)
+    {
+        if (bytes <= cap && p != nullptr)
+            return 0;
+        if (p)
+        {
+            HIP_TRY(hipFree(p));
+            p = nullptr, cap = 0;
+        }
+        if (bytes == 0)
+            bytes = 16;
+        HIP_TRY(hipMalloc(&p, bytes));
+        cap = bytes;
+        return 0;
+    }
+    void release()
+    {
+        if (p)
+            (void)hipFree(p);
+        p = nullptr, cap = 0;
+    }
+    template <typename T>
+    T *as() const
+    {
+        return (T *)p;
+    }
+};
+
+// brings `bytes` at `src` to the device if it is host memory; returns the device pointer to use
+int to_device(const void *src, size_t bytes, DevBuf &stage, hipStream_t s, const void **out)
+{
+    if (src == nullptr)
+    {
+        *out = nullptr;
+        return 0;
+    }
+    if (is_device_ptr(src))
+    {
+        *out = src;
+        return 0;
+    }
+    TRY(stage.ensure(bytes));
+    HIP_TRY(hipMemcpyAsync(stage.p, src, bytes, hipMemcpyHostToDevice, s));
+    *out = stage.p;
+    return 0;
+}
+
+int num_cus()
+{
+    static int cus = -1;
+    if (cus < 0)
+    {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess)
+            return 256;
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess)
+            return 256;
+        cus = prop.multiProcessorCount;
+    }
+    return cus;
+}
+
+bool is_8bit(int dt)
+{
+    return dt == MI355_U8 || dt == MI355_S8;
+}
+
+// The part of a GEMM that both the dense handle and the convolution handle need
+struct GemmCore
+{
+    int     M = 0, N = 0, K = 0, batch = 1;
+    int     epi       = EPI_S32;
+    int     dst_dtype = MI355_S32;
+    bool    flip_a = false, flip_b = false;
+    int32_t a_offset = 0, b_offset = 0; // as given (added convention)
+    mi355_requant rq{};
+    float   scale = 1.f, act_min = -INFINITY, act_max = INFINITY;
+    int     path = MI355_PATH_AUTO, cfg_idx = 0;
+    int     Kp = 0, Np = 0;
+    bool    b_shared = true; // one B for all batches
+    bool    has_bias = false, has_pc = false, prepared = false;
+    std::string kname;
+    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap;
+
+    int32_t a_off_eff() const { return (int32_t)((uint32_t)a_offset + (flip_a ? 128u : 0u)); }
+    int32_t b_off_eff() const { return (int32_t)((uint32_t)b_offset + (flip_b ? 128u : 0u)); }
+    int     nb() const { return b_shared ? 1 : batch; }
+
+    void release()
+    {
+        Bp.release(), Bs.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
+        shift.release(), bias.release(), Ap.release();
+    }
+
+    int choose_kernel()
+    {
+        Kp = round_up(K, PACK_K_ALIGN);
+        Np = round_up(N, PACK_N_ALIGN);
+        if (path == MI355_PATH_AUTO)
+            path = (M <= SKINNY_MAX_M && batch == 1) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
+        if (path == MI355_PATH_SKINNY && (M > SKINNY_MAX_M || batch != 1))
+            return fail("skinny path needs M <= %d and batch == 1", SKINNY_MAX_M);
+        if (path == MI355_PATH_SIMPLE)
+            kname = "simple";
+        else if (path == MI355_PATH_SKINNY)
+            kname = "skinny_16xN_splitk8";
+        else
+        {
+            const int   cus   = num_cus();
+            int         best  = -1;
+            long        most  = -1;
+            const char *force = getenv("MI355_GEMM_CFG");
+            for (int i = 0; i < mfma_num_configs(); ++i)
+            {
+                const MfmaConfig c     = mfma_config(i);
+                const long       tiles = (long)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN) * batch;
+                if (N <= 64 && c.BN > 64)
+                    continue;
+                if (tiles >= cus)
+                {
+                    best = i;
+                    break;
+                }
+                if (tiles > most)
+                    most = tiles, best = i;
+            }
+            if (force && atoi(force) >= 0 && atoi(force) < mfma_num_configs())
+                best = atoi(force);
+            cfg_idx = best;
+            kname   = mfma_config(best).name;
+        }
+        return 0;
+    }
+
+    // after Bp / colsum have been written for every B: per-column vectors
+    int finish_prepare(const int32_t *bias_in, const int32_t *mult_in, const int32_t *shift_in, hipStream_t s)
+    {
+        has_bias = bias_in != nullptr;
+        if (has_bias)
+        {
+            TRY(bias.ensure(sizeof(int32_t) * (size_t)N));
+            HIP_TRY(hipMemcpyAsync(bias.p, bias_in, sizeof(int32_t) * (size_t)N, hipMemcpyDefault, s));
+        }
+        has_pc = epi == EPI_FIXEDPOINT && rq.per_channel != 0;
+        if (has_pc)
+        {
+            if (mult_in == nullptr || shift_in == nullptr)
+                return fail("per-channel requantisation needs multiplier and shift arrays");
+            TRY(mult.ensure(sizeof(int32_t) * (size_t)N));
+            TRY(shift.ensure(sizeof(int32_t) * (size_t)N));
+            HIP_TRY(hipMemcpyAsync(mult.p, mult_in, sizeof(int32_t) * (size_t)N, hipMemcpyDefault, s));
+            HIP_TRY(hipMemcpyAsync(shift.p, shift_in, sizeof(int32_t) * (size_t)N, hipMemcpyDefault, s));
+        }
+        if (path == MI355_PATH_SKINNY)
+        {
+            TRY(Bs.ensure((size_t)Np * Kp));
+            HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>(), Kp, Np, Bs.as<int8_t>(), s));
+        }
+        TRY(refresh_colvec(s));
+        prepared = true;
+        return 0;
+    }
+
+    int refresh_colvec(hipStream_t s)
+    {
+        TRY(colvec.ensure(sizeof(int32_t) * (size_t)Np * nb()));
+        for (int b = 0; b < nb(); ++b)
+            HIP_TRY(colvec_launch(colsum.as<int32_t>() + (size_t)b * Np,
+                                  (has_bias && epi == EPI_FIXEDPOINT) ? bias.as<int32_t>() : nullptr, a_off_eff(),
+                                  b_off_eff(), K, N, colvec.as<int32_t>() + (size_t)b * Np, s));
+        return 0;
+    }
+
+    void fill_epi(EpiParams &p, const float *bias_f32) const
+    {
+        p.colvec              = colvec.as<int32_t>();
+        p.rowvec              = nullptr;
+        p.mult                = has_pc ? mult.as<int32_t>() : nullptr;
+        p.shift               = has_pc ? shift.as<int32_t>() : nullptr;
+        p.bias_f32            = bias_f32;
+        p.colvec_batch_stride = b_shared ? 0 : Np;
+        p.rowvec_batch_stride = M;
+        p.mult_s              = rq.multiplier;
+        p.shift_s             = rq.shift;
+        p.result_offset       = rq.result_offset;
+        const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
+        p.lo                  = rq.min_bound > tlo ? rq.min_bound : tlo;
+        p.hi                  = rq.max_bound < thi ? rq.max_bound : thi;
+        p.scale               = scale;
+        p.act_min             = act_min;
+        p.act_max             = act_max;
+        p.has_offsets         = (a_offset != 0 || b_offset != 0) ? 1 : 0;
+        p.dst_signed          = dst_dtype == MI355_S8;
+    }
+
+    // A, D and bias_f32 are device pointers here
+    int run_dense(const int8_t *A, int64_t lda, int64_t a_bs, void *D, int64_t ldd, int64_t d_bs,
+                  const float *bias_f32, hipStream_t s)
+    {
+        if (!prepared)
+            return fail("run before prepare");
+        GemmArgs g{};
+        fill_epi(g.epi, bias_f32);
+        bool flip_in_loader = flip_a;
+        int  k_valid        = K;
+        const bool direct =
+            path == MI355_PATH_SIMPLE || ((((uintptr_t)A | (uintptr_t)lda | (uintptr_t)a_bs) & 3) == 0);
+        const bool need_rowvec = b_off_eff() != 0;
+        if (need_rowvec)
+            TRY(rowvec.ensure(sizeof(int32_t) * (size_t)M * batch));
+        if (!direct)
+        {
+            // rows not dword aligned: padded, sign-normalised copy (and the row sums in the same pass)
+            TRY(Ap.ensure((size_t)batch * M * Kp));
+            for (int b = 0; b < batch; ++b)
+                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, Ap.as<int8_t>() + (size_t)b * M * Kp,
+                                         Kp, need_rowvec ? rowvec.as<int32_t>() + (size_t)b * M : nullptr, b_off_eff(),
+                                         s));
+            A = Ap.as<int8_t>(), lda = Kp, a_bs = (int64_t)M * Kp, k_valid = Kp, flip_in_loader = false;
+        }
+        else if (need_rowvec)
+        {
+            for (int b = 0; b < batch; ++b)
+                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, nullptr, Kp,
+                                         rowvec.as<int32_t>() + (size_t)b * M, b_off_eff(), s));
+        }
+        if (need_rowvec)
+            g.epi.rowvec = rowvec.as<int32_t>();
+        g.A = A, g.lda = lda, g.a_batch_stride = a_bs;
+        g.Bp = Bp.as<int8_t>(), g.Kp = Kp, g.bp_batch_stride = b_shared ? 0 : (int64_t)Np * Kp;
+        g.D = D, g.ldd = ldd, g.d_batch_stride = d_bs;
+        g.M = M, g.N = N, g.K = k_valid;
+        return launch(g, flip_in_loader, false, s);
+    }
+
+    int launch(GemmArgs &g, bool flip_in_loader, bool conv, hipStream_t s)
+    {
+        if (path == MI355_PATH_SIMPLE)
+            HIP_TRY(simple_gemm_launch(epi, flip_in_loader, g, batch, s));
+        else if (path == MI355_PATH_SKINNY)
+        {
+            g.Bp = Bs.as<int8_t>();
+            HIP_TRY(skinny_launch(epi, flip_in_loader, g, s));
+        }
+        else
+        {
+            const MfmaConfig c = mfma_config(cfg_idx);
+            g.tiles_m          = (g.M + c.BM - 1) / c.BM;
+            g.tiles_n          = (g.N + c.BN - 1) / c.BN;
+            HIP_TRY(mfma_launch(cfg_idx, epi, flip_in_loader, conv, g, batch, s));
+        }
+        return 0;
+    }
+};
+
+int check_requant(const mi355_requant &rq, int dst_dtype)
+{
+    if (rq.min_bound > rq.max_bound)
+        return fail("min_bound > max_bound");
+    const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
+    if (rq.max_bound < tlo || rq.min_bound > thi)
+        return fail("clamp bounds [%d,%d] do not intersect the destination type's range", rq.min_bound, rq.max_bound);
+    return 0;
+}
+} // namespace
+
+struct mi355_gemm_handle
+{
+    mi355_gemm_desc d;
+    GemmCore        core;
+    DevBuf          stageA, stageB, stageD, stageBiasF, stageBias, stageMult, stageShift;
+};
+
+struct mi355_conv_handle
+{
+    mi355_conv_desc d;
+    GemmCore        core;
+    ConvGeom        geom;
+    bool            implicit = false;
+    DevBuf          stageSrc, stageW, stageDst, stageBias, stageMult, stageShift, cols;
+};
+
+extern "C"
+{
+const char *mi355_last_error(void)
+{
+    return g_err.c_str();
+}
+
+int mi355_device_info(char *name, size_t name_len)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        fail("no HIP device");
+        return -1;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess)
+    {
+        fail("hipGetDeviceProperties failed");
+        return -1;
+    }
+    if (name && name_len)
+    {
+        strncpy(name, prop.gcnArchName, name_len - 1);
+        name[name_len - 1] = 0;
+    }
+    return prop.multiProcessorCount;
+}
+
+int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
+{
+    if (!desc || !out)
+        return fail("null argument");
+    const mi355_gemm_desc &d = *desc;
+    if (d.M < 1 || d.N < 1 || d.K < 1 || d.batch < 1)
+        return fail("M, N, K, batch must be positive (got %d %d %d %d)", d.M, d.N, d.K, d.batch);
+    if (!is_8bit(d.a_dtype) || !is_8bit(d.b_dtype))
+        return fail("A and B must be 8-bit");
+    if (d.lda < d.K || d.ldb < d.N || d.ldd < d.N)
+        return fail("row stride smaller than the row");
+    switch (d.epilogue)
+    {
+        case MI355_EPI_S32:
+            if (d.dst_dtype != MI355_S32)
+                return fail("S32 epilogue needs an S32 destination");
+            break;
+        case MI355_EPI_FIXEDPOINT:
+            if (!is_8bit(d.dst_dtype))
+                return fail("FIXEDPOINT epilogue needs an 8-bit destination");
+            if (check_requant(d.requant, d.dst_dtype))
+                return 1;
+            break;
+        case MI355_EPI_F32:
+            if (d.dst_dtype != MI355_F32)
+                return fail("F32 epilogue needs an F32 destination");
+            break;
+        default:
+            return fail("unknown epilogue %d", d.epilogue);
+    }
+    if (d.batch > 1 && (d.a_batch_stride < (int64_t)(d.M - 1) * d.lda + d.K || d.d_batch_stride < (int64_t)(d.M - 1) * d.ldd + d.N))
+        return fail("batch stride smaller than one matrix");
+    if (d.batch > 1 && d.b_batch_stride != 0 && d.b_batch_stride < (int64_t)(d.K - 1) * d.ldb + d.N)
+        return fail("B batch stride smaller than one matrix");
+    mi355_gemm_handle *h = new (std::nothrow) mi355_gemm_handle();
+    if (!h)
+        return fail("out of host memory");
+    h->d        = d;
+    GemmCore &c = h->core;
+    c.M = d.M, c.N = d.N, c.K = d.K, c.batch = d.batch;
+    c.epi = d.epilogue, c.dst_dtype = d.dst_dtype;
+    c.flip_a = d.a_dtype == MI355_U8, c.flip_b = d.b_dtype == MI355_U8;
+    c.a_offset = d.a_offset, c.b_offset = d.b_offset;
+    c.rq = d.requant, c.scale = d.scale, c.act_min = d.act_min, c.act_max = d.act_max;
+    c.path     = d.path;
+    c.b_shared = d.batch == 1 || d.b_batch_stride == 0;
+    if (c.choose_kernel())
+    {
+        delete h;
+        return 1;
+    }
+    *out = h;
+    return 0;
+}
+
+int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *bias, const int32_t *mult,
+                           const int32_t *shift, void *stream)
+{
+    if (!h || !B)
+        return fail("null argument");
+    hipStream_t            s = (hipStream_t)stream;
+    GemmCore              &c = h->core;
+    const mi355_gemm_desc &d = h->d;
+    const int              nb = c.nb();
+    const size_t           b_bytes = (size_t)(nb - 1) * d.b_batch_stride + (size_t)(d.K - 1) * d.ldb + d.N;
+    const void            *Bd, *biasd, *multd, *shiftd;
+    TRY(to_device(B, b_bytes, h->stageB, s, &Bd));
+    TRY(to_device(bias, sizeof(int32_t) * d.N, h->stageBias, s, &biasd));
+    TRY(to_device(c.rq.per_channel ? mult : nullptr, sizeof(int32_t) * d.N, h->stageMult, s, &multd));
+    TRY(to_device(c.rq.per_channel ? shift : nullptr, sizeof(int32_t) * d.N, h->stageShift, s, &shiftd));
+    TRY(c.Bp.ensure((size_t)nb * c.Np * c.Kp));
+    TRY(c.colsum.ensure(sizeof(int32_t) * (size_t)nb * c.Np));
+    for (int b = 0; b < nb; ++b)
+        HIP_TRY(pack_b_launch((const uint8_t *)Bd + (size_t)b * d.b_batch_stride, d.ldb, d.K, d.N, c.Kp, c.Np, c.flip_b,
+                              c.Bp.as<int8_t>() + (size_t)b * c.Np * c.Kp, c.colsum.as<int32_t>() + (size_t)b * c.Np, s));
+    if (c.path == MI355_PATH_SKINNY && nb != 1)
+        return fail("skinny path does not batch");
+    TRY(c.finish_prepare((const int32_t *)biasd, (const int32_t *)multd, (const int32_t *)shiftd, s));
+    // staging buffers are reused by later calls: make sure the copies out of them have finished
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t b_offset, const mi355_requant *requant,
+                                float scale, void *stream)
+{
+    if (!h)
+        return fail("null argument");
+    GemmCore &c = h->core;
+    if (requant)
+    {
+        if (c.epi == EPI_FIXEDPOINT && check_requant(*requant, c.dst_dtype))
+            return 1;
+        if (requant->per_channel != c.rq.per_channel)
+            return fail("update cannot switch between per-tensor and per-channel requantisation");
+        c.rq = *requant;
+    }
+    c.a_offset = a_offset, c.b_offset = b_offset, c.scale = scale;
+    h->d.a_offset = a_offset, h->d.b_offset = b_offset, h->d.scale = scale;
+    if (c.prepared)
+        TRY(c.refresh_colvec((hipStream_t)stream));
+    return 0;
+}
+
+int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream)
+{
+    if (!h || !A || !D)
+        return fail("null argument");
+    hipStream_t            s = (hipStream_t)stream;
+    GemmCore              &c = h->core;
+    const mi355_gemm_desc &d = h->d;
+    if (bias_f32 && c.epi != EPI_F32)
+        return fail("float bias is only valid with the F32 epilogue");
+    const size_t esz     = d.dst_dtype == MI355_S32 || d.dst_dtype == MI355_F32 ? 4 : 1;
+    const size_t a_bytes = (size_t)(d.batch - 1) * d.a_batch_stride + (size_t)(d.M - 1) * d.lda + d.K;
+    const size_t d_elems = (size_t)(d.batch - 1) * d.d_batch_stride + (size_t)(d.M - 1) * d.ldd + d.N;
+    const void  *Ad, *bfd;
+    TRY(to_device(A, a_bytes, h->stageA, s, &Ad));
+    TRY(to_device(bias_f32, sizeof(float) * d.N, h->stageBiasF, s, &bfd));
+    const bool d_host = !is_device_ptr(D);
+    void      *Dd     = D;
+    if (d_host)
+    {
+        TRY(h->stageD.ensure(d_elems * esz));
+        Dd = h->stageD.p;
+        if (d.ldd != d.N || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
+            HIP_TRY(hipMemcpyAsync(Dd, D, d_elems * esz, hipMemcpyHostToDevice, s)); // keep the caller's padding
+    }
+    TRY(c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, Dd, d.ldd, d.d_batch_stride, (const float *)bfd, s));
+    if (d_host)
+    {
+        HIP_TRY(hipMemcpyAsync(D, Dd, d_elems * esz, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
+    else if (Ad != A || bfd != bias_f32)
+        HIP_TRY(hipStreamSynchronize(s)); // staged inputs must be consumed before the caller may reuse them
+    return 0;
+}
+
+void mi355_gemmlowp_destroy(mi355_gemm_handle *h)
+{
+    if (!h)
+        return;
+    h->core.release();
+    h->stageA.release(), h->stageB.release(), h->stageD.release(), h->stageBiasF.release(), h->stageBias.release();
+    h->stageMult.release(), h->stageShift.release();
+    delete h;
+}
+
+const char *mi355_gemmlowp_kernel_name(const mi355_gemm_handle *h)
+{
+    return h ? h->core.kname.c_str() : "";
+}
+
+int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *src, const int32_t *bias, void *dst,
+                           void *stream)
+{
+    if (!desc || !src || !dst)
+        return fail("null argument");
+    const mi355_output_stage_desc &d = *desc;
+    if (d.M < 1 || d.N < 1 || d.ld_src < d.N || d.ld_dst < d.N)
+        return fail("bad output-stage shape");
+    if (!is_8bit(d.dst_dtype))
+        return fail("output stage writes QASYMM8 or QASYMM8_SIGNED");
+    if (d.requant.per_channel)
+        return fail("the stand-alone output stage is per-tensor");
+    if (check_requant(d.requant, d.dst_dtype))
+        return 1;
+    hipStream_t s = (hipStream_t)stream;
+    DevBuf      sSrc, sBias, sDst;
+    const void *srcd, *biasd;
+    const size_t s_elems = (size_t)(d.M - 1) * d.ld_src + d.N, d_elems = (size_t)(d.M - 1) * d.ld_dst + d.N;
+    int          rc      = 0;
+    void        *Dd      = dst;
+    const bool   d_host  = !is_device_ptr(dst);
+    EpiParams    p{};
+    p.mult_s = d.requant.multiplier, p.shift_s = d.requant.shift, p.result_offset = d.requant.result_offset;
+    const int32_t tlo = d.dst_dtype == MI355_S8 ? -128 : 0, thi = d.dst_dtype == MI355_S8 ? 127 : 255;
+    p.lo = d.requant.min_bound > tlo ? d.requant.min_bound : tlo;
+    p.hi = d.requant.max_bound < thi ? d.requant.max_bound : thi;
+    auto body = [&]() -> int
+    {
+        TRY(to_device(src, s_elems * 4, sSrc, s, &srcd));
+        TRY(to_device(bias, sizeof(int32_t) * d.N, sBias, s, &biasd));
+        if (d_host)
+        {
+            TRY(sDst.ensure(d_elems));
+            Dd = sDst.p;
+            if (d.ld_dst != d.N)
+                HIP_TRY(hipMemcpyAsync(Dd, dst, d_elems, hipMemcpyHostToDevice, s));
+        }
+        HIP_TRY(output_stage_launch((const int32_t *)srcd, d.ld_src, (const int32_t *)biasd, Dd, d.ld_dst, d.M, d.N, p, s));
+        if (d_host)
+            HIP_TRY(hipMemcpyAsync(dst, Dd, d_elems, hipMemcpyDeviceToHost, s));
+        if (d_host || srcd != src || biasd != bias)
+            HIP_TRY(hipStreamSynchronize(s));
+        return 0;
+    };
+    rc = body();
+    sSrc.release(), sBias.release(), sDst.release();
+    return rc;
+}
+
+static void conv_geom(const mi355_conv_desc &d, ConvGeom &g)
+{
+    g.H = d.H, g.W = d.W, g.C = d.C, g.KH = d.KH, g.KW = d.KW;
+    g.stride_x = d.stride_x, g.stride_y = d.stride_y, g.pad_left = d.pad_left, g.pad_top = d.pad_top;
+    g.dil_x = d.dilation_x, g.dil_y = d.dilation_y;
+    // FLOOR rounding of PadStrideInfo (src/core/Utils.cpp:288-332)
+    int w = (int)std::floor((float)(d.W + d.pad_left + d.pad_right - (d.dilation_x * (d.KW - 1) + 1)) / (float)d.stride_x + 1.f);
+    int h = (int)std::floor((float)(d.H + d.pad_top + d.pad_bottom - (d.dilation_y * (d.KH - 1) + 1)) / (float)d.stride_y + 1.f);
+    g.OW = w < 1 ? 1 : w;
+    g.OH = h < 1 ? 1 : h;
+}
+
+void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW)
+{
+    ConvGeom g{};
+    conv_geom(*desc, g);
+    if (OH)
+        *OH = g.OH;
+    if (OW)
+        *OW = g.OW;
+}
+
+static int conv_check(const mi355_conv_desc &d)
+{
+    if (d.batch < 1 || d.H < 1 || d.W < 1 || d.C < 1 || d.OFM < 1 || d.KH < 1 || d.KW < 1)
+        return fail("convolution dimensions must be positive");
+    if (d.stride_x < 1 || d.stride_y < 1 || d.dilation_x < 1 || d.dilation_y < 1)
+        return fail("stride and dilation must be >= 1");
+    if (d.pad_left < 0 || d.pad_top < 0 || d.pad_right < 0 || d.pad_bottom < 0)
+        return fail("negative padding");
+    if (!is_8bit(d.src_dtype) || !is_8bit(d.weights_dtype) || !is_8bit(d.dst_dtype))
+        return fail("convolution tensors must be 8-bit");
+    return 0;
+}
+
+int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
+{
+    if (!desc || !out)
+        return fail("null argument");
+    const mi355_conv_desc &d = *desc;
+    TRY(conv_check(d));
+    TRY(check_requant(d.requant, d.dst_dtype));
+    mi355_conv_handle *h = new (std::nothrow) mi355_conv_handle();
+    if (!h)
+        return fail("out of host memory");
+    h->d = d;
+    conv_geom(d, h->geom);
+    GemmCore     &c  = h->core;
+    const int64_t M64 = (int64_t)d.batch * h->geom.OH * h->geom.OW;
+    const int64_t K64 = (int64_t)d.KH * d.KW * d.C;
+    if (M64 > INT32_MAX || K64 > INT32_MAX)
+    {
+        delete h;
+        return fail("convolution too large");
+    }
+    c.M = (int)M64, c.N = d.OFM, c.K = (int)K64, c.batch = 1;
+    c.epi = EPI_FIXEDPOINT, c.dst_dtype = d.dst_dtype;
+    c.flip_a = d.src_dtype == MI355_U8, c.flip_b = d.weights_dtype == MI355_U8;
+    c.a_offset = d.src_offset, c.b_offset = d.weights_offset;
+    c.rq = d.requant, c.path = MI355_PATH_MFMA, c.b_shared = true;
+    if (c.choose_kernel())
+    {
+        delete h;
+        return 1;
+    }
+    // the on-the-fly loader moves 16-byte pieces of one tap: needs C % 16 == 0; it has no row sums: needs b_off == 0
+    h->implicit         = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0;
+    const uint32_t pb   = ((uint32_t)d.pad_value & 0xFFu) ^ ((h->implicit && c.flip_a) ? 0x80u : 0u);
+    h->geom.pad_word    = pb * 0x01010101u;
+    c.kname             = std::string(h->implicit ? "implicit_" : "im2col+") + c.kname;
+    *out                = h;
+    return 0;
+}
+
+int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t *bias, const int32_t *mult,
+                       const int32_t *shift, void *stream)
+{
+    if (!h || !weights)
+        return fail("null argument");
+    hipStream_t s = (hipStream_t)stream;
+    GemmCore   &c = h->core;
+    const void *wd, *biasd, *multd, *shiftd;
+    TRY(to_device(weights, (size_t)c.N * c.K, h->stageW, s, &wd));
+    TRY(to_device(bias, sizeof(int32_t) * c.N, h->stageBias, s, &biasd));
+    TRY(to_device(c.rq.per_channel ? mult : nullptr, sizeof(int32_t) * c.N, h->stageMult, s, &multd));
+    TRY(to_device(c.rq.per_channel ? shift : nullptr, sizeof(int32_t) * c.N, h->stageShift, s, &shiftd));
+    TRY(c.Bp.ensure((size_t)c.Np * c.Kp));
+    TRY(c.colsum.ensure(sizeof(int32_t) * (size_t)c.Np));
+    // weights [OFM][KH][KW][C] are already the K-contiguous layout with k = c + kx*C + ky*C*KW
+    // (src/cpu/kernels/CpuWeightsReshapeKernel.cpp:150-166)
+    HIP_TRY(pack_bt_launch(wd, c.K, c.K, c.N, c.Kp, c.Np, c.flip_b, c.Bp.as<int8_t>(), c.colsum.as<int32_t>(), s));
+    TRY(c.finish_prepare((const int32_t *)biasd, (const int32_t *)multd, (const int32_t *)shiftd, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream)
+{
+    if (!h || !src || !dst)
+        return fail("null argument");
+    hipStream_t            s = (hipStream_t)stream;
+    GemmCore              &c = h->core;
+    const mi355_conv_desc &d = h->d;
+    if (!c.prepared)
+        return fail("run before prepare");
+    const size_t src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N;
+    const void  *srcd;
+    TRY(to_device(src, src_bytes, h->stageSrc, s, &srcd));
+    const bool d_host = !is_device_ptr(dst);
+    void      *Dd     = dst;
+    if (d_host)
+    {
+        TRY(h->stageDst.ensure(dst_bytes));
+        Dd = h->stageDst.p;
+    }
+    if (h->implicit && (((uintptr_t)srcd) & 15) == 0)
+    {
+        GemmArgs g{};
+        c.fill_epi(g.epi, nullptr);
+        g.A = (const int8_t *)srcd, g.lda = 0, g.a_batch_stride = 0;
+        g.Bp = c.Bp.as<int8_t>(), g.Kp = c.Kp, g.bp_batch_stride = 0;
+        g.D = Dd, g.ldd = c.N, g.d_batch_stride = 0;
+        g.M = c.M, g.N = c.N, g.K = c.K;
+        g.conv = h->geom;
+        TRY(c.launch(g, c.flip_a, true, s));
+    }
+    else
+    {
+        // explicit lowering: patch matrix [M][Kp] in workspace, then the dense path
+        ConvGeom g2   = h->geom;
+        g2.pad_word   = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
+        const int ldc = round_up(c.K, 16);
+        TRY(h->cols.ensure((size_t)c.M * ldc));
+        HIP_TRY(im2col_nhwc_launch(srcd, h->cols.p, d.batch, g2, ldc, s));
+        TRY(c.run_dense(h->cols.as<int8_t>(), ldc, 0, Dd, c.N, 0, nullptr, s));
+    }
+    if (d_host)
+    {
+        HIP_TRY(hipMemcpyAsync(dst, Dd, dst_bytes, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
+    else if (srcd != src)
+        HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
+void mi355_conv_destroy(mi355_conv_handle *h)
+{
+    if (!h)
+        return;
+    h->core.release();
+    h->stageSrc.release(), h->stageW.release(), h->stageDst.release(), h->stageBias.release();
+    h->stageMult.release(), h->stageShift.release(), h->cols.release();
+    delete h;
+}
+
+const char *mi355_conv_kernel_name(const mi355_conv_handle *h)
+{
+    return h ? h->core.kname.c_str() : "";
+}
+
+int mi355_im2col_nhwc_run(const mi355_conv_desc *desc, const void *src, void *dst, void *stream)
+{
+    if (!desc || !src || !dst)
+        return fail("null argument");
+    const mi355_conv_desc &d = *desc;
+    TRY(conv_check(d));
+    ConvGeom g{};
+    conv_geom(d, g);
+    g.pad_word      = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
+    hipStream_t s   = (hipStream_t)stream;
+    const size_t K  = (size_t)d.KH * d.KW * d.C, rows = (size_t)d.batch * g.OH * g.OW;
+    DevBuf       sSrc, sDst;
+    const void  *srcd;
+    void        *Dd     = dst;
+    const bool   d_host = !is_device_ptr(dst);
+    auto         body   = [&]() -> int
+    {
+        TRY(to_device(src, (size_t)d.batch * d.H * d.W * d.C, sSrc, s, &srcd));
+        if (d_host)
+        {
+            TRY(sDst.ensure(rows * K));
+            Dd = sDst.p;
+        }
+        HIP_TRY(im2col_nhwc_launch(srcd, Dd, d.batch, g, (int64_t)K, s));
+        if (d_host)
+            HIP_TRY(hipMemcpyAsync(dst, Dd, rows * K, hipMemcpyDeviceToHost, s));
+        if (d_host || srcd != src)
+            HIP_TRY(hipStreamSynchronize(s));
+        return 0;
+    };
+    const int rc = body();
+    sSrc.release(), sDst.release();
+    return rc;
+}
+} // extern "C"

@@ -1,0 +1,101 @@
+// Device-side arithmetic shared by every kernel of the quantized-GEMM path: the fixed-point
+// requantisation primitive and the three ways an int32 accumulator leaves the chip.
+//
+// The integer semantics restate the reference's NEON code:
+//   SQDMULH (no rounding) then SRSHL (round half up), src/core/NEON/NEAsymm.h:95-128, :233-296,
+//   src/core/NEON/NEMath.inl:430-440; saturating narrow then bounded-relu clamp, NEAsymm.h:130-147.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355
+{
+enum : int
+{
+    EPI_S32        = 0,
+    EPI_FIXEDPOINT = 1,
+    EPI_F32        = 2
+};
+
+struct EpiParams
+{
+    const int32_t *colvec; // [N]  a_off*colsum[j] + a_off*b_off*K (+ int32 bias[j] for EPI_FIXEDPOINT)
+    const int32_t *rowvec; // [M]  b_off*rowsum[i], or nullptr when b_off == 0
+    const int32_t *mult;   // [N]  per-channel multipliers, or nullptr (then mult_s)
+    const int32_t *shift;  // [N]  per-channel shifts, or nullptr (then shift_s)
+    const float   *bias_f32;
+    int64_t        colvec_batch_stride; // elements between batches (0: shared B)
+    int64_t        rowvec_batch_stride;
+    int32_t        mult_s, shift_s;
+    int32_t        result_offset;
+    int32_t        lo, hi; // clamp range, already intersected with the destination type's range
+    float          scale;
+    float          act_min, act_max;
+    int32_t        has_offsets; // EPI_F32: whether the offset term is added at all
+    int32_t        dst_signed;
+};
+
+// (a * b * 2) >> 32 with the single saturating case, without 64-bit VALU arithmetic
+__device__ __forceinline__ int32_t sqdmulh(int32_t a, int32_t b)
+{
+    const int32_t  hi = __mulhi(a, b);
+    const uint32_t lo = (uint32_t)a * (uint32_t)b;
+    const int32_t  r  = (int32_t)(((uint32_t)hi << 1) | (lo >> 31));
+    return (a == INT32_MIN && b == INT32_MIN) ? INT32_MAX : r;
+}
+
+// (x + 2^(e-1)) >> e without intermediate overflow
+__device__ __forceinline__ int32_t rounding_shift_right(int32_t x, int32_t e)
+{
+    if (e <= 0)
+        return x;
+    if (e >= 32)
+        return 0;
+    return (x >> e) + ((x >> (e - 1)) & 1);
+}
+
+__device__ __forceinline__ int32_t requant_fixedpoint(int32_t v, int32_t mult, int32_t shift, int32_t result_offset)
+{
+    int32_t r;
+    if (shift < 0)
+    {
+        const int32_t pre = (-shift >= 32) ? 0 : (int32_t)((uint32_t)v << (-shift));
+        r                 = sqdmulh(pre, mult);
+    }
+    else
+    {
+        r = rounding_shift_right(sqdmulh(v, mult), shift);
+    }
+    return (int32_t)((uint32_t)r + (uint32_t)result_offset);
+}
+
+__device__ __forceinline__ int32_t clamp_i32(int32_t v, int32_t lo, int32_t hi)
+{
+    return min(max(v, lo), hi);
+}
+
+// One element of the FIXEDPOINT epilogue: acc (raw dot product) -> 8-bit value as int32
+__device__ __forceinline__ int32_t epi_fixedpoint(int32_t acc, int32_t colv, int32_t rowv, int32_t mult, int32_t shift,
+                                                  const EpiParams &p)
+{
+    const int32_t v = (int32_t)((uint32_t)acc + (uint32_t)colv + (uint32_t)rowv);
+    return clamp_i32(requant_fixedpoint(v, mult, shift, p.result_offset), p.lo, p.hi);
+}
+
+// float(acc)*scale (+bias) then + float(offset terms)*scale, two separate roundings and no fused multiply-add, in the
+// order of src/core/NEON/kernels/arm_gemm/quantized.cpp:1000-1012 followed by
+// src/cpu/kernels/gemmlowp/generic/neon/fp32.cpp:31-54
+__device__ __forceinline__ float epi_f32(int32_t acc, int32_t off, float bias, bool has_bias, const EpiParams &p)
+{
+#pragma clang fp contract(off) // the multiply and the add must round separately, as the two NEON instructions do
+    float r = (float)acc * p.scale;
+    if (has_bias)
+        r = r + bias;
+    if (p.has_offsets)
+    {
+        const float scaled = (float)off * p.scale;
+        r                  = r + scaled;
+    }
+    return fminf(fmaxf(r, p.act_min), p.act_max);
+}
+} // namespace mi355

@@ -1,0 +1,103 @@
+// Declarations shared between the C-ABI layer (capi.hip) and the kernel translation units.
+#pragma once
+#include "epilogue.hpp"
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355
+{
+// Padding of the packed B matrix Bp[Np][Kp] (int8, K contiguous, zero filled beyond N and K)
+constexpr int PACK_N_ALIGN = 256;
+constexpr int PACK_K_ALIGN = 128;
+
+inline int round_up(int v, int a)
+{
+    return (v + a - 1) / a * a;
+}
+
+// Geometry of the on-the-fly im2col A loader (implicit GEMM). row m = (n, oy, ox), k = (ky, kx, c).
+struct ConvGeom
+{
+    int32_t H, W, C, KH, KW, OH, OW;
+    int32_t stride_x, stride_y, pad_left, pad_top, dil_x, dil_y;
+    uint32_t pad_word; // the padding byte (already sign-flipped if the loader flips) replicated into 4 bytes
+};
+
+struct GemmArgs
+{
+    const int8_t *A;  // dense: [batch][M][lda] ; conv: NHWC source
+    const int8_t *Bp; // [batch?][Np][Kp]
+    void         *D;
+    int64_t       lda, a_batch_stride;
+    int64_t       Kp, bp_batch_stride;
+    int64_t       ldd, d_batch_stride;
+    int32_t       M, N, K; // K: valid depth of A (bytes readable per row)
+    int32_t       tiles_m, tiles_n;
+    EpiParams     epi;
+    ConvGeom      conv;
+};
+
+struct MfmaConfig
+{
+    const char *name;
+    int         BM, BN, BK;
+};
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes of an A row of which only the first `rem` (0 < rem < 16) exist; p is 4-byte aligned. Bytes past the
+// row's end read as zero (they meet the zero padding of the packed B, so their value is irrelevant, but the
+// access itself must stay inside the tensor).
+__device__ __forceinline__ v4i_t load16_partial(const int8_t *p, int rem)
+{
+    v4i_t v = {0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+    {
+        const int r = rem - 4 * t;
+        if (r >= 4)
+            v[t] = *(const int *)(p + 4 * t);
+        else if (r > 0)
+        {
+            uint32_t w = 0;
+            for (int b = 0; b < r; ++b)
+                w |= (uint32_t)(uint8_t)p[4 * t + b] << (8 * b);
+            v[t] = (int)w;
+        }
+    }
+    return v;
+}
+
+// gemm_mfma.hip
+int         mfma_num_configs();
+MfmaConfig  mfma_config(int idx);
+// epi: EPI_*, flip_a: xor 0x80 on A bytes in the loader, conv: implicit-GEMM loader. Returns hipError_t as int.
+int         mfma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
+
+// gemm_skinny.hip — M <= 16, B packed in matrix-core operand order (see pack_b_skinny)
+constexpr int SKINNY_MAX_M = 16;
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
+
+// kernels_aux.hip
+// B [K][ldb] (row-major, N contiguous) -> Bp [Np][Kp] int8 (flip: xor 0x80), colsum[Np] (sums of the packed int8 values)
+int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+                  hipStream_t s);
+// B given as [N][ldk] with K contiguous (conv weights [OFM][KH*KW*C])
+int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+                   hipStream_t s);
+// Bp [Np][Kp] -> operand order for the skinny kernel: [Np/16][Kp/64][64 lanes][16 bytes]
+int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream_t s);
+// colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j])
+int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int32_t b_off, int K, int N,
+                  int32_t *colvec, hipStream_t s);
+// A pre-pass: optional padded + flipped copy Ap[M][Kp] and/or rowvec[i] = b_off * sum_k(flip(A[i][k]))
+int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
+                     int32_t b_off, hipStream_t s);
+int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
+                        int N, const EpiParams &epi, hipStream_t s);
+int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);
+// one thread per output; A dense [M][lda] (unflipped or flipped per flip_a), Bp packed
+int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s);
+int fill_i32_launch(int32_t *p, int32_t v, int64_t n, hipStream_t s);
+} // namespace mi355

@@ -1,0 +1,412 @@
+// Bandwidth-bound helper kernels of the quantized-GEMM path: B packing + column sums (prepare time), the A pre-pass
+// (row sums / padded copy), the stand-alone output stage, explicit im2col, and a one-thread-per-output GEMM used only
+// for cross-checking the matrix-core kernels.
+#include "internal.hpp"
+
+namespace mi355
+{
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+static inline int launch_status()
+{
+    return (int)hipGetLastError();
+}
+
+// sum of the four int8 lanes of a dword
+__device__ __forceinline__ int32_t sum4_i8(int32_t w)
+{
+    return __builtin_amdgcn_sdot4(w, 0x01010101, 0, false);
+}
+
+__global__ void fill_i32_kernel(int32_t *p, int32_t v, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        p[i] = v;
+}
+int fill_i32_launch(int32_t *p, int32_t v, int64_t n, hipStream_t s)
+{
+    if (n <= 0)
+        return 0;
+    fill_i32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(p, v, n);
+    return launch_status();
+}
+
+// ---- P1: B[K][ldb] -> Bp[Np][Kp] (transpose to K-contiguous, optional sign flip, zero padding) + column sums ----------
+// Replaces pretranspose_B_array (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:594-617) / CpuGemmTranspose1xWKernel and
+// CpuGemmLowpMatrixBReductionKernel (src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:273-446) in one pass over B.
+__global__ __launch_bounds__(256) void pack_b_kernel(const uint8_t *__restrict__ B, int64_t ldb, int K, int N, int Kp,
+                                                     uint8_t flip, int8_t *__restrict__ Bp,
+                                                     int32_t *__restrict__ colsum)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile[64][64 + 16]; // [n][k]
+    const int          n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+    const int          tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk)
+    {
+        const int k = k0 + ty * 16 + kk, n = n0 + tx;
+        uint8_t   v = 0;
+        if (k < K && n < N)
+            v = B[(int64_t)k * ldb + n] ^ flip;
+        tile[tx][ty * 16 + kk] = v;
+    }
+    __syncthreads();
+    const int n = threadIdx.x >> 2, kc = (threadIdx.x & 3) * 16;
+    const v4i v = *(const v4i *)&tile[n][kc];
+    *(v4i *)(Bp + (int64_t)(n0 + n) * Kp + k0 + kc) = v;
+    int32_t s = sum4_i8(v.x) + sum4_i8(v.y) + sum4_i8(v.z) + sum4_i8(v.w);
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    if ((threadIdx.x & 3) == 0 && s != 0)
+        atomicAdd(colsum + n0 + n, s);
+}
+
+int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+                  hipStream_t s)
+{
+    if (Np % 64 || Kp % 64 || Np < N || Kp < K)
+        return (int)hipErrorInvalidValue;
+    int e = fill_i32_launch(colsum, 0, Np, s);
+    if (e)
+        return e;
+    pack_b_kernel<<<dim3(Np / 64, Kp / 64), dim3(256), 0, s>>>((const uint8_t *)B, ldb, K, N, Kp, flip ? 0x80 : 0, Bp,
+                                                               colsum);
+    return launch_status();
+}
+
+// B already K-contiguous: Bt[N][ldk] (convolution weights [OFM][KH*KW*C], the layout CpuWeightsReshapeKernel
+// produces transposed: src/cpu/kernels/CpuWeightsReshapeKernel.cpp:150-166)
+__global__ __launch_bounds__(256) void pack_bt_kernel(const uint8_t *__restrict__ Bt, int64_t ldk, int K, int N, int Kp,
+                                                      int Np, uint8_t flip, int8_t *__restrict__ Bp,
+                                                      int32_t *__restrict__ colsum)
+{
+    const int     cpr = Kp / 16;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)Np * cpr)
+        return;
+    const int n = (int)(idx / cpr), kc = (int)(idx % cpr) * 16;
+    union
+    {
+        v4i     v;
+        uint8_t b[16];
+    } u;
+    int32_t s = 0;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+    {
+        uint8_t x = 0;
+        if (n < N && kc + t < K)
+            x = Bt[(int64_t)n * ldk + kc + t] ^ flip;
+        u.b[t] = x;
+        s += (int8_t)x;
+    }
+    *(v4i *)(Bp + (int64_t)n * Kp + kc) = u.v;
+    if (s != 0)
+        atomicAdd(colsum + n, s);
+}
+
+int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+                   hipStream_t s)
+{
+    if (Kp % 16 || Np < N || Kp < K)
+        return (int)hipErrorInvalidValue;
+    int e = fill_i32_launch(colsum, 0, Np, s);
+    if (e)
+        return e;
+    const int64_t total = (int64_t)Np * (Kp / 16);
+    pack_bt_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)Bt, ldk, K, N, Kp, Np,
+                                                                               flip ? 0x80 : 0, Bp, colsum);
+    return launch_status();
+}
+
+// Bp[Np][Kp] -> Bs[Np/16][Kp/64][64][16]: 1 KiB blocks holding 16 columns x 64 k in the lane order the 16x16x64 matrix
+// instruction reads its B operand (lane l: column l%16, bytes 16*(l/16) .. +16 of the k block)
+__global__ __launch_bounds__(256) void pack_b_skinny_kernel(const int8_t *__restrict__ Bp, int Kp, int Np,
+                                                            int8_t *__restrict__ Bs)
+{
+    const int64_t idx   = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)Np * Kp / 16;
+    if (idx >= total)
+        return;
+    const int     lane = (int)(idx & 63);
+    const int64_t blk  = idx >> 6;
+    const int     KB   = Kp / 64;
+    const int     kb = (int)(blk % KB), ng = (int)(blk / KB);
+    const int     col = lane & 15, kc = lane >> 4;
+    *(v4i *)(Bs + idx * 16) = *(const v4i *)(Bp + (int64_t)(ng * 16 + col) * Kp + kb * 64 + kc * 16);
+}
+
+int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream_t s)
+{
+    if (Kp % 64 || Np % 16)
+        return (int)hipErrorInvalidValue;
+    const int64_t total = (int64_t)Np * Kp / 16;
+    pack_b_skinny_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>(Bp, Kp, Np, Bs);
+    return launch_status();
+}
+
+// colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j]); the per-column part of the offset contribution, folded with the
+// bias like arm_gemm's col_bias (src/core/NEON/kernels/arm_gemm/quantized.cpp:963-968)
+__global__ void colvec_kernel(const int32_t *__restrict__ colsum, const int32_t *__restrict__ bias, uint32_t a_off,
+                              uint32_t b_off, uint32_t K, int N, int32_t *__restrict__ colvec)
+{
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= N)
+        return;
+    uint32_t v = a_off * (uint32_t)colsum[j] + a_off * b_off * K;
+    if (bias)
+        v += (uint32_t)bias[j];
+    colvec[j] = (int32_t)v;
+}
+
+int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int32_t b_off, int K, int N,
+                  int32_t *colvec, hipStream_t s)
+{
+    colvec_kernel<<<dim3((N + 255) / 256), dim3(256), 0, s>>>(colsum, bias, (uint32_t)a_off, (uint32_t)b_off,
+                                                              (uint32_t)K, N, colvec);
+    return launch_status();
+}
+
+// ---- A pre-pass -----------------------------------------------------------------------------------------------------
+// One block per row. Optionally writes the row sign-flipped and zero-padded to Kp (for A whose rows are not 16-byte
+// aligned), optionally reduces it: rowvec[i] = b_off * sum_k flip(A[i][k])
+// (CpuGemmLowpMatrixAReductionKernel, src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:133-204).
+template <int VEC>
+__global__ __launch_bounds__(256) void a_prepass_kernel(const uint8_t *__restrict__ A, int64_t lda, int K, uint8_t flip,
+                                                        int8_t *__restrict__ Ap, int Kp, int32_t *__restrict__ rowvec,
+                                                        uint32_t b_off)
+{
+    const int      row  = blockIdx.x;
+    const uint8_t *src  = A + (int64_t)row * lda;
+    const int      kmax = Ap ? Kp : K;
+    int32_t        s    = 0;
+    for (int k = threadIdx.x * VEC; k < kmax; k += 256 * VEC)
+    {
+        union
+        {
+            uint8_t  b[VEC];
+            uint32_t w[VEC >= 4 ? VEC / 4 : 1];
+        } u;
+        if (k < K)
+        {
+            if (VEC == 1)
+                u.b[0] = src[k] ^ flip;
+            else
+            {
+#pragma unroll
+                for (int t = 0; t < VEC / 4; ++t)
+                    u.w[t] = *(const uint32_t *)(src + k + 4 * t) ^ (flip * 0x01010101u);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int t = 0; t < (VEC >= 4 ? VEC / 4 : 1); ++t)
+                u.w[t] = 0;
+            if (VEC == 1)
+                u.b[0] = 0;
+        }
+        if (VEC == 1)
+            s += (int8_t)u.b[0];
+        else
+        {
+#pragma unroll
+            for (int t = 0; t < VEC / 4; ++t)
+                s += sum4_i8((int32_t)u.w[t]);
+        }
+        if (Ap)
+        {
+            if (VEC == 1)
+                Ap[(int64_t)row * Kp + k] = (int8_t)u.b[0];
+            else
+            {
+#pragma unroll
+                for (int t = 0; t < VEC / 4; ++t)
+                    *(uint32_t *)(Ap + (int64_t)row * Kp + k + 4 * t) = u.w[t];
+            }
+        }
+    }
+    if (rowvec)
+    {
+        __shared__ int32_t part[4];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            s += __shfl_xor(s, o);
+        if ((threadIdx.x & 63) == 0)
+            part[threadIdx.x >> 6] = s;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            rowvec[row] = (int32_t)(b_off * (uint32_t)(part[0] + part[1] + part[2] + part[3]));
+    }
+}
+
+int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
+                     int32_t b_off, hipStream_t s)
+{
+    if (M <= 0)
+        return 0;
+    const uintptr_t mix  = (uintptr_t)A | (uintptr_t)lda | (uintptr_t)K;
+    const uint8_t   f    = flip ? 0x80 : 0;
+    const dim3      grid(M), block(256);
+    if ((mix & 15) == 0)
+        a_prepass_kernel<16><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+    else if ((mix & 7) == 0)
+        a_prepass_kernel<8><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+    else if ((mix & 3) == 0)
+        a_prepass_kernel<4><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+    else
+        a_prepass_kernel<1><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+    return launch_status();
+}
+
+// ---- K2: stand-alone output stage --------------------------------------------------------------------------------------
+// CpuGemmLowpQuantizeDownInt32To{Int8,Uint8}ScaleByFixedPointKernel
+// (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt8ScaleByFixedPointKernel.cpp:79-181): 4 B read + 1 B written per element
+template <bool VEC4>
+__global__ __launch_bounds__(256) void output_stage_kernel(const int32_t *__restrict__ src, int64_t ld_src,
+                                                           const int32_t *__restrict__ bias, int8_t *__restrict__ dst,
+                                                           int64_t ld_dst, int M, int N, EpiParams p)
+{
+    const int     per_row = VEC4 ? N / 4 : N;
+    const int64_t idx     = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)M * per_row)
+        return;
+    const int i = (int)(idx / per_row), q = (int)(idx % per_row);
+    if (VEC4)
+    {
+        const int j = q * 4;
+        v4i       v = *(const v4i *)(src + (int64_t)i * ld_src + j);
+        v4i       b = {0, 0, 0, 0};
+        if (bias)
+            b = *(const v4i *)(bias + j);
+        uint32_t out = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+        {
+            const int32_t mu = p.mult ? p.mult[j + t] : p.mult_s;
+            const int32_t sh = p.shift ? p.shift[j + t] : p.shift_s;
+            out |= ((uint32_t)epi_fixedpoint(v[t], b[t], 0, mu, sh, p) & 0xFFu) << (8 * t);
+        }
+        *(uint32_t *)(dst + (int64_t)i * ld_dst + j) = out;
+    }
+    else
+    {
+        const int32_t mu = p.mult ? p.mult[q] : p.mult_s;
+        const int32_t sh = p.shift ? p.shift[q] : p.shift_s;
+        dst[(int64_t)i * ld_dst + q] =
+            (int8_t)epi_fixedpoint(src[(int64_t)i * ld_src + q], bias ? bias[q] : 0, 0, mu, sh, p);
+    }
+}
+
+int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
+                        int N, const EpiParams &epi, hipStream_t s)
+{
+    if (M <= 0 || N <= 0)
+        return 0;
+    const bool vec = (N % 4 == 0) && (ld_src % 4 == 0) && (ld_dst % 4 == 0) && (((uintptr_t)src & 15) == 0) &&
+                     (((uintptr_t)dst & 3) == 0) && (bias == nullptr || ((uintptr_t)bias & 15) == 0);
+    const int64_t total = (int64_t)M * (vec ? N / 4 : N);
+    const dim3    grid((unsigned)((total + 255) / 256)), block(256);
+    if (vec)
+        output_stage_kernel<true><<<grid, block, 0, s>>>(src, ld_src, bias, (int8_t *)dst, ld_dst, M, N, epi);
+    else
+        output_stage_kernel<false><<<grid, block, 0, s>>>(src, ld_src, bias, (int8_t *)dst, ld_dst, M, N, epi);
+    return launch_status();
+}
+
+// ---- explicit im2col (NHWC) ----------------------------------------------------------------------------------------------
+// CpuIm2ColKernel / linearize_volume_nhwc (src/cpu/kernels/directconv2d/impl.h:148-220,307-389). Used when the implicit
+// loader does not apply (channel count not a multiple of 16, asymmetric weights) and exported on its own.
+template <int VEC>
+__global__ __launch_bounds__(256) void im2col_nhwc_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                          int64_t rows, ConvGeom g, int64_t ld_dst)
+{
+    const int     K    = g.KH * g.KW * g.C;
+    const int     upr  = K / VEC; // units per row
+    const int64_t idx  = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * upr)
+        return;
+    const int64_t m = idx / upr;
+    const int     k = (int)(idx % upr) * VEC;
+    const int     tap = k / g.C, c0 = k - tap * g.C;
+    const int     ky = tap / g.KW, kx = tap - ky * g.KW;
+    const int     ox = (int)(m % g.OW);
+    const int64_t t  = m / g.OW;
+    const int     oy = (int)(t % g.OH);
+    const int64_t n  = t / g.OH;
+    const int     iy = oy * g.stride_y - g.pad_top + ky * g.dil_y;
+    const int     ix = ox * g.stride_x - g.pad_left + kx * g.dil_x;
+    const bool    in = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+    const uint8_t *s = src + ((n * g.H + iy) * g.W + ix) * g.C + c0;
+    uint8_t       *d = dst + m * ld_dst + k;
+    if (VEC == 16)
+    {
+        const int pw = (int)g.pad_word;
+        v4i       v  = {pw, pw, pw, pw};
+        if (in)
+            v = *(const v4i *)s;
+        *(v4i *)d = v;
+    }
+    else
+        *d = in ? *s : (uint8_t)(g.pad_word & 0xFF);
+}
+
+int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s)
+{
+    const int64_t rows = (int64_t)batch * g.OH * g.OW;
+    const int     K    = g.KH * g.KW * g.C;
+    if (rows <= 0 || K <= 0)
+        return 0;
+    const bool vec = (g.C % 16 == 0) && (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 15) == 0) &&
+                     (ld_dst % 16 == 0);
+    const int64_t total = rows * (vec ? K / 16 : K);
+    const dim3    grid((unsigned)((total + 255) / 256)), block(256);
+    if (vec)
+        im2col_nhwc_kernel<16><<<grid, block, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, rows, g, ld_dst);
+    else
+        im2col_nhwc_kernel<1><<<grid, block, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, rows, g, ld_dst);
+    return launch_status();
+}
+
+// ---- one thread per output: the plainest possible statement of the path, for cross-checking only ----------------------
+template <int EPI>
+__global__ __launch_bounds__(256) void simple_gemm_kernel(GemmArgs g, uint8_t flip)
+{
+    const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int bz = blockIdx.z;
+    if (i >= g.M || j >= g.N)
+        return;
+    const uint8_t *a = (const uint8_t *)g.A + (int64_t)bz * g.a_batch_stride + (int64_t)i * g.lda;
+    const int8_t  *b = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)j * g.Kp;
+    int32_t        acc = 0;
+    for (int k = 0; k < g.K; ++k)
+        acc += (int32_t)(int8_t)(a[k] ^ flip) * (int32_t)b[k];
+    const EpiParams &p   = g.epi;
+    const int32_t    cv  = p.colvec[(int64_t)bz * p.colvec_batch_stride + j];
+    const int32_t    rv  = p.rowvec ? p.rowvec[(int64_t)bz * p.rowvec_batch_stride + i] : 0;
+    const int64_t    idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j;
+    if (EPI == EPI_S32)
+        ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc + (uint32_t)cv + (uint32_t)rv);
+    else if (EPI == EPI_FIXEDPOINT)
+        ((int8_t *)g.D)[idx] =
+            (int8_t)epi_fixedpoint(acc, cv, rv, p.mult ? p.mult[j] : p.mult_s, p.shift ? p.shift[j] : p.shift_s, p);
+    else
+        ((float *)g.D)[idx] = epi_f32(acc, (int32_t)((uint32_t)cv + (uint32_t)rv), p.bias_f32 ? p.bias_f32[j] : 0.f,
+                                      p.bias_f32 != nullptr, p);
+}
+
+int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s)
+{
+    const dim3    grid((args.N + 15) / 16, (args.M + 15) / 16, batch), block(256);
+    const uint8_t f = flip_a ? 0x80 : 0;
+    if (epi == EPI_S32)
+        simple_gemm_kernel<EPI_S32><<<grid, block, 0, s>>>(args, f);
+    else if (epi == EPI_FIXEDPOINT)
+        simple_gemm_kernel<EPI_FIXEDPOINT><<<grid, block, 0, s>>>(args, f);
+    else
+        simple_gemm_kernel<EPI_F32><<<grid, block, 0, s>>>(args, f);
+    return launch_status();
+}
+} // namespace mi355

@@ -1,0 +1,180 @@
+/*
+ * mi355_gemmlowp.h — C ABI of the MI355X (gfx950) quantized-GEMM path.
+ *
+ * This is the only boundary below which HIP is used. The C++ host layer that mirrors the
+ * arm_compute function classes (NEGEMMLowpMatrixMultiplyCore, NEGEMMLowpOutputStage,
+ * NEGEMMConvolutionLayer) calls these entry points; so can any other language through its FFI.
+ *
+ * The lifecycle follows the object the reference's operators drive for this path,
+ * arm_gemm::GemmCommon (src/cpu/kernels/assembly/arm_gemm/gemm_common.hpp:56-302):
+ *   configure -> pretranspose_B_array / set_quantized_bias -> set_arrays -> execute
+ * becomes
+ *   mi355_gemmlowp_create -> mi355_gemmlowp_prepare -> mi355_gemmlowp_run.
+ *
+ * Conventions
+ *  - Matrices are row-major. A is M x K, B is K x N, D is M x N ("ld*" = row stride in elements,
+ *    "*_batch_stride" = distance between consecutive matrices in elements; b_batch_stride 0
+ *    shares one B between all batches).
+ *  - a_offset / b_offset are ADDED to every element before the product, exactly as
+ *    NEGEMMLowpMatrixMultiplyCore treats QuantizationInfo::offset
+ *    (arm_compute/runtime/NEON/functions/NEGEMMLowpMatrixMultiplyCore.h:95-97).
+ *  - Every data pointer may be a host pointer or a device pointer; the library finds out with
+ *    hipPointerGetAttributes. Host buffers are staged through device memory owned by the
+ *    handle (synchronous, like the reference's run()); device buffers are used in place and
+ *    the call only enqueues work on `stream` (a hipStream_t passed as void*, NULL = default
+ *    stream).
+ *  - All functions return 0 on success, non-zero on failure; mi355_last_error() then returns
+ *    a thread-local message. No exception crosses this boundary.
+ *  - A handle is single-caller: one call at a time per handle. Distinct handles may be used
+ *    from distinct threads / streams.
+ */
+#ifndef MI355_GEMMLOWP_H
+#define MI355_GEMMLOWP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mi355_dtype
+{
+    MI355_U8  = 0, /* QASYMM8 */
+    MI355_S8  = 1, /* QASYMM8_SIGNED, QSYMM8, QSYMM8_PER_CHANNEL */
+    MI355_S32 = 2,
+    MI355_F32 = 3
+} mi355_dtype;
+
+/* What happens to the int32 accumulators. Replaces the choice the reference makes between
+ * CpuGemmLowpOffsetContributionKernel (S32 / F32) and
+ * CpuGemmLowpOffsetContributionOutputStageKernel (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:281-321). */
+typedef enum mi355_epilogue
+{
+    MI355_EPI_S32        = 0, /* dst = acc + offset contribution                       (int32) */
+    MI355_EPI_FIXEDPOINT = 1, /* + bias, QUANTIZE_DOWN_FIXEDPOINT, clamp               (uint8 / int8) */
+    MI355_EPI_F32        = 2  /* float(acc)*scale (+ f32 bias) + float(offsets)*scale, activation clamp (float) */
+} mi355_epilogue;
+
+typedef enum mi355_path
+{
+    MI355_PATH_AUTO   = 0, /* MFMA tiled kernel, or the skinny kernel when M <= 16 */
+    MI355_PATH_SIMPLE = 1, /* one thread per output; for cross-checking only */
+    MI355_PATH_MFMA   = 2,
+    MI355_PATH_SKINNY = 3
+} mi355_path;
+
+/* Mirrors the fields of GEMMLowpOutputStageInfo the FIXEDPOINT stage reads
+ * (arm_compute/function_info/GEMMInfo.h:49-82). With per_channel != 0 the per-column
+ * multiplier / shift arrays are passed to mi355_gemmlowp_prepare instead. */
+typedef struct mi355_requant
+{
+    int32_t per_channel;
+    int32_t multiplier;
+    int32_t shift; /* > 0: rounding right shift after the multiply; < 0: left shift before it */
+    int32_t result_offset;
+    int32_t min_bound;
+    int32_t max_bound;
+} mi355_requant;
+
+typedef struct mi355_gemm_desc
+{
+    int32_t       M, N, K, batch;
+    int32_t       a_dtype, b_dtype, dst_dtype; /* mi355_dtype */
+    int32_t       epilogue;                    /* mi355_epilogue */
+    int64_t       lda, ldb, ldd;
+    int64_t       a_batch_stride, b_batch_stride, d_batch_stride;
+    int32_t       a_offset, b_offset;
+    mi355_requant requant;          /* MI355_EPI_FIXEDPOINT only */
+    float         scale;            /* MI355_EPI_F32 only: a.scale * b.scale */
+    float         act_min, act_max; /* MI355_EPI_F32 only: activation clamp, +-INFINITY for none */
+    int32_t       path;             /* mi355_path */
+    int32_t       reserved;
+} mi355_gemm_desc;
+
+typedef struct mi355_gemm_handle mi355_gemm_handle;
+
+/* Replaces CpuGemmLowpMatrixMultiplyCore::configure (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:116-360):
+ * checks the descriptor, picks the kernel, sizes the device workspace. Allocates nothing on the device yet. */
+int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out);
+
+/* Replaces CpuGemmLowpMatrixMultiplyCore::prepare (:813-846) = pretranspose_B_array + column sums of B
+ * (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:594-617, src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:273-446)
+ * + set_quantized_bias (:963-968 of src/core/NEON/kernels/arm_gemm/quantized.cpp): re-lays B out for the
+ * matrix cores, reduces its columns, and folds a_offset*colsum + a_offset*b_offset*K + bias into one per-column
+ * int32 vector. bias (N int32) may be NULL; mult / shift (N int32 each) are read only when requant.per_channel.
+ * Call again whenever B, bias or the per-channel vectors change (a non-constant B: before every run). */
+int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *bias, const int32_t *mult,
+                           const int32_t *shift, void *stream);
+
+/* Replaces CpuGemmLowpMatrixMultiplyCore::update_quantization_parameters (:852-876): new offsets, per-tensor
+ * requantisation and dequantisation scale without re-packing B. */
+int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t b_offset,
+                                const mi355_requant *requant, float scale, void *stream);
+
+/* Replaces CpuGemmLowpMatrixMultiplyCore::run (:647-811). bias_f32 (N floats, MI355_EPI_F32 only) may be NULL. */
+int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
+
+void mi355_gemmlowp_destroy(mi355_gemm_handle *h);
+
+/* Name of the kernel variant the handle dispatches to, e.g. "mfma_256x128x64" (static string). */
+const char *mi355_gemmlowp_kernel_name(const mi355_gemm_handle *h);
+
+/* Stand-alone output stage on an int32 matrix. Replaces CpuGemmLowpOutputStage::run ->
+ * CpuGemmLowpQuantizeDownInt32To{Int8,Uint8}ScaleByFixedPointKernel
+ * (src/cpu/operators/CpuGemmLowpOutputStage.cpp:163-167,
+ *  src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt8ScaleByFixedPointKernel.cpp:79-181). Stateless. */
+typedef struct mi355_output_stage_desc
+{
+    int32_t       M, N;
+    int64_t       ld_src, ld_dst;
+    int32_t       dst_dtype; /* MI355_U8 or MI355_S8 */
+    mi355_requant requant;   /* per-tensor */
+} mi355_output_stage_desc;
+
+int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *src, const int32_t *bias, void *dst,
+                           void *stream);
+
+/* Quantized NHWC convolution lowered to GEMM. Replaces CpuGemmConv2d::{configure,prepare,run}
+ * (src/cpu/operators/CpuGemmConv2d.cpp:461-651, :1011-1101, :923-1008): CpuIm2ColKernel + CpuWeightsReshapeKernel
+ * + CpuGemmLowpMatrixMultiplyCore. src is [batch][H][W][C], weights [OFM][KH][KW][C], dst [batch][OH][OW][OFM].
+ * src_offset / weights_offset are the ADDED offsets (the negated zero points, as configure_mm passes them,
+ * :266-280); pad_value is the byte im2col writes for out-of-image taps (the src zero point,
+ * src/cpu/kernels/directconv2d/impl.h:333-334). */
+typedef struct mi355_conv_desc
+{
+    int32_t       batch, H, W, C, OFM, KH, KW;
+    int32_t       stride_x, stride_y, pad_left, pad_top, pad_right, pad_bottom, dilation_x, dilation_y;
+    int32_t       src_dtype, weights_dtype, dst_dtype; /* mi355_dtype (8-bit) */
+    int32_t       src_offset, weights_offset;
+    int32_t       pad_value;
+    mi355_requant requant;
+    int32_t       path; /* 0 auto (implicit GEMM where the shape allows), 1 force explicit im2col + GEMM */
+    int32_t       reserved;
+} mi355_conv_desc;
+
+typedef struct mi355_conv_handle mi355_conv_handle;
+
+int  mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out);
+int  mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t *bias, const int32_t *mult,
+                        const int32_t *shift, void *stream);
+int  mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream);
+void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW);
+void mi355_conv_destroy(mi355_conv_handle *h);
+const char *mi355_conv_kernel_name(const mi355_conv_handle *h);
+
+/* The im2col kernel on its own. Replaces CpuIm2ColKernel::run_op for NHWC
+ * (src/cpu/kernels/CpuIm2ColKernel.cpp:408-420 -> src/cpu/kernels/directconv2d/impl.h:307-389).
+ * dst is [batch*OH*OW][KH*KW*C], K ordered (ky, kx, c). */
+int mi355_im2col_nhwc_run(const mi355_conv_desc *desc, const void *src, void *dst, void *stream);
+
+/* Thread-local text of the last error on this thread ("" if none). */
+const char *mi355_last_error(void);
+
+/* Library / device identification: fills name with the HIP device's gcnArchName; returns its CU count or -1. */
+int mi355_device_info(char *name, size_t name_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_GEMMLOWP_H */

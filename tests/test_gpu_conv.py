@@ -1,0 +1,102 @@
+"""GPU parity of the convolution lowering (implicit GEMM and explicit im2col + GEMM) and the im2col kernel."""
+import numpy as np
+import pytest
+
+import oracle
+from computelibrary_amd import capi
+from gpu_util import announce, to_dev
+
+pytestmark = pytest.mark.gpu
+CODE = {np.dtype(np.uint8): capi.U8, np.dtype(np.int8): capi.S8}
+
+
+def run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dilation=(1, 1), path=0,
+             device=True):
+    B_, H, W, C = src.shape
+    OFM, KH, KW, _ = w.shape
+    pc = len(np.atleast_1d(mult)) > 1
+    rq = capi.requant(0 if pc else int(np.atleast_1d(mult)[0]), 0 if pc else int(np.atleast_1d(shift)[0]), out_zp, lo,
+                      hi, pc)
+    d = capi.conv_desc(B_, H, W, C, OFM, KH, KW, stride, pad, dilation, CODE[src.dtype], CODE[w.dtype],
+                       CODE[src.dtype], -in_zp, -w_zp, in_zp, rq, path)
+    cv = capi.Conv(d)
+    OH, OW = cv.out_dims()
+    m = np.ascontiguousarray(mult, dtype=np.int32) if pc else None
+    s = np.ascontiguousarray(shift, dtype=np.int32) if pc else None
+    b = np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.zeros((B_, OH, OW, OFM), dtype=src.dtype)
+    if device:
+        import torch
+        sd, wd, od = to_dev(src), to_dev(w), to_dev(out)
+        keep = [to_dev(b), to_dev(m), to_dev(s)]
+        cv.prepare(wd, *keep)
+        cv.run(sd, od)
+        torch.cuda.synchronize()
+        out = od.cpu().numpy()
+    else:
+        cv.prepare(np.ascontiguousarray(w), b, m, s)
+        cv.run(np.ascontiguousarray(src), out)
+    name = cv.kernel_name
+    cv.close()
+    return out, name
+
+
+def test_im2col_fixture(golden):
+    g = golden("im2col_nhwc.npz")
+    for n in range(int(g["count"])):
+        KH, KW, sx, sy, pl, pt, pr, pb, zp = (int(x) for x in g["p%d" % n])
+        src, want = g["src%d" % n], g["dst%d" % n]
+        B_, H, W, C = src.shape
+        d = capi.conv_desc(B_, H, W, C, 1, KH, KW, (sx, sy), (pl, pt, pr, pb), pad_value=zp)
+        for device in (False, True):
+            announce("im2col fixture", n, src.shape, "device", device)
+            if device:
+                out = to_dev(np.zeros_like(want))
+                capi.im2col_nhwc(d, to_dev(src), out)
+                got = out.cpu().numpy()
+            else:
+                got = np.zeros_like(want)
+                capi.im2col_nhwc(d, np.ascontiguousarray(src), got)
+            np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_conv_fixture(golden, path):
+    g = golden("conv_nhwc.npz")
+    names = set()
+    for n in range(int(g["count"])):
+        sx, sy, pl, pt, pr, pb, in_zp, w_zp, out_zp, pc = (int(x) for x in g["p%d" % n])
+        src, w, bias, want = g["src%d" % n], g["w%d" % n], g["bias%d" % n], g["dst%d" % n]
+        in_scale, out_scale = g["scales%d" % n]
+        mult, shift = oracle.calculate_quantized_multipliers(in_scale, g["wscale%d" % n], out_scale)
+        lo, hi = (-128, 127) if src.dtype == np.int8 else (0, 255)
+        for device in (True, False):
+            announce("conv fixture", n, src.shape, w.shape, "path", path, "device", device)
+            got, name = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, (sx, sy), (pl, pt, pr, pb),
+                                 path=path, device=device)
+            names.add(name.split("_")[0].split("+")[0])
+            np.testing.assert_array_equal(got, want)
+    if path == 0:
+        assert "implicit" in names  # the 64-channel cases really took the on-the-fly loader
+
+
+def test_conv_seeded_strides_dilation_uint8():
+    rng = np.random.default_rng(51)
+    for (shape, wshape, stride, pad, dil, dt) in [
+            ((2, 13, 11, 32), (24, 3, 3, 32), (2, 1), (1, 1, 1, 1), (1, 1), np.uint8),
+            ((1, 12, 12, 16), (40, 3, 3, 16), (1, 1), (2, 2, 2, 2), (2, 2), np.int8),
+            ((3, 9, 7, 48), (64, 1, 1, 48), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),
+            ((1, 10, 10, 6), (7, 3, 3, 6), (1, 1), (1, 1, 1, 1), (1, 1), np.int8)]:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(-127, 128, size=wshape).astype(np.int8)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multipliers(0.02, rng.uniform(0.01, 1, wshape[0]), 1.1)
+        zp = 5 if dt == np.int8 else 131
+        lo, hi = (-128, 127) if dt == np.int8 else (0, 255)
+        want = oracle.conv_nhwc_direct(src, w, bias, zp, 0, mult, shift, -5 if dt == np.int8 else 9, lo, hi, stride,
+                                       pad, dil)
+        for path in (0, 1):
+            announce("conv seeded", shape, wshape, stride, pad, dil, "path", path)
+            got, _ = run_conv(src, w, bias, zp, 0, mult, shift, -5 if dt == np.int8 else 9, lo, hi, stride, pad, dil,
+                              path=path)
+            np.testing.assert_array_equal(got, want)

@@ -1,0 +1,196 @@
+"""GPU parity: the HIP path through the C ABI against the golden fixtures (outputs of the reference's own
+portable code) and against the CPU oracle on seeded inputs. Integer outputs must be bit-exact."""
+import numpy as np
+import pytest
+
+import oracle
+from computelibrary_amd import capi
+from gpu_util import announce, run_gemm
+
+pytestmark = pytest.mark.gpu
+
+PATHS = [capi.PATH_SIMPLE, capi.PATH_MFMA, capi.PATH_SKINNY]
+
+
+def paths_for(M, batch=1):
+    return [p for p in PATHS if p != capi.PATH_SKINNY or (M <= 16 and batch == 1)]
+
+
+def test_device_is_gfx950():
+    name, cus = capi.device_info()
+    assert name.startswith("gfx950"), name
+    assert cus >= 200
+
+
+@pytest.mark.parametrize("device", [False, True])
+def test_s32_fixture(golden, device):
+    g = golden("gemmlowp_s32.npz")
+    for n in range(int(g["count"])):
+        A, B = g["a%d" % n], g["b%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        for path in paths_for(A.shape[0]):
+            announce("s32 fixture", n, A.shape, B.shape, A.dtype, B.dtype, ao, bo, "path", path, "device", device)
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=path, device=device)
+            np.testing.assert_array_equal(got, g["dst%d" % n])
+
+
+def test_s32_batched_fixture(golden):
+    g = golden("gemmlowp_batched.npz")
+    for n in range(int(g["count"])):
+        A, B = g["a%d" % n], g["b%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        for path in (capi.PATH_SIMPLE, capi.PATH_MFMA):
+            announce("batched fixture", n, A.shape, B.shape, "path", path)
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=path, device=True)
+            np.testing.assert_array_equal(got, g["dst%d" % n])
+
+
+@pytest.mark.parametrize("device", [False, True])
+def test_fused_fixedpoint_fixture(golden, device):
+    g = golden("gemmlowp_fused_fixedpoint.npz")
+    for n in range(int(g["count"])):
+        ao, bo, roff, lo, hi, pc = (int(x) for x in g["p%d" % n])
+        A, B, dst = g["a%d" % n], g["b%d" % n], g["dst%d" % n]
+        for path in paths_for(A.shape[0]):
+            announce("fused fixture", n, A.shape, B.shape, dst.dtype, "pc", pc, "path", path, "device", device)
+            got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, dst.dtype, ao, bo, g["bias%d" % n], g["mult%d" % n],
+                              g["shift%d" % n], roff, lo, hi, path=path, device=device)
+            np.testing.assert_array_equal(got, dst)
+
+
+def test_f32_fixture(golden):
+    g = golden("gemmlowp_f32.npz")
+    scale = float(g["scale"])
+    for n in range(int(g["count"])):
+        A, B = g["a%d" % n], g["b%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        want_ref = g["dst%d" % n]
+        want_orc = oracle.gemmlowp_f32(A, B, None, ao, bo, scale)
+        for path in paths_for(A.shape[0]):
+            announce("f32 fixture", n, A.shape, B.shape, ao, bo, "path", path)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=scale, path=path, device=True)
+            # same float operations in the same order as the oracle: identical bits
+            np.testing.assert_array_equal(got, want_orc)
+            # and within the stated 1e-5 relative error of the reference's own test oracle
+            tol = 1e-5 * np.maximum(np.abs(want_ref), np.abs(A.astype(np.float64) @ B.astype(np.float64)) * scale)
+            assert (np.abs(got - want_ref) <= tol + 1e-30).all()
+
+
+@pytest.mark.parametrize("a_dt,b_dt", [(np.uint8, np.uint8), (np.int8, np.int8), (np.uint8, np.int8),
+                                        (np.int8, np.uint8)])
+def test_seeded_against_oracle_all_sign_combinations(a_dt, b_dt):
+    rng = np.random.default_rng(41)
+    for (M, N, K) in [(300, 200, 520), (129, 257, 1000), (64, 64, 64), (5, 1000, 333)]:
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(np.iinfo(b_dt).min, np.iinfo(b_dt).max + 1, size=(K, N)).astype(b_dt)
+        ao, bo = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+        want = oracle.gemmlowp_s32(A, B, ao, bo)
+        bias = rng.integers(-5000, 5000, size=N, dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multiplier(float(rng.uniform(0.0005, 0.01)))
+        want_q = oracle.gemmlowp_fixedpoint(A, B, bias, ao, bo, [mult], [shift], 3, 0, 255, np.uint8)
+        for path in paths_for(M):
+            announce("seeded", a_dt.__name__, b_dt.__name__, (M, N, K), ao, bo, "path", path)
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=path, device=True)
+            np.testing.assert_array_equal(got, want)
+            got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.uint8, ao, bo, bias, [mult], [shift], 3, 0, 255,
+                              path=path, device=True)
+            np.testing.assert_array_equal(got, want_q)
+
+
+@pytest.mark.parametrize("K,lda", [(1000, 1000), (1001, 1001), (998, 1000), (64, 80), (17, 17), (1, 1)])
+def test_row_strides_and_k_tails(K, lda):
+    """A rows that are not 16-byte aligned (dword-aligned: direct loads with a guarded tail; otherwise the padded
+    copy), x-padding on A and on the destination (tests/validation/fixtures/GEMMLowpFixture.h:302)."""
+    rng = np.random.default_rng(42)
+    M, N = 70, 90
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    want = oracle.gemmlowp_s32(A, B, 7, -3)
+    for path in (capi.PATH_MFMA, capi.PATH_SIMPLE):
+        for device in (True, False):
+            announce("strides", K, lda, "path", path, "device", device)
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, 7, -3, path=path, device=device, lda=lda, ldd=N + 5)
+            np.testing.assert_array_equal(got, want)
+    announce("strides skinny", K, lda)
+    got, _ = run_gemm(A[:9], B, capi.EPI_S32, np.int32, 7, -3, path=capi.PATH_SKINNY, device=True, lda=lda)
+    np.testing.assert_array_equal(got, want[:9])
+
+
+def test_per_channel_left_and_right_shifts():
+    rng = np.random.default_rng(43)
+    M, N, K = 150, 130, 200
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    bias = rng.integers(-2000, 2000, size=N, dtype=np.int32)
+    reals = np.exp(rng.uniform(np.log(1e-4), np.log(3.0), size=N))
+    mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+    assert (shift < 0).any() and (shift > 0).any()
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -3, 0, mult, shift, -5, -128, 127, np.int8)
+    for path in (capi.PATH_MFMA, capi.PATH_SIMPLE):
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, -3, 0, bias, mult, shift, -5, -128, 127, path=path,
+                          device=True)
+        np.testing.assert_array_equal(got, want)
+
+
+def test_requant_extremes_on_device():
+    """Accumulators and multipliers at the edges of int32 (saturating SQDMULH, shift 0 / 31, wrap-around adds)
+    through the stand-alone output stage."""
+    import torch
+    I32_MIN, I32_MAX = -(1 << 31), (1 << 31) - 1
+    vals = np.array([I32_MIN, I32_MIN + 1, -(1 << 30), -65537, -3, -2, -1, 0, 1, 2, 3, 65535, 1 << 30, I32_MAX - 1,
+                     I32_MAX, 123456789], dtype=np.int32).reshape(1, -1)
+    for m in (1 << 30, 1518500250, I32_MAX, I32_MIN, 1, -1):
+        for s in (-3, -1, 0, 1, 8, 30, 31):
+            for dt, lo, hi in ((np.int8, -128, 127), (np.uint8, 0, 255)):
+                want = oracle.output_stage_fixedpoint(vals, None, [m], [s], 10, lo, hi, dt)
+                dst = torch.zeros(vals.shape, dtype=torch.int8 if dt == np.int8 else torch.uint8, device="cuda")
+                capi.output_stage(torch.from_numpy(vals).cuda(), None, dst, capi.requant(m, s, 10, lo, hi))
+                np.testing.assert_array_equal(dst.cpu().numpy(), want)
+
+
+def test_output_stage_fixture(golden):
+    g = golden("output_stage.npz")
+    for n in range(int(g["count"])):
+        mult, shift, roff, lo, hi, with_bias = (int(x) for x in g["p%d" % n])
+        src, dst = g["src%d" % n], g["dst%d" % n]
+        out = np.zeros_like(dst)
+        announce("output stage fixture", n, src.shape, dst.dtype)
+        capi.output_stage(np.ascontiguousarray(src), np.ascontiguousarray(g["bias%d" % n]) if with_bias else None,
+                          out, capi.requant(mult, shift, roff, lo, hi))
+        np.testing.assert_array_equal(out, dst)
+
+
+def test_update_quant_and_rerun():
+    """update_quantization_parameters: new offsets / multiplier without re-packing B; run twice gives identical bytes
+    (tests/validation/NEON/GEMMLowp.cpp:211-297 MultipleExecutionWithConfigure)."""
+    import torch
+    rng = np.random.default_rng(44)
+    M, N, K = 96, 80, 144
+    A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, size=(K, N), dtype=np.uint8)
+    bias = rng.integers(-500, 500, size=N, dtype=np.int32)
+    g = capi.Gemm(M, N, K, capi.U8, capi.U8, capi.U8, capi.EPI_FIXEDPOINT, -10, -20,
+                  capi.requant(1518500250, 9, 5, 0, 255))
+    Ad, Bd, bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), torch.from_numpy(bias).cuda()
+    D1 = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+    D2 = torch.zeros_like(D1)
+    g.prepare(Bd, bd)
+    g.run(Ad, D1)
+    g.run(Ad, D2)
+    torch.cuda.synchronize()
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -10, -20, [1518500250], [9], 5, 0, 255, np.uint8)
+    np.testing.assert_array_equal(D1.cpu().numpy(), want)
+    np.testing.assert_array_equal(D2.cpu().numpy(), want)
+    g.update_quant(-100, -128, capi.requant(1288490240, 10, 17, 3, 250))
+    g.run(Ad, D1)
+    torch.cuda.synchronize()
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -100, -128, [1288490240], [10], 17, 3, 250, np.uint8)
+    np.testing.assert_array_equal(D1.cpu().numpy(), want)
+    g.close()
+
+
+def test_run_before_prepare_is_an_error():
+    g = capi.Gemm(32, 32, 32, capi.S8, capi.S8, capi.S32, capi.EPI_S32)
+    with pytest.raises(capi.Mi355Error):
+        g.run(np.zeros((32, 32), np.int8), np.zeros((32, 32), np.int32))
+    g.close()

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libmi355gemmlowp.so")
-SOURCES = ["gemm_mfma.hip", "gemm_skinny.hip", "kernels_aux.hip", "capi.hip"]
+SOURCES = ["gemm_dma.hip", "gemm_mfma.hip", "gemm_skinny.hip", "kernels_aux.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -138,12 +138,15 @@ struct GemmCore
     int32_t a_offset = 0, b_offset = 0; // as given (added convention)
     mi355_requant rq{};
     float   scale = 1.f, act_min = -INFINITY, act_max = INFINITY;
-    int     path = MI355_PATH_AUTO, cfg_idx = 0;
+    int     path = MI355_PATH_AUTO, cfg_idx = 0, dma_idx = -1;
     int     Kp = 0, Np = 0;
     bool    b_shared = true; // one B for all batches
     bool    has_bias = false, has_pc = false, prepared = false;
     std::string kname;
-    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap;
+    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp;
+    bool    qp_ok = false; // all multipliers >= 0: the branch-free epilogue applies
+    std::string kname_mfma, kname_dma, kprefix;
+    uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
 
     int32_t a_off_eff() const { return (int32_t)((uint32_t)a_offset + (flip_a ? 128u : 0u)); }
     int32_t b_off_eff() const { return (int32_t)((uint32_t)b_offset + (flip_b ? 128u : 0u)); }
@@ -152,7 +155,7 @@ struct GemmCore
     void release()
     {
         Bp.release(), Bs.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
-        shift.release(), bias.release(), Ap.release();
+        shift.release(), bias.release(), Ap.release(), fill.release(), qp.release();
     }
 
     int choose_kernel()
@@ -169,28 +172,37 @@ struct GemmCore
             kname = "skinny_16xN_splitk8";
         else
         {
-            const int   cus   = num_cus();
-            int         best  = -1;
-            long        most  = -1;
-            const char *force = getenv("MI355_GEMM_CFG");
-            for (int i = 0; i < mfma_num_configs(); ++i)
+            const int cus = num_cus();
+            auto      pick = [&](int count, MfmaConfig (*get)(int), const char *env) -> int
             {
-                const MfmaConfig c     = mfma_config(i);
-                const long       tiles = (long)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN) * batch;
-                if (N <= 64 && c.BN > 64)
-                    continue;
-                if (tiles >= cus)
+                int  best = -1;
+                long most = -1;
+                for (int i = 0; i < count; ++i)
                 {
-                    best = i;
-                    break;
+                    const MfmaConfig c     = get(i);
+                    const long       tiles = (long)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN) * batch;
+                    if (N <= 64 && c.BN > 64)
+                        continue;
+                    if (tiles >= cus)
+                        return i;
+                    if (tiles > most)
+                        most = tiles, best = i;
                 }
-                if (tiles > most)
-                    most = tiles, best = i;
-            }
-            if (force && atoi(force) >= 0 && atoi(force) < mfma_num_configs())
-                best = atoi(force);
-            cfg_idx = best;
-            kname   = mfma_config(best).name;
+                (void)env;
+                return best;
+            };
+            cfg_idx = pick(mfma_num_configs(), mfma_config, nullptr);
+            dma_idx = pick(DMA_AUTO_CONFIGS, dma_config, nullptr);
+            const char *f1 = getenv("MI355_GEMM_CFG"), *f2 = getenv("MI355_DMA_CFG");
+            if (f1 && atoi(f1) >= 0 && atoi(f1) < mfma_num_configs())
+                cfg_idx = atoi(f1);
+            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs())
+                dma_idx = atoi(f2);
+            if (getenv("MI355_NO_DMA") || K % 16 != 0)
+                dma_idx = -1;
+            kname_mfma = mfma_config(cfg_idx).name;
+            kname_dma  = dma_idx >= 0 ? dma_config(dma_idx).name : "";
+            kname      = dma_idx >= 0 ? kname_dma : kname_mfma;
         }
         return 0;
     }
@@ -209,8 +221,11 @@ struct GemmCore
         {
             if (mult_in == nullptr || shift_in == nullptr)
                 return fail("per-channel requantisation needs multiplier and shift arrays");
-            TRY(mult.ensure(sizeof(int32_t) * (size_t)N));
-            TRY(shift.ensure(sizeof(int32_t) * (size_t)N));
+            // padded like the packed B panel: the epilogue reads these as 16-byte vectors
+            TRY(mult.ensure(sizeof(int32_t) * (size_t)Np));
+            TRY(shift.ensure(sizeof(int32_t) * (size_t)Np));
+            HIP_TRY(fill_i32_launch(mult.as<int32_t>(), 0, Np, s));
+            HIP_TRY(fill_i32_launch(shift.as<int32_t>(), 0, Np, s));
             HIP_TRY(hipMemcpyAsync(mult.p, mult_in, sizeof(int32_t) * (size_t)N, hipMemcpyDefault, s));
             HIP_TRY(hipMemcpyAsync(shift.p, shift_in, sizeof(int32_t) * (size_t)N, hipMemcpyDefault, s));
         }
@@ -219,7 +234,10 @@ struct GemmCore
             TRY(Bs.ensure((size_t)Np * Kp));
             HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>(), Kp, Np, Bs.as<int8_t>(), s));
         }
+        TRY(fill.ensure(16));
+        HIP_TRY(fill_i32_launch(fill.as<int32_t>(), (int32_t)(0x01010101u * fill_byte), 4, s));
         TRY(refresh_colvec(s));
+        TRY(refresh_qparams(s));
         prepared = true;
         return 0;
     }
@@ -234,8 +252,27 @@ struct GemmCore
         return 0;
     }
 
+    // digest multipliers / shifts for the pipelined kernel's epilogue; synchronises the stream to learn whether it applies
+    int refresh_qparams(hipStream_t s)
+    {
+        qp_ok = false;
+        if (epi != EPI_FIXEDPOINT)
+            return 0;
+        TRY(qp.ensure(sizeof(int32_t) * ((size_t)QP_COUNT * Np + 4)));
+        int32_t *flag = qp.as<int32_t>() + (size_t)QP_COUNT * Np;
+        HIP_TRY(qparams_launch(has_pc ? mult.as<int32_t>() : nullptr, has_pc ? shift.as<int32_t>() : nullptr,
+                               rq.multiplier, rq.shift, N, Np, qp.as<int32_t>(), flag, s));
+        int32_t neg = 1;
+        HIP_TRY(hipMemcpyAsync(&neg, flag, sizeof(neg), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+        qp_ok = neg == 0;
+        return 0;
+    }
+
     void fill_epi(EpiParams &p, const float *bias_f32) const
     {
+        p.qp                  = qp_ok ? qp.as<int32_t>() : nullptr;
+        p.qp_stride           = Np;
         p.colvec              = colvec.as<int32_t>();
         p.rowvec              = nullptr;
         p.mult                = has_pc ? mult.as<int32_t>() : nullptr;
@@ -293,7 +330,15 @@ struct GemmCore
         g.Bp = Bp.as<int8_t>(), g.Kp = Kp, g.bp_batch_stride = b_shared ? 0 : (int64_t)Np * Kp;
         g.D = D, g.ldd = ldd, g.d_batch_stride = d_bs;
         g.M = M, g.N = N, g.K = k_valid;
+        set_vec_store(g);
         return launch(g, flip_in_loader, false, s);
+    }
+
+    // 4 consecutive outputs of a row may leave as one store when every row start is aligned to 4 elements
+    void set_vec_store(GemmArgs &g) const
+    {
+        const size_t esz = (epi == EPI_FIXEDPOINT) ? 1 : 4;
+        g.epi.vec_store  = (((uintptr_t)g.D % (4 * esz)) == 0 && g.ldd % 4 == 0 && g.d_batch_stride % 4 == 0) ? 1 : 0;
     }
 
     int launch(GemmArgs &g, bool flip_in_loader, bool conv, hipStream_t s)
@@ -307,10 +352,29 @@ struct GemmCore
         }
         else
         {
-            const MfmaConfig c = mfma_config(cfg_idx);
-            g.tiles_m          = (g.M + c.BM - 1) / c.BM;
-            g.tiles_n          = (g.N + c.BN - 1) / c.BN;
-            HIP_TRY(mfma_launch(cfg_idx, epi, flip_in_loader, conv, g, batch, s));
+            g.fill16 = fill.as<int8_t>();
+            // the pipelined kernel moves whole aligned 16-byte columns straight into LDS
+            const bool aligned =
+                conv ? (g.conv.C % 16 == 0 && ((uintptr_t)g.A & 15) == 0)
+                     : ((((uintptr_t)g.A | (uintptr_t)g.lda | (uintptr_t)g.a_batch_stride) & 15) == 0);
+            if (dma_idx >= 0 && aligned && g.K % 16 == 0)
+            {
+                const MfmaConfig c = dma_config(dma_idx);
+                g.tiles_m          = (g.M + c.BM - 1) / c.BM;
+                g.tiles_n          = (g.N + c.BN - 1) / c.BN;
+                kname              = kprefix + kname_dma;
+                HIP_TRY(dma_launch(dma_idx, epi, flip_in_loader, conv, g, batch, s));
+            }
+            else
+            {
+                const MfmaConfig c = mfma_config(cfg_idx);
+                g.tiles_m          = (g.M + c.BM - 1) / c.BM;
+                g.tiles_n          = (g.N + c.BN - 1) / c.BN;
+                kname              = kprefix + kname_mfma;
+                if (conv)
+                    g.conv.pad_word = (0x01010101u * fill_byte) ^ (flip_in_loader ? 0x80808080u : 0u);
+                HIP_TRY(mfma_launch(cfg_idx, epi, flip_in_loader, conv, g, batch, s));
+            }
         }
         return 0;
     }
@@ -473,7 +537,10 @@ int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t 
     c.a_offset = a_offset, c.b_offset = b_offset, c.scale = scale;
     h->d.a_offset = a_offset, h->d.b_offset = b_offset, h->d.scale = scale;
     if (c.prepared)
+    {
         TRY(c.refresh_colvec((hipStream_t)stream));
+        TRY(c.refresh_qparams((hipStream_t)stream));
+    }
     return 0;
 }
 
@@ -642,10 +709,12 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         return 1;
     }
     // the on-the-fly loader moves 16-byte pieces of one tap: needs C % 16 == 0; it has no row sums: needs b_off == 0
-    h->implicit         = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0;
-    const uint32_t pb   = ((uint32_t)d.pad_value & 0xFFu) ^ ((h->implicit && c.flip_a) ? 0x80u : 0u);
-    h->geom.pad_word    = pb * 0x01010101u;
-    c.kname             = std::string(h->implicit ? "implicit_" : "im2col+") + c.kname;
+    h->implicit      = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0;
+    h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
+    if (h->implicit)
+        c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
+    c.kprefix = h->implicit ? "implicit_" : "im2col+";
+    c.kname   = c.kprefix + c.kname;
     *out                = h;
     return 0;
 }
@@ -700,6 +769,7 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         g.D = Dd, g.ldd = c.N, g.d_batch_stride = 0;
         g.M = c.M, g.N = c.N, g.K = c.K;
         g.conv = h->geom;
+        c.set_vec_store(g);
         TRY(c.launch(g, c.flip_a, true, s));
     }
     else

@@ -33,7 +33,37 @@ struct EpiParams
     float          act_min, act_max;
     int32_t        has_offsets; // EPI_F32: whether the offset term is added at all
     int32_t        dst_signed;
+    int32_t        vec_store; // destination rows / base / batch stride allow 4-element vector stores
+    // Pre-digested per-column requantisation vectors qp[5][qp_stride] (see fast_requant below), or nullptr when some
+    // multiplier is negative and the general formula has to be used
+    const int32_t *qp;
+    int64_t        qp_stride;
 };
+
+// Per-column constants of the branch-free requantisation used by the pipelined kernel's epilogue, valid for
+// multipliers >= 0 (everything calculate_quantized_multiplier produces):
+//   s2    = (int32)(2*mult mod 2^32), cmask = (2*mult >= 2^31) ? -1 : 0   so that  sqdmulh(a, mult) = mulhi(a, s2) + (a & cmask)
+//   ls    = max(-shift, 0)                                              left shift before the multiply
+//   rsm1  = max(shift - 1, 0), rmask = shift > 0 ? 1 : 0                 so that  rshr(x) = ((x >> rsm1) + rmask) >> rmask
+// Shifts of 32 or more in either direction give 0 in the reference arithmetic: encoded as a zero multiplier.
+enum : int
+{
+    QP_S2 = 0,
+    QP_CMASK,
+    QP_LS,
+    QP_RSM1,
+    QP_RMASK,
+    QP_COUNT
+};
+
+__device__ __forceinline__ int32_t fast_requant(int32_t v, int32_t s2, int32_t cmask, int32_t ls, int32_t rsm1,
+                                                int32_t rmask, int32_t result_offset, int32_t lo, int32_t hi)
+{
+    const int32_t pre = (int32_t)((uint32_t)v << ls);
+    const int32_t h   = __mulhi(pre, s2) + (pre & cmask);
+    const int32_t r   = ((h >> rsm1) + rmask) >> rmask;
+    return min(max((int32_t)((uint32_t)r + (uint32_t)result_offset), lo), hi);
+}
 
 // (a * b * 2) >> 32 with the single saturating case, without 64-bit VALU arithmetic
 __device__ __forceinline__ int32_t sqdmulh(int32_t a, int32_t b)

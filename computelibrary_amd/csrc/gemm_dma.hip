@@ -1,0 +1,374 @@
+// K1 / K4, pipelined variant: the same int8 MFMA GEMM + fused epilogue as gemm_mfma.hip, organised for throughput.
+// This is the kernel that runs whenever A rows are 16-byte aligned and K is a multiple of 16; gemm_mfma.hip remains the
+// fallback for everything else.
+//
+// Global -> LDS: direct-to-LDS loads (global_load_lds_dwordx4: no staging registers, no ds_write) into an NS-stage ring,
+// so NS-1 K steps of loads are in flight while one is being multiplied. One wave instruction moves 64 lanes x 16 B =
+// 1 KiB into consecutive LDS bytes (the hardware adds lane*16 to the LDS base held in M0); a unit therefore covers
+// 1024/BK tile rows, and the bank swizzle of mfma_common.hpp is applied on the global side: lane l fetches the 16-byte
+// column that belongs at its LDS slot, which stays inside the same BK-byte row segment, so the global access is still
+// one contiguous segment per row. The loads are issued from inline assembly with hand-placed s_waitcnt vmcnt(n): the
+// compiler cannot tell which stage a direct-to-LDS load writes and would force vmcnt(0) before every LDS read.
+//
+// Roles: a block has 8 consumer waves and 4 producer waves (3 waves per SIMD). The producers do nothing but issue the
+// direct-to-LDS loads: such a load occupies its wave for as long as the texture addresser takes to accept it (about 18
+// clocks per 1 KiB on this part), which would otherwise stall the wave's matrix instructions.
+//
+// LDS -> matrix cores: the consumers form two groups of four (one wave of each group per SIMD) that run half a K step
+// apart ("ping-pong"): while one group streams its 16 matrix instructions for a K step out of registers, the other
+// group reads its operands for the next step from LDS. Two workgroup barriers per K step keep the groups in
+// anti-phase; group 1 takes one extra barrier before the loop and group 0 one after it, so every wave executes the
+// same number of barriers.
+//
+// Accumulators are kept transposed (the B panel is fed as the first matrix operand), so each lane ends up with 4
+// consecutive output columns per register quad: the epilogue packs 4 int8 results into one 32-bit store and reads the
+// per-column parameters as 16-byte vectors.
+#include "mfma_common.hpp"
+
+namespace mi355
+{
+__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void block_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// GWM x GWN consumer waves per group, 2 groups stacked along M, plus NP = GWM*GWN producer waves
+template <int BM, int BN, int BK, int GWM, int GWN, int NS, int EPI, bool FLIP_A, bool CONV>
+__global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
+{
+    constexpr int GW    = GWM * GWN; // waves per consumer group
+    constexpr int NW    = 2 * GW;    // consumer waves
+    constexpr int NP    = GW;        // producer waves (one per SIMD when GW == 4)
+    constexpr int CPR   = BK / 16;   // 16-byte columns per tile row
+    constexpr int RPU   = 1024 / BK; // tile rows per staging unit
+    constexpr int AU = BM / RPU, BU = BN / RPU; // staging units of the A and the B part of a stage
+    constexpr int LPP = (AU + BU) / NP;         // loads per producer wave per stage: unit u belongs to producer u % NP
+    constexpr int TM = BM / 2 / GWM, TN = BN / GWN;
+    constexpr int FM = TM / 32, FN = TN / 32;
+    constexpr int KK    = BK / 32;
+    constexpr int STAGE = (BM + BN) * BK;
+    static_assert((AU + BU) % NP == 0, "staging shape");
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && FM >= 1 && FN >= 1, "wave tile");
+    static_assert(NS >= 3 && (NS - 2) * LPP < 64, "ring depth / vmcnt range");
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    int tm, tn;
+    tile_coords(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int bz = blockIdx.z;
+    const int nk = (g.K + BK - 1) / BK;
+
+    // Barrier protocol (b = number of barriers a wave has executed): consumer group 0 reads stage kt between barriers
+    // 2kt and 2kt+1 and multiplies it between 2kt+1 and 2kt+2; group 1 does the same one barrier later. Producers make
+    // stage kt+1 complete before barrier 2kt+2 and overwrite the ring slot of stage kt-1 after barrier 2kt (its last
+    // reader, group 1, finished before that barrier). Every wave executes 2*nk + 2 barriers.
+    if (wave >= NW)
+    {
+        // ================= producer: global -> LDS =================
+        const int8_t *__restrict__ A  = g.A + (int64_t)bz * g.a_batch_stride;
+        const int8_t *__restrict__ Bp = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
+        const int     pw = wave - NW;
+        const int     ur = lane / CPR; // row inside a unit
+        const int     up = lane % CPR; // LDS column slot inside the row
+        const int8_t *pu[LPP];
+        int           a_c16[LPP]; // byte offset of this lane's column inside a K step
+        int           a_iy0[LPP], a_ix0[LPP];
+#pragma unroll
+        for (int i = 0; i < LPP; ++i)
+        {
+            const int u = pw + i * NP; // wave-uniform
+            if (u < AU)
+            {
+                const int row = u * RPU + ur;
+                const int c   = up ^ swz<CPR>(row);
+                a_c16[i]      = c * 16;
+                const int gr  = min(m0 + row, g.M - 1);
+                if (CONV)
+                {
+                    const int ox = gr % g.conv.OW;
+                    const int t  = gr / g.conv.OW;
+                    const int oy = t % g.conv.OH;
+                    const int n  = t / g.conv.OH;
+                    pu[i]        = A + (int64_t)n * g.conv.H * g.conv.W * g.conv.C;
+                    a_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
+                    a_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
+                }
+                else
+                {
+                    pu[i]    = A + (int64_t)gr * g.lda + c * 16;
+                    a_iy0[i] = a_ix0[i] = 0;
+                }
+            }
+            else
+            {
+                const int row = (u - AU) * RPU + ur;
+                const int c   = up ^ swz<CPR>(row);
+                pu[i]         = Bp + (int64_t)row * g.Kp + c * 16;
+                a_c16[i] = a_iy0[i] = a_ix0[i] = 0;
+            }
+        }
+        auto issue = [&](int kt)
+        {
+            const int      k0   = kt * BK;
+            const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
+#pragma unroll
+            for (int i = 0; i < LPP; ++i)
+            {
+                const int     u   = pw + i * NP;
+                const int8_t *src = pu[i] + k0; // B unit: always inside the zero-padded packed panel
+                if (u < AU)
+                {
+                    const int k = k0 + a_c16[i];
+                    src         = g.fill16;
+                    if (k < g.K)
+                    {
+                        if (CONV)
+                        {
+                            const int tap = k / g.conv.C;
+                            const int c0  = k - tap * g.conv.C;
+                            const int ky  = tap / g.conv.KW;
+                            const int kx  = tap - ky * g.conv.KW;
+                            const int iy  = a_iy0[i] + ky * g.conv.dil_y;
+                            const int ix  = a_ix0[i] + kx * g.conv.dil_x;
+                            if (iy >= 0 && iy < g.conv.H && ix >= 0 && ix < g.conv.W)
+                                src = pu[i] + ((int64_t)iy * g.conv.W + ix) * g.conv.C + c0;
+                        }
+                        else
+                            src = pu[i] + k0;
+                    }
+                }
+                dma16(src, base + (uint32_t)u * 1024u);
+            }
+        };
+#pragma unroll
+        for (int s = 0; s < NS - 1; ++s)
+            if (s < nk)
+                issue(s);
+        if (nk >= NS - 1)
+            wait_vmcnt<(NS - 2) * LPP>(); // stage 0 complete, the NS-2 younger stages may still be in flight
+        else
+            wait_vmcnt<0>();
+        block_barrier(); // barrier 0
+        for (int kt = 0; kt < nk; ++kt)
+        {
+            const bool more = kt + NS - 1 < nk;
+            if (more)
+                issue(kt + NS - 1); // ring slot of stage kt-1
+            block_barrier();        // barrier 2kt+1
+            if (more)
+                wait_vmcnt<(NS - 2) * LPP>(); // stage kt+1 complete
+            else
+                wait_vmcnt<0>();
+            block_barrier(); // barrier 2kt+2
+        }
+        block_barrier(); // barrier 2nk+1
+        if (EPI == EPI_FIXEDPOINT && g.epi.qp != nullptr)
+            __syncthreads(); // the consumers' staging of the epilogue constants
+        return;
+    }
+
+    // ================= consumers: LDS -> matrix cores =================
+    const int group = wave / GW; // waves w and w + GW share a SIMD (waves are placed on the 4 SIMDs round-robin)
+    const int wq    = wave % GW;
+    const int row_w = group * (BM / 2) + (wq / GWN) * TM; // this wave's sub-tile inside the block tile
+    const int col_w = (wq % GWN) * TN;
+
+    // per-column epilogue constants of this block: fetched now, parked in registers, staged in LDS after the loop
+    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
+    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
+    int32_t       par_reg[PPT > 0 ? PPT : 1];
+    const bool    fast = EPI == EPI_FIXEDPOINT && g.epi.qp != nullptr;
+    if (fast)
+    {
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            const int idx = tid + t * NW * 64;
+            par_reg[t]    = 0;
+            if (idx < NPAR * BN)
+            {
+                const int par = idx / BN, col = idx % BN;
+                par_reg[t]    = par == 0 ? g.epi.colvec[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
+                                         : g.epi.qp[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
+            }
+        }
+    }
+
+    v16i acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+
+    // operand read addresses: lane -> (row lane%32, 16-byte column lane/32) of a 32 x 32 operand block
+    const int lr = lane & 31, lh = lane >> 5;
+    int       a_rd[FM], b_rd[FN], a_sw[FM], b_sw[FN];
+#pragma unroll
+    for (int f = 0; f < FM; ++f)
+    {
+        const int row = row_w + f * 32 + lr;
+        a_rd[f]       = row * BK;
+        a_sw[f]       = swz<CPR>(row);
+    }
+#pragma unroll
+    for (int f = 0; f < FN; ++f)
+    {
+        const int row = col_w + f * 32 + lr;
+        b_rd[f]       = BM * BK + row * BK;
+        b_sw[f]       = swz<CPR>(row);
+    }
+
+    block_barrier(); // barrier 0: stage 0 is in LDS
+    if (group == 1)
+        block_barrier(); // group 1 runs one slot behind group 0
+
+    v4i fa[KK][FM], fb[KK][FN];
+    for (int kt = 0; kt < nk; ++kt)
+    {
+        // ---- load slot: operands of K step kt from LDS into registers ----
+        const char *s = smem + (kt % NS) * STAGE;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+        {
+#pragma unroll
+            for (int f = 0; f < FM; ++f)
+                fa[kk][f] = *(const v4i *)(s + a_rd[f] + (((kk * 2 + lh) ^ a_sw[f]) << 4));
+#pragma unroll
+            for (int f = 0; f < FN; ++f)
+                fb[kk][f] = *(const v4i *)(s + b_rd[f] + (((kk * 2 + lh) ^ b_sw[f]) << 4));
+        }
+        if (FLIP_A)
+        {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+                for (int f = 0; f < FM; ++f)
+                    fa[kk][f] ^= (int)0x80808080;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+
+        // ---- compute slot: a pure stream of matrix instructions ----
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+    }
+    if (group == 0)
+        block_barrier(); // barrier 2nk+1; every operand read of every wave is complete beyond this point
+
+    if (fast)
+    {
+        int32_t *par = (int32_t *)smem;
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            const int idx = tid + t * NW * 64;
+            if (idx < NPAR * BN)
+                par[idx] = par_reg[t];
+        }
+        __syncthreads();
+        if (EPI == EPI_FIXEDPOINT)
+            epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+    }
+    else
+        epilogue_store_t<EPI, FM, FN>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
+}
+
+// ---- instantiation table -------------------------------------------------------------------------------------------
+struct DmaEntry
+{
+    MfmaConfig  cfg;
+    int         threads;
+    int         lds_bytes;
+    const void *fn[3][2][2]; // [epi][flip][conv]
+};
+
+#define MI355_DFN(BM, BN, BK, WM, WN, NS, E, F, C) (const void *)gemm_dma_kernel<BM, BN, BK, WM, WN, NS, E, F, C>
+#define MI355_DCFG(NAME, BM, BN, BK, WM, WN, NS)                                                                     \
+    {                                                                                                                \
+        {NAME, BM, BN, BK}, WM *WN * 192, NS * (BM + BN) * BK,                                                        \
+        {                                                                                                            \
+            {{MI355_DFN(BM, BN, BK, WM, WN, NS, 0, false, false), nullptr},                                           \
+             {MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, false), nullptr}},                                           \
+                {{MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, true)}, \
+                 {MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, true)}}, \
+                {{MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, false), nullptr},                                       \
+                 {MI355_DFN(BM, BN, BK, WM, WN, NS, 2, true, false), nullptr}},                                       \
+        }                                                                                                            \
+    }
+
+static const DmaEntry g_dma[] = {
+    MI355_DCFG("pp_256x128x128_s3", 256, 128, 128, 2, 2, 3),
+    MI355_DCFG("pp_128x128x128_s3", 128, 128, 128, 2, 2, 3),
+    MI355_DCFG("pp_128x64x128_s3", 128, 64, 128, 2, 2, 3),
+    MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
+    MI355_DCFG("pp_256x128x64_s4", 256, 128, 64, 2, 2, 4),
+};
+
+int dma_num_configs()
+{
+    return (int)(sizeof(g_dma) / sizeof(g_dma[0]));
+}
+MfmaConfig dma_config(int idx)
+{
+    return g_dma[idx].cfg;
+}
+
+int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s)
+{
+    if (cfg_idx < 0 || cfg_idx >= dma_num_configs() || epi < 0 || epi > 2)
+        return (int)hipErrorInvalidValue;
+    const DmaEntry &c  = g_dma[cfg_idx];
+    const void     *fn = c.fn[epi][flip_a ? 1 : 0][conv ? 1 : 0];
+    if (fn == nullptr || args.fill16 == nullptr)
+        return (int)hipErrorInvalidValue;
+    // shapes the kernel assumes: whole 16-byte columns, 16-byte aligned rows, tiles that cover the output and stay
+    // inside the packed B panel
+    if (args.K % 16 != 0 || args.K > args.Kp || args.Kp % c.cfg.BK != 0 || args.tiles_m * c.cfg.BM < args.M ||
+        args.tiles_n * c.cfg.BN < args.N || args.tiles_n * c.cfg.BN > round_up(args.N, PACK_N_ALIGN) || args.M < 1)
+        return (int)hipErrorInvalidValue;
+    if (conv ? (args.conv.C % 16 != 0 || ((uintptr_t)args.A & 15) != 0)
+             : ((((uintptr_t)args.A | (uintptr_t)args.lda | (uintptr_t)args.a_batch_stride) & 15) != 0))
+        return (int)hipErrorInvalidValue;
+    if (c.lds_bytes > 48 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, c.lds_bytes);
+        if (e != hipSuccess)
+            return (int)e;
+    }
+    GemmArgs a       = args;
+    void    *kargs[] = {&a};
+    dim3     grid(args.tiles_m * args.tiles_n, 1, batch), block(c.threads);
+    return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);
+}
+} // namespace mi355

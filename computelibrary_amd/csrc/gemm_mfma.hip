@@ -13,38 +13,10 @@
 // K step it stages BM x BK of A and BN x BK of B in LDS (two stages), 16 bytes per lane per access, with an XOR swizzle
 // of the 16-byte column index so that both the staging writes and the operand reads are bank-conflict free.
 // Each wave owns a (BM/WM) x (BN/WN) sub-tile as 32x32 accumulator blocks fed by v_mfma_i32_32x32x32_i8.
-#include "internal.hpp"
+#include "mfma_common.hpp"
 
 namespace mi355
 {
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-template <int CPR>
-__device__ __forceinline__ int swz(int row)
-{
-    // CPR 16-byte columns per LDS row; 8 columns span all banks once
-    return (CPR >= 8) ? (row & 7) : ((row * CPR / 8) & (CPR - 1));
-}
-
-// Tile -> workgroup mapping. Workgroups are handed to the 8 XCDs round-robin, each XCD has its own L2: give every
-// XCD a contiguous run of logical tile ids, and walk the tile grid in groups of GM row panels so that a run covers a
-// compact GM x (run/GM) patch whose A and B panels are shared inside one L2.
-__device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, int tiles_n, int &tm, int &tn)
-{
-    int l = bid;
-    if ((nblocks & 7) == 0)
-        l = (bid & 7) * (nblocks >> 3) + (bid >> 3);
-    const int GM      = 4;
-    const int per_grp = GM * tiles_n;
-    const int grp     = l / per_grp;
-    const int first   = grp * GM;
-    const int gsize   = min(tiles_m - first, GM);
-    const int in_grp  = l - grp * per_grp;
-    tm                = first + in_grp % gsize;
-    tn                = in_grp / gsize;
-}
-
 template <int BM, int BN, int BK, int WM, int WN, int EPI, bool FLIP_A, bool CONV>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_mfma_kernel(GemmArgs g)
 {
@@ -195,7 +167,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_mfma_kernel(GemmArgs g)
         b_sw[f]       = swz<CPR>(row);
     }
 
-    const int nk = (int)(g.Kp / BK);
+    const int nk = (g.K + BK - 1) / BK; // k tiles that hold real data (the packed B is zero beyond K)
     load_tiles(0);
     store_tiles(0);
     __syncthreads();
@@ -226,52 +198,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_mfma_kernel(GemmArgs g)
         __syncthreads();
     }
 
-    // ---- epilogue: accumulator (fm, fn, r) of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block ----
-    const EpiParams &p      = g.epi;
-    const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
-    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
-    char            *D      = (char *)g.D;
-#pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
-    {
-        const int  j  = n0 + wn * TN + fn * 32 + lr;
-        const bool vj = j < g.N;
-        int32_t    cv = 0, mu = p.mult_s, sh = p.shift_s;
-        float      bf = 0.f;
-        if (vj)
-        {
-            cv = colvec[j];
-            if (EPI == EPI_FIXEDPOINT && p.mult)
-            {
-                mu = p.mult[j];
-                sh = p.shift[j];
-            }
-            if (EPI == EPI_F32 && p.bias_f32)
-                bf = p.bias_f32[j];
-        }
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm)
-        {
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                const int i = m0 + wm * TM + fm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                if (vj && i < g.M)
-                {
-                    const int32_t rv  = rowvec ? rowvec[i] : 0;
-                    const int32_t a   = acc[fm][fn][r];
-                    const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j;
-                    if (EPI == EPI_S32)
-                        ((int32_t *)D)[idx] = (int32_t)((uint32_t)a + (uint32_t)cv + (uint32_t)rv);
-                    else if (EPI == EPI_FIXEDPOINT)
-                        ((int8_t *)D)[idx] = (int8_t)epi_fixedpoint(a, cv, rv, mu, sh, p);
-                    else
-                        ((float *)D)[idx] =
-                            epi_f32(a, (int32_t)((uint32_t)cv + (uint32_t)rv), bf, p.bias_f32 != nullptr, p);
-                }
-            }
-        }
-    }
+    epilogue_store<EPI, FM, FN>(acc, g, m0 + wm * TM, n0 + wn * TN, lane, bz);
 }
 
 // ---- instantiation table -------------------------------------------------------------------------------------------

@@ -36,6 +36,7 @@ struct GemmArgs
     int32_t       tiles_m, tiles_n;
     EpiParams     epi;
     ConvGeom      conv;
+    const int8_t *fill16; // 16 readable bytes: what a staged 16-byte column reads where A has no data (zeros / pad value)
 };
 
 struct MfmaConfig
@@ -75,6 +76,12 @@ MfmaConfig  mfma_config(int idx);
 // epi: EPI_*, flip_a: xor 0x80 on A bytes in the loader, conv: implicit-GEMM loader. Returns hipError_t as int.
 int         mfma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
 
+// gemm_dma.hip — same contract as mfma_launch; additionally needs 16-byte aligned A rows, K % 16 == 0 and args.fill16
+int         dma_num_configs();
+MfmaConfig  dma_config(int idx);
+int         dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
+constexpr int DMA_AUTO_CONFIGS = 4; // the first entries are the ones the heuristic picks from; the rest are experiments
+
 // gemm_skinny.hip — M <= 16, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 16;
 int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
@@ -91,6 +98,9 @@ int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream
 // colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j])
 int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int32_t b_off, int K, int N,
                   int32_t *colvec, hipStream_t s);
+// (multiplier, shift) per column -> qp[QP_COUNT][Np]; *neg != 0 afterwards if any multiplier is negative
+int qparams_launch(const int32_t *mult, const int32_t *shift, int32_t mult_s, int32_t shift_s, int N, int Np,
+                   int32_t *qp, int32_t *neg, hipStream_t s);
 // A pre-pass: optional padded + flipped copy Ap[M][Kp] and/or rowvec[i] = b_off * sum_k(flip(A[i][k]))
 int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
                      int32_t b_off, hipStream_t s);

@@ -168,6 +168,42 @@ int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int
     return launch_status();
 }
 
+// Digest (multiplier, shift) per column into the QP_* vectors of epilogue.hpp; *neg is set when a multiplier is negative
+// (then the branch-free form does not apply). mult / shift may be nullptr: per-tensor values mult_s / shift_s.
+__global__ void qparams_kernel(const int32_t *__restrict__ mult, const int32_t *__restrict__ shift, int32_t mult_s,
+                               int32_t shift_s, int N, int Np, int32_t *__restrict__ qp, int32_t *__restrict__ neg)
+{
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= Np)
+        return;
+    int32_t m = 0, s = 0;
+    if (j < N)
+    {
+        m = mult ? mult[j] : mult_s;
+        s = shift ? shift[j] : shift_s;
+    }
+    if (m < 0)
+        atomicOr(neg, 1);
+    if (s >= 32 || s <= -32)
+        m = 0, s = 0; // the reference arithmetic yields 0 for these
+    const uint32_t m2          = (uint32_t)m << 1;
+    qp[QP_S2 * (int64_t)Np + j]    = (int32_t)m2;
+    qp[QP_CMASK * (int64_t)Np + j] = ((uint32_t)m >= 0x40000000u) ? -1 : 0;
+    qp[QP_LS * (int64_t)Np + j]    = s < 0 ? -s : 0;
+    qp[QP_RSM1 * (int64_t)Np + j]  = s > 1 ? s - 1 : 0;
+    qp[QP_RMASK * (int64_t)Np + j] = s > 0 ? 1 : 0;
+}
+
+int qparams_launch(const int32_t *mult, const int32_t *shift, int32_t mult_s, int32_t shift_s, int N, int Np,
+                   int32_t *qp, int32_t *neg, hipStream_t s)
+{
+    int e = fill_i32_launch(neg, 0, 1, s);
+    if (e)
+        return e;
+    qparams_kernel<<<dim3((Np + 255) / 256), dim3(256), 0, s>>>(mult, shift, mult_s, shift_s, N, Np, qp, neg);
+    return launch_status();
+}
+
 // ---- A pre-pass -----------------------------------------------------------------------------------------------------
 // One block per row. Optionally writes the row sign-flipped and zero-padded to Kp (for A whose rows are not 16-byte
 // aligned), optionally reduces it: rowvec[i] = b_off * sum_k flip(A[i][k])

@@ -1,0 +1,259 @@
+// Pieces shared by the matrix-core GEMM kernels: LDS swizzle, tile -> workgroup mapping, accumulator epilogue.
+#pragma once
+#include "internal.hpp"
+
+namespace mi355
+{
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// LDS tiles are rows of CPR 16-byte columns. Column c of row r is stored at column c ^ swz(r). The LDS serves a 16-byte
+// access 16 lanes (256 bytes, all 64 banks) per clock: 16 consecutive rows reading the same logical column must land in
+// 16 different 16-byte bank groups. 16/CPR rows share one 256-byte span, so rows r and r + 16/CPR (same position in the
+// span) get different rotations; a staging write (consecutive columns of consecutive rows) is conflict free as well.
+template <int CPR>
+__device__ __forceinline__ int swz(int row)
+{
+    return (row / (16 / CPR)) & (CPR - 1);
+}
+
+// Tile -> workgroup mapping. Workgroups are handed to the 8 XCDs round-robin and each XCD has its own L2: give every
+// XCD a contiguous run of logical tile ids, and walk the tile grid in groups of GM row panels so that a run covers a
+// compact GM x (run/GM) patch whose A and B panels are shared inside one L2.
+__device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, int tiles_n, int &tm, int &tn)
+{
+    int l = bid;
+    if ((nblocks & 7) == 0)
+        l = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+    const int GM      = 4;
+    const int per_grp = GM * tiles_n;
+    const int grp     = l / per_grp;
+    const int first   = grp * GM;
+    const int gsize   = min(tiles_m - first, GM);
+    const int in_grp  = l - grp * per_grp;
+    tm                = first + in_grp % gsize;
+    tn                = in_grp / gsize;
+}
+
+// Accumulator (fm, fn, r) of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 block.
+// (row0, col0) is the wave's top-left output coordinate.
+template <int EPI, int FM, int FN>
+__device__ __forceinline__ void epilogue_store(const v16i (&acc)[FM][FN], const GemmArgs &g, int row0, int col0, int lane,
+                                               int bz)
+{
+    const int        lr = lane & 31, lh = lane >> 5;
+    const EpiParams &p      = g.epi;
+    const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    char            *D      = (char *)g.D;
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn)
+    {
+        const int  j  = col0 + fn * 32 + lr;
+        const bool vj = j < g.N;
+        int32_t    cv = 0, mu = p.mult_s, sh = p.shift_s;
+        float      bf = 0.f;
+        if (vj)
+        {
+            cv = colvec[j];
+            if (EPI == EPI_FIXEDPOINT && p.mult)
+            {
+                mu = p.mult[j];
+                sh = p.shift[j];
+            }
+            if (EPI == EPI_F32 && p.bias_f32)
+                bf = p.bias_f32[j];
+        }
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+        {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const int i = row0 + fm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                if (vj && i < g.M)
+                {
+                    const int32_t rv  = rowvec ? rowvec[i] : 0;
+                    const int32_t a   = acc[fm][fn][r];
+                    const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j;
+                    if (EPI == EPI_S32)
+                        ((int32_t *)D)[idx] = (int32_t)((uint32_t)a + (uint32_t)cv + (uint32_t)rv);
+                    else if (EPI == EPI_FIXEDPOINT)
+                        ((int8_t *)D)[idx] = (int8_t)epi_fixedpoint(a, cv, rv, mu, sh, p);
+                    else
+                        ((float *)D)[idx] =
+                            epi_f32(a, (int32_t)((uint32_t)cv + (uint32_t)rv), bf, p.bias_f32 != nullptr, p);
+                }
+            }
+        }
+    }
+}
+// Transposed accumulators (the B panel was the first matrix operand): accumulator (fm, fn, r) of lane l holds output
+// row l%32 of row block fm and output column 8*(r/4) + 4*(l/32) + r%4 of column block fn, i.e. every register quad is
+// 4 consecutive columns of one row: per-column parameters are read as 16-byte vectors and 4 results leave in one store.
+template <int EPI, int FM, int FN>
+__device__ __forceinline__ void epilogue_store_t(const v16i (&acc)[FM][FN], const GemmArgs &g, int row0, int col0,
+                                                 int lane, int bz)
+{
+    const int        lr = lane & 31, lh = lane >> 5;
+    const EpiParams &p      = g.epi;
+    const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    char            *D      = (char *)g.D;
+    int32_t          rv[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+    {
+        const int i = row0 + fm * 32 + lr;
+        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int j0 = col0 + fn * 32 + 8 * q + 4 * lh; // first of 4 consecutive columns; inside the padded vectors
+            const v4i cv = *(const v4i *)(colvec + j0);
+            v4i       mu = {p.mult_s, p.mult_s, p.mult_s, p.mult_s};
+            v4i       sh = {p.shift_s, p.shift_s, p.shift_s, p.shift_s};
+            float     bf[4] = {0.f, 0.f, 0.f, 0.f};
+            if (EPI == EPI_FIXEDPOINT && p.mult)
+            {
+                mu = *(const v4i *)(p.mult + j0);
+                sh = *(const v4i *)(p.shift + j0);
+            }
+            if (EPI == EPI_F32 && p.bias_f32)
+            {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (j0 + t < g.N)
+                        bf[t] = p.bias_f32[j0 + t];
+            }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm)
+            {
+                const int i = row0 + fm * 32 + lr;
+                if (i >= g.M || j0 >= g.N)
+                    continue;
+                const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
+                const bool    vec = p.vec_store && (j0 + 3 < g.N);
+                if (EPI == EPI_FIXEDPOINT)
+                {
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        packed |= ((uint32_t)epi_fixedpoint(acc[fm][fn][4 * q + t], cv[t], rv[fm], mu[t], sh[t], p) & 0xFFu)
+                                  << (8 * t);
+                    if (vec)
+                        *(uint32_t *)(D + idx) = packed;
+                    else
+                    {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (j0 + t < g.N)
+                                D[idx + t] = (char)(packed >> (8 * t));
+                    }
+                }
+                else if (EPI == EPI_S32)
+                {
+                    v4i o;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
+                    if (vec)
+                        *(v4i *)((int32_t *)D + idx) = o;
+                    else
+                    {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (j0 + t < g.N)
+                                ((int32_t *)D)[idx + t] = o[t];
+                    }
+                }
+                else
+                {
+                    typedef float v4f __attribute__((ext_vector_type(4)));
+                    v4f o;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        o[t] = epi_f32(acc[fm][fn][4 * q + t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv[fm]), bf[t],
+                                       p.bias_f32 != nullptr, p);
+                    if (vec)
+                        *(v4f *)((float *)D + idx) = o;
+                    else
+                    {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (j0 + t < g.N)
+                                ((float *)D)[idx + t] = o[t];
+                    }
+                }
+            }
+        }
+    }
+}
+// FIXEDPOINT epilogue of the pipelined kernel for multipliers >= 0. The block's per-column constants were staged in LDS
+// as par[6][BN]: row 0 the folded offset/bias vector, rows 1..5 the QP_* vectors; col_in_tile is the wave's first
+// column inside the block tile. Same accumulator layout as epilogue_store_t.
+template <int FM, int FN, int BN>
+__device__ __forceinline__ void epilogue_store_fast(const v16i (&acc)[FM][FN], const GemmArgs &g, const int32_t *par,
+                                                    int row0, int col0, int col_in_tile, int lane, int bz)
+{
+    const int        lr = lane & 31, lh = lane >> 5;
+    const EpiParams &p      = g.epi;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    char            *D      = (char *)g.D;
+    int32_t          rv[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+    {
+        const int i = row0 + fm * 32 + lr;
+        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int c  = col_in_tile + fn * 32 + 8 * q + 4 * lh;
+            const int j0 = col0 + fn * 32 + 8 * q + 4 * lh;
+            const v4i cv = *(const v4i *)(par + 0 * BN + c);
+            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
+            const v4i cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
+            const v4i ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
+            const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
+            const v4i rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm)
+            {
+                const int i = row0 + fm * 32 + lr;
+                int32_t   o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                {
+                    const int32_t v = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
+                    o[t]            = fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
+                }
+                // low bytes of o[0..3] -> one dword
+                const uint32_t p01    = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
+                const uint32_t p23    = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
+                const uint32_t packed = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+                if (i >= g.M || j0 >= g.N)
+                    continue;
+                const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
+                if (p.vec_store && (j0 + 3 < g.N))
+                    *(uint32_t *)(D + idx) = packed;
+                else
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (j0 + t < g.N)
+                            D[idx + t] = (char)(packed >> (8 * t));
+                }
+            }
+        }
+    }
+}
+} // namespace mi355

@@ -15,7 +15,7 @@ PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
 EXPORTS = [
     "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_run",
     "mi355_gemmlowp_destroy", "mi355_gemmlowp_kernel_name", "mi355_output_stage_run", "mi355_conv_create",
-    "mi355_conv_prepare", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
+    "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
     "mi355_im2col_nhwc_run", "mi355_last_error", "mi355_device_info",
 ]
 
@@ -77,6 +77,7 @@ def lib():
         l.mi355_conv_create.argtypes = [C.POINTER(ConvDesc), C.POINTER(vp)]
         l.mi355_conv_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
         l.mi355_conv_run.argtypes = [vp, vp, vp, vp]
+        l.mi355_conv_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Requant), i32p, i32p, vp]
         l.mi355_conv_out_dims.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         l.mi355_conv_out_dims.restype = None
         l.mi355_conv_destroy.argtypes = [vp]
@@ -192,6 +193,10 @@ class Conv:
 
     def prepare(self, weights, bias=None, mult=None, shift=None, stream=None):
         _check(lib().mi355_conv_prepare(self._h, ptr(weights), ptr(bias), ptr(mult), ptr(shift), stream))
+
+    def update_quant(self, src_offset, weights_offset, pad_value, rq, mult=None, shift=None, stream=None):
+        _check(lib().mi355_conv_update_quant(self._h, src_offset, weights_offset, pad_value, C.byref(rq), ptr(mult),
+                                             ptr(shift), stream))
 
     def run(self, src, dst, stream=None):
         _check(lib().mi355_conv_run(self._h, ptr(src), ptr(dst), stream))

@@ -741,6 +741,41 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t 
     return 0;
 }
 
+int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t weights_offset, int32_t pad_value,
+                            const mi355_requant *requant, const int32_t *mult, const int32_t *shift, void *stream)
+{
+    if (!h || !requant)
+        return fail("null argument");
+    hipStream_t s = (hipStream_t)stream;
+    GemmCore   &c = h->core;
+    TRY(check_requant(*requant, c.dst_dtype));
+    if ((requant->per_channel != 0) != (c.rq.per_channel != 0))
+        return fail("update cannot switch between per-tensor and per-channel requantisation");
+    h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
+    c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
+    h->implicit      = h->d.path == 0 && (h->d.C % 16 == 0) && c.b_off_eff() == 0;
+    h->geom.pad_word = ((uint32_t)pad_value & 0xFFu) * 0x01010101u;
+    c.fill_byte      = (uint8_t)(pad_value & 0xFF);
+    c.kprefix        = h->implicit ? "implicit_" : "im2col+";
+    if (!c.prepared)
+        return 0;
+    if (c.rq.per_channel)
+    {
+        if (!mult || !shift)
+            return fail("per-channel requantisation needs multiplier and shift arrays");
+        const void *multd, *shiftd;
+        TRY(to_device(mult, sizeof(int32_t) * c.N, h->stageMult, s, &multd));
+        TRY(to_device(shift, sizeof(int32_t) * c.N, h->stageShift, s, &shiftd));
+        HIP_TRY(hipMemcpyAsync(c.mult.p, multd, sizeof(int32_t) * (size_t)c.N, hipMemcpyDeviceToDevice, s));
+        HIP_TRY(hipMemcpyAsync(c.shift.p, shiftd, sizeof(int32_t) * (size_t)c.N, hipMemcpyDeviceToDevice, s));
+    }
+    HIP_TRY(fill_i32_launch(c.fill.as<int32_t>(), (int32_t)(0x01010101u * c.fill_byte), 4, s));
+    TRY(c.refresh_colvec(s));
+    TRY(c.refresh_qparams(s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
 int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream)
 {
     if (!h || !src || !dst)

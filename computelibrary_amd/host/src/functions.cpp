@@ -1,0 +1,725 @@
+// NEGEMMLowpMatrixMultiplyCore, NEGEMMLowpOutputStage and NEGEMMConvolutionLayer on top of the MI355X C ABI
+// (include/mi355_gemmlowp.h). The classes keep the reference's calling conventions: non-owning tensor pointers captured
+// at configure() and dereferenced at run(), buffers that may be allocated after configure(), validate() that returns a
+// Status and never throws, configure() that throws std::runtime_error on invalid input, synchronous run().
+#include "arm_compute/core/utils/quantization/AsymmHelpers.h"
+#include "arm_compute/runtime/NEON/NEFunctions.h"
+#include "mi355_gemmlowp.h"
+
+#include <cmath>
+#include <limits>
+#include <set>
+#include <string>
+#include <vector>
+
+namespace arm_compute
+{
+namespace
+{
+int to_mi355(DataType dt)
+{
+    switch (dt)
+    {
+        case DataType::QASYMM8:
+        case DataType::U8:
+            return MI355_U8;
+        case DataType::QASYMM8_SIGNED:
+        case DataType::QSYMM8:
+        case DataType::QSYMM8_PER_CHANNEL:
+        case DataType::S8:
+            return MI355_S8;
+        case DataType::S32:
+            return MI355_S32;
+        case DataType::F32:
+            return MI355_F32;
+        default:
+            return -1;
+    }
+}
+
+bool is_one_of(DataType dt, std::initializer_list<DataType> list)
+{
+    for (DataType d : list)
+        if (d == dt)
+            return true;
+    return false;
+}
+
+void check_abi(int rc, const char *what)
+{
+    if (rc != 0)
+        throw std::runtime_error(std::string(what) + ": " + mi355_last_error());
+}
+
+uint8_t *first_element(const ITensor *t)
+{
+    return t->buffer() + t->info()->offset_first_element_in_bytes();
+}
+
+mi355_requant make_requant(const GEMMLowpOutputStageInfo &s)
+{
+    mi355_requant rq{};
+    rq.per_channel   = s.is_quantized_per_channel ? 1 : 0;
+    rq.multiplier    = s.gemmlowp_multiplier;
+    rq.shift         = s.gemmlowp_shift;
+    rq.result_offset = s.gemmlowp_offset;
+    rq.min_bound     = s.gemmlowp_min_bound;
+    rq.max_bound     = s.gemmlowp_max_bound;
+    return rq;
+}
+
+// rows of the matrix must be contiguous along x, everything above dimension 1 is one batch index
+Status check_matrix_layout(const ITensorInfo *t, const char *name)
+{
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->strides_in_bytes()[0] != t->element_size(),
+                                    std::string(name) + ": elements of a row must be contiguous");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->strides_in_bytes()[1] % t->element_size() != 0,
+                                    std::string(name) + ": row stride must be a whole number of elements");
+    return Status{};
+}
+
+const std::set<ActivationLayerInfo::ActivationFunction> fusable_acts = {
+    ActivationLayerInfo::ActivationFunction::RELU, ActivationLayerInfo::ActivationFunction::BOUNDED_RELU,
+    ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU};
+} // namespace
+
+// =====================================================================================================================
+// NEGEMMLowpMatrixMultiplyCore
+// =====================================================================================================================
+struct NEGEMMLowpMatrixMultiplyCore::Impl
+{
+    const ITensor      *a{nullptr}, *b{nullptr}, *c{nullptr};
+    ITensor            *output{nullptr};
+    GEMMInfo            info{};
+    mi355_gemm_desc     desc{};
+    mi355_gemm_handle  *handle{nullptr};
+    bool                is_prepared{false};
+    bool                b_constant{true};
+    std::vector<int32_t> multipliers, shifts; // per-channel, exactly N entries
+
+    ~Impl()
+    {
+        if (handle)
+            mi355_gemmlowp_destroy(handle);
+    }
+};
+
+NEGEMMLowpMatrixMultiplyCore::NEGEMMLowpMatrixMultiplyCore(std::shared_ptr<IMemoryManager> memory_manager,
+                                                           IWeightsManager                *weights_manager)
+    : _impl(std::make_unique<Impl>())
+{
+    // device workspace is owned by the handle; a host memory manager has nothing to manage here
+    ARM_COMPUTE_UNUSED(memory_manager, weights_manager);
+}
+NEGEMMLowpMatrixMultiplyCore::~NEGEMMLowpMatrixMultiplyCore() = default;
+
+// Accept / reject rules of src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:362-645 and of the kernels it validates
+// (CpuGemmLowpOffsetContributionOutputStageKernel.cpp:829-905, CpuGemmLowpMatrixMultiplyKernel.cpp:690-692).
+Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITensorInfo *b, const ITensorInfo *c,
+                                              const ITensorInfo *output, const GEMMInfo &gemm_info)
+{
+    ARM_COMPUTE_RETURN_ERROR_ON_NULLPTR(a, b, output);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(a->is_dynamic() || b->is_dynamic() || output->is_dynamic() ||
+                                        (c != nullptr && c->is_dynamic()),
+                                    "Dynamic tensor shapes are not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(a->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}) ||
+                                        a->num_channels() != 1,
+                                    "Matrix A must be QASYMM8 or QASYMM8_SIGNED");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(b->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED,
+                                                                DataType::QSYMM8, DataType::QSYMM8_PER_CHANNEL}) ||
+                                        b->num_channels() != 1,
+                                    "Matrix B must be QASYMM8, QASYMM8_SIGNED, QSYMM8 or QSYMM8_PER_CHANNEL");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::F16, "F16 output is not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::S32, DataType::QASYMM8,
+                                                                     DataType::QASYMM8_SIGNED, DataType::F32}),
+                                    "Output must be S32, QASYMM8, QASYMM8_SIGNED or F32");
+    const GEMMLowpOutputStageInfo stage = gemm_info.gemmlowp_output_stage();
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(c != nullptr && output->data_type() != DataType::F32 &&
+                                        stage.type == GEMMLowpOutputStageType::NONE,
+                                    "Bias addition not supported in NEGEMMLowpMatrixMultiplyCore for output S32");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(
+        a->dimension(0) != b->dimension(1),
+        "The product AB is defined only if the number of columns in A is equal to the number of rows in B");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.is_a_reshaped(), "Matrix A already reshaped is not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.is_b_reshaped(), "Matrix B already reshaped is not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.pretranspose_A(), "Matrix A already pretransposed is not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.pretranspose_B(), "Matrix B already pretransposed is not supported");
+    // signed A with unsigned B has no kernel in the reference (CpuGemmLowpMatrixMultiplyKernel.cpp:690-692)
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(a->data_type() == DataType::QASYMM8_SIGNED && b->data_type() == DataType::QASYMM8,
+                                    "QASYMM8_SIGNED lhs with QASYMM8 rhs is not supported");
+    if (gemm_info.accumulate())
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.type != GEMMLowpOutputStageType::NONE,
+                                        "Accumulation is not supported for output QASYMM8/QASYMM8_SIGNED");
+        ARM_COMPUTE_RETURN_ERROR_MSG("Accumulation into the destination is not built in this library");
+    }
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.reinterpret_input_as_3d(),
+                                    "reinterpret_input_as_3d is not built in this library");
+
+    // shapes
+    ARM_COMPUTE_RETURN_ERROR_ON(b->dimension(0) != output->dimension(0));
+    if (gemm_info.depth_output_gemm3d() != 0)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1) * output->dimension(2));
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->strides_in_bytes()[2] !=
+                                            output->dimension(1) * output->strides_in_bytes()[1],
+                                        "GEMM3D output planes must be contiguous (no y padding)");
+    }
+    else
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1));
+        ARM_COMPUTE_RETURN_ERROR_ON(a->tensor_shape().total_size_upper(2) != output->tensor_shape().total_size_upper(2));
+    }
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(b->num_dimensions() > 2 &&
+                                        b->tensor_shape().total_size_upper(2) != a->tensor_shape().total_size_upper(2),
+                                    "Batched B must have as many matrices as A");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(a->num_dimensions() > 3 || b->num_dimensions() > 3,
+                                    "More than one batch dimension is not supported");
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(a, "a"));
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(b, "b"));
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(output, "output"));
+
+    // output stage
+    switch (stage.type)
+    {
+        case GEMMLowpOutputStageType::NONE:
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::S32, DataType::F32}),
+                                            "A quantized output needs an output stage");
+            if (c != nullptr)
+            {
+                ARM_COMPUTE_RETURN_ERROR_ON(c->data_type() != DataType::F32);
+                ARM_COMPUTE_RETURN_ERROR_ON(c->num_dimensions() > 1 || c->dimension(0) != b->dimension(0));
+            }
+            break;
+        case GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT:
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}),
+                                            "The fixed-point output stage writes QASYMM8 or QASYMM8_SIGNED");
+            ARM_COMPUTE_RETURN_ERROR_ON(stage.gemmlowp_min_bound > stage.gemmlowp_max_bound);
+            if (c != nullptr)
+            {
+                ARM_COMPUTE_RETURN_ERROR_ON(c->data_type() != DataType::S32);
+                ARM_COMPUTE_RETURN_ERROR_ON(c->num_dimensions() > 1 || c->dimension(0) != b->dimension(0));
+            }
+            if (stage.is_quantized_per_channel)
+            {
+                ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.gemmlowp_multipliers.size() < b->dimension(0) ||
+                                                    stage.gemmlowp_shifts.size() < b->dimension(0),
+                                                "Per-channel multipliers / shifts shorter than the number of columns");
+                // CpuGemmLowpOffsetContributionOutputStageKernel.cpp:832-836
+                ARM_COMPUTE_RETURN_ERROR_ON_MSG(b->quantization_info().uniform().offset != 0 &&
+                                                    !is_data_type_quantized_per_channel(b->data_type()),
+                                                "Per-channel requantization needs a zero rhs offset");
+            }
+            break;
+        case GEMMLowpOutputStageType::QUANTIZE_DOWN:
+            ARM_COMPUTE_RETURN_ERROR_MSG("QUANTIZE_DOWN (integer multiplier) is not built in this library");
+        default:
+            ARM_COMPUTE_RETURN_ERROR_MSG("Unsupported output stage");
+    }
+    return Status{};
+}
+
+void NEGEMMLowpMatrixMultiplyCore::configure(const ITensor *a, const ITensor *b, const ITensor *c, ITensor *output,
+                                             const GEMMInfo &gemm_info)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(a, b, output);
+    ARM_COMPUTE_ERROR_THROW_ON(
+        validate(a->info(), b->info(), c != nullptr ? c->info() : nullptr, output->info(), gemm_info));
+    Impl &s = *_impl;
+    if (s.handle)
+    {
+        mi355_gemmlowp_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.a = a, s.b = b, s.c = c, s.output = output, s.info = gemm_info;
+    s.is_prepared = false;
+    s.b_constant  = gemm_info.reshape_b_only_on_first_run(); // NEGEMMLowpMatrixMultiplyCore.cpp:77-81 of the reference
+
+    const ITensorInfo *ai = a->info(), *bi = b->info(), *oi = output->info();
+    const GEMMLowpOutputStageInfo stage = gemm_info.gemmlowp_output_stage();
+    mi355_gemm_desc &d = s.desc;
+    d                  = mi355_gemm_desc{};
+    d.K                = static_cast<int32_t>(ai->dimension(0));
+    d.N                = static_cast<int32_t>(bi->dimension(0));
+    d.M                = static_cast<int32_t>(ai->dimension(1));
+    d.batch            = static_cast<int32_t>(ai->tensor_shape().total_size_upper(2));
+    d.a_dtype          = to_mi355(ai->data_type());
+    d.b_dtype          = to_mi355(bi->data_type());
+    d.dst_dtype        = to_mi355(oi->data_type());
+    d.lda              = ai->strides_in_bytes()[1];
+    d.ldb              = bi->strides_in_bytes()[1];
+    d.ldd              = oi->strides_in_bytes()[1] / oi->element_size();
+    d.a_batch_stride   = ai->strides_in_bytes()[2];
+    d.b_batch_stride   = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
+    if (gemm_info.depth_output_gemm3d() != 0)
+        d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
+    else
+        d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
+    d.a_offset = ai->quantization_info().uniform().offset;
+    d.b_offset = is_data_type_quantized_per_channel(bi->data_type()) ? 0 : bi->quantization_info().uniform().offset;
+    d.act_min  = -std::numeric_limits<float>::infinity();
+    d.act_max  = std::numeric_limits<float>::infinity();
+    d.scale    = 1.f;
+    d.path     = MI355_PATH_AUTO;
+    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT)
+    {
+        d.epilogue = MI355_EPI_FIXEDPOINT;
+        d.requant  = make_requant(stage);
+        if (stage.is_quantized_per_channel)
+        {
+            s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.N);
+            s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.N);
+        }
+    }
+    else if (oi->data_type() == DataType::F32)
+    {
+        d.epilogue = MI355_EPI_F32;
+        d.scale    = ai->quantization_info().uniform().scale * bi->quantization_info().uniform().scale;
+        const ActivationLayerInfo act = gemm_info.activation_info();
+        if (act.enabled())
+        {
+            switch (act.activation())
+            {
+                case ActivationLayerInfo::ActivationFunction::RELU:
+                    d.act_min = 0.f;
+                    break;
+                case ActivationLayerInfo::ActivationFunction::BOUNDED_RELU:
+                    d.act_min = 0.f, d.act_max = act.a();
+                    break;
+                case ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU:
+                    d.act_min = act.b(), d.act_max = act.a();
+                    break;
+                default:
+                    ARM_COMPUTE_ERROR("Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
+            }
+        }
+    }
+    else
+        d.epilogue = MI355_EPI_S32;
+    check_abi(mi355_gemmlowp_create(&d, &s.handle), "NEGEMMLowpMatrixMultiplyCore::configure");
+}
+
+void NEGEMMLowpMatrixMultiplyCore::prepare()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMLowpMatrixMultiplyCore::prepare() before configure()");
+    if (s.is_prepared)
+        return;
+    ARM_COMPUTE_ERROR_ON_MSG(s.b->buffer() == nullptr, "matrix B has no memory");
+    const int32_t *bias = nullptr;
+    if (s.desc.epilogue == MI355_EPI_FIXEDPOINT && s.c != nullptr)
+    {
+        ARM_COMPUTE_ERROR_ON_MSG(s.c->buffer() == nullptr, "bias has no memory");
+        bias = reinterpret_cast<const int32_t *>(first_element(s.c));
+    }
+    check_abi(mi355_gemmlowp_prepare(s.handle, first_element(s.b), bias,
+                                     s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                     s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "NEGEMMLowpMatrixMultiplyCore::prepare");
+    if (s.b_constant)
+    {
+        s.b->mark_as_unused(); // the packed copy lives on the device from here on
+        s.is_prepared = true;
+    }
+}
+
+void NEGEMMLowpMatrixMultiplyCore::update_quantization_parameters()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "update_quantization_parameters() before configure()");
+    const QuantizationInfo iq = s.a->info()->quantization_info();
+    const QuantizationInfo wq = s.b->info()->quantization_info();
+    const QuantizationInfo oq = (s.output->info()->total_size() == 0) ? iq : s.output->info()->quantization_info();
+    const DataType         dt = s.a->info()->data_type();
+    int32_t                lo = get_min_max(dt).first, hi = get_min_max(dt).second;
+    const UniformQuantizationInfo uo = oq.uniform();
+    if (fusable_acts.count(s.info.activation_info().activation()) != 0)
+        std::tie(lo, hi) = get_quantized_activation_min_max(s.info.activation_info(), dt, uo);
+    s.desc.a_offset = iq.uniform().offset;
+    s.desc.b_offset = is_data_type_quantized_per_channel(s.b->info()->data_type()) ? 0 : wq.uniform().offset;
+    if (s.desc.epilogue == MI355_EPI_FIXEDPOINT)
+    {
+        ARM_COMPUTE_ERROR_ON_MSG(s.desc.requant.per_channel, "per-channel output stages cannot be updated in place");
+        GEMMLowpOutputStageInfo out;
+        out.type                     = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+        out.gemmlowp_offset          = uo.offset;
+        out.gemmlowp_min_bound       = lo;
+        out.gemmlowp_max_bound       = hi;
+        out.is_quantized_per_channel = false;
+        out.output_data_type         = s.output->info()->data_type();
+        ARM_COMPUTE_ERROR_THROW_ON(quantization::calculate_quantized_multipliers(iq, wq, oq, out));
+        s.desc.requant = make_requant(out);
+        s.info.set_gemmlowp_output_stage(out);
+    }
+    if (s.desc.epilogue == MI355_EPI_F32)
+        s.desc.scale = iq.uniform().scale * wq.uniform().scale;
+    check_abi(mi355_gemmlowp_update_quant(s.handle, s.desc.a_offset, s.desc.b_offset,
+                                          s.desc.epilogue == MI355_EPI_FIXEDPOINT ? &s.desc.requant : nullptr,
+                                          s.desc.scale, nullptr),
+              "NEGEMMLowpMatrixMultiplyCore::update_quantization_parameters");
+}
+
+void NEGEMMLowpMatrixMultiplyCore::run()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMLowpMatrixMultiplyCore::run() before configure()");
+    ARM_COMPUTE_ERROR_ON_MSG(s.a->buffer() == nullptr || s.output->buffer() == nullptr, "tensor without memory");
+    // dynamic quantization: offsets are re-read on every run (CpuGemmLowpMatrixMultiplyCore.cpp:668-674 of the reference)
+    if (s.a->info()->quantization_info().is_dynamic() || s.b->info()->quantization_info().is_dynamic())
+    {
+        const int32_t ao = s.a->info()->quantization_info().uniform().offset;
+        const int32_t bo = is_data_type_quantized_per_channel(s.b->info()->data_type())
+                               ? 0
+                               : s.b->info()->quantization_info().uniform().offset;
+        if (ao != s.desc.a_offset || bo != s.desc.b_offset)
+        {
+            s.desc.a_offset = ao, s.desc.b_offset = bo;
+            if (s.desc.epilogue == MI355_EPI_F32)
+                s.desc.scale = s.a->info()->quantization_info().uniform().scale *
+                               s.b->info()->quantization_info().uniform().scale;
+            check_abi(mi355_gemmlowp_update_quant(s.handle, ao, bo, nullptr, s.desc.scale, nullptr),
+                      "NEGEMMLowpMatrixMultiplyCore::run");
+        }
+    }
+    prepare();
+    const float *bias_f32 = nullptr;
+    if (s.desc.epilogue == MI355_EPI_F32 && s.c != nullptr)
+        bias_f32 = reinterpret_cast<const float *>(first_element(s.c));
+    check_abi(mi355_gemmlowp_run(s.handle, first_element(s.a), bias_f32, first_element(s.output), nullptr),
+              "NEGEMMLowpMatrixMultiplyCore::run");
+}
+
+const char *NEGEMMLowpMatrixMultiplyCore::kernel_name() const
+{
+    return _impl->handle ? mi355_gemmlowp_kernel_name(_impl->handle) : "";
+}
+
+// =====================================================================================================================
+// NEGEMMLowpOutputStage
+// =====================================================================================================================
+struct NEGEMMLowpOutputStage::Impl
+{
+    const ITensor          *src{nullptr}, *bias{nullptr};
+    ITensor                *dst{nullptr};
+    mi355_output_stage_desc desc{};
+    bool                    configured{false};
+};
+
+NEGEMMLowpOutputStage::NEGEMMLowpOutputStage() : _impl(std::make_unique<Impl>()) {}
+NEGEMMLowpOutputStage::~NEGEMMLowpOutputStage() = default;
+
+// src/cpu/operators/CpuGemmLowpOutputStage.cpp:114-161 and
+// src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt8ScaleByFixedPointKernel.cpp:52-76 of the reference
+Status NEGEMMLowpOutputStage::validate(const ITensorInfo *input, const ITensorInfo *bias, const ITensorInfo *output,
+                                       const GEMMLowpOutputStageInfo &info)
+{
+    ARM_COMPUTE_RETURN_ERROR_ON_NULLPTR(input, output);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::UNKNOWN,
+                                    "NEGEMMLowpOutputStage cannot be used with UNKNOWN output data type.");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED,
+                                                                     DataType::QSYMM16}),
+                                    "Output must be QASYMM8, QASYMM8_SIGNED or QSYMM16");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type != GEMMLowpOutputStageType::QUANTIZE_DOWN &&
+                                        info.type != GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT,
+                                    "Unsupported output stage type");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type == GEMMLowpOutputStageType::QUANTIZE_DOWN,
+                                    "QUANTIZE_DOWN (integer multiplier) is not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::QSYMM16, "QSYMM16 output is not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON(input->data_type() != DataType::S32 || input->num_channels() != 1);
+    ARM_COMPUTE_RETURN_ERROR_ON(info.gemmlowp_min_bound > info.gemmlowp_max_bound);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.is_quantized_per_channel, "The stand-alone output stage is per-tensor");
+    if (bias != nullptr)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(bias->data_type() != input->data_type());
+        ARM_COMPUTE_RETURN_ERROR_ON(bias->num_dimensions() > 1);
+        ARM_COMPUTE_RETURN_ERROR_ON(input->dimension(0) != bias->dimension(0));
+    }
+    if (output->total_size() != 0)
+        ARM_COMPUTE_RETURN_ERROR_ON(output->tensor_shape() != input->tensor_shape());
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(input, "input"));
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(output, "output"));
+    return Status{};
+}
+
+void NEGEMMLowpOutputStage::configure(const ITensor *input, const ITensor *bias, ITensor *output,
+                                      const GEMMLowpOutputStageInfo &info)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(input, output);
+    // like the reference, an uninitialised output takes the input's shape and the requested data type
+    if (output->info()->total_size() == 0 && output->info()->is_resizable())
+    {
+        output->info()->set_tensor_shape(input->info()->tensor_shape());
+        output->info()->set_num_channels(1);
+        output->info()->set_data_type(info.output_data_type);
+    }
+    ARM_COMPUTE_ERROR_THROW_ON(validate(input->info(), bias != nullptr ? bias->info() : nullptr, output->info(), info));
+    Impl &s = *_impl;
+    s.src = input, s.bias = bias, s.dst = output;
+    const ITensorInfo *ii = input->info(), *oi = output->info();
+    // every dimension above x is a row as long as rows are evenly spaced
+    const size_t rows = ii->tensor_shape().total_size_upper(1);
+    for (size_t i = 2; i < ii->num_dimensions(); ++i)
+    {
+        ARM_COMPUTE_ERROR_ON_MSG(ii->strides_in_bytes()[i] != ii->dimension(i - 1) * ii->strides_in_bytes()[i - 1] ||
+                                     oi->strides_in_bytes()[i] != oi->dimension(i - 1) * oi->strides_in_bytes()[i - 1],
+                                 "padding between planes is not supported by the stand-alone output stage");
+    }
+    s.desc           = mi355_output_stage_desc{};
+    s.desc.M         = static_cast<int32_t>(rows);
+    s.desc.N         = static_cast<int32_t>(ii->dimension(0));
+    s.desc.ld_src    = ii->strides_in_bytes()[1] / ii->element_size();
+    s.desc.ld_dst    = oi->strides_in_bytes()[1] / oi->element_size();
+    s.desc.dst_dtype = to_mi355(oi->data_type());
+    s.desc.requant   = make_requant(info);
+    s.configured     = true;
+}
+
+void NEGEMMLowpOutputStage::run()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(!s.configured, "NEGEMMLowpOutputStage::run() before configure()");
+    ARM_COMPUTE_ERROR_ON_MSG(s.src->buffer() == nullptr || s.dst->buffer() == nullptr, "tensor without memory");
+    check_abi(mi355_output_stage_run(&s.desc, reinterpret_cast<const int32_t *>(first_element(s.src)),
+                                     s.bias ? reinterpret_cast<const int32_t *>(first_element(s.bias)) : nullptr,
+                                     first_element(s.dst), nullptr),
+              "NEGEMMLowpOutputStage::run");
+}
+
+// =====================================================================================================================
+// NEGEMMConvolutionLayer
+// =====================================================================================================================
+struct NEGEMMConvolutionLayer::Impl
+{
+    const ITensor       *src{nullptr}, *weights{nullptr}, *biases{nullptr};
+    ITensor             *dst{nullptr};
+    ActivationLayerInfo  act{};
+    mi355_conv_desc      desc{};
+    mi355_conv_handle   *handle{nullptr};
+    bool                 is_prepared{false};
+    std::vector<int32_t> multipliers, shifts;
+
+    ~Impl()
+    {
+        if (handle)
+            mi355_conv_destroy(handle);
+    }
+};
+
+NEGEMMConvolutionLayer::NEGEMMConvolutionLayer(const std::shared_ptr<IMemoryManager> &memory_manager,
+                                               IWeightsManager                       *weights_manager)
+    : _impl(std::make_unique<Impl>())
+{
+    ARM_COMPUTE_UNUSED(memory_manager, weights_manager);
+}
+NEGEMMConvolutionLayer::~NEGEMMConvolutionLayer() = default;
+
+namespace
+{
+// requantisation of a quantized convolution, as CpuGemmConv2d::configure_mm derives it
+// (src/cpu/operators/CpuGemmConv2d.cpp:266-313 of the reference)
+Status conv_output_stage(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *dst,
+                         const ActivationLayerInfo &act, GEMMLowpOutputStageInfo &out)
+{
+    const QuantizationInfo iq = src->quantization_info();
+    const QuantizationInfo wq = weights->quantization_info();
+    const QuantizationInfo oq = (dst->total_size() == 0) ? iq : dst->quantization_info();
+    const DataType         dt = src->data_type();
+    int32_t                lo = get_min_max(dt).first, hi = get_min_max(dt).second;
+    if (fusable_acts.count(act.activation()) != 0)
+        std::tie(lo, hi) = get_quantized_activation_min_max(act, dt, oq.uniform());
+    out.type                     = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    out.gemmlowp_offset          = oq.uniform().offset;
+    out.gemmlowp_min_bound       = lo;
+    out.gemmlowp_max_bound       = hi;
+    out.is_quantized_per_channel = weights->data_type() == DataType::QSYMM8_PER_CHANNEL;
+    return quantization::calculate_quantized_multipliers(iq, wq, oq, out);
+}
+} // namespace
+
+// src/cpu/operators/CpuGemmConv2d.cpp:697-856 of the reference, restricted to what this library builds
+Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorInfo *weights, const ITensorInfo *biases,
+                                        const ITensorInfo *output, const PadStrideInfo &conv_info,
+                                        const WeightsInfo &weights_info, const Size2D &dilation,
+                                        const ActivationLayerInfo &act_info, bool enable_fast_math,
+                                        unsigned int num_groups)
+{
+    ARM_COMPUTE_UNUSED(enable_fast_math);
+    ARM_COMPUTE_RETURN_ERROR_ON_NULLPTR(input, weights, output);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights_info.are_reshaped(), "Weights already reshaped are not supported!");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(is_one_of(input->data_type(), {DataType::BFLOAT16, DataType::F16, DataType::F32}),
+                                    "Floating-point convolution is not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(input->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}),
+                                    "Input must be QASYMM8 or QASYMM8_SIGNED");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(weights->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED,
+                                                                      DataType::QSYMM8_PER_CHANNEL}),
+                                    "Weights must be QASYMM8, QASYMM8_SIGNED or QSYMM8_PER_CHANNEL");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != weights->data_layout(), "Mismatching data layouts");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(num_groups > 1, "Grouping (num_groups != 1) is not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC, "Only the NHWC layout is built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_type() == DataType::QASYMM8_SIGNED && weights->data_type() == DataType::QASYMM8,
+                                    "QASYMM8_SIGNED input with QASYMM8 weights is not supported");
+    ARM_COMPUTE_RETURN_ERROR_ON(weights->dimension(0) != input->dimension(0)); // channels
+    ARM_COMPUTE_RETURN_ERROR_ON(weights->num_dimensions() > 4);
+    ARM_COMPUTE_RETURN_ERROR_ON(input->num_dimensions() > 4);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() != input->data_type(),
+                                    "Output must have the input's data type (the F32 destination is not built)");
+    if (biases != nullptr)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->data_type() != DataType::S32);
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->dimension(0) != weights->dimension(3));
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->num_dimensions() > 1);
+    }
+    if (weights->data_type() == DataType::QSYMM8_PER_CHANNEL)
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights->quantization_info().scale().size() != weights->dimension(3),
+                                        "One weight scale per output channel is required");
+    if (act_info.enabled())
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(fusable_acts.count(act_info.activation()) == 0,
+                                        "Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
+    unsigned int conv_w = 0, conv_h = 0;
+    std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(input->dimension(1)), static_cast<int>(input->dimension(2)),
+                                                 static_cast<int>(weights->dimension(1)), static_cast<int>(weights->dimension(2)),
+                                                 conv_info, dilation);
+    if (output->total_size() != 0)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(0) != weights->dimension(3));
+        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(1) != conv_w || output->dimension(2) != conv_h);
+        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(3) != input->dimension(3));
+    }
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->has_padding() || weights->has_padding() || output->has_padding(),
+                                    "Padded tensors are not supported by the convolution of this library");
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_RETURN_ON_ERROR(conv_output_stage(input, weights, output, act_info, stage));
+    return Status{};
+}
+
+Status NEGEMMConvolutionLayer::has_opt_impl(WeightFormat &expected_weight_format, const ITensorInfo *src,
+                                            const ITensorInfo *weights, const ITensorInfo *biases,
+                                            const ITensorInfo *dst, const PadStrideInfo &conv_info,
+                                            const WeightsInfo &weights_info, const Size2D &dilation,
+                                            const ActivationLayerInfo &act_info, bool enable_fast_math)
+{
+    // no fixed-format weights in this library: the packed layout is private to the device workspace
+    expected_weight_format = WeightFormat::UNSPECIFIED;
+    ARM_COMPUTE_RETURN_ON_ERROR(validate(src, weights, biases, dst, conv_info, weights_info, dilation, act_info,
+                                         enable_fast_math, 1));
+    ARM_COMPUTE_RETURN_ERROR_MSG("No fixed-format kernel available");
+}
+
+void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weights, const ITensor *biases,
+                                       ITensor *output, const PadStrideInfo &conv_info, const WeightsInfo &weights_info,
+                                       const Size2D &dilation, const ActivationLayerInfo &act_info,
+                                       bool enable_fast_math, unsigned int num_groups)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(input, weights, output);
+    const ITensorInfo *ii = input->info(), *wi = weights->info();
+    if (output->info()->total_size() == 0 && output->info()->is_resizable())
+    {
+        unsigned int conv_w = 0, conv_h = 0;
+        std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(ii->dimension(1)), static_cast<int>(ii->dimension(2)),
+                                                     static_cast<int>(wi->dimension(1)), static_cast<int>(wi->dimension(2)),
+                                                     conv_info, dilation);
+        const QuantizationInfo keep = output->info()->quantization_info();
+        output->info()->set_tensor_shape(TensorShape(wi->dimension(3), conv_w, conv_h, ii->dimension(3)));
+        output->info()->set_num_channels(1);
+        output->info()->set_data_type(ii->data_type());
+        output->info()->set_data_layout(ii->data_layout());
+        output->info()->set_quantization_info(keep.empty() ? ii->quantization_info() : keep);
+    }
+    ARM_COMPUTE_ERROR_THROW_ON(validate(ii, wi, biases != nullptr ? biases->info() : nullptr, output->info(), conv_info,
+                                        weights_info, dilation, act_info, enable_fast_math, num_groups));
+    Impl &s = *_impl;
+    if (s.handle)
+    {
+        mi355_conv_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.src = input, s.weights = weights, s.biases = biases, s.dst = output, s.act = act_info;
+    s.is_prepared = false;
+
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, output->info(), act_info, stage));
+    mi355_conv_desc &d = s.desc;
+    d                  = mi355_conv_desc{};
+    d.C = static_cast<int32_t>(ii->dimension(0)), d.W = static_cast<int32_t>(ii->dimension(1));
+    d.H = static_cast<int32_t>(ii->dimension(2)), d.batch = static_cast<int32_t>(ii->tensor_shape().total_size_upper(3));
+    d.KW = static_cast<int32_t>(wi->dimension(1)), d.KH = static_cast<int32_t>(wi->dimension(2));
+    d.OFM      = static_cast<int32_t>(wi->dimension(3));
+    d.stride_x = conv_info.stride().first, d.stride_y = conv_info.stride().second;
+    d.pad_left = conv_info.pad_left(), d.pad_top = conv_info.pad_top();
+    d.pad_right = conv_info.pad_right(), d.pad_bottom = conv_info.pad_bottom();
+    d.dilation_x = static_cast<int32_t>(dilation.x()), d.dilation_y = static_cast<int32_t>(dilation.y());
+    d.src_dtype = to_mi355(ii->data_type()), d.weights_dtype = to_mi355(wi->data_type());
+    d.dst_dtype = to_mi355(output->info()->data_type());
+    // the GEMM adds its offsets: hand it the negated zero points (CpuGemmConv2d.cpp:266-280 of the reference);
+    // im2col pads with the un-negated input zero point (src/cpu/kernels/directconv2d/impl.h:333-334)
+    const int32_t in_zp = ii->quantization_info().uniform().offset;
+    d.src_offset        = -in_zp;
+    d.weights_offset =
+        is_data_type_quantized_per_channel(wi->data_type()) ? 0 : -wi->quantization_info().uniform().offset;
+    d.pad_value = in_zp;
+    d.requant   = make_requant(stage);
+    d.path      = 0;
+    if (stage.is_quantized_per_channel)
+    {
+        s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
+        s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.OFM);
+    }
+    else
+        s.multipliers.clear(), s.shifts.clear();
+    check_abi(mi355_conv_create(&d, &s.handle), "NEGEMMConvolutionLayer::configure");
+}
+
+void NEGEMMConvolutionLayer::prepare()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMConvolutionLayer::prepare() before configure()");
+    if (s.is_prepared)
+        return;
+    ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");
+    check_abi(mi355_conv_prepare(s.handle, first_element(s.weights),
+                                 s.biases ? reinterpret_cast<const int32_t *>(first_element(s.biases)) : nullptr,
+                                 s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                 s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "NEGEMMConvolutionLayer::prepare");
+    s.weights->mark_as_unused();
+    s.is_prepared = true;
+}
+
+void NEGEMMConvolutionLayer::update_quantization_parameters()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "update_quantization_parameters() before configure()");
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(s.src->info(), s.weights->info(), s.dst->info(), s.act, stage));
+    const int32_t in_zp   = s.src->info()->quantization_info().uniform().offset;
+    s.desc.src_offset     = -in_zp;
+    s.desc.pad_value      = in_zp;
+    s.desc.weights_offset = is_data_type_quantized_per_channel(s.weights->info()->data_type())
+                                ? 0
+                                : -s.weights->info()->quantization_info().uniform().offset;
+    s.desc.requant = make_requant(stage);
+    if (stage.is_quantized_per_channel)
+    {
+        s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + s.desc.OFM);
+        s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + s.desc.OFM);
+    }
+    check_abi(mi355_conv_update_quant(s.handle, s.desc.src_offset, s.desc.weights_offset, s.desc.pad_value,
+                                      &s.desc.requant, s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                      s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "NEGEMMConvolutionLayer::update_quantization_parameters");
+}
+
+void NEGEMMConvolutionLayer::run()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMConvolutionLayer::run() before configure()");
+    ARM_COMPUTE_ERROR_ON_MSG(s.src->buffer() == nullptr || s.dst->buffer() == nullptr, "tensor without memory");
+    prepare();
+    check_abi(mi355_conv_run(s.handle, first_element(s.src), first_element(s.dst), nullptr), "NEGEMMConvolutionLayer::run");
+}
+
+const char *NEGEMMConvolutionLayer::kernel_name() const
+{
+    return _impl->handle ? mi355_conv_kernel_name(_impl->handle) : "";
+}
+} // namespace arm_compute

@@ -158,6 +158,10 @@ typedef struct mi355_conv_handle mi355_conv_handle;
 int  mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out);
 int  mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t *bias, const int32_t *mult,
                         const int32_t *shift, void *stream);
+/* Replaces CpuGemmConv2d::update_quantization_parameters (:858-908): new offsets, pad value and requantisation without
+ * touching the packed weights. mult / shift (OFM int32 each) are read only when requant->per_channel. */
+int  mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t weights_offset, int32_t pad_value,
+                             const mi355_requant *requant, const int32_t *mult, const int32_t *shift, void *stream);
 int  mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream);
 void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW);
 void mi355_conv_destroy(mi355_conv_handle *h);

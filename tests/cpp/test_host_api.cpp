@@ -1,0 +1,573 @@
+// Tests of the arm_compute-compatible host layer, written the way the reference's validation suites are
+// (tests/validation/NEON/GEMMLowp.cpp, ConvolutionLayer.cpp): build the function on real Tensors, fill them from a
+// seed, run, and compare against the oracle (oracle/gemmlowp_oracle.h) with tolerance zero.
+//   test_host_api --cpu   : validate() tables, TensorInfo layout, quantization helpers (no GPU needed)
+//   test_host_api --gpu   : configure / prepare / run on the device, host buffers and imported device buffers
+#include "arm_compute/core/utils/quantization/AsymmHelpers.h"
+#include "arm_compute/runtime/NEON/NEFunctions.h"
+#include "arm_compute/runtime/Tensor.h"
+#include "gemmlowp_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+using namespace arm_compute;
+
+static int g_failures = 0, g_checks = 0;
+#define EXPECT(cond)                                                              \
+    do                                                                            \
+    {                                                                             \
+        ++g_checks;                                                               \
+        if (!(cond))                                                              \
+        {                                                                         \
+            ++g_failures;                                                         \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);         \
+        }                                                                         \
+    } while (0)
+#define SECTION(name) std::printf("[case] %s\n", name), std::fflush(stdout)
+
+// ---------------------------------------------------------------------------------------------------------------------
+static void test_tensor_info()
+{
+    SECTION("TensorInfo strides, padding, shapes");
+    TensorInfo info(TensorShape(21U, 13U), 1, DataType::QASYMM8);
+    EXPECT(info.dimension(0) == 21 && info.dimension(1) == 13 && info.num_dimensions() == 2);
+    EXPECT(info.strides_in_bytes()[0] == 1 && info.strides_in_bytes()[1] == 21 && info.total_size() == 21 * 13);
+    EXPECT(info.offset_first_element_in_bytes() == 0);
+    info.extend_padding(PaddingSize(0, 3, 0, 2)); // top, right, bottom, left
+    EXPECT(info.strides_in_bytes()[1] == 26 && info.offset_first_element_in_bytes() == 2 && info.has_padding());
+    TensorInfo s32(TensorShape(33U, 13U, 4U), 1, DataType::S32);
+    EXPECT(s32.element_size() == 4 && s32.strides_in_bytes()[1] == 132 && s32.strides_in_bytes()[2] == 132 * 13);
+    EXPECT(s32.total_size() == 132u * 13 * 4);
+    EXPECT(TensorShape(5U, 1U, 1U).num_dimensions() == 1); // trailing ones are not counted
+    EXPECT(TensorShape(5U, 3U, 2U).total_size_upper(1) == 6);
+    EXPECT(info.clone()->set_is_resizable(false).is_resizable() == false);
+    TensorInfo nhwc(TensorShape(64U, 56U, 48U, 2U), 1, DataType::QASYMM8_SIGNED, DataLayout::NHWC);
+    EXPECT(nhwc.dimension(DataLayoutDimension::CHANNEL) == 64 && nhwc.dimension(DataLayoutDimension::WIDTH) == 56 &&
+           nhwc.dimension(DataLayoutDimension::HEIGHT) == 48 && nhwc.dimension(DataLayoutDimension::BATCHES) == 2);
+    QuantizationInfo q(0.5f, -3);
+    EXPECT(q.uniform().scale == 0.5f && q.uniform().offset == -3 && !q.is_dynamic());
+    QuantizationInfo pc(std::vector<float>{0.1f, 0.2f});
+    EXPECT(pc.scale().size() == 2 && pc.offset().empty() && pc.uniform().offset == 0);
+}
+
+static void test_quant_helpers()
+{
+    SECTION("calculate_quantized_multiplier against the oracle");
+    std::mt19937                          rng(7);
+    std::uniform_real_distribution<float> u(std::log(1e-6f), std::log(8.f));
+    for (int i = 0; i < 20000; ++i)
+    {
+        const float real = std::exp(u(rng));
+        int32_t     m = 0, s = 0, om = 0, os = 0;
+        const bool  ok  = bool(quantization::calculate_quantized_multiplier(real, &m, &s));
+        const bool  ook = orc_calculate_quantized_multiplier(real, &om, &os) == 0;
+        EXPECT(ok == ook);
+        if (ok && ook)
+            EXPECT(m == om && s == os);
+    }
+    int32_t m = 0, s = 0;
+    EXPECT(bool(quantization::calculate_quantized_multiplier(0.0007f, &m, &s)) && m == 1539316224 && s == 10);
+    EXPECT(bool(quantization::calculate_quantized_multiplier(1.0f, &m, &s)) && m == (1 << 30) && s == -1);
+    EXPECT(!bool(quantization::calculate_quantized_multiplier(-0.5f, &m, &s)));
+
+    SECTION("calculate_quantized_multipliers pads per-channel vectors by 32");
+    GEMMLowpOutputStageInfo st;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(QuantizationInfo(0.02f, 1),
+                                                              QuantizationInfo(std::vector<float>{0.1f, 0.5f, 0.9f}),
+                                                              QuantizationInfo(0.5f, 3), st)));
+    EXPECT(st.gemmlowp_multipliers.size() == 3 + 32 && st.gemmlowp_shifts.size() == 3 + 32);
+    EXPECT(st.gemmlowp_multiplier == st.gemmlowp_multipliers[0] && st.gemmlowp_shift == st.gemmlowp_shifts[0]);
+
+    SECTION("get_quantized_activation_min_max");
+    const UniformQuantizationInfo oq(0.1f, 10);
+    auto r = get_quantized_activation_min_max(ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU),
+                                              DataType::QASYMM8, oq);
+    EXPECT(r.first == 10 && r.second == 255);
+    r = get_quantized_activation_min_max(ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 6.f),
+                                         DataType::QASYMM8, oq);
+    EXPECT(r.first == 10 && r.second == 70);
+    r = get_quantized_activation_min_max(
+        ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU, 6.f, -1.f), DataType::QASYMM8_SIGNED, oq);
+    EXPECT(r.first == 0 && r.second == 70);
+    auto d = scaled_dimensions(56, 56, 3, 3, PadStrideInfo(1, 1, 1, 1));
+    EXPECT(d.first == 56 && d.second == 56);
+    d = scaled_dimensions(23, 27, 3, 3, PadStrideInfo(2, 1, 0, 0));
+    EXPECT(d.first == 11 && d.second == 25);
+}
+
+// the reference's own validate tables: tests/validation/NEON/GEMMLowp.cpp:168-200 and :533-568
+static void test_validate_tables()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore::validate table (S32)");
+    const QuantizationInfo qa(1.f / 255, 10), qb(1.f / 256, 10);
+    struct Row
+    {
+        TensorInfo a, b, o;
+        bool       expected;
+    };
+    const std::vector<Row> rows = {
+        {TensorInfo(TensorShape(21U, 13U), 1, DataType::QASYMM8, qa), TensorInfo(TensorShape(33U, 21U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(33U, 13U), 1, DataType::S32), true},
+        {TensorInfo(TensorShape(21U, 13U), 1, DataType::S32), TensorInfo(TensorShape(33U, 21U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(33U, 13U), 1, DataType::S32), false},
+        {TensorInfo(TensorShape(20U, 13U), 1, DataType::QASYMM8, qa), TensorInfo(TensorShape(33U, 21U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(33U, 13U), 1, DataType::S32), false},
+        {TensorInfo(TensorShape(21U, 13U), 1, DataType::QASYMM8, qa), TensorInfo(TensorShape(33U, 21U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(8U, 11U), 1, DataType::S32), false},
+        {TensorInfo(TensorShape(16U, 32U), 1, DataType::QASYMM8, qa), TensorInfo(TensorShape(64U, 16U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(64U, 32U), 1, DataType::S32), true},
+        {TensorInfo(TensorShape(16U, 32U), 1, DataType::QASYMM8_SIGNED, qa), TensorInfo(TensorShape(64U, 16U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(64U, 32U), 1, DataType::S32), false},
+    };
+    for (const Row &r : rows)
+    {
+        const Status st = NEGEMMLowpMatrixMultiplyCore::validate(&r.a.clone()->set_is_resizable(false),
+                                                                 &r.b.clone()->set_is_resizable(false), nullptr,
+                                                                 &r.o.clone()->set_is_resizable(false));
+        EXPECT(bool(st) == r.expected);
+    }
+    SECTION("NEGEMMLowpMatrixMultiplyCore::validate table (F32 dequant)");
+    const std::vector<Row> frows = {
+        {TensorInfo(TensorShape(16U, 32U), 1, DataType::QASYMM8, qa), TensorInfo(TensorShape(64U, 16U), 1, DataType::QASYMM8_SIGNED, qb),
+         TensorInfo(TensorShape(64U, 32U), 1, DataType::F32), true},
+        {TensorInfo(TensorShape(16U, 32U), 1, DataType::QASYMM8_SIGNED, qa), TensorInfo(TensorShape(64U, 16U), 1, DataType::QASYMM8_SIGNED, qb),
+         TensorInfo(TensorShape(64U, 32U), 1, DataType::F32), true},
+        {TensorInfo(TensorShape(16U, 32U), 1, DataType::QASYMM8_SIGNED, qa), TensorInfo(TensorShape(64U, 16U), 1, DataType::QASYMM8, qb),
+         TensorInfo(TensorShape(64U, 32U), 1, DataType::F32), false},
+    };
+    for (const Row &r : frows)
+        EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(&r.a, &r.b, nullptr, &r.o)) == r.expected);
+
+    SECTION("validate: bias, reshape flags, accumulate, output stage rules");
+    const TensorInfo a(TensorShape(16U, 32U), 1, DataType::QASYMM8, qa), b(TensorShape(64U, 16U), 1, DataType::QASYMM8, qb);
+    const TensorInfo o32(TensorShape(64U, 32U), 1, DataType::S32), o8(TensorShape(64U, 32U), 1, DataType::QASYMM8, qa);
+    const TensorInfo bias(TensorShape(64U), 1, DataType::S32), bias_bad(TensorShape(63U), 1, DataType::S32);
+    // bias with S32 output and no output stage: CpuGemmLowpMatrixMultiplyCore.cpp:376-378
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o32)));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o32, GEMMInfo(true, false, true))));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o32, GEMMInfo(false, true, true))));
+    GEMMInfo pre;
+    pre.set_pretranspose_B(true);
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o32, pre)));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o8))); // quantized output without a stage
+    GEMMLowpOutputStageInfo st;
+    st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    st.gemmlowp_multiplier = 1518500250, st.gemmlowp_shift = 8, st.gemmlowp_offset = 10;
+    st.gemmlowp_min_bound = 0, st.gemmlowp_max_bound = 255, st.output_data_type = DataType::QASYMM8;
+    GEMMInfo fused(false, false, true, 0, false, false, st);
+    EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, fused)));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias_bad, &o8, fused)));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o32, fused)));
+    st.gemmlowp_min_bound = 5, st.gemmlowp_max_bound = 4;
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, GEMMInfo(false, false, true, 0, false, false, st))));
+    GEMMInfo acc;
+    acc.set_accumulate(true);
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o8, acc)));
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(nullptr, &b, nullptr, &o32)));
+
+    SECTION("NEGEMMLowpOutputStage::validate");
+    GEMMLowpOutputStageInfo os;
+    os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    os.gemmlowp_multiplier = 1 << 30, os.gemmlowp_shift = 3, os.gemmlowp_min_bound = 0, os.gemmlowp_max_bound = 255;
+    os.output_data_type = DataType::QASYMM8;
+    EXPECT(bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o8, &bias, &o8, os)));       // src must be S32
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias_bad, &o8, os)));  // bias length
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o32, os)));     // dst type
+    os.type = GEMMLowpOutputStageType::NONE;
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
+    os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    os.gemmlowp_min_bound = 9, os.gemmlowp_max_bound = 1;
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
+
+    SECTION("NEGEMMConvolutionLayer::validate");
+    TensorInfo src(TensorShape(64U, 8U, 8U, 2U), 1, DataType::QASYMM8_SIGNED, QuantizationInfo(0.02f, -1));
+    TensorInfo w(TensorShape(64U, 3U, 3U, 32U), 1, DataType::QSYMM8_PER_CHANNEL, QuantizationInfo(std::vector<float>(32, 0.01f)));
+    TensorInfo cb(TensorShape(32U), 1, DataType::S32);
+    TensorInfo dst(TensorShape(32U, 8U, 8U, 2U), 1, DataType::QASYMM8_SIGNED, QuantizationInfo(0.5f, -5));
+    for (TensorInfo *t : {&src, &w, &dst})
+        t->set_data_layout(DataLayout::NHWC);
+    const PadStrideInfo ps(1, 1, 1, 1);
+    EXPECT(bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb, &dst, ps)));
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb, &dst, ps, WeightsInfo(true, 3, 3, 32))));
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb, &dst, ps, WeightsInfo(), Size2D(1, 1), ActivationLayerInfo(), false, 2)));
+    TensorInfo w_badc(TensorShape(32U, 3U, 3U, 32U), 1, DataType::QSYMM8_PER_CHANNEL, QuantizationInfo(std::vector<float>(32, 0.01f)));
+    w_badc.set_data_layout(DataLayout::NHWC);
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w_badc, &cb, &dst, ps)));
+    TensorInfo cb_bad(TensorShape(31U), 1, DataType::S32);
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb_bad, &dst, ps)));
+    TensorInfo dst_bad(TensorShape(32U, 7U, 8U, 2U), 1, DataType::QASYMM8_SIGNED, QuantizationInfo(0.5f, -5));
+    dst_bad.set_data_layout(DataLayout::NHWC);
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb, &dst_bad, ps)));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// GPU tests
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename T>
+static void fill_uniform(Tensor &t, int lo, int hi, unsigned seed)
+{
+    // element-wise through the tensor's strides, so padded tensors are filled correctly
+    std::mt19937                       rng(seed);
+    std::uniform_int_distribution<int> u(lo, hi);
+    const ITensorInfo                 *i = t.info();
+    const size_t rows = i->tensor_shape().total_size_upper(1);
+    for (size_t r = 0; r < rows; ++r)
+    {
+        // decompose r into coordinates of dims 1..5
+        size_t  rem = r;
+        int32_t off = static_cast<int32_t>(i->offset_first_element_in_bytes());
+        for (size_t d = 1; d < MAX_DIMS; ++d)
+        {
+            const size_t dim = i->tensor_shape()[d];
+            off += static_cast<int32_t>((rem % dim) * i->strides_in_bytes()[d]);
+            rem /= dim;
+        }
+        T *row = reinterpret_cast<T *>(t.buffer() + off);
+        for (size_t x = 0; x < i->dimension(0); ++x)
+            row[x] = static_cast<T>(u(rng));
+    }
+}
+
+template <typename T>
+static std::vector<T> dense_copy(const Tensor &t)
+{
+    const ITensorInfo *i = t.info();
+    std::vector<T>     out(i->tensor_shape().total_size());
+    const size_t       rows = i->tensor_shape().total_size_upper(1), w = i->dimension(0);
+    for (size_t r = 0; r < rows; ++r)
+    {
+        size_t  rem = r;
+        int32_t off = static_cast<int32_t>(i->offset_first_element_in_bytes());
+        for (size_t d = 1; d < MAX_DIMS; ++d)
+        {
+            const size_t dim = i->tensor_shape()[d];
+            off += static_cast<int32_t>((rem % dim) * i->strides_in_bytes()[d]);
+            rem /= dim;
+        }
+        std::memcpy(out.data() + r * w, t.buffer() + off, w * sizeof(T));
+    }
+    return out;
+}
+
+static void init_tensor(Tensor &t, const TensorShape &shape, DataType dt, const QuantizationInfo &q = QuantizationInfo(),
+                        const PaddingSize &pad = PaddingSize(0))
+{
+    TensorInfo info(shape, 1, dt, q);
+    t.allocator()->init(info);
+    if (!pad.empty())
+        t.info()->extend_padding(pad);
+}
+
+// the flow of examples/neon_gemm_qasymm8.cpp of the reference: configure first, allocate afterwards, run twice
+static void test_gemmlowp_fused_u8(bool padded)
+{
+    SECTION(padded ? "NEGEMMLowpMatrixMultiplyCore fused QASYMM8 (x-padded tensors)" : "NEGEMMLowpMatrixMultiplyCore fused QASYMM8");
+    const int   M = 72, N = 33, K = 52;
+    Tensor      a, b, bias, dst;
+    const PaddingSize pad = padded ? PaddingSize(0, 5, 0, 3) : PaddingSize(0);
+    init_tensor(a, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(1.f / 255, -9), pad);
+    init_tensor(b, TensorShape(N, K), DataType::QASYMM8, QuantizationInfo(1.f / 255, 1), pad);
+    init_tensor(bias, TensorShape(N), DataType::S32);
+    init_tensor(dst, TensorShape(N, M), DataType::QASYMM8, QuantizationInfo(0.3f, 10), pad);
+    GEMMLowpOutputStageInfo st;
+    st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    st.gemmlowp_multiplier = 1518500250, st.gemmlowp_shift = 8, st.gemmlowp_offset = 10;
+    st.gemmlowp_min_bound = 0, st.gemmlowp_max_bound = 255, st.output_data_type = DataType::QASYMM8;
+    NEGEMMLowpMatrixMultiplyCore gemm;
+    gemm.configure(&a, &b, &bias, &dst, GEMMInfo(false, false, true, 0, false, false, st));
+    a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<uint8_t>(a, 0, 255, 1), fill_uniform<uint8_t>(b, 0, 255, 2), fill_uniform<int32_t>(bias, -1000, 1000, 3);
+    const auto A = dense_copy<uint8_t>(a), B = dense_copy<uint8_t>(b);
+    const auto C = dense_copy<int32_t>(bias);
+    std::vector<uint8_t> want(M * N);
+    const int32_t mult = st.gemmlowp_multiplier, shift = st.gemmlowp_shift;
+    orc_gemmlowp_fixedpoint(A.data(), 0, K, B.data(), 0, N, C.data(), want.data(), N, 0, M, N, K, -9, 1, &mult, &shift, 1, 10, 0, 255);
+    gemm.run();
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    EXPECT(!b.is_used()); // B was packed once and handed back (NEGEMMLowpMatrixMultiplyCore.cpp:176-183 of the reference)
+    // run again with a new A: identical function object, new data
+    fill_uniform<uint8_t>(a, 0, 255, 11);
+    const auto A2 = dense_copy<uint8_t>(a);
+    orc_gemmlowp_fixedpoint(A2.data(), 0, K, B.data(), 0, N, C.data(), want.data(), N, 0, M, N, K, -9, 1, &mult, &shift, 1, 10, 0, 255);
+    gemm.run();
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    std::printf("       kernel: %s\n", gemm.kernel_name());
+}
+
+static void test_gemmlowp_s32_batched()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore S32 output, batched, non-constant B");
+    const int M = 17, N = 29, K = 15, batch = 3;
+    Tensor    a, b, dst;
+    init_tensor(a, TensorShape(K, M, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.1f, 5));
+    init_tensor(b, TensorShape(N, K, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.2f, -7));
+    init_tensor(dst, TensorShape(N, M, batch), DataType::S32);
+    a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+    NEGEMMLowpMatrixMultiplyCore gemm;
+    gemm.configure(&a, &b, nullptr, &dst, GEMMInfo(false, false, false /* B changes between runs */));
+    for (int rep = 0; rep < 2; ++rep)
+    {
+        fill_uniform<int8_t>(a, -128, 127, 20 + rep), fill_uniform<int8_t>(b, -128, 127, 30 + rep);
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        std::vector<int32_t> want(batch * M * N);
+        for (int z = 0; z < batch; ++z)
+            orc_gemmlowp_s32(A.data() + z * M * K, 1, K, B.data() + z * K * N, 1, N, want.data() + z * M * N, N, M, N, K, 5, -7);
+        gemm.run();
+        EXPECT(dense_copy<int32_t>(dst) == want);
+        EXPECT(b.is_used());
+    }
+}
+
+static void test_gemmlowp_per_channel_and_update()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore per-channel QSYMM8_PER_CHANNEL rhs");
+    const int M = 150, N = 130, K = 208;
+    std::mt19937 rng(5);
+    std::uniform_real_distribution<float> us(1e-4f, 2e-2f);
+    std::vector<float> wscale(N);
+    for (auto &v : wscale)
+        v = us(rng);
+    Tensor a, b, bias, dst;
+    init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(0.05f, -3)); // offsets are ADDED: zero point 3
+    init_tensor(b, TensorShape(N, K), DataType::QSYMM8_PER_CHANNEL, QuantizationInfo(wscale));
+    init_tensor(bias, TensorShape(N), DataType::S32);
+    init_tensor(dst, TensorShape(N, M), DataType::QASYMM8_SIGNED, QuantizationInfo(0.7f, -5));
+    GEMMLowpOutputStageInfo st;
+    st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    st.gemmlowp_offset = -5, st.gemmlowp_min_bound = -128, st.gemmlowp_max_bound = 127;
+    st.is_quantized_per_channel = true, st.output_data_type = DataType::QASYMM8_SIGNED;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(QuantizationInfo(0.05f, 3), QuantizationInfo(wscale),
+                                                              QuantizationInfo(0.7f, -5), st)));
+    a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int8_t>(a, -128, 127, 41), fill_uniform<int8_t>(b, -127, 127, 42), fill_uniform<int32_t>(bias, -2000, 2000, 43);
+    NEGEMMLowpMatrixMultiplyCore gemm;
+    gemm.configure(&a, &b, &bias, &dst, GEMMInfo(false, false, true, 0, false, false, st));
+    gemm.run();
+    const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+    const auto C = dense_copy<int32_t>(bias);
+    std::vector<int8_t> want(M * N);
+    orc_gemmlowp_fixedpoint(A.data(), 1, K, B.data(), 1, N, C.data(), want.data(), N, 1, M, N, K, -3, 0,
+                            st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(), N, -5, -128, 127);
+    EXPECT(dense_copy<int8_t>(dst) == want);
+
+    SECTION("update_quantization_parameters (per tensor) after configure");
+    Tensor a2, b2, dst2;
+    init_tensor(a2, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(0.05f, 2));
+    init_tensor(b2, TensorShape(N, K), DataType::QASYMM8, QuantizationInfo(0.01f, 4));
+    init_tensor(dst2, TensorShape(N, M), DataType::QASYMM8, QuantizationInfo(0.9f, 7));
+    GEMMLowpOutputStageInfo st2;
+    st2.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    st2.gemmlowp_multiplier = 1 << 30, st2.gemmlowp_shift = 12, st2.gemmlowp_offset = 0;
+    st2.gemmlowp_min_bound = 0, st2.gemmlowp_max_bound = 255, st2.output_data_type = DataType::QASYMM8;
+    a2.allocator()->allocate(), b2.allocator()->allocate(), dst2.allocator()->allocate();
+    fill_uniform<uint8_t>(a2, 0, 255, 51), fill_uniform<uint8_t>(b2, 0, 255, 52);
+    NEGEMMLowpMatrixMultiplyCore g2;
+    g2.configure(&a2, &b2, nullptr, &dst2, GEMMInfo(false, false, true, 0, false, false, st2));
+    g2.run();
+    // new quantization on the tensors, as the reference's UpdateStaticQuantInfoAfterConfigure tests do
+    a2.info()->set_quantization_info(QuantizationInfo(0.04f, -100));
+    b2.info()->set_quantization_info(QuantizationInfo(0.02f, -120));
+    dst2.info()->set_quantization_info(QuantizationInfo(1.3f, 17));
+    g2.update_quantization_parameters();
+    g2.run();
+    int32_t m = 0, s = 0;
+    EXPECT(bool(quantization::calculate_quantized_multiplier(0.04f * 0.02f / 1.3f, &m, &s)));
+    const auto A2 = dense_copy<uint8_t>(a2), B2 = dense_copy<uint8_t>(b2);
+    std::vector<uint8_t> want2(M * N);
+    orc_gemmlowp_fixedpoint(A2.data(), 0, K, B2.data(), 0, N, nullptr, want2.data(), N, 0, M, N, K, -100, -120, &m, &s, 1, 17, 0, 255);
+    EXPECT(dense_copy<uint8_t>(dst2) == want2);
+}
+
+static void test_gemmlowp_f32()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore F32 dequantized output with F32 bias and fused RELU");
+    const int M = 40, N = 65, K = 1000;
+    Tensor    a, b, bias, dst;
+    init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(0.02f, 3));
+    init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(0.005f, -2));
+    init_tensor(bias, TensorShape(N), DataType::F32);
+    init_tensor(dst, TensorShape(N, M), DataType::F32);
+    a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int8_t>(a, -128, 127, 61), fill_uniform<int8_t>(b, -128, 127, 62);
+    std::mt19937 rng(63);
+    std::normal_distribution<float> nd(0.f, 2.f);
+    for (int j = 0; j < N; ++j)
+        reinterpret_cast<float *>(bias.buffer())[j] = nd(rng);
+    GEMMInfo info(false, false, true, 0, false, false, GEMMLowpOutputStageInfo(), false, false, false,
+                  ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU));
+    NEGEMMLowpMatrixMultiplyCore gemm;
+    gemm.configure(&a, &b, &bias, &dst, info);
+    gemm.run();
+    const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+    std::vector<float> want(M * N);
+    orc_gemmlowp_f32(A.data(), 1, K, B.data(), 1, N, reinterpret_cast<const float *>(bias.buffer()), want.data(), N, M, N, K, 3,
+                     -2, 0.02f * 0.005f, 0.f, INFINITY);
+    const auto got = dense_copy<float>(dst);
+    bool       ok  = true;
+    for (size_t i = 0; i < want.size(); ++i)
+        ok = ok && std::fabs(got[i] - want[i]) <= 1e-5f * std::fabs(want[i]) + 1e-30f; // the stated 1e-5 relative bar
+    EXPECT(ok);
+    EXPECT(got == want); // and in fact identical bits: same float operations in the same order
+}
+
+static void test_output_stage()
+{
+    SECTION("NEGEMMLowpOutputStage S32 -> QASYMM8_SIGNED with bias (output auto-initialised)");
+    const int M = 13, N = 130;
+    Tensor    src, bias, dst;
+    init_tensor(src, TensorShape(N, M), DataType::S32);
+    init_tensor(bias, TensorShape(N), DataType::S32);
+    GEMMLowpOutputStageInfo os;
+    os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    os.gemmlowp_multiplier = 1288490240, os.gemmlowp_shift = 4, os.gemmlowp_offset = -3;
+    os.gemmlowp_min_bound = -100, os.gemmlowp_max_bound = 120, os.output_data_type = DataType::QASYMM8_SIGNED;
+    NEGEMMLowpOutputStage stage;
+    stage.configure(&src, &bias, &dst, os);
+    EXPECT(dst.info()->data_type() == DataType::QASYMM8_SIGNED && dst.info()->dimension(0) == (size_t)N);
+    src.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int32_t>(src, -6000, 6000, 71), fill_uniform<int32_t>(bias, -6000, 6000, 72);
+    stage.run();
+    std::vector<int8_t> want(M * N);
+    orc_output_stage_fixedpoint(reinterpret_cast<const int32_t *>(src.buffer()), N, reinterpret_cast<const int32_t *>(bias.buffer()),
+                                want.data(), N, 1, M, N, &os.gemmlowp_multiplier, &os.gemmlowp_shift, 1, -3, -100, 120);
+    EXPECT(dense_copy<int8_t>(dst) == want);
+}
+
+static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act)
+{
+    SECTION(per_channel ? "NEGEMMConvolutionLayer NHWC per-channel weights" : "NEGEMMConvolutionLayer NHWC per-tensor weights");
+    const bool is_signed = dt == DataType::QASYMM8_SIGNED;
+    const int  batch = 2, H = 9, W = 8, OFM = 24, KH = 3, KW = 3;
+    const int  in_zp = is_signed ? -1 : 127, out_zp = is_signed ? -5 : 9, w_zp = (per_channel || is_signed) ? 0 : 120;
+    std::mt19937 rng(81);
+    std::uniform_real_distribution<float> us(0.01f, 1.f);
+    std::vector<float> wscale(per_channel ? OFM : 1);
+    for (auto &v : wscale)
+        v = us(rng) * 0.05f;
+    Tensor src, w, bias, dst;
+    init_tensor(src, TensorShape(C, W, H, batch), dt, QuantizationInfo(0.02f, in_zp));
+    init_tensor(w, TensorShape(C, KW, KH, OFM), per_channel ? DataType::QSYMM8_PER_CHANNEL : dt,
+                per_channel ? QuantizationInfo(wscale) : QuantizationInfo(wscale[0], w_zp));
+    init_tensor(bias, TensorShape(OFM), DataType::S32);
+    init_tensor(dst, TensorShape(), dt, QuantizationInfo(0.9f, out_zp)); // shape filled in by configure()
+    for (Tensor *t : {&src, &w, &dst})
+        t->info()->set_data_layout(DataLayout::NHWC);
+    NEGEMMConvolutionLayer conv;
+    conv.configure(&src, &w, &bias, &dst, PadStrideInfo(1, 1, 1, 1), WeightsInfo(), Size2D(1, 1), act);
+    EXPECT(dst.info()->dimension(0) == (size_t)OFM && dst.info()->dimension(1) == (size_t)W && dst.info()->dimension(2) == (size_t)H);
+    src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    if (is_signed)
+        fill_uniform<int8_t>(src, -128, 127, 82);
+    else
+        fill_uniform<uint8_t>(src, 0, 255, 82);
+    if (per_channel || is_signed)
+        fill_uniform<int8_t>(w, -127, 127, 83);
+    else
+        fill_uniform<uint8_t>(w, 0, 255, 83);
+    fill_uniform<int32_t>(bias, -500, 500, 84);
+    conv.run();
+    EXPECT(!w.is_used());
+    // expected: direct convolution of the oracle with the multipliers the reference's helper derives
+    GEMMLowpOutputStageInfo st;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(
+        QuantizationInfo(0.02f, in_zp), per_channel ? QuantizationInfo(wscale) : QuantizationInfo(wscale[0], w_zp),
+        QuantizationInfo(0.9f, out_zp), st)));
+    int32_t lo = is_signed ? -128 : 0, hi = is_signed ? 127 : 255;
+    if (act.enabled())
+        std::tie(lo, hi) = get_quantized_activation_min_max(act, dt, UniformQuantizationInfo(0.9f, out_zp));
+    std::vector<uint8_t> want(batch * H * W * OFM);
+    orc_conv_nhwc_direct(src.buffer(), is_signed, w.buffer(), (per_channel || is_signed) ? 1 : 0,
+                         reinterpret_cast<const int32_t *>(bias.buffer()), want.data(), is_signed, batch, H, W, C, OFM, KH, KW,
+                         1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp, st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(),
+                         per_channel ? OFM : 1, out_zp, lo, hi);
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    std::printf("       kernel: %s\n", conv.kernel_name());
+
+    // new output quantization after configure
+    dst.info()->set_quantization_info(QuantizationInfo(1.7f, out_zp + 2));
+    conv.update_quantization_parameters();
+    conv.run();
+    EXPECT(bool(quantization::calculate_quantized_multipliers(
+        QuantizationInfo(0.02f, in_zp), per_channel ? QuantizationInfo(wscale) : QuantizationInfo(wscale[0], w_zp),
+        QuantizationInfo(1.7f, out_zp + 2), st)));
+    lo = is_signed ? -128 : 0, hi = is_signed ? 127 : 255;
+    if (act.enabled())
+        std::tie(lo, hi) = get_quantized_activation_min_max(act, dt, UniformQuantizationInfo(1.7f, out_zp + 2));
+    orc_conv_nhwc_direct(src.buffer(), is_signed, w.buffer(), (per_channel || is_signed) ? 1 : 0,
+                         reinterpret_cast<const int32_t *>(bias.buffer()), want.data(), is_signed, batch, H, W, C, OFM, KH, KW,
+                         1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp, st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(),
+                         per_channel ? OFM : 1, out_zp + 2, lo, hi);
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+}
+
+static void test_error_paths()
+{
+    SECTION("configure() throws on invalid input; run() before configure() throws");
+    Tensor a, b, dst;
+    init_tensor(a, TensorShape(20U, 13U), DataType::QASYMM8, QuantizationInfo(1.f, 0));
+    init_tensor(b, TensorShape(33U, 21U), DataType::QASYMM8, QuantizationInfo(1.f, 0));
+    init_tensor(dst, TensorShape(33U, 13U), DataType::S32);
+    NEGEMMLowpMatrixMultiplyCore gemm;
+    bool threw = false;
+    try
+    {
+        gemm.configure(&a, &b, nullptr, &dst);
+    }
+    catch (const std::runtime_error &)
+    {
+        threw = true;
+    }
+    EXPECT(threw);
+    threw = false;
+    try
+    {
+        gemm.run();
+    }
+    catch (const std::runtime_error &)
+    {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
+int main(int argc, char **argv)
+{
+    const std::string mode = argc > 1 ? argv[1] : "--cpu";
+    try
+    {
+        if (mode == "--cpu")
+        {
+            test_tensor_info();
+            test_quant_helpers();
+            test_validate_tables();
+            test_error_paths();
+        }
+        else
+        {
+            test_gemmlowp_fused_u8(false);
+            test_gemmlowp_fused_u8(true);
+            test_gemmlowp_s32_batched();
+            test_gemmlowp_per_channel_and_update();
+            test_gemmlowp_f32();
+            test_output_stage();
+            test_convolution(DataType::QASYMM8_SIGNED, true, 64, ActivationLayerInfo());
+            test_convolution(DataType::QASYMM8_SIGNED, false, 16, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU));
+            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
+            test_convolution(DataType::QASYMM8, true, 32,
+                             ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
+        }
+    }
+    catch (const std::exception &e)
+    {
+        std::printf("FAILED: unexpected exception: %s\n", e.what());
+        ++g_failures;
+    }
+    std::printf("%d checks, %d failures\n", g_checks, g_failures);
+    return g_failures == 0 ? 0 : 1;
+}

@@ -61,6 +61,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check against it")
     ap.add_argument("--no-secondary", action="store_true", help="skip the M=8 bandwidth measurement")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 256 MiB device-to-device copy a few times (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -73,6 +76,16 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
+
+    if args.copy_calibration:
+        src = torch.arange(64 * 1024 * 1024, dtype=torch.int32, device="cuda")  # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(max(args.steps, 1)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4,
+                          "launches": max(args.steps, 1)}))
+        return
 
     M, N, K = 2048, 4096, 4096
     A, B, bias, mult, shift = synth_config2(M, N, K)
@@ -108,7 +121,7 @@ def main():
         import oracle
         fg = oracle.FastGemm(B)
         reps, cpu_s, want = 0, 0.0, None
-        while cpu_s < 10.0 and reps < 40:
+        while cpu_s < 10.0 and reps < 400:
             t0 = time.perf_counter()
             want = fg.run(A, bias, -3, 0, mult, shift, -5, -128, 127, np.int8)
             cpu_s += time.perf_counter() - t0

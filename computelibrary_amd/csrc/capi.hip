@@ -145,6 +145,7 @@ struct GemmCore
     std::string kname;
     DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp;
     bool    qp_ok = false; // all multipliers >= 0: the branch-free epilogue applies
+    bool    qp_std = false; // ... and every column has a normalised multiplier (>= 2^30) and a right shift of 2..31
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
 
@@ -255,7 +256,7 @@ struct GemmCore
     // digest multipliers / shifts for the pipelined kernel's epilogue; synchronises the stream to learn whether it applies
     int refresh_qparams(hipStream_t s)
     {
-        qp_ok = false;
+        qp_ok = qp_std = false;
         if (epi != EPI_FIXEDPOINT)
             return 0;
         TRY(qp.ensure(sizeof(int32_t) * ((size_t)QP_COUNT * Np + 4)));
@@ -265,13 +266,15 @@ struct GemmCore
         int32_t neg = 1;
         HIP_TRY(hipMemcpyAsync(&neg, flag, sizeof(neg), hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
-        qp_ok = neg == 0;
+        qp_ok  = (neg & 1) == 0;
+        qp_std = neg == 0;
         return 0;
     }
 
     void fill_epi(EpiParams &p, const float *bias_f32) const
     {
         p.qp                  = qp_ok ? qp.as<int32_t>() : nullptr;
+        p.qp_std              = (qp_ok && qp_std && rq.result_offset > -(1 << 28) && rq.result_offset < (1 << 28)) ? 1 : 0;
         p.qp_stride           = Np;
         p.colvec              = colvec.as<int32_t>();
         p.rowvec              = nullptr;
@@ -339,6 +342,7 @@ struct GemmCore
     {
         const size_t esz = (epi == EPI_FIXEDPOINT) ? 1 : 4;
         g.epi.vec_store  = (((uintptr_t)g.D % (4 * esz)) == 0 && g.ldd % 4 == 0 && g.d_batch_stride % 4 == 0) ? 1 : 0;
+        g.epi.vec_store16 = (esz == 1 && ((uintptr_t)g.D % 16) == 0 && g.ldd % 16 == 0 && g.d_batch_stride % 16 == 0) ? 1 : 0;
     }
 
     int launch(GemmArgs &g, bool flip_in_loader, bool conv, hipStream_t s)
@@ -357,7 +361,11 @@ struct GemmCore
             const bool aligned =
                 conv ? (g.conv.C % 16 == 0 && ((uintptr_t)g.A & 15) == 0)
                      : ((((uintptr_t)g.A | (uintptr_t)g.lda | (uintptr_t)g.a_batch_stride) & 15) == 0);
-            if (dma_idx >= 0 && aligned && g.K % 16 == 0)
+            // its producers address a block's A rows (dense) or the whole image batch (convolution) with 32-bit offsets
+            const int64_t span = conv ? (int64_t)((g.M + g.conv.OH * g.conv.OW - 1) / (g.conv.OH * g.conv.OW)) *
+                                            g.conv.H * g.conv.W * g.conv.C
+                                      : (int64_t)g.lda * 256 + g.K;
+            if (dma_idx >= 0 && aligned && g.K % 16 == 0 && span < ((int64_t)1 << 32))
             {
                 const MfmaConfig c = dma_config(dma_idx);
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;

@@ -34,10 +34,12 @@ struct EpiParams
     int32_t        has_offsets; // EPI_F32: whether the offset term is added at all
     int32_t        dst_signed;
     int32_t        vec_store; // destination rows / base / batch stride allow 4-element vector stores
+    int32_t        vec_store16; // ... and 16-byte stores of 8-bit results
     // Pre-digested per-column requantisation vectors qp[5][qp_stride] (see fast_requant below), or nullptr when some
     // multiplier is negative and the general formula has to be used
     const int32_t *qp;
     int64_t        qp_stride;
+    int32_t        qp_std; // every column: multiplier >= 2^30, shift in [2, 31]; |result_offset| < 2^28 (see std_requant)
 };
 
 // Per-column constants of the branch-free requantisation used by the pipelined kernel's epilogue, valid for
@@ -63,6 +65,15 @@ __device__ __forceinline__ int32_t fast_requant(int32_t v, int32_t s2, int32_t c
     const int32_t h   = __mulhi(pre, s2) + (pre & cmask);
     const int32_t r   = ((h >> rsm1) + rmask) >> rmask;
     return min(max((int32_t)((uint32_t)r + (uint32_t)result_offset), lo), hi);
+}
+
+// The common case of fast_requant (cmask = -1, ls = 0, rmask = 1, rsm1 >= 1): the rounding increment and the result
+// offset are one constant, off2p1 = 2*result_offset + 1, added before the last shift:
+// ((x + 1) >> 1) + off == (x + 1 + 2*off) >> 1, and |x| <= 2^30 here, so nothing overflows.
+__device__ __forceinline__ int32_t std_requant(int32_t v, int32_t s2, int32_t rsm1, int32_t off2p1, int32_t lo, int32_t hi)
+{
+    const int32_t h = __mulhi(v, s2) + v;
+    return min(max(((h >> rsm1) + off2p1) >> 1, lo), hi);
 }
 
 // (a * b * 2) >> 32 with the single saturating case, without 64-bit VALU arithmetic

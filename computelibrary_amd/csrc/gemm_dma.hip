@@ -21,8 +21,9 @@
 // same number of barriers.
 //
 // Accumulators are kept transposed (the B panel is fed as the first matrix operand), so each lane ends up with 4
-// consecutive output columns per register quad: the epilogue packs 4 int8 results into one 32-bit store and reads the
-// per-column parameters as 16-byte vectors.
+// consecutive output columns per register quad: the epilogue reads the per-column parameters as 16-byte vectors and
+// packs 4 int8 results into one dword. Those dwords go to LDS first (the ring is free by then) and leave as whole
+// 128-byte tile rows, 16 bytes per lane; where the destination is not 16-byte aligned they are stored directly.
 #include "mfma_common.hpp"
 
 namespace mi355
@@ -30,6 +31,12 @@ namespace mi355
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
 {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+}
+
+// scalar-base form: address = sbase (SGPR pair, wave-uniform) + zero-extended per-lane 32-bit offset
+__device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
 }
 
 template <int N>
@@ -45,6 +52,121 @@ __device__ __forceinline__ void block_barrier()
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }
+
+// Stages the A and B panels of one block tile. All NP producer waves of a block hold one of these. The loads use the
+// scalar-base form of the instruction (wave-uniform 64-bit base in SGPRs + one 32-bit offset register per lane): with
+// per-lane 64-bit addresses every load costs the SIMD's matrix pipe about 50 clocks, with scalar bases the stream
+// overlaps the matrix instructions almost completely. The K offset of a step is added to the scalar base, so a dense
+// producer executes no vector ALU work at all inside the loop. Lanes that must read padding instead (K tail of A,
+// out-of-image taps of the implicit convolution) need a different base: a wave with any such lane falls back to
+// per-lane addresses for that one load.
+template <int BM, int BN, int BK, int NP, int NS, bool CONV>
+struct PanelProducer
+{
+    static constexpr int CPR   = BK / 16;   // 16-byte columns per tile row
+    static constexpr int RPU   = 1024 / BK; // tile rows per staging unit (one wave instruction = 1 KiB)
+    static constexpr int AU    = BM / RPU;  // staging units of the A part of a stage
+    static constexpr int BU    = BN / RPU;
+    static constexpr int LPP   = (AU + BU) / NP; // loads per producer wave per stage: unit u belongs to producer u % NP
+    static constexpr int STAGE = (BM + BN) * BK;
+    static_assert((AU + BU) % NP == 0, "staging shape");
+
+    const int8_t *a_base, *b_base, *fill16; // wave-uniform
+    uint32_t      off[LPP];                 // this lane's byte offset from the base (dense A rows, B rows, conv image)
+    int           a_c16[LPP];               // byte offset of this lane's column inside a K step
+    int           a_iy0[LPP], a_ix0[LPP];   // conv: top-left input coordinate of this lane's output pixel
+    uint32_t      lds0;
+    int           pw, K;
+    ConvGeom      conv;
+
+    __device__ __forceinline__ void init(const GemmArgs &g, int m0, int n0, int bz, int producer_wave, int lane,
+                                         uint32_t lds_base)
+    {
+        pw     = producer_wave;
+        lds0   = lds_base;
+        K      = g.K;
+        conv   = g.conv;
+        fill16 = g.fill16;
+        a_base = g.A + (int64_t)bz * g.a_batch_stride + (CONV ? (int64_t)0 : (int64_t)m0 * g.lda);
+        b_base = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
+        const int ur = lane / CPR; // row inside a unit
+        const int up = lane % CPR; // LDS column slot inside the row
+#pragma unroll
+        for (int i = 0; i < LPP; ++i)
+        {
+            const int u = pw + i * NP; // wave-uniform
+            if (u < AU)
+            {
+                const int row = u * RPU + ur;
+                const int c   = up ^ swz<CPR>(row);
+                a_c16[i]      = c * 16;
+                const int gr  = min(m0 + row, g.M - 1);
+                if (CONV)
+                {
+                    const int ox = gr % g.conv.OW;
+                    const int t  = gr / g.conv.OW;
+                    const int oy = t % g.conv.OH;
+                    const int n  = t / g.conv.OH;
+                    off[i]       = (uint32_t)n * (uint32_t)(g.conv.H * g.conv.W * g.conv.C);
+                    a_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
+                    a_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
+                }
+                else
+                {
+                    off[i]   = (uint32_t)(gr - m0) * (uint32_t)g.lda + (uint32_t)(c * 16);
+                    a_iy0[i] = a_ix0[i] = 0;
+                }
+            }
+            else
+            {
+                const int row = (u - AU) * RPU + ur;
+                const int c   = up ^ swz<CPR>(row);
+                off[i]        = (uint32_t)row * (uint32_t)g.Kp + (uint32_t)(c * 16);
+                a_c16[i] = a_iy0[i] = a_ix0[i] = 0;
+            }
+        }
+    }
+
+    __device__ __forceinline__ void issue(int kt) const
+    {
+        const int      k0   = kt * BK;
+        const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
+        const int8_t  *a_k  = a_base + (CONV ? 0 : k0);
+        const int8_t  *b_k  = b_base + k0; // always inside the zero-padded packed panel
+        const bool     full = k0 + BK <= K;
+#pragma unroll
+        for (int i = 0; i < LPP; ++i)
+        {
+            const int      u   = pw + i * NP;
+            const uint32_t dst = base + (uint32_t)u * 1024u;
+            if (u >= AU)
+                dma16s(b_k, off[i], dst);
+            else if (!CONV)
+            {
+                if (full)
+                    dma16s(a_k, off[i], dst);
+                else
+                    dma16(k0 + a_c16[i] < K ? a_k + off[i] : fill16, dst);
+            }
+            else
+            {
+                const int k     = k0 + a_c16[i];
+                const int tap   = k / conv.C;
+                const int c0    = k - tap * conv.C;
+                const int ky    = tap / conv.KW;
+                const int kx    = tap - ky * conv.KW;
+                const int iy    = a_iy0[i] + ky * conv.dil_y;
+                const int ix    = a_ix0[i] + kx * conv.dil_x;
+                const bool ok   = k < K && iy >= 0 && iy < conv.H && ix >= 0 && ix < conv.W;
+                const uint32_t o = off[i] + (uint32_t)((iy * conv.W + ix) * conv.C + c0);
+                if (__builtin_amdgcn_ballot_w64(ok) == ~0ull)
+                    dma16s(a_k, o, dst);
+                else
+                    dma16(ok ? a_k + o : fill16, dst);
+            }
+        }
+    }
+};
 
 // GWM x GWN consumer waves per group, 2 groups stacked along M, plus NP = GWM*GWN producer waves
 template <int BM, int BN, int BK, int GWM, int GWN, int NS, int EPI, bool FLIP_A, bool CONV>
@@ -85,85 +207,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     if (wave >= NW)
     {
         // ================= producer: global -> LDS =================
-        const int8_t *__restrict__ A  = g.A + (int64_t)bz * g.a_batch_stride;
-        const int8_t *__restrict__ Bp = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
-        const int     pw = wave - NW;
-        const int     ur = lane / CPR; // row inside a unit
-        const int     up = lane % CPR; // LDS column slot inside the row
-        const int8_t *pu[LPP];
-        int           a_c16[LPP]; // byte offset of this lane's column inside a K step
-        int           a_iy0[LPP], a_ix0[LPP];
-#pragma unroll
-        for (int i = 0; i < LPP; ++i)
-        {
-            const int u = pw + i * NP; // wave-uniform
-            if (u < AU)
-            {
-                const int row = u * RPU + ur;
-                const int c   = up ^ swz<CPR>(row);
-                a_c16[i]      = c * 16;
-                const int gr  = min(m0 + row, g.M - 1);
-                if (CONV)
-                {
-                    const int ox = gr % g.conv.OW;
-                    const int t  = gr / g.conv.OW;
-                    const int oy = t % g.conv.OH;
-                    const int n  = t / g.conv.OH;
-                    pu[i]        = A + (int64_t)n * g.conv.H * g.conv.W * g.conv.C;
-                    a_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
-                    a_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
-                }
-                else
-                {
-                    pu[i]    = A + (int64_t)gr * g.lda + c * 16;
-                    a_iy0[i] = a_ix0[i] = 0;
-                }
-            }
-            else
-            {
-                const int row = (u - AU) * RPU + ur;
-                const int c   = up ^ swz<CPR>(row);
-                pu[i]         = Bp + (int64_t)row * g.Kp + c * 16;
-                a_c16[i] = a_iy0[i] = a_ix0[i] = 0;
-            }
-        }
-        auto issue = [&](int kt)
-        {
-            const int      k0   = kt * BK;
-            const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
-#pragma unroll
-            for (int i = 0; i < LPP; ++i)
-            {
-                const int     u   = pw + i * NP;
-                const int8_t *src = pu[i] + k0; // B unit: always inside the zero-padded packed panel
-                if (u < AU)
-                {
-                    const int k = k0 + a_c16[i];
-                    src         = g.fill16;
-                    if (k < g.K)
-                    {
-                        if (CONV)
-                        {
-                            const int tap = k / g.conv.C;
-                            const int c0  = k - tap * g.conv.C;
-                            const int ky  = tap / g.conv.KW;
-                            const int kx  = tap - ky * g.conv.KW;
-                            const int iy  = a_iy0[i] + ky * g.conv.dil_y;
-                            const int ix  = a_ix0[i] + kx * g.conv.dil_x;
-                            if (iy >= 0 && iy < g.conv.H && ix >= 0 && ix < g.conv.W)
-                                src = pu[i] + ((int64_t)iy * g.conv.W + ix) * g.conv.C + c0;
-                        }
-                        else
-                            src = pu[i] + k0;
-                    }
-                }
-                dma16(src, base + (uint32_t)u * 1024u);
-            }
-        };
+        PanelProducer<BM, BN, BK, NP, NS, CONV> prod;
+        prod.init(g, m0, n0, bz, wave - NW, lane, lds0);
 #pragma unroll
         for (int s = 0; s < NS - 1; ++s)
             if (s < nk)
-                issue(s);
+                prod.issue(s);
         if (nk >= NS - 1)
             wait_vmcnt<(NS - 2) * LPP>(); // stage 0 complete, the NS-2 younger stages may still be in flight
         else
@@ -173,7 +222,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         {
             const bool more = kt + NS - 1 < nk;
             if (more)
-                issue(kt + NS - 1); // ring slot of stage kt-1
+                prod.issue(kt + NS - 1); // ring slot of stage kt-1
             block_barrier();        // barrier 2kt+1
             if (more)
                 wait_vmcnt<(NS - 2) * LPP>(); // stage kt+1 complete
@@ -183,7 +232,11 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         }
         block_barrier(); // barrier 2nk+1
         if (EPI == EPI_FIXEDPOINT && g.epi.qp != nullptr)
+        {
             __syncthreads(); // the consumers' staging of the epilogue constants
+            if (g.epi.vec_store16)
+                __syncthreads(); // ... and of the output tile
+        }
         return;
     }
 
@@ -298,7 +351,17 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         }
         __syncthreads();
         if (EPI == EPI_FIXEDPOINT)
-            epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+        {
+            char *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
+            if (g.epi.vec_store16 && g.epi.qp_std)
+                epilogue_store_staged<true, FM, FN, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                [] { __syncthreads(); });
+            else if (g.epi.vec_store16)
+                epilogue_store_staged<false, FM, FN, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                 [] { __syncthreads(); });
+            else
+                epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+        }
     }
     else
         epilogue_store_t<EPI, FM, FN>(acc, g, m0 + row_w, n0 + col_w, lane, bz);

@@ -184,6 +184,8 @@ __global__ void qparams_kernel(const int32_t *__restrict__ mult, const int32_t *
     }
     if (m < 0)
         atomicOr(neg, 1);
+    if (j < N && !(m >= 0x40000000 && s >= 2 && s < 32))
+        atomicOr(neg, 2); // not the common case (normalised multiplier, right shift by 2 or more)
     if (s >= 32 || s <= -32)
         m = 0, s = 0; // the reference arithmetic yields 0 for these
     const uint32_t m2          = (uint32_t)m << 1;

@@ -256,4 +256,84 @@ __device__ __forceinline__ void epilogue_store_fast(const v16i (&acc)[FM][FN], c
         }
     }
 }
+// The same arithmetic as epilogue_store_fast, but the packed 8-bit results of the whole BM x BN block tile are first
+// laid out in LDS (row pitch BN + 16 bytes) and then written with 16 bytes per lane, BN/16 lanes per output row, so a
+// wave instruction writes whole rows of the tile instead of 8-byte pieces of 32 different rows. All NW consumer waves
+// of the block call this together; `barrier` is executed once between the two phases by every wave of the block.
+// Requires p.vec_store16. stage must not overlap par.
+template <bool STD, int FM, int FN, int BM, int BN, int NW, typename Barrier>
+__device__ __forceinline__ void epilogue_store_staged(const v16i (&acc)[FM][FN], const GemmArgs &g, const int32_t *par,
+                                                      char *stage, int m0, int n0, int row_in_tile, int col_in_tile,
+                                                      int wave, int lane, int bz, Barrier barrier)
+{
+    constexpr int    PITCH = BN + 16;
+    const int        lr = lane & 31, lh = lane >> 5;
+    const EpiParams &p      = g.epi;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    int32_t          rv[FM];
+    const int32_t    off2p1 = 2 * p.result_offset + 1;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+    {
+        const int i = m0 + row_in_tile + fm * 32 + lr;
+        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int c  = col_in_tile + fn * 32 + 8 * q + 4 * lh;
+            const v4i cv = *(const v4i *)(par + 0 * BN + c);
+            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
+            const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
+            v4i       cm = {0, 0, 0, 0}, ls = cm, rm = cm;
+            if (!STD)
+            {
+                cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
+                ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
+                rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
+            }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm)
+            {
+                int32_t o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                {
+                    const int32_t v = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
+                    o[t] = STD ? std_requant(v, s2[t], r1[t], off2p1, p.lo, p.hi)
+                               : fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
+                }
+                const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
+                const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
+                *(uint32_t *)(stage + (row_in_tile + fm * 32 + lr) * PITCH + c) =
+                    __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+            }
+        }
+    }
+    barrier();
+    constexpr int LPR = BN / 16;  // lanes per output row
+    constexpr int RPI = 64 / LPR; // rows per wave instruction
+    char         *D   = (char *)g.D + (int64_t)bz * g.d_batch_stride;
+    const int     rr = lane / LPR, cc = (lane % LPR) * 16;
+#pragma unroll
+    for (int it = 0; it < BM / (NW * RPI); ++it)
+    {
+        const int r = (it * NW + wave) * RPI + rr;
+        const int i = m0 + r, j0 = n0 + cc;
+        if (i >= g.M || j0 >= g.N)
+            continue;
+        const v4i     val = *(const v4i *)(stage + r * PITCH + cc);
+        const int64_t idx = (int64_t)i * g.ldd + j0;
+        if (j0 + 16 <= g.N)
+            *(v4i *)(D + idx) = val;
+        else
+        {
+            for (int t = 0; t < g.N - j0; ++t)
+                D[idx + t] = (char)(val[t >> 2] >> (8 * (t & 3)));
+        }
+    }
+}
 } // namespace mi355

@@ -1,5 +1,7 @@
 """GPU parity: the HIP path through the C ABI against the golden fixtures (outputs of the reference's own
 portable code) and against the CPU oracle on seeded inputs. Integer outputs must be bit-exact."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -131,6 +133,38 @@ def test_per_channel_left_and_right_shifts():
                           device=True)
         np.testing.assert_array_equal(got, want)
 
+
+@pytest.mark.parametrize("case", ["std", "mixed_shifts", "negative_mult", "big_offset", "uint8_out"])
+@pytest.mark.parametrize("N,ldd", [(256, 256), (250, 256), (250, 252), (250, 251), (130, 144)])
+def test_pipelined_kernel_epilogue_variants(case, N, ldd):
+    """Every store path of the pipelined kernel's fused output stage (LDS-staged 16-byte rows with and without a ragged
+    right edge, packed dwords, single bytes) crossed with every arithmetic path (common case, general branch-free
+    case with left / zero / one-bit shifts, negative multipliers, offsets too large for the folded rounding)."""
+    rng = np.random.default_rng(zlib.crc32(repr((case, N, ldd)).encode()))
+    M, K = 300, 512
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, size=N, dtype=np.int32)
+    reals = np.exp(rng.uniform(np.log(2e-4), np.log(2e-3), size=N))
+    off, dt, lo, hi = -5, np.int8, -128, 127
+    if case == "mixed_shifts":
+        reals = np.exp(rng.uniform(np.log(1e-4), np.log(3.0), size=N))
+    mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+    if case == "mixed_shifts":
+        shift[:4] = [0, 1, 2, 31]
+        assert (shift < 0).any() and (shift > 1).any()
+    elif case == "negative_mult":
+        mult[::7] = -mult[::7]
+    elif case == "big_offset":
+        off, lo, hi = (1 << 29) + 77, -128, 127
+    elif case == "uint8_out":
+        off, dt, lo, hi = 128, np.uint8, 3, 250
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -3, 0, mult, shift, off, lo, hi, dt)
+    announce("pipelined epilogue", case, N, ldd)
+    got, name = run_gemm(A, B, capi.EPI_FIXEDPOINT, dt, -3, 0, bias, mult, shift, off, lo, hi, path=capi.PATH_MFMA,
+                         device=True, ldd=ldd)
+    assert name.startswith("pp_"), name
+    np.testing.assert_array_equal(got, want)
 
 def test_requant_extremes_on_device():
     """Accumulators and multipliers at the edges of int32 (saturating SQDMULH, shift 0 / 31, wrap-around adds)

@@ -170,7 +170,7 @@ struct GemmCore
         if (path == MI355_PATH_SIMPLE)
             kname = "simple";
         else if (path == MI355_PATH_SKINNY)
-            kname = "skinny_16xN_splitk8";
+            kname = "skinny_16xN_splitk";
         else
         {
             const int cus = num_cus();

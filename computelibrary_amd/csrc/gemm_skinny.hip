@@ -5,28 +5,54 @@
 //
 // B is packed at prepare time into 1 KiB blocks of 16 columns x 64 k in matrix-core operand order
 // (Bs[Np/16][Kp/64][64 lanes][16 bytes]), so every wave-wide load is one contiguous, fully coalesced 1 KiB read and a
-// column group's K range is one contiguous stream. A block owns one group of 16 output columns; its waves split the
-// k blocks, each keeping UNROLL loads in flight, multiply with v_mfma_i32_16x16x64_i8 (A rows padded to 16 with
-// zeros; A itself is tiny and stays in L2), reduce the partial 16 x 16 accumulators through LDS, and wave 0 applies the
-// fused offset / requantisation epilogue.
+// column group's K range is one contiguous stream. A block owns NG groups of 16 output columns; its WAVES waves split
+// the k blocks, each keeping UNROLL steps of loads in flight, multiply with v_mfma_i32_16x16x64_i8 (A rows padded to 16
+// with zeros; A itself is tiny and stays in L2), reduce the partial 16 x 16 accumulators through LDS, and wave 0 applies
+// the fused offset / requantisation epilogue. The kernel lives on memory-level parallelism: every block of the grid
+// should be resident at once, so the register footprint is kept small (the K tail has its own one-step loop) and the
+// number of waves per block is chosen from the number of column groups.
 #include "internal.hpp"
+
+#include <cstdlib>
 
 namespace mi355
 {
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int SK_WAVES  = 8;
-constexpr int SK_UNROLL = 8;
 
-template <int EPI, bool FLIP_A>
+template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 {
-    __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][64][4];
+    __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int ng   = blockIdx.x;
+    const int ng0  = blockIdx.x * NG; // first of this block's NG groups of 16 columns
     const int KB   = (int)(g.Kp / 64);
+    const int NGT  = (int)((g.N + 15) / 16);
+
+    // wave 0 applies the epilogue to column ng0*16 + (lane%16) + 16*n: fetch its per-column constants now, so that
+    // their latency is hidden behind the B stream instead of following it
+    const EpiParams &p = g.epi;
+    int32_t          cv[NG], mu[NG], sh[NG];
+    float            bf[NG];
+#pragma unroll
+    for (int n = 0; n < NG; ++n)
+    {
+        const int j = min((ng0 + n) * 16 + (lane & 15), g.N - 1);
+        cv[n] = 0, mu[n] = p.mult_s, sh[n] = p.shift_s, bf[n] = 0.f;
+        if (wave == 0)
+        {
+            cv[n] = p.colvec[j];
+            if (EPI == EPI_FIXEDPOINT && p.mult)
+            {
+                mu[n] = p.mult[j];
+                sh[n] = p.shift[j];
+            }
+            if (EPI == EPI_F32 && p.bias_f32)
+                bf[n] = p.bias_f32[j];
+        }
+    }
 
     // this wave's contiguous range of k blocks
     const int per  = (KB + SK_WAVES - 1) / SK_WAVES;
@@ -37,86 +63,109 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     const int   akc    = (lane >> 4) * 16;
     const bool  a_live = arow < g.M;
     const int8_t *__restrict__ a_ptr = g.A + (int64_t)min(arow, g.M - 1) * g.lda + akc;
-    const int8_t *__restrict__ b_ptr = g.Bp + ((int64_t)ng * KB * 64 + lane) * 16;
+    const int8_t *b_ptr[NG];
+#pragma unroll
+    for (int n = 0; n < NG; ++n)
+        b_ptr[n] = g.Bp + ((int64_t)min(ng0 + n, NGT - 1) * KB * 64 + lane) * 16;
 
-    v4i acc = {0, 0, 0, 0};
-    for (int kb = kb0; kb < kb1; kb += SK_UNROLL)
+    v4i acc[NG];
+#pragma unroll
+    for (int n = 0; n < NG; ++n)
+        acc[n] = (v4i){0, 0, 0, 0};
+    const v4i zero4 = {0, 0, 0, 0};
+    int       kb    = kb0;
+    // whole steps inside the wave's range and inside K: straight-line loads, all in flight together
+    for (; kb + SK_UNROLL <= kb1 && (kb + SK_UNROLL) * 64 <= g.K; kb += SK_UNROLL)
     {
-        v4i fa[SK_UNROLL], fb[SK_UNROLL];
+        v4i fa[SK_UNROLL], fb[SK_UNROLL][NG];
 #pragma unroll
         for (int u = 0; u < SK_UNROLL; ++u)
         {
-            const int kk = kb + u;
-            fb[u]        = (v4i){0, 0, 0, 0};
-            fa[u]        = (v4i){0, 0, 0, 0};
-            if (kk < kb1)
+            fa[u] = zero4;
+#pragma unroll
+            for (int n = 0; n < NG; ++n)
+                fb[u][n] = __builtin_nontemporal_load((const v4i *)(b_ptr[n] + (int64_t)(kb + u) * 1024));
+        }
+        if (a_live)
+        {
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u)
             {
-                fb[u] = *(const v4i *)(b_ptr + (int64_t)kk * 1024);
-                const int rem = g.K - (kk * 64 + akc);
-                if (a_live && rem > 0)
-                {
-                    fa[u] = rem >= 16 ? *(const v4i *)(a_ptr + (int64_t)kk * 64)
-                                      : load16_partial(a_ptr + (int64_t)kk * 64, rem);
-                    if (FLIP_A)
-                        fa[u] ^= (int)0x80808080;
-                }
+                fa[u] = *(const v4i *)(a_ptr + (int64_t)(kb + u) * 64);
+                if (FLIP_A)
+                    fa[u] ^= (int)0x80808080;
             }
         }
 #pragma unroll
         for (int u = 0; u < SK_UNROLL; ++u)
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u], acc, 0, 0, 0);
+#pragma unroll
+            for (int n = 0; n < NG; ++n)
+                acc[n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u][n], acc[n], 0, 0, 0);
+    }
+    // remaining k blocks one at a time, with the guarded loads of the K tail
+    for (; kb < kb1; ++kb)
+    {
+        v4i fa = zero4, fb[NG];
+#pragma unroll
+        for (int n = 0; n < NG; ++n)
+            fb[n] = *(const v4i *)(b_ptr[n] + (int64_t)kb * 1024);
+        const int rem = g.K - (kb * 64 + akc);
+        if (a_live && rem > 0)
+        {
+            fa = rem >= 16 ? *(const v4i *)(a_ptr + (int64_t)kb * 64) : load16_partial(a_ptr + (int64_t)kb * 64, rem);
+            if (FLIP_A)
+                fa ^= (int)0x80808080;
+        }
+#pragma unroll
+        for (int n = 0; n < NG; ++n)
+            acc[n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[n], acc[n], 0, 0, 0);
     }
 
-    *(v4i *)&red[wave][lane][0] = acc;
+#pragma unroll
+    for (int n = 0; n < NG; ++n)
+        *(v4i *)&red[wave][n][lane][0] = acc[n];
     __syncthreads();
     if (wave != 0)
         return;
 #pragma unroll
     for (int w = 1; w < SK_WAVES; ++w)
-    {
-        const v4i o = *(const v4i *)&red[w][lane][0];
-        acc += o;
-    }
+#pragma unroll
+        for (int n = 0; n < NG; ++n)
+            acc[n] += *(const v4i *)&red[w][n][lane][0];
 
     // accumulator r of lane l is row 4*(l/16) + r, column l%16
-    const EpiParams &p = g.epi;
-    const int        j = ng * 16 + (lane & 15);
-    if (j >= g.N)
-        return;
-    const int32_t cv = p.colvec[j];
-    int32_t       mu = p.mult_s, sh = p.shift_s;
-    if (EPI == EPI_FIXEDPOINT && p.mult)
-    {
-        mu = p.mult[j];
-        sh = p.shift[j];
-    }
-    const float bf = (EPI == EPI_F32 && p.bias_f32) ? p.bias_f32[j] : 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int n = 0; n < NG; ++n)
     {
-        const int i = 4 * (lane >> 4) + r;
-        if (i < g.M)
+        const int j = (ng0 + n) * 16 + (lane & 15);
+        if (j >= g.N)
+            continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
         {
-            const int32_t rv  = p.rowvec ? p.rowvec[i] : 0;
-            const int64_t idx = (int64_t)i * g.ldd + j;
-            if (EPI == EPI_S32)
-                ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc[r] + (uint32_t)cv + (uint32_t)rv);
-            else if (EPI == EPI_FIXEDPOINT)
-                ((int8_t *)g.D)[idx] = (int8_t)epi_fixedpoint(acc[r], cv, rv, mu, sh, p);
-            else
-                ((float *)g.D)[idx] =
-                    epi_f32(acc[r], (int32_t)((uint32_t)cv + (uint32_t)rv), bf, p.bias_f32 != nullptr, p);
+            const int i = 4 * (lane >> 4) + r;
+            if (i < g.M)
+            {
+                const int32_t rv  = p.rowvec ? p.rowvec[i] : 0;
+                const int64_t idx = (int64_t)i * g.ldd + j;
+                if (EPI == EPI_S32)
+                    ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc[n][r] + (uint32_t)cv[n] + (uint32_t)rv);
+                else if (EPI == EPI_FIXEDPOINT)
+                    ((int8_t *)g.D)[idx] = (int8_t)epi_fixedpoint(acc[n][r], cv[n], rv, mu[n], sh[n], p);
+                else
+                    ((float *)g.D)[idx] = epi_f32(acc[n][r], (int32_t)((uint32_t)cv[n] + (uint32_t)rv), bf[n],
+                                                  p.bias_f32 != nullptr, p);
+            }
         }
     }
 }
 
-int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
+template <int NG, int WAVES, int UNROLL>
+static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
 {
-    if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
-        return (int)hipErrorInvalidValue;
-    const dim3 grid((args.N + 15) / 16), block(SK_WAVES * 64);
-    GemmArgs   a = args;
-#define MI355_SK(E, F) gemm_skinny_kernel<E, F><<<grid, block, 0, s>>>(a)
+    const int  groups = (a.N + 15) / 16;
+    const dim3 grid((groups + NG - 1) / NG), block(WAVES * 64);
+#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL><<<grid, block, 0, s>>>(a)
     if (epi == EPI_S32)
         flip_a ? MI355_SK(EPI_S32, true) : MI355_SK(EPI_S32, false);
     else if (epi == EPI_FIXEDPOINT)
@@ -127,5 +176,17 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
         return (int)hipErrorInvalidValue;
 #undef MI355_SK
     return (int)hipGetLastError();
+}
+
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
+{
+    if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
+        return (int)hipErrorInvalidValue;
+    // about 2000-4000 waves fill the 256 compute units with enough loads in flight: split K over 4 waves per block
+    // when there are many column groups, over 8 otherwise
+    static const char *force  = getenv("MI355_SKINNY_WAVES");
+    const int          groups = (args.N + 15) / 16;
+    const int          waves  = force ? atoi(force) : (groups >= 512 ? 4 : 8);
+    return waves == 4 ? skinny_launch_v<1, 4, 8>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8>(epi, flip_a, args, s);
 }
 } // namespace mi355

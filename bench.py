@@ -23,17 +23,30 @@ sys.path.insert(0, ROOT)
 
 INT8_DENSE_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix rate (5.0 POP/s)
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+# HBM-side bytes of one launch of the config-2 kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the
+# same counters read for a plain copy (profiles/gemm_pp_256x128x128_cfg2_hbm_traffic.txt holds the runs)
+CFG2_MEASURED_TRAFFIC_BYTES = None
+
+
+def quantized_multipliers(scales):
+    """(multiplier, shift) per real multiplier, as quantization::calculate_quantized_multiplier derives them
+    (src/core/utils/quantization/AsymmHelpers.cpp:43-115): real = q * 2^e with q in [0.5, 1), multiplier = round(q * 2^31),
+    shift = -e. Only used to synthesise inputs."""
+    q, e = np.frexp(np.asarray(scales, dtype=np.float32).astype(np.float64))
+    m = np.floor(q * float(1 << 31) + 0.5).astype(np.int64)
+    e = np.where(m == (1 << 31), e + 1, e)
+    m = np.where(m == (1 << 31), m // 2, m)
+    return m.astype(np.int32), (-e).astype(np.int32)
 
 
 def synth_config2(M, N, K, seed=2):
     """BASELINE config 2/3 distributions: A int8 U[-128,127] zero point 3; B int8 ~N(0,32) clipped to +-127;
     per-column scale U[1e-4,1e-3] -> (multiplier, shift); bias int32 ~N(0,2000); output offset -5, clamp [-128,127]."""
-    import oracle
     rng = np.random.default_rng(seed)
     A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
     B = np.clip(np.rint(rng.normal(0.0, 32.0, size=(K, N))), -127, 127).astype(np.int8)
     scales = rng.uniform(1e-4, 1e-3, size=N).astype(np.float32)
-    mult, shift = oracle.calculate_quantized_multipliers(1.0, scales, 1.0)
+    mult, shift = quantized_multipliers(scales)
     bias = np.rint(rng.normal(0.0, 2000.0, size=N)).astype(np.int32)
     return A, B, bias, mult, shift
 
@@ -113,7 +126,7 @@ def main():
         "config": {"workload": "gemmlowp s8 x per-channel s8 -> s8, M=2048 N=4096 K=4096, fused offset + "
                                "FIXEDPOINT requant", "kernel": g.kernel_name, "prepare_ms": round(prepare_ms, 3)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_DENSE_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved / INT8_DENSE_PEAK_TOPS, 4), "traffic": None,
+                     "frac": round(achieved / INT8_DENSE_PEAK_TOPS, 4), "traffic": CFG2_MEASURED_TRAFFIC_BYTES,
                      "kernel_us": round(kern_s * 1e6, 3)},
     }
 
@@ -166,6 +179,43 @@ def main():
             "note": "B rotated over 9 packed copies (405 MB) so reads come from HBM"}}
         for h in handles:
             h.close()
+
+        # config 4: NHWC 3x3 convolution as an implicit GEMM (M = 32*56*56, N = 64, K = 576), near the roofline ridge
+        rng = np.random.default_rng(4)
+        src = torch.from_numpy(rng.integers(-128, 128, size=(32, 56, 56, 64), dtype=np.int8)).cuda()
+        wts = torch.from_numpy(np.clip(np.rint(rng.normal(0.0, 24.0, size=(64, 3, 3, 64))), -127, 127).astype(np.int8)).cuda()
+        m4, s4 = quantized_multipliers(rng.uniform(1e-4, 1e-3, size=64).astype(np.float32))
+        b4 = torch.from_numpy(np.rint(rng.normal(0.0, 500.0, size=64)).astype(np.int32)).cuda()
+        cv = capi.Conv(capi.conv_desc(32, 56, 56, 64, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.S8,
+                                      1, 0, -1, rq, 0))
+        dst4 = torch.zeros((32, 56, 56, 64), dtype=torch.int8, device="cuda")
+        cv.prepare(wts, b4, torch.from_numpy(m4).cuda(), torch.from_numpy(s4).cuda(), stream)
+        _, evt4 = time_launches(torch, lambda: cv.run(src, dst4, stream), args.steps, args.warmup)
+        ops4, bytes4 = 2.0 * 32 * 56 * 56 * 64 * 576, 2 * 32 * 56 * 56 * 64 + 64 * 576 + 3 * 4 * 64
+        out["secondary"]["conv_cfg4"] = {
+            "workload": "NHWC s8 [32,56,56,64] * 3x3x64x64 per-channel, s1 p1 -> s8", "kernel": cv.kernel_name,
+            "kernel_us": round(evt4 / args.steps * 1e6, 3), "TOPS": round(ops4 / (evt4 / args.steps) / 1e12, 1),
+            "frac_mfma": round(ops4 / (evt4 / args.steps) / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "GBs": round(bytes4 / (evt4 / args.steps) / 1e9, 1),
+            "frac_hbm": round(bytes4 / (evt4 / args.steps) / 1e9 / HBM_PEAK_GBS, 4)}
+        cv.close()
+
+        # config 5: 16 x (1024 x 1000) * (1000 x 1024) s8 -> f32 dequantised, store-bound
+        A5 = torch.from_numpy(rng.integers(-128, 128, size=(16, 1024, 1000), dtype=np.int8)).cuda()
+        B5 = torch.from_numpy(rng.integers(-128, 128, size=(16, 1000, 1024), dtype=np.int8)).cuda()
+        D5 = torch.zeros((16, 1024, 1024), dtype=torch.float32, device="cuda")
+        g5 = capi.Gemm(1024, 1024, 1000, capi.S8, capi.S8, capi.F32, capi.EPI_F32, 0, 0, None,
+                       float(np.float32(0.02) * np.float32(0.005)), batch=16, b_batched=True)
+        g5.prepare(B5, None, None, None, stream)
+        _, evt5 = time_launches(torch, lambda: g5.run(A5, D5, None, stream), args.steps, args.warmup)
+        ops5, bytes5 = 2.0 * 16 * 1024 * 1024 * 1000, 16 * (2 * 1024 * 1000 + 4 * 1024 * 1024)
+        out["secondary"]["batched_f32_cfg5"] = {
+            "workload": "16 x (1024x1000)*(1000x1024) s8 -> f32 dequantised", "kernel": g5.kernel_name,
+            "kernel_us": round(evt5 / args.steps * 1e6, 3), "TOPS": round(ops5 / (evt5 / args.steps) / 1e12, 1),
+            "frac_mfma": round(ops5 / (evt5 / args.steps) / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "GBs": round(bytes5 / (evt5 / args.steps) / 1e9, 1),
+            "frac_hbm": round(bytes5 / (evt5 / args.steps) / 1e9 / HBM_PEAK_GBS, 4)}
+        g5.close()
 
     g.close()
     print(json.dumps(out))

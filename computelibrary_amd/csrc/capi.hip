@@ -199,7 +199,7 @@ struct GemmCore
                 cfg_idx = atoi(f1);
             if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs())
                 dma_idx = atoi(f2);
-            if (getenv("MI355_NO_DMA") || K % 16 != 0)
+            if (getenv("MI355_NO_DMA") || K < 16)
                 dma_idx = -1;
             kname_mfma = mfma_config(cfg_idx).name;
             kname_dma  = dma_idx >= 0 ? dma_config(dma_idx).name : "";
@@ -357,15 +357,16 @@ struct GemmCore
         else
         {
             g.fill16 = fill.as<int8_t>();
-            // the pipelined kernel moves whole aligned 16-byte columns straight into LDS
+            // the pipelined kernel moves 16-byte columns of dword-aligned rows straight into LDS
             const bool aligned =
-                conv ? (g.conv.C % 16 == 0 && ((uintptr_t)g.A & 15) == 0)
-                     : ((((uintptr_t)g.A | (uintptr_t)g.lda | (uintptr_t)g.a_batch_stride) & 15) == 0);
+                conv ? (g.conv.C % 16 == 0 && ((uintptr_t)g.A & 15) == 0 && g.K % 16 == 0)
+                     : ((((uintptr_t)g.A | (uintptr_t)g.lda | (uintptr_t)g.a_batch_stride) & 3) == 0);
+            g.a_end = conv ? nullptr : g.A + (int64_t)(batch - 1) * g.a_batch_stride + (int64_t)(g.M - 1) * g.lda + g.K;
             // its producers address a block's A rows (dense) or the whole image batch (convolution) with 32-bit offsets
             const int64_t span = conv ? (int64_t)((g.M + g.conv.OH * g.conv.OW - 1) / (g.conv.OH * g.conv.OW)) *
                                             g.conv.H * g.conv.W * g.conv.C
                                       : (int64_t)g.lda * 256 + g.K;
-            if (dma_idx >= 0 && aligned && g.K % 16 == 0 && span < ((int64_t)1 << 32))
+            if (dma_idx >= 0 && aligned && g.K >= 16 && span < ((int64_t)1 << 32))
             {
                 const MfmaConfig c = dma_config(dma_idx);
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;
@@ -661,6 +662,15 @@ static void conv_geom(const mi355_conv_desc &d, ConvGeom &g)
     int h = (int)std::floor((float)(d.H + d.pad_top + d.pad_bottom - (d.dilation_y * (d.KH - 1) + 1)) / (float)d.stride_y + 1.f);
     g.OW = w < 1 ? 1 : w;
     g.OH = h < 1 ? 1 : h;
+    auto magic = [](int32_t dv) -> uint32_t { return dv == 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / (uint64_t)dv) + 1u; };
+    g.magic_C = magic(g.C), g.magic_KW = magic(g.KW), g.magic_OW = magic(g.OW), g.magic_OH = magic(g.OH);
+}
+
+// the implicit-GEMM loader divides by C, KW, OW and OH with 32-bit reciprocal multiplies: exact while x * d < 2^32
+static bool conv_fast_div_ok(const mi355_conv_desc &d, const ConvGeom &g)
+{
+    const int64_t M = (int64_t)d.batch * g.OH * g.OW, K = (int64_t)d.KH * d.KW * d.C, lim = (int64_t)1 << 32;
+    return M * g.OW < lim && (M / g.OW + 1) * g.OH < lim && (K + 256) * d.C < lim && ((int64_t)d.KH * d.KW + 256) * d.KW < lim;
 }
 
 void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW)
@@ -717,7 +727,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         return 1;
     }
     // the on-the-fly loader moves 16-byte pieces of one tap: needs C % 16 == 0; it has no row sums: needs b_off == 0
-    h->implicit      = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0;
+    h->implicit      = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(d, h->geom);
     h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
     if (h->implicit)
         c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
@@ -761,7 +771,7 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
         return fail("update cannot switch between per-tensor and per-channel requantisation");
     h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
     c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
-    h->implicit      = h->d.path == 0 && (h->d.C % 16 == 0) && c.b_off_eff() == 0;
+    h->implicit      = h->d.path == 0 && (h->d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(h->d, h->geom);
     h->geom.pad_word = ((uint32_t)pad_value & 0xFFu) * 0x01010101u;
     c.fill_byte      = (uint8_t)(pad_value & 0xFF);
     c.kprefix        = h->implicit ? "implicit_" : "im2col+";

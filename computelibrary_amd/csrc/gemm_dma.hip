@@ -71,12 +71,12 @@ struct PanelProducer
     static constexpr int STAGE = (BM + BN) * BK;
     static_assert((AU + BU) % NP == 0, "staging shape");
 
-    const int8_t *a_base, *b_base, *fill16; // wave-uniform
+    const int8_t *a_base, *b_base, *fill16, *a_end; // wave-uniform
     uint32_t      off[LPP];                 // this lane's byte offset from the base (dense A rows, B rows, conv image)
     int           a_c16[LPP];               // byte offset of this lane's column inside a K step
     int           a_iy0[LPP], a_ix0[LPP];   // conv: top-left input coordinate of this lane's output pixel
     uint32_t      lds0;
-    int           pw, K;
+    int           pw, K, lane_id;
     ConvGeom      conv;
 
     __device__ __forceinline__ void init(const GemmArgs &g, int m0, int n0, int bz, int producer_wave, int lane,
@@ -87,6 +87,8 @@ struct PanelProducer
         K      = g.K;
         conv   = g.conv;
         fill16 = g.fill16;
+        a_end  = g.a_end;
+        lane_id = lane;
         a_base = g.A + (int64_t)bz * g.a_batch_stride + (CONV ? (int64_t)0 : (int64_t)m0 * g.lda);
         b_base = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
         const int ur = lane / CPR; // row inside a unit
@@ -103,10 +105,10 @@ struct PanelProducer
                 const int gr  = min(m0 + row, g.M - 1);
                 if (CONV)
                 {
-                    const int ox = gr % g.conv.OW;
-                    const int t  = gr / g.conv.OW;
-                    const int oy = t % g.conv.OH;
-                    const int n  = t / g.conv.OH;
+                    const int t  = fast_div(gr, g.conv.magic_OW);
+                    const int ox = gr - t * g.conv.OW;
+                    const int n  = fast_div(t, g.conv.magic_OH);
+                    const int oy = t - n * g.conv.OH;
                     off[i]       = (uint32_t)n * (uint32_t)(g.conv.H * g.conv.W * g.conv.C);
                     a_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
                     a_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
@@ -146,14 +148,28 @@ struct PanelProducer
                 if (full)
                     dma16s(a_k, off[i], dst);
                 else
-                    dma16(k0 + a_c16[i] < K ? a_k + off[i] : fill16, dst);
+                {
+                    // last K step. Columns at or beyond K read the fill bytes. A column that straddles K reads on into
+                    // the next row (those bytes meet the zero rows of the packed B) - except at the very end of A, where
+                    // the lane fetches just the valid bytes and writes its LDS slot itself.
+                    const int     k   = k0 + a_c16[i];
+                    const int8_t *ptr = a_k + off[i];
+                    if (k >= K || ptr + 16 <= a_end)
+                        dma16(k < K ? ptr : fill16, dst);
+                    else
+                    {
+                        const v4i v = load16_partial(ptr, K - k);
+                        *(__attribute__((address_space(3))) v4i *)(size_t)(dst + (uint32_t)lane_id * 16u) = v;
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    }
+                }
             }
             else
             {
                 const int k     = k0 + a_c16[i];
-                const int tap   = k / conv.C;
+                const int tap   = fast_div(k, conv.magic_C);
                 const int c0    = k - tap * conv.C;
-                const int ky    = tap / conv.KW;
+                const int ky    = fast_div(tap, conv.magic_KW);
                 const int kx    = tap - ky * conv.KW;
                 const int iy    = a_iy0[i] + ky * conv.dil_y;
                 const int ix    = a_ix0[i] + kx * conv.dil_x;
@@ -186,6 +202,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     static_assert((AU + BU) % NP == 0, "staging shape");
     static_assert(TM % 32 == 0 && TN % 32 == 0 && FM >= 1 && FN >= 1, "wave tile");
     static_assert(NS >= 3 && (NS - 2) * LPP < 64, "ring depth / vmcnt range");
+    static_assert(NW * 32 * (FN * 128 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
@@ -363,6 +380,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
                 epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
         }
     }
+    else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store)
+    {
+        // the ring is free beyond the last barrier: 32 x (FN*128 + 16) bytes per wave
+        if constexpr (EPI != EPI_FIXEDPOINT)
+            epilogue_store_wave32<EPI, FM, FN>(acc, g, smem + wave * 32 * (FN * 128 + 16), m0 + row_w, n0 + col_w, lane, bz);
+    }
     else
         epilogue_store_t<EPI, FM, FN>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
 }
@@ -396,6 +419,9 @@ static const DmaEntry g_dma[] = {
     MI355_DCFG("pp_128x64x128_s3", 128, 64, 128, 2, 2, 3),
     MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
     MI355_DCFG("pp_256x128x64_s4", 256, 128, 64, 2, 2, 4),
+    MI355_DCFG("pp_256x64x64_s4", 256, 64, 64, 2, 1, 4),
+    MI355_DCFG("pp_128x64x64_s4", 128, 64, 64, 1, 1, 4),
+    MI355_DCFG("pp_256x64x128_s3", 256, 64, 128, 2, 1, 3),
 };
 
 int dma_num_configs()
@@ -415,13 +441,13 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     const void     *fn = c.fn[epi][flip_a ? 1 : 0][conv ? 1 : 0];
     if (fn == nullptr || args.fill16 == nullptr)
         return (int)hipErrorInvalidValue;
-    // shapes the kernel assumes: whole 16-byte columns, 16-byte aligned rows, tiles that cover the output and stay
-    // inside the packed B panel
-    if (args.K % 16 != 0 || args.K > args.Kp || args.Kp % c.cfg.BK != 0 || args.tiles_m * c.cfg.BM < args.M ||
+    // shapes the kernel assumes: dword-aligned rows of at least one 16-byte column (whole columns of one tap for the
+    // convolution), tiles that cover the output and stay inside the packed B panel
+    if (args.K < 16 || args.K > args.Kp || args.Kp % c.cfg.BK != 0 || args.tiles_m * c.cfg.BM < args.M ||
         args.tiles_n * c.cfg.BN < args.N || args.tiles_n * c.cfg.BN > round_up(args.N, PACK_N_ALIGN) || args.M < 1)
         return (int)hipErrorInvalidValue;
-    if (conv ? (args.conv.C % 16 != 0 || ((uintptr_t)args.A & 15) != 0)
-             : ((((uintptr_t)args.A | (uintptr_t)args.lda | (uintptr_t)args.a_batch_stride) & 15) != 0))
+    if (conv ? (args.conv.C % 16 != 0 || ((uintptr_t)args.A & 15) != 0 || args.K % 16 != 0)
+             : ((((uintptr_t)args.A | (uintptr_t)args.lda | (uintptr_t)args.a_batch_stride) & 3) != 0 || args.a_end == nullptr))
         return (int)hipErrorInvalidValue;
     if (c.lds_bytes > 48 * 1024)
     {

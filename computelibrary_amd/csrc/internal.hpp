@@ -22,7 +22,15 @@ struct ConvGeom
     int32_t H, W, C, KH, KW, OH, OW;
     int32_t stride_x, stride_y, pad_left, pad_top, dil_x, dil_y;
     uint32_t pad_word; // the padding byte (already sign-flipped if the loader flips) replicated into 4 bytes
+    // floor(2^32 / d) + 1 for d = C, KW, OW, OH (0 when d == 1): x / d == mulhi(x, magic) exactly while x * d < 2^32
+    uint32_t magic_C, magic_KW, magic_OW, magic_OH;
 };
+
+// x / d for the divisors above (see ConvGeom::magic_*); the caller guarantees x * d < 2^32
+__device__ __forceinline__ int fast_div(int x, uint32_t magic)
+{
+    return magic ? (int)__umulhi((uint32_t)x, magic) : x;
+}
 
 struct GemmArgs
 {
@@ -37,6 +45,7 @@ struct GemmArgs
     EpiParams     epi;
     ConvGeom      conv;
     const int8_t *fill16; // 16 readable bytes: what a staged 16-byte column reads where A has no data (zeros / pad value)
+    const int8_t *a_end;  // dense A: one past the last byte of the last row of the last batch (no 16-byte read may cross it)
 };
 
 struct MfmaConfig

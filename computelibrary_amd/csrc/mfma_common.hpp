@@ -336,4 +336,74 @@ __device__ __forceinline__ void epilogue_store_staged(const v16i (&acc)[FM][FN],
         }
     }
 }
+// S32 / F32 results of one wave's (FM*32) x (FN*32) sub-tile, 32 rows at a time through a wave-private LDS area
+// (32 rows, pitch FN*128 + 16 bytes) so that they leave as 16 bytes per lane along whole row segments of FN*128 bytes
+// instead of 32-byte pieces of 32 different rows. Needs no synchronisation with other waves. Requires p.vec_store.
+template <int EPI, int FM, int FN>
+__device__ __forceinline__ void epilogue_store_wave32(const v16i (&acc)[FM][FN], const GemmArgs &g, char *stage, int row0,
+                                                      int col0, int lane, int bz)
+{
+    static_assert(EPI == EPI_S32 || EPI == EPI_F32, "32-bit outputs only");
+    constexpr int    PITCH = FN * 128 + 16;
+    constexpr int    LPR   = FN * 8;   // lanes per output row segment
+    constexpr int    RPI   = 64 / LPR; // rows per wave instruction
+    const int        lr = lane & 31, lh = lane >> 5;
+    const EpiParams &p      = g.epi;
+    const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    char            *D      = (char *)g.D + (int64_t)bz * g.d_batch_stride * 4;
+    const int        rr = lane / LPR, cc = lane % LPR;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+    {
+        const int     i  = row0 + fm * 32 + lr;
+        const int32_t rv = (rowvec && i < g.M) ? rowvec[i] : 0;
+#pragma unroll
+        for (int fn = 0; fn < FN; ++fn)
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int c  = fn * 32 + 8 * q + 4 * lh;
+                const int j0 = col0 + c; // inside the padded vectors
+                const v4i cv = *(const v4i *)(colvec + j0);
+                v4i       o;
+                if (EPI == EPI_S32)
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv);
+                }
+                else
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                    {
+                        const float bf = (p.bias_f32 && j0 + t < g.N) ? p.bias_f32[j0 + t] : 0.f;
+                        o[t] = __float_as_int(epi_f32(acc[fm][fn][4 * q + t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bf,
+                                                      p.bias_f32 != nullptr, p));
+                    }
+                }
+                *(v4i *)(stage + lr * PITCH + c * 4) = o;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it)
+        {
+            const int r  = it * RPI + rr;
+            const int gi = row0 + fm * 32 + r, j0 = col0 + cc * 4;
+            if (gi >= g.M || j0 >= g.N)
+                continue;
+            const v4i     val = *(const v4i *)(stage + r * PITCH + cc * 16);
+            const int64_t idx = ((int64_t)gi * g.ldd + j0) * 4;
+            if (j0 + 3 < g.N)
+                *(v4i *)(D + idx) = val;
+            else
+            {
+                for (int t = 0; t < g.N - j0; ++t)
+                    *(int32_t *)(D + idx + 4 * t) = val[t];
+            }
+        }
+    }
+}
 } // namespace mi355

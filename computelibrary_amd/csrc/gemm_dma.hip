@@ -56,10 +56,13 @@ __device__ __forceinline__ void block_barrier()
 // Stages the A and B panels of one block tile. All NP producer waves of a block hold one of these. The loads use the
 // scalar-base form of the instruction (wave-uniform 64-bit base in SGPRs + one 32-bit offset register per lane): with
 // per-lane 64-bit addresses every load costs the SIMD's matrix pipe about 50 clocks, with scalar bases the stream
-// overlaps the matrix instructions almost completely. The K offset of a step is added to the scalar base, so a dense
-// producer executes no vector ALU work at all inside the loop. Lanes that must read padding instead (K tail of A,
-// out-of-image taps of the implicit convolution) need a different base: a wave with any such lane falls back to
-// per-lane addresses for that one load.
+// overlaps the matrix instructions almost completely. Unit u of a stage (1 KiB = RPU tile rows) belongs to producer
+// u % NP. Inside a unit, lane l covers row l / CPR at LDS column slot l % CPR, i.e. global column (l % CPR) ^ swz(row);
+// that column is the same for every unit of a wave (see SAME_COL), so a dense producer keeps ONE offset register for A
+// and one for B and moves from unit to unit and from K step to K step by scalar additions to the base: no vector
+// registers per load (arrays of per-load offsets were spilled to scratch memory, and every reload waited for all the
+// loads in flight). Lanes that must read padding instead (K tail of A, out-of-image taps of the implicit convolution)
+// need a different base: a wave with any such lane falls back to per-lane addresses for that one load.
 template <int BM, int BN, int BK, int NP, int NS, bool CONV>
 struct PanelProducer
 {
@@ -67,14 +70,22 @@ struct PanelProducer
     static constexpr int RPU   = 1024 / BK; // tile rows per staging unit (one wave instruction = 1 KiB)
     static constexpr int AU    = BM / RPU;  // staging units of the A part of a stage
     static constexpr int BU    = BN / RPU;
-    static constexpr int LPP   = (AU + BU) / NP; // loads per producer wave per stage: unit u belongs to producer u % NP
+    static constexpr int LPP   = (AU + BU) / NP; // loads per producer wave per stage
+    static constexpr int LPA   = (AU + NP - 1) / NP; // at most this many of them are A units
     static constexpr int STAGE = (BM + BN) * BK;
     static_assert((AU + BU) % NP == 0, "staging shape");
+    // swz(row) of row = u*RPU + r depends on u only through (4u) & (CPR-1): constant for CPR <= 4, the parity of u for
+    // CPR == 8 - and u = pw + i*NP keeps its parity when NP is even
+    static_assert(CPR <= 4 || (CPR == 8 && NP % 2 == 0), "every unit of a producer wave must share the lane -> column map");
 
     const int8_t *a_base, *b_base, *fill16, *a_end; // wave-uniform
-    uint32_t      off[LPP];                 // this lane's byte offset from the base (dense A rows, B rows, conv image)
-    int           a_c16[LPP];               // byte offset of this lane's column inside a K step
-    int           a_iy0[LPP], a_ix0[LPP];   // conv: top-left input coordinate of this lane's output pixel
+    uint32_t      lane_a, lane_b; // dense A: (l / CPR) * lda + column bytes; B: (l / CPR) * Kp + column bytes
+    int           c16;            // byte offset of this lane's column inside a K step
+    int           ur;             // this lane's row inside a unit
+    int           rows_left;      // M - m0: rows of A at and below the tile's first row
+    int64_t       lda, Kp;
+    uint32_t      c_off[CONV ? LPA : 1]; // conv: image offset of the (possibly out-of-image) top-left tap of the lane's pixel
+    int           c_iy0[CONV ? LPA : 1], c_ix0[CONV ? LPA : 1]; // conv: its input coordinates
     uint32_t      lds0;
     int           pw, K, lane_id;
     ConvGeom      conv;
@@ -82,78 +93,87 @@ struct PanelProducer
     __device__ __forceinline__ void init(const GemmArgs &g, int m0, int n0, int bz, int producer_wave, int lane,
                                          uint32_t lds_base)
     {
-        pw     = producer_wave;
-        lds0   = lds_base;
-        K      = g.K;
-        conv   = g.conv;
-        fill16 = g.fill16;
-        a_end  = g.a_end;
-        lane_id = lane;
-        a_base = g.A + (int64_t)bz * g.a_batch_stride + (CONV ? (int64_t)0 : (int64_t)m0 * g.lda);
-        b_base = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
-        const int ur = lane / CPR; // row inside a unit
-        const int up = lane % CPR; // LDS column slot inside the row
-#pragma unroll
-        for (int i = 0; i < LPP; ++i)
+        pw        = producer_wave;
+        lds0      = lds_base;
+        K         = g.K;
+        conv      = g.conv;
+        fill16    = g.fill16;
+        a_end     = g.a_end;
+        lane_id   = lane;
+        lda       = g.lda;
+        Kp        = g.Kp;
+        rows_left = g.M - m0;
+        a_base    = g.A + (int64_t)bz * g.a_batch_stride + (CONV ? (int64_t)0 : (int64_t)m0 * g.lda);
+        b_base    = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp;
+        ur        = lane / CPR;
+        const int c = (lane % CPR) ^ swz<CPR>(pw * RPU + ur);
+        c16       = c * 16;
+        lane_a    = (uint32_t)ur * (uint32_t)g.lda + (uint32_t)c16;
+        lane_b    = (uint32_t)ur * (uint32_t)g.Kp + (uint32_t)c16;
+        if (CONV)
         {
-            const int u = pw + i * NP; // wave-uniform
-            if (u < AU)
+#pragma unroll
+            for (int i = 0; i < LPA; ++i)
             {
-                const int row = u * RPU + ur;
-                const int c   = up ^ swz<CPR>(row);
-                a_c16[i]      = c * 16;
-                const int gr  = min(m0 + row, g.M - 1);
-                if (CONV)
-                {
-                    const int t  = fast_div(gr, g.conv.magic_OW);
-                    const int ox = gr - t * g.conv.OW;
-                    const int n  = fast_div(t, g.conv.magic_OH);
-                    const int oy = t - n * g.conv.OH;
-                    off[i]       = (uint32_t)n * (uint32_t)(g.conv.H * g.conv.W * g.conv.C);
-                    a_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
-                    a_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
-                }
-                else
-                {
-                    off[i]   = (uint32_t)(gr - m0) * (uint32_t)g.lda + (uint32_t)(c * 16);
-                    a_iy0[i] = a_ix0[i] = 0;
-                }
-            }
-            else
-            {
-                const int row = (u - AU) * RPU + ur;
-                const int c   = up ^ swz<CPR>(row);
-                off[i]        = (uint32_t)row * (uint32_t)g.Kp + (uint32_t)(c * 16);
-                a_c16[i] = a_iy0[i] = a_ix0[i] = 0;
+                const int gr = min(m0 + (pw + i * NP) * RPU + ur, g.M - 1);
+                const int t  = fast_div(gr, g.conv.magic_OW);
+                const int ox = gr - t * g.conv.OW;
+                const int n  = fast_div(t, g.conv.magic_OH);
+                const int oy = t - n * g.conv.OH;
+                c_iy0[i]     = oy * g.conv.stride_y - g.conv.pad_top;
+                c_ix0[i]     = ox * g.conv.stride_x - g.conv.pad_left;
+                c_off[i]     = (uint32_t)n * (uint32_t)(g.conv.H * g.conv.W * g.conv.C) +
+                           (uint32_t)((c_iy0[i] * g.conv.W + c_ix0[i]) * g.conv.C);
             }
         }
     }
 
-    __device__ __forceinline__ void issue(int kt) const
+    // K step kt of the tile into ring slot `slot`
+    __device__ __forceinline__ void issue(int kt, int slot) const
     {
         const int      k0   = kt * BK;
-        const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
+        const uint32_t base = lds0 + (uint32_t)slot * STAGE;
         const int8_t  *a_k  = a_base + (CONV ? 0 : k0);
         const int8_t  *b_k  = b_base + k0; // always inside the zero-padded packed panel
         const bool     full = k0 + BK <= K;
+        // convolution: one tap decode per K step (the lane's column is the same in every unit)
+        bool     t_in = false;
+        int      t_dy = 0, t_dx = 0;
+        uint32_t t_off = 0;
+        if (CONV)
+        {
+            const int k   = k0 + c16;
+            const int tap = fast_div(k, conv.magic_C);
+            const int c0  = k - tap * conv.C;
+            const int ky  = fast_div(tap, conv.magic_KW);
+            const int kx  = tap - ky * conv.KW;
+            t_dy          = ky * conv.dil_y;
+            t_dx          = kx * conv.dil_x;
+            t_off         = (uint32_t)((t_dy * conv.W + t_dx) * conv.C + c0);
+            t_in          = k < K;
+        }
 #pragma unroll
         for (int i = 0; i < LPP; ++i)
         {
-            const int      u   = pw + i * NP;
+            const int      u   = pw + i * NP; // wave-uniform
             const uint32_t dst = base + (uint32_t)u * 1024u;
             if (u >= AU)
-                dma16s(b_k, off[i], dst);
+                dma16s(b_k + (int64_t)(u - AU) * RPU * Kp, lane_b, dst);
             else if (!CONV)
             {
+                // rows beyond M re-read row M-1 (their results are never stored): only the last row tile has any
+                const bool     edge = (u + 1) * RPU > rows_left;
+                const int8_t  *ub   = edge ? a_k : a_k + (int64_t)u * RPU * lda;
+                const uint32_t o    = edge ? (uint32_t)min(u * RPU + ur, rows_left - 1) * (uint32_t)lda + (uint32_t)c16 : lane_a;
                 if (full)
-                    dma16s(a_k, off[i], dst);
+                    dma16s(ub, o, dst);
                 else
                 {
                     // last K step. Columns at or beyond K read the fill bytes. A column that straddles K reads on into
                     // the next row (those bytes meet the zero rows of the packed B) - except at the very end of A, where
                     // the lane fetches just the valid bytes and writes its LDS slot itself.
-                    const int     k   = k0 + a_c16[i];
-                    const int8_t *ptr = a_k + off[i];
+                    const int     k   = k0 + c16;
+                    const int8_t *ptr = ub + o;
                     if (k >= K || ptr + 16 <= a_end)
                         dma16(k < K ? ptr : fill16, dst);
                     else
@@ -166,15 +186,9 @@ struct PanelProducer
             }
             else
             {
-                const int k     = k0 + a_c16[i];
-                const int tap   = fast_div(k, conv.magic_C);
-                const int c0    = k - tap * conv.C;
-                const int ky    = fast_div(tap, conv.magic_KW);
-                const int kx    = tap - ky * conv.KW;
-                const int iy    = a_iy0[i] + ky * conv.dil_y;
-                const int ix    = a_ix0[i] + kx * conv.dil_x;
-                const bool ok   = k < K && iy >= 0 && iy < conv.H && ix >= 0 && ix < conv.W;
-                const uint32_t o = off[i] + (uint32_t)((iy * conv.W + ix) * conv.C + c0);
+                const int      iy = c_iy0[i < LPA ? i : 0] + t_dy, ix = c_ix0[i < LPA ? i : 0] + t_dx;
+                const bool     ok = t_in && (unsigned)iy < (unsigned)conv.H && (unsigned)ix < (unsigned)conv.W;
+                const uint32_t o  = c_off[i < LPA ? i : 0] + t_off;
                 if (__builtin_amdgcn_ballot_w64(ok) == ~0ull)
                     dma16s(a_k, o, dst);
                 else
@@ -229,7 +243,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
 #pragma unroll
         for (int s = 0; s < NS - 1; ++s)
             if (s < nk)
-                prod.issue(s);
+                prod.issue(s, s % NS);
         if (nk >= NS - 1)
             wait_vmcnt<(NS - 2) * LPP>(); // stage 0 complete, the NS-2 younger stages may still be in flight
         else
@@ -239,7 +253,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         {
             const bool more = kt + NS - 1 < nk;
             if (more)
-                prod.issue(kt + NS - 1); // ring slot of stage kt-1
+                prod.issue(kt + NS - 1, (kt + NS - 1) % NS); // ring slot of stage kt-1
             block_barrier();        // barrier 2kt+1
             if (more)
                 wait_vmcnt<(NS - 2) * LPP>(); // stage kt+1 complete

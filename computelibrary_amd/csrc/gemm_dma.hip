@@ -128,7 +128,8 @@ struct PanelProducer
         }
     }
 
-    // K step kt of the tile into ring slot `slot`
+    // K step kt of the tile into ring slot `slot`: loads [I0, I1) of this wave's LPP
+    template <int I0 = 0, int I1 = LPP>
     __device__ __forceinline__ void issue(int kt, int slot) const
     {
         const int      k0   = kt * BK;
@@ -153,7 +154,7 @@ struct PanelProducer
             t_in          = k < K;
         }
 #pragma unroll
-        for (int i = 0; i < LPP; ++i)
+        for (int i = I0; i < I1; ++i)
         {
             const int      u   = pw + i * NP; // wave-uniform
             const uint32_t dst = base + (uint32_t)u * 1024u;
@@ -251,10 +252,15 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         block_barrier(); // barrier 0
         for (int kt = 0; kt < nk; ++kt)
         {
+            // A wave gets one direct-to-LDS load accepted about every 90 clocks, so LPP of them take as long as the
+            // consumers' whole K step: issue half on either side of the mid-step barrier instead of making both
+            // consumer groups wait for all of them. Ring slot of stage kt-1: free since barrier 2kt.
             const bool more = kt + NS - 1 < nk;
             if (more)
-                prod.issue(kt + NS - 1, (kt + NS - 1) % NS); // ring slot of stage kt-1
-            block_barrier();        // barrier 2kt+1
+                prod.template issue<0, LPP / 2>(kt + NS - 1, (kt + NS - 1) % NS);
+            block_barrier(); // barrier 2kt+1
+            if (more)
+                prod.template issue<LPP / 2, LPP>(kt + NS - 1, (kt + NS - 1) % NS);
             if (more)
                 wait_vmcnt<(NS - 2) * LPP>(); // stage kt+1 complete
             else

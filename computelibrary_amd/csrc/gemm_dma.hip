@@ -439,9 +439,6 @@ static const DmaEntry g_dma[] = {
     MI355_DCFG("pp_128x64x128_s3", 128, 64, 128, 2, 2, 3),
     MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
     MI355_DCFG("pp_256x128x64_s4", 256, 128, 64, 2, 2, 4),
-    MI355_DCFG("pp_256x64x64_s4", 256, 64, 64, 2, 1, 4),
-    MI355_DCFG("pp_128x64x64_s4", 128, 64, 64, 1, 1, 4),
-    MI355_DCFG("pp_256x64x128_s3", 256, 64, 128, 2, 1, 3),
 };
 
 int dma_num_configs()

@@ -328,7 +328,7 @@ __device__ __forceinline__ void epilogue_store_staged(const v16i (&acc)[FM][FN],
         const v4i     val = *(const v4i *)(stage + r * PITCH + cc);
         const int64_t idx = (int64_t)i * g.ldd + j0;
         if (j0 + 16 <= g.N)
-            *(v4i *)(D + idx) = val;
+            __builtin_nontemporal_store(val, (v4i *)(D + idx));
         else
         {
             for (int t = 0; t < g.N - j0; ++t)
@@ -397,7 +397,7 @@ __device__ __forceinline__ void epilogue_store_wave32(const v16i (&acc)[FM][FN],
             const v4i     val = *(const v4i *)(stage + r * PITCH + cc * 16);
             const int64_t idx = ((int64_t)gi * g.ldd + j0) * 4;
             if (j0 + 3 < g.N)
-                *(v4i *)(D + idx) = val;
+                __builtin_nontemporal_store(val, (v4i *)(D + idx));
             else
             {
                 for (int t = 0; t < g.N - j0; ++t)

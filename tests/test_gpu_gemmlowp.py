@@ -166,6 +166,41 @@ def test_pipelined_kernel_epilogue_variants(case, N, ldd):
     assert name.startswith("pp_"), name
     np.testing.assert_array_equal(got, want)
 
+def test_run_can_be_captured_in_a_hip_graph():
+    """run() with device buffers only enqueues kernels on the given stream, so it can be captured; every replay, with
+    eager work and synchronisations in between, must reproduce the eager result."""
+    import torch
+    rng = np.random.default_rng(47)
+    M, N, K = 300, 256, 512
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    bias = rng.integers(-5000, 5000, size=N).astype(np.int32)
+    mult, shift = oracle.calculate_quantized_multipliers(1.0, rng.uniform(2e-4, 2e-3, size=N).astype(np.float32), 1.0)
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -3, 0, mult, shift, -5, -128, 127, np.int8)
+    g = capi.Gemm(M, N, K, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0,
+                  capi.requant(0, 0, -5, -128, 127, per_channel=True))
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    vecs = [torch.from_numpy(x).cuda() for x in (bias, mult, shift)]
+    Dd = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    g.prepare(Bd, *vecs)
+    g.run(Ad, Dd)  # first run outside the capture: allocates the handle's workspace
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(Dd.cpu().numpy(), want)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    announce("graph capture")
+    with torch.cuda.graph(graph, stream=side):
+        g.run(Ad, Dd, None, torch.cuda.current_stream().cuda_stream)
+    for rep in range(4):
+        Dd.fill_(77)                                # eager work between replays
+        A2 = torch.roll(Ad, rep, 0) if rep else Ad  # and new input contents in the same buffer
+        Ad.copy_(A2)
+        torch.cuda.synchronize()
+        announce("graph replay", rep)
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(Dd.cpu().numpy(), np.roll(want, sum(range(rep + 1)), 0))
+    g.close()
+
 def test_requant_extremes_on_device():
     """Accumulators and multipliers at the edges of int32 (saturating SQDMULH, shift 0 / 31, wrap-around adds)
     through the stand-alone output stage."""

@@ -226,10 +226,9 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    int tm, tn;
-    tile_coords(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+    int tm, tn, bz;
+    tile_coords_batched(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, bz, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int bz = blockIdx.z;
     const int nk = (g.K + BK - 1) / BK;
 
     // Barrier protocol (b = number of barriers a wave has executed): consumer group 0 reads stage kt between barriers
@@ -474,7 +473,7 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     }
     GemmArgs a       = args;
     void    *kargs[] = {&a};
-    dim3     grid(args.tiles_m * args.tiles_n, 1, batch), block(c.threads);
+    dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block(c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);
 }
 } // namespace mi355

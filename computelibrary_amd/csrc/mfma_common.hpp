@@ -35,6 +35,27 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
     tn                = in_grp / gsize;
 }
 
+// The same for a batch of GEMMs launched as one 1-D grid of batch * tiles_m * tiles_n workgroups: the logical ids run
+// batch-major, so an XCD's contiguous run covers whole batch entries (their A and B are then fetched into one L2 only).
+__device__ __forceinline__ void tile_coords_batched(int bid, int nblocks, int tiles_m, int tiles_n, int &bz, int &tm,
+                                                    int &tn)
+{
+    int l = bid;
+    if ((nblocks & 7) == 0)
+        l = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+    const int tpb = tiles_m * tiles_n;
+    bz            = l / tpb;
+    l -= bz * tpb;
+    const int GM      = 4;
+    const int per_grp = GM * tiles_n;
+    const int grp     = l / per_grp;
+    const int first   = grp * GM;
+    const int gsize   = min(tiles_m - first, GM);
+    const int in_grp  = l - grp * per_grp;
+    tm                = first + in_grp % gsize;
+    tn                = in_grp / gsize;
+}
+
 // Accumulator (fm, fn, r) of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 block.
 // (row0, col0) is the wave's top-left output coordinate.
 template <int EPI, int FM, int FN>

@@ -32,7 +32,8 @@ class GemmDesc(C.Structure):
                 ("a_batch_stride", C.c_int64), ("b_batch_stride", C.c_int64), ("d_batch_stride", C.c_int64),
                 ("a_offset", C.c_int32), ("b_offset", C.c_int32), ("requant", Requant),
                 ("scale", C.c_float), ("act_min", C.c_float), ("act_max", C.c_float),
-                ("path", C.c_int32), ("reserved", C.c_int32)]
+                ("path", C.c_int32), ("b_transposed", C.c_int32), ("b_k_interleave", C.c_int32),
+                ("reserved", C.c_int32)]
 
 
 class OutputStageDesc(C.Structure):
@@ -129,11 +130,12 @@ class Gemm:
 
     def __init__(self, M, N, K, a_dtype, b_dtype, dst_dtype, epilogue, a_offset=0, b_offset=0, rq=None, scale=1.0,
                  act_min=-np.inf, act_max=np.inf, batch=1, b_batched=False, lda=None, ldb=None, ldd=None,
-                 path=PATH_AUTO):
-        lda, ldb, ldd = lda or K, ldb or N, ldd or N
+                 path=PATH_AUTO, b_transposed=False, b_k_interleave=0):
+        lda, ldb, ldd = lda or K, ldb or (K if b_transposed else N), ldd or N
+        b_rows = N if b_transposed else K
         self.desc = GemmDesc(M, N, K, batch, a_dtype, b_dtype, dst_dtype, epilogue, lda, ldb, ldd, M * lda,
-                             K * ldb if b_batched else 0, M * ldd, a_offset, b_offset, rq or requant(), scale,
-                             act_min, act_max, path, 0)
+                             b_rows * ldb if b_batched else 0, M * ldd, a_offset, b_offset, rq or requant(), scale,
+                             act_min, act_max, path, 1 if b_transposed else 0, b_k_interleave, 0)
         self._h = C.c_void_p()
         _check(lib().mi355_gemmlowp_create(C.byref(self.desc), C.byref(self._h)))
 

@@ -455,8 +455,10 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
         return fail("M, N, K, batch must be positive (got %d %d %d %d)", d.M, d.N, d.K, d.batch);
     if (!is_8bit(d.a_dtype) || !is_8bit(d.b_dtype))
         return fail("A and B must be 8-bit");
-    if (d.lda < d.K || d.ldb < d.N || d.ldd < d.N)
+    if (d.lda < d.K || d.ldb < (d.b_transposed ? d.K : d.N) || d.ldd < d.N)
         return fail("row stride smaller than the row");
+    if (d.b_k_interleave < 0 || (d.b_k_interleave > 1 && d.K % d.b_k_interleave != 0))
+        return fail("b_k_interleave must divide K");
     switch (d.epilogue)
     {
         case MI355_EPI_S32:
@@ -478,7 +480,8 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
     }
     if (d.batch > 1 && (d.a_batch_stride < (int64_t)(d.M - 1) * d.lda + d.K || d.d_batch_stride < (int64_t)(d.M - 1) * d.ldd + d.N))
         return fail("batch stride smaller than one matrix");
-    if (d.batch > 1 && d.b_batch_stride != 0 && d.b_batch_stride < (int64_t)(d.K - 1) * d.ldb + d.N)
+    if (d.batch > 1 && d.b_batch_stride != 0 &&
+        d.b_batch_stride < (d.b_transposed ? (int64_t)(d.N - 1) * d.ldb + d.K : (int64_t)(d.K - 1) * d.ldb + d.N))
         return fail("B batch stride smaller than one matrix");
     mi355_gemm_handle *h = new (std::nothrow) mi355_gemm_handle();
     if (!h)
@@ -510,7 +513,8 @@ int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *b
     GemmCore              &c = h->core;
     const mi355_gemm_desc &d = h->d;
     const int              nb = c.nb();
-    const size_t           b_bytes = (size_t)(nb - 1) * d.b_batch_stride + (size_t)(d.K - 1) * d.ldb + d.N;
+    const size_t           b_bytes = (size_t)(nb - 1) * d.b_batch_stride +
+                           (d.b_transposed ? (size_t)(d.N - 1) * d.ldb + d.K : (size_t)(d.K - 1) * d.ldb + d.N);
     const void            *Bd, *biasd, *multd, *shiftd;
     TRY(to_device(B, b_bytes, h->stageB, s, &Bd));
     TRY(to_device(bias, sizeof(int32_t) * d.N, h->stageBias, s, &biasd));
@@ -519,8 +523,15 @@ int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *b
     TRY(c.Bp.ensure((size_t)nb * c.Np * c.Kp));
     TRY(c.colsum.ensure(sizeof(int32_t) * (size_t)nb * c.Np));
     for (int b = 0; b < nb; ++b)
-        HIP_TRY(pack_b_launch((const uint8_t *)Bd + (size_t)b * d.b_batch_stride, d.ldb, d.K, d.N, c.Kp, c.Np, c.flip_b,
-                              c.Bp.as<int8_t>() + (size_t)b * c.Np * c.Kp, c.colsum.as<int32_t>() + (size_t)b * c.Np, s));
+    {
+        const uint8_t *src = (const uint8_t *)Bd + (size_t)b * d.b_batch_stride;
+        int8_t        *dst = c.Bp.as<int8_t>() + (size_t)b * c.Np * c.Kp;
+        int32_t       *cs  = c.colsum.as<int32_t>() + (size_t)b * c.Np;
+        if (d.b_transposed)
+            HIP_TRY(pack_bt_launch(src, d.ldb, d.K, d.N, c.Kp, c.Np, c.flip_b, d.b_k_interleave, dst, cs, s));
+        else
+            HIP_TRY(pack_b_launch(src, d.ldb, d.K, d.N, c.Kp, c.Np, c.flip_b, d.b_k_interleave, dst, cs, s));
+    }
     if (c.path == MI355_PATH_SKINNY && nb != 1)
         return fail("skinny path does not batch");
     TRY(c.finish_prepare((const int32_t *)biasd, (const int32_t *)multd, (const int32_t *)shiftd, s));
@@ -753,7 +764,7 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t 
     TRY(c.colsum.ensure(sizeof(int32_t) * (size_t)c.Np));
     // weights [OFM][KH][KW][C] are already the K-contiguous layout with k = c + kx*C + ky*C*KW
     // (src/cpu/kernels/CpuWeightsReshapeKernel.cpp:150-166)
-    HIP_TRY(pack_bt_launch(wd, c.K, c.K, c.N, c.Kp, c.Np, c.flip_b, c.Bp.as<int8_t>(), c.colsum.as<int32_t>(), s));
+    HIP_TRY(pack_bt_launch(wd, c.K, c.K, c.N, c.Kp, c.Np, c.flip_b, 0, c.Bp.as<int8_t>(), c.colsum.as<int32_t>(), s));
     TRY(c.finish_prepare((const int32_t *)biasd, (const int32_t *)multd, (const int32_t *)shiftd, s));
     HIP_TRY(hipStreamSynchronize(s));
     return 0;

@@ -97,10 +97,10 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
 
 // kernels_aux.hip
 // B [K][ldb] (row-major, N contiguous) -> Bp [Np][Kp] int8 (flip: xor 0x80), colsum[Np] (sums of the packed int8 values)
-int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int kf, int8_t *Bp, int32_t *colsum,
                   hipStream_t s);
 // B given as [N][ldk] with K contiguous (conv weights [OFM][KH*KW*C])
-int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
+int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int kf, int8_t *Bp, int32_t *colsum,
                    hipStream_t s);
 // Bp [Np][Kp] -> operand order for the skinny kernel: [Np/16][Kp/64][64 lanes][16 bytes]
 int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream_t s);

@@ -35,8 +35,16 @@ int fill_i32_launch(int32_t *p, int32_t v, int64_t n, hipStream_t s)
 // ---- P1: B[K][ldb] -> Bp[Np][Kp] (transpose to K-contiguous, optional sign flip, zero padding) + column sums ----------
 // Replaces pretranspose_B_array (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:594-617) / CpuGemmTranspose1xWKernel and
 // CpuGemmLowpMatrixBReductionKernel (src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:273-446) in one pass over B.
+// kf > 1 re-orders K on the way: packed row k = a*kf + b (b < kf) is source row b*(K/kf) + a, which is what
+// CpuConvertFullyConnectedWeightsKernel does to weights trained in the other data layout
+// (src/cpu/kernels/CpuConvertFullyConnectedWeightsKernel.cpp:60-66,118-121 with kf = its _factor2).
+__device__ __forceinline__ int k_source(int k, int K, int kf)
+{
+    return kf > 1 ? (k % kf) * (K / kf) + k / kf : k;
+}
+
 __global__ __launch_bounds__(256) void pack_b_kernel(const uint8_t *__restrict__ B, int64_t ldb, int K, int N, int Kp,
-                                                     uint8_t flip, int8_t *__restrict__ Bp,
+                                                     uint8_t flip, int kf, int8_t *__restrict__ Bp,
                                                      int32_t *__restrict__ colsum)
 {
     __shared__ __attribute__((aligned(16))) uint8_t tile[64][64 + 16]; // [n][k]
@@ -48,7 +56,7 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const uint8_t *__restrict__
         const int k = k0 + ty * 16 + kk, n = n0 + tx;
         uint8_t   v = 0;
         if (k < K && n < N)
-            v = B[(int64_t)k * ldb + n] ^ flip;
+            v = B[(int64_t)k_source(k, K, kf) * ldb + n] ^ flip;
         tile[tx][ty * 16 + kk] = v;
     }
     __syncthreads();
@@ -62,23 +70,23 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const uint8_t *__restrict__
         atomicAdd(colsum + n0 + n, s);
 }
 
-int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
-                  hipStream_t s)
+int pack_b_launch(const void *B, int64_t ldb, int K, int N, int Kp, int Np, bool flip, int kf, int8_t *Bp,
+                  int32_t *colsum, hipStream_t s)
 {
-    if (Np % 64 || Kp % 64 || Np < N || Kp < K)
+    if (Np % 64 || Kp % 64 || Np < N || Kp < K || (kf > 1 && K % kf != 0))
         return (int)hipErrorInvalidValue;
     int e = fill_i32_launch(colsum, 0, Np, s);
     if (e)
         return e;
-    pack_b_kernel<<<dim3(Np / 64, Kp / 64), dim3(256), 0, s>>>((const uint8_t *)B, ldb, K, N, Kp, flip ? 0x80 : 0, Bp,
-                                                               colsum);
+    pack_b_kernel<<<dim3(Np / 64, Kp / 64), dim3(256), 0, s>>>((const uint8_t *)B, ldb, K, N, Kp, flip ? 0x80 : 0, kf,
+                                                               Bp, colsum);
     return launch_status();
 }
 
 // B already K-contiguous: Bt[N][ldk] (convolution weights [OFM][KH*KW*C], the layout CpuWeightsReshapeKernel
 // produces transposed: src/cpu/kernels/CpuWeightsReshapeKernel.cpp:150-166)
 __global__ __launch_bounds__(256) void pack_bt_kernel(const uint8_t *__restrict__ Bt, int64_t ldk, int K, int N, int Kp,
-                                                      int Np, uint8_t flip, int8_t *__restrict__ Bp,
+                                                      int Np, uint8_t flip, int kf, int8_t *__restrict__ Bp,
                                                       int32_t *__restrict__ colsum)
 {
     const int     cpr = Kp / 16;
@@ -91,32 +99,48 @@ __global__ __launch_bounds__(256) void pack_bt_kernel(const uint8_t *__restrict_
         v4i     v;
         uint8_t b[16];
     } u;
-    int32_t s = 0;
-#pragma unroll
-    for (int t = 0; t < 16; ++t)
+    int32_t        s   = 0;
+    const uint8_t *row = Bt + (int64_t)n * ldk + kc;
+    if (n < N && kc + 16 <= K && (((uintptr_t)row) & 15) == 0 && kf <= 1)
     {
-        uint8_t x = 0;
-        if (n < N && kc + t < K)
-            x = Bt[(int64_t)n * ldk + kc + t] ^ flip;
-        u.b[t] = x;
-        s += (int8_t)x;
+        // whole aligned 16-byte piece of a row
+        u.v = *(const v4i *)row;
+        const int f4 = (int)(flip * 0x01010101u);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            u.v[t] ^= f4;
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            s += (int8_t)u.b[t];
+    }
+    else
+    {
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+        {
+            uint8_t x = 0;
+            if (n < N && kc + t < K)
+                x = Bt[(int64_t)n * ldk + k_source(kc + t, K, kf)] ^ flip;
+            u.b[t] = x;
+            s += (int8_t)x;
+        }
     }
     *(v4i *)(Bp + (int64_t)n * Kp + kc) = u.v;
     if (s != 0)
         atomicAdd(colsum + n, s);
 }
 
-int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int8_t *Bp, int32_t *colsum,
-                   hipStream_t s)
+int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bool flip, int kf, int8_t *Bp,
+                   int32_t *colsum, hipStream_t s)
 {
-    if (Kp % 16 || Np < N || Kp < K)
+    if (Kp % 16 || Np < N || Kp < K || (kf > 1 && K % kf != 0))
         return (int)hipErrorInvalidValue;
     int e = fill_i32_launch(colsum, 0, Np, s);
     if (e)
         return e;
     const int64_t total = (int64_t)Np * (Kp / 16);
     pack_bt_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)Bt, ldk, K, N, Kp, Np,
-                                                                               flip ? 0x80 : 0, Bp, colsum);
+                                                                               flip ? 0x80 : 0, kf, Bp, colsum);
     return launch_status();
 }
 

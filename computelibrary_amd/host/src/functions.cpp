@@ -1,4 +1,5 @@
-// NEGEMMLowpMatrixMultiplyCore, NEGEMMLowpOutputStage and NEGEMMConvolutionLayer on top of the MI355X C ABI
+// NEGEMMLowpMatrixMultiplyCore, NEGEMMLowpOutputStage, NEGEMMConvolutionLayer and NEFullyConnectedLayer on top of the
+// MI355X C ABI
 // (include/mi355_gemmlowp.h). The classes keep the reference's calling conventions: non-owning tensor pointers captured
 // at configure() and dereferenced at run(), buffers that may be allocated after configure(), validate() that returns a
 // Status and never throws, configure() that throws std::runtime_error on invalid input, synchronous run().
@@ -721,5 +722,255 @@ void NEGEMMConvolutionLayer::run()
 const char *NEGEMMConvolutionLayer::kernel_name() const
 {
     return _impl->handle ? mi355_conv_kernel_name(_impl->handle) : "";
+}
+// =====================================================================================================================
+// NEFullyConnectedLayer
+// =====================================================================================================================
+struct NEFullyConnectedLayer::Impl
+{
+    const ITensor     *src{nullptr}, *weights{nullptr}, *biases{nullptr};
+    ITensor           *dst{nullptr};
+    mi355_gemm_desc    desc{};
+    mi355_gemm_handle *handle{nullptr};
+    bool               is_prepared{false};
+    bool               dynamic_weights{false};
+
+    ~Impl()
+    {
+        if (handle)
+            mi355_gemmlowp_destroy(handle);
+    }
+};
+
+NEFullyConnectedLayer::NEFullyConnectedLayer(std::shared_ptr<IMemoryManager> memory_manager, IWeightsManager *weights_manager)
+    : _impl(std::make_unique<Impl>())
+{
+    ARM_COMPUTE_UNUSED(memory_manager, weights_manager);
+}
+NEFullyConnectedLayer::~NEFullyConnectedLayer() = default;
+
+namespace
+{
+// what CpuFullyConnected::validate / configure derive from the tensor infos
+// (src/cpu/operators/CpuFullyConnected.cpp:232-262, 420-489 of the reference)
+struct FcGeometry
+{
+    bool   weights_reshaped{true}; // the weights tensor is already [num_inputs rows][num_outputs], i.e. B itself
+    bool   is_fc_after_conv{true};
+    bool   convert_weights{false}; // trained in the other data layout
+    size_t K{0}, N{0}, M{0};
+    size_t k_interleave{0};        // _factor2 of CpuConvertFullyConnectedWeightsKernel
+};
+
+Status fc_geometry(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *dst,
+                   const FullyConnectedLayerInfo &fc_info, FcGeometry &g)
+{
+    g.weights_reshaped             = fc_info.transpose_weights ? fc_info.are_weights_reshaped : true;
+    const bool is_batched_fc_layer = dst->dimension(1) > 1;
+    if (is_batched_fc_layer)
+    {
+        g.is_fc_after_conv = true;
+        for (size_t i = 3; i < Dimensions<size_t>::num_max_dimensions; ++i)
+            if (src->tensor_shape()[i] != dst->tensor_shape()[i - 2])
+                g.is_fc_after_conv = false;
+    }
+    else
+        g.is_fc_after_conv = src->num_dimensions() > 1;
+    // after the (possibly implicit) transpose the weights are [K rows][N]
+    g.K = g.weights_reshaped ? weights->dimension(1) : weights->dimension(0);
+    g.N = g.weights_reshaped ? weights->dimension(0) : weights->dimension(1);
+    if (g.is_fc_after_conv)
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(g.K != src->dimension(0) * src->dimension(1) * src->dimension(2),
+                                        "weights do not match the flattened input");
+    else
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(src->dimension(0) != g.K, "weights do not match the input");
+    g.M = src->tensor_shape().total_size() / g.K;
+    g.convert_weights = g.is_fc_after_conv && src->data_layout() != fc_info.weights_trained_layout;
+    if (g.convert_weights)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(fc_info.weights_trained_layout == DataLayout::UNKNOWN);
+        // the tensor's own layout is the one the weights were NOT trained with
+        const DataLayout in_layout = fc_info.weights_trained_layout == DataLayout::NCHW ? DataLayout::NHWC : DataLayout::NCHW;
+        const size_t plane = src->dimension(get_data_layout_dimension_index(in_layout, DataLayoutDimension::WIDTH)) *
+                             src->dimension(get_data_layout_dimension_index(in_layout, DataLayoutDimension::HEIGHT));
+        const size_t chans = src->dimension(get_data_layout_dimension_index(in_layout, DataLayoutDimension::CHANNEL));
+        g.k_interleave     = fc_info.weights_trained_layout == DataLayout::NCHW ? chans : plane;
+    }
+    return Status{};
+}
+
+Status fc_output_stage(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *dst,
+                       const ActivationLayerInfo &act, GEMMLowpOutputStageInfo &out)
+{
+    const UniformQuantizationInfo iq = src->quantization_info().uniform();
+    const UniformQuantizationInfo wq = weights->quantization_info().uniform();
+    const UniformQuantizationInfo oq = dst->quantization_info().uniform();
+    const float                   multiplier = (iq.scale * wq.scale) / oq.scale;
+    int32_t                       m = 0, sft = 0;
+    ARM_COMPUTE_RETURN_ON_ERROR(quantization::calculate_quantized_multiplier(multiplier, &m, &sft));
+    int32_t lo = get_min_max(src->data_type()).first, hi = get_min_max(src->data_type()).second;
+    if (act.enabled())
+    {
+        // quantization::get_quantized_asymmetric_output_min_max (src/core/utils/quantization/AsymmHelpers.cpp:183-221)
+        const bool is_signed = src->data_type() == DataType::QASYMM8_SIGNED;
+        auto       q = [&](float v) -> int32_t { return is_signed ? quantize_qasymm8_signed(v, oq) : quantize_qasymm8(v, oq); };
+        switch (act.activation())
+        {
+            case ActivationLayerInfo::ActivationFunction::RELU:
+                lo = oq.offset;
+                break;
+            case ActivationLayerInfo::ActivationFunction::BOUNDED_RELU:
+                lo = oq.offset;
+                hi = q(act.a());
+                break;
+            case ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU:
+                lo = q(act.b());
+                hi = q(act.a());
+                break;
+            default:
+                ARM_COMPUTE_RETURN_ERROR_MSG("Activation function not supported.");
+        }
+    }
+    out.type                = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    out.gemmlowp_multiplier = m;
+    out.gemmlowp_shift      = sft;
+    out.gemmlowp_offset     = oq.offset;
+    out.gemmlowp_min_bound  = lo;
+    out.gemmlowp_max_bound  = hi;
+    return Status{};
+}
+} // namespace
+
+// src/cpu/operators/CpuFullyConnected.cpp:384-489 of the reference, restricted to what this library builds
+Status NEFullyConnectedLayer::validate(const ITensorInfo *input, const ITensorInfo *weights, const ITensorInfo *biases,
+                                       const ITensorInfo *output, FullyConnectedLayerInfo fc_info,
+                                       const WeightsInfo &weights_info)
+{
+    ARM_COMPUTE_RETURN_ERROR_ON_NULLPTR(input, weights, output);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights_info.weight_format() != WeightFormat::UNSPECIFIED,
+                                    "Fixed-format weights are not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(is_one_of(input->data_type(), {DataType::F16, DataType::F32, DataType::BFLOAT16}),
+                                    "Floating-point fully connected layers are not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(input->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}),
+                                    "Input must be QASYMM8 or QASYMM8_SIGNED");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights->data_type() != input->data_type() || output->data_type() != input->data_type(),
+                                    "Mismatching data types");
+    ARM_COMPUTE_RETURN_ERROR_ON(weights->num_dimensions() > 2);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(fc_info.activation_info.enabled() &&
+                                        fusable_acts.count(fc_info.activation_info.activation()) == 0,
+                                    "Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
+    if (biases != nullptr)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->num_dimensions() > 1);
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(biases->data_type() != DataType::S32, "Biases must be S32");
+    }
+    FcGeometry g;
+    ARM_COMPUTE_RETURN_ON_ERROR(fc_geometry(input, weights, output, fc_info, g));
+    if (biases != nullptr)
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->dimension(0) != g.N);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->dimension(0) != g.N, "The output's first dimension must be the number of outputs");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->tensor_shape().total_size() != g.M * g.N, "Mismatching number of batches");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->has_padding(), "A padded input cannot be flattened in place");
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(weights, "weights"));
+    ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(output, "output"));
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(g.M > 1 && output->num_dimensions() > 2 && output->has_padding(),
+                                    "A padded output with more than two dimensions is not supported");
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_RETURN_ON_ERROR(fc_output_stage(input, weights, output, fc_info.activation_info, stage));
+    return Status{};
+}
+
+Status NEFullyConnectedLayer::has_opt_impl(WeightFormat &expected_weight_format, const ITensorInfo *input,
+                                           const ITensorInfo *weights, const ITensorInfo *biases, const ITensorInfo *output,
+                                           const FullyConnectedLayerInfo &fc_info, const WeightsInfo &weights_info)
+{
+    // no fixed-format weights in this library: the packed layout is private to the device workspace
+    expected_weight_format = WeightFormat::UNSPECIFIED;
+    ARM_COMPUTE_RETURN_ON_ERROR(validate(input, weights, biases, output, fc_info, weights_info));
+    ARM_COMPUTE_RETURN_ERROR_MSG("No fixed-format kernel available");
+}
+
+void NEFullyConnectedLayer::configure(const ITensor *input, const ITensor *weights, const ITensor *biases, ITensor *output,
+                                      FullyConnectedLayerInfo fc_info, const WeightsInfo &weights_info)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(input, weights, output);
+    const ITensorInfo *ii = input->info(), *wi = weights->info(), *oi = output->info();
+    ARM_COMPUTE_ERROR_THROW_ON(validate(ii, wi, biases != nullptr ? biases->info() : nullptr, oi, fc_info, weights_info));
+    FcGeometry g;
+    ARM_COMPUTE_ERROR_THROW_ON(fc_geometry(ii, wi, oi, fc_info, g));
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_ERROR_THROW_ON(fc_output_stage(ii, wi, oi, fc_info.activation_info, stage));
+
+    mi355_gemm_desc d{};
+    d.M = static_cast<int32_t>(g.M), d.N = static_cast<int32_t>(g.N), d.K = static_cast<int32_t>(g.K), d.batch = 1;
+    d.a_dtype = to_mi355(ii->data_type()), d.b_dtype = to_mi355(wi->data_type()), d.dst_dtype = to_mi355(oi->data_type());
+    d.epilogue = MI355_EPI_FIXEDPOINT;
+    d.lda      = static_cast<int64_t>(g.K); // flattening an unpadded tensor is the identity on its bytes
+    d.ldb      = static_cast<int64_t>(wi->strides_in_bytes()[1] / wi->element_size());
+    d.ldd      = static_cast<int64_t>(g.M > 1 ? oi->strides_in_bytes()[1] / oi->element_size() : g.N);
+    d.a_batch_stride = d.b_batch_stride = d.d_batch_stride = 0;
+    // the GEMM adds its offsets: negated zero points (CpuFullyConnected.cpp:98-103,166-171 of the reference)
+    d.a_offset       = -ii->quantization_info().uniform().offset;
+    d.b_offset       = -wi->quantization_info().uniform().offset;
+    d.requant        = make_requant(stage);
+    d.scale          = 1.f;
+    d.act_min        = -std::numeric_limits<float>::infinity();
+    d.act_max        = std::numeric_limits<float>::infinity();
+    d.path           = MI355_PATH_AUTO;
+    d.b_transposed   = g.weights_reshaped ? 0 : 1; // [num_outputs rows][num_inputs]: the transpose happens while packing
+    d.b_k_interleave = g.convert_weights ? static_cast<int32_t>(g.k_interleave) : 0;
+
+    Impl      &s    = *_impl;
+    const bool keep = fc_info.retain_internal_weights && s.handle != nullptr && s.is_prepared && s.desc.M == d.M &&
+                      s.desc.N == d.N && s.desc.K == d.K && s.desc.b_dtype == d.b_dtype;
+    s.src = input, s.weights = weights, s.biases = biases, s.dst = output;
+    s.dynamic_weights = !wi->are_values_constant() && !g.weights_reshaped;
+    if (keep)
+    {
+        // packed weights of the previous configuration stay; offsets and requantisation may have changed
+        s.desc.a_offset = d.a_offset, s.desc.b_offset = d.b_offset, s.desc.requant = d.requant;
+        check_abi(mi355_gemmlowp_update_quant(s.handle, d.a_offset, d.b_offset, &d.requant, 1.f, nullptr),
+                  "NEFullyConnectedLayer::configure");
+        return;
+    }
+    if (s.handle)
+    {
+        mi355_gemmlowp_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.desc        = d;
+    s.is_prepared = false;
+    check_abi(mi355_gemmlowp_create(&d, &s.handle), "NEFullyConnectedLayer::configure");
+}
+
+void NEFullyConnectedLayer::prepare()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEFullyConnectedLayer::prepare() before configure()");
+    if (s.is_prepared && !s.dynamic_weights)
+        return;
+    ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");
+    check_abi(mi355_gemmlowp_prepare(s.handle, first_element(s.weights),
+                                     s.biases ? reinterpret_cast<const int32_t *>(first_element(s.biases)) : nullptr,
+                                     nullptr, nullptr, nullptr),
+              "NEFullyConnectedLayer::prepare");
+    if (!s.dynamic_weights)
+        s.weights->mark_as_unused();
+    s.is_prepared = true;
+}
+
+void NEFullyConnectedLayer::run()
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEFullyConnectedLayer::run() before configure()");
+    ARM_COMPUTE_ERROR_ON_MSG(s.src->buffer() == nullptr || s.dst->buffer() == nullptr, "tensor without memory");
+    prepare();
+    check_abi(mi355_gemmlowp_run(s.handle, first_element(s.src), nullptr, first_element(s.dst), nullptr),
+              "NEFullyConnectedLayer::run");
+}
+
+const char *NEFullyConnectedLayer::kernel_name() const
+{
+    return _impl->handle ? mi355_gemmlowp_kernel_name(_impl->handle) : "";
 }
 } // namespace arm_compute

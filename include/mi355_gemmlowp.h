@@ -12,7 +12,7 @@
  *   mi355_gemmlowp_create -> mi355_gemmlowp_prepare -> mi355_gemmlowp_run.
  *
  * Conventions
- *  - Matrices are row-major. A is M x K, B is K x N, D is M x N ("ld*" = row stride in elements,
+ *  - Matrices are row-major. A is M x K, B is K x N (or N x K with b_transposed), D is M x N ("ld*" = row stride in elements,
  *    "*_batch_stride" = distance between consecutive matrices in elements; b_batch_stride 0
  *    shares one B between all batches).
  *  - a_offset / b_offset are ADDED to every element before the product, exactly as
@@ -89,6 +89,14 @@ typedef struct mi355_gemm_desc
     float         scale;            /* MI355_EPI_F32 only: a.scale * b.scale */
     float         act_min, act_max; /* MI355_EPI_F32 only: activation clamp, +-INFINITY for none */
     int32_t       path;             /* mi355_path */
+    int32_t       b_transposed;     /* != 0: B is handed over as its transpose, N rows of K elements (ldb = row stride
+                                       >= K, b_batch_stride between such matrices) - how fully connected weights arrive
+                                       before CpuTransposeKernel (src/cpu/operators/CpuFullyConnected.cpp:283-292) */
+    int32_t       b_k_interleave;   /* f > 1: the rows of B (its K index) are re-ordered while packing: row a*f + b
+                                       (b < f) of the matrix that is multiplied is row b*(K/f) + a of the matrix handed
+                                       over. Replaces CpuConvertFullyConnectedWeights
+                                       (src/cpu/kernels/CpuConvertFullyConnectedWeightsKernel.cpp:60-66,118-121; f is its
+                                       _factor2). 0 or 1: none. Must divide K. */
     int32_t       reserved;
 } mi355_gemm_desc;
 

@@ -206,6 +206,47 @@ static void test_validate_tables()
     EXPECT(!bool(NEGEMMConvolutionLayer::validate(&src, &w, &cb, &dst_bad, ps)));
 }
 
+// accept / reject rules of CpuFullyConnected::validate (src/cpu/operators/CpuFullyConnected.cpp:384-489 of the reference)
+static void test_fully_connected_validate()
+{
+    SECTION("NEFullyConnectedLayer::validate accept / reject");
+    const QuantizationInfo q(0.1f, 3);
+    TensorInfo src(TensorShape(200U, 4U), 1, DataType::QASYMM8, q), w(TensorShape(200U, 30U), 1, DataType::QASYMM8, q);
+    TensorInfo b(TensorShape(30U), 1, DataType::S32), dst(TensorShape(30U, 4U), 1, DataType::QASYMM8, q);
+    EXPECT(bool(NEFullyConnectedLayer::validate(&src, &w, &b, &dst)));
+    EXPECT(bool(NEFullyConnectedLayer::validate(&src, &w, nullptr, &dst)));
+    TensorInfo w_bad_k(TensorShape(201U, 30U), 1, DataType::QASYMM8, q);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w_bad_k, &b, &dst)));          // num_inputs mismatch
+    TensorInfo w3(TensorShape(200U, 30U, 2U), 1, DataType::QASYMM8, q);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w3, &b, &dst)));               // weights with more than 2 dimensions
+    TensorInfo w_s8(TensorShape(200U, 30U), 1, DataType::QASYMM8_SIGNED, q);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w_s8, &b, &dst)));             // mismatching data types
+    TensorInfo b_f32(TensorShape(30U), 1, DataType::F32);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w, &b_f32, &dst)));            // quantized needs S32 biases
+    TensorInfo b2(TensorShape(30U, 2U), 1, DataType::S32);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w, &b2, &dst)));               // biases with more than 1 dimension
+    TensorInfo dst_bad(TensorShape(31U, 4U), 1, DataType::QASYMM8, q);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w, &b, &dst_bad)));
+    FullyConnectedLayerInfo tanh_info;
+    tanh_info.activation_info = ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::TANH);
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&src, &w, &b, &dst, tanh_info)));     // only the RELU family fuses
+    FullyConnectedLayerInfo relu_info;
+    relu_info.activation_info = ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU, 6.f, -1.f);
+    EXPECT(bool(NEFullyConnectedLayer::validate(&src, &w, &b, &dst, relu_info)));
+    TensorInfo f_src(TensorShape(200U, 4U), 1, DataType::F32), f_w(TensorShape(200U, 30U), 1, DataType::F32);
+    TensorInfo f_dst(TensorShape(30U, 4U), 1, DataType::F32);
+    const Status st = NEFullyConnectedLayer::validate(&f_src, &f_w, nullptr, &f_dst);
+    EXPECT(!bool(st) && st.error_description().find("not built") != std::string::npos); // out of scope, and says so
+    // after a convolution: the flattened input must match the weights
+    TensorInfo conv_src(TensorShape(16U, 3U, 5U, 4U), 1, DataType::QASYMM8, q), conv_w(TensorShape(240U, 30U), 1, DataType::QASYMM8, q);
+    conv_src.set_data_layout(DataLayout::NHWC);
+    EXPECT(bool(NEFullyConnectedLayer::validate(&conv_src, &conv_w, &b, &dst)));
+    EXPECT(!bool(NEFullyConnectedLayer::validate(&conv_src, &w, &b, &dst)));
+    WeightFormat wf = WeightFormat::ANY;
+    EXPECT(!bool(NEFullyConnectedLayer::has_opt_impl(wf, &src, &w, &b, &dst, FullyConnectedLayerInfo(), WeightsInfo())));
+    EXPECT(wf == WeightFormat::UNSPECIFIED);
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 // GPU tests
 // ---------------------------------------------------------------------------------------------------------------------
@@ -506,6 +547,112 @@ static void test_convolution(DataType dt, bool per_channel, int C, const Activat
     EXPECT(dense_copy<uint8_t>(dst) == want);
 }
 
+// NEFullyConnectedLayer against the oracle GEMM on explicitly transposed / re-ordered weights
+// (the reference's own FullyConnectedLayer fixture compares against a reference built the same way:
+//  tests/validation/fixtures/FullyConnectedLayerFixture.h of the reference)
+enum class FcCase
+{
+    AfterFc,          // src [K, batch], weights [K, N] (one row of num_inputs per output), RELU
+    AfterConvNhwc,    // src NHWC [C, W, H, batch], weights trained NCHW (the default): K re-ordered while packing
+    AfterConvNchw,    // src NCHW [W, H, C, batch], weights trained NHWC
+    WeightsReshaped   // transpose_weights = false: weights [N, K]
+};
+
+static void test_fully_connected(DataType dt, FcCase which)
+{
+    SECTION(which == FcCase::AfterFc         ? "NEFullyConnectedLayer after FC, RELU"
+            : which == FcCase::AfterConvNhwc ? "NEFullyConnectedLayer after conv, NHWC input, NCHW-trained weights"
+            : which == FcCase::AfterConvNchw ? "NEFullyConnectedLayer after conv, NCHW input, NHWC-trained weights, BOUNDED_RELU"
+                                             : "NEFullyConnectedLayer with weights already transposed");
+    const bool is_signed = dt == DataType::QASYMM8_SIGNED;
+    const int  C = 16, W = 3, H = 5, batch = 7, N = 45;
+    const int  K = (which == FcCase::AfterConvNhwc || which == FcCase::AfterConvNchw) ? C * W * H : 200;
+    const int  in_zp = is_signed ? -7 : 120, w_zp = is_signed ? 3 : 131, out_zp = is_signed ? -2 : 9;
+    const QuantizationInfo iq(0.02f, in_zp), wq(0.011f, w_zp), oq(0.31f, out_zp);
+    Tensor src, weights, bias, dst;
+    FullyConnectedLayerInfo fc;
+    if (which == FcCase::AfterConvNhwc)
+    {
+        init_tensor(src, TensorShape(C, W, H, batch), dt, iq);
+        src.info()->set_data_layout(DataLayout::NHWC);
+    }
+    else if (which == FcCase::AfterConvNchw)
+    {
+        init_tensor(src, TensorShape(W, H, C, batch), dt, iq);
+        src.info()->set_data_layout(DataLayout::NCHW);
+        fc.weights_trained_layout = DataLayout::NHWC;
+        fc.activation_info        = ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 60.f);
+    }
+    else
+        init_tensor(src, TensorShape(K, batch), dt, iq);
+    if (which == FcCase::WeightsReshaped)
+    {
+        init_tensor(weights, TensorShape(N, K), dt, wq);
+        fc.transpose_weights = false;
+    }
+    else
+        init_tensor(weights, TensorShape(K, N), dt, wq);
+    if (which == FcCase::AfterFc)
+        fc.activation_info = ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU);
+    init_tensor(bias, TensorShape(N), DataType::S32);
+    init_tensor(dst, TensorShape(N, batch), dt, oq);
+    EXPECT(bool(NEFullyConnectedLayer::validate(src.info(), weights.info(), bias.info(), dst.info(), fc)));
+    NEFullyConnectedLayer fcl;
+    fcl.configure(&src, &weights, &bias, &dst, fc);
+    src.allocator()->allocate(), weights.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    if (is_signed)
+        fill_uniform<int8_t>(src, -128, 127, 21), fill_uniform<int8_t>(weights, -128, 127, 22);
+    else
+        fill_uniform<uint8_t>(src, 0, 255, 21), fill_uniform<uint8_t>(weights, 0, 255, 22);
+    fill_uniform<int32_t>(bias, -3000, 3000, 23);
+    const auto A = dense_copy<uint8_t>(src), Wt = dense_copy<uint8_t>(weights);
+    const auto Cb = dense_copy<int32_t>(bias);
+    // B[k][n] as the GEMM of the reference sees it after transpose + layout conversion
+    std::vector<uint8_t> B(static_cast<size_t>(K) * N);
+    for (int k = 0; k < K; ++k)
+        for (int n = 0; n < N; ++n)
+        {
+            int ks = k;
+            if (which == FcCase::AfterConvNhwc) // flattened NHWC index k = (h*W + w)*C + c takes the NCHW-trained row
+                ks = (k % C) * (W * H) + k / C;
+            else if (which == FcCase::AfterConvNchw) // flattened NCHW index k = c*H*W + p takes the NHWC-trained row
+                ks = (k % (W * H)) * C + k / (W * H);
+            B[static_cast<size_t>(k) * N + n] =
+                which == FcCase::WeightsReshaped ? Wt[static_cast<size_t>(ks) * N + n] : Wt[static_cast<size_t>(n) * K + ks];
+        }
+    int32_t mult = 0, shift = 0;
+    EXPECT(bool(quantization::calculate_quantized_multiplier(0.02f * 0.011f / 0.31f, &mult, &shift)));
+    int32_t lo = is_signed ? -128 : 0, hi = is_signed ? 127 : 255;
+    if (which == FcCase::AfterFc)
+        lo = out_zp;
+    if (which == FcCase::AfterConvNchw)
+    {
+        lo = out_zp;
+        hi = is_signed ? quantize_qasymm8_signed(60.f, oq.uniform()) : quantize_qasymm8(60.f, oq.uniform());
+    }
+    std::vector<uint8_t> want(static_cast<size_t>(batch) * N);
+    orc_gemmlowp_fixedpoint(A.data(), is_signed, K, B.data(), is_signed, N, Cb.data(), want.data(), N, is_signed, batch, N, K,
+                            -in_zp, -w_zp, &mult, &shift, 1, out_zp, lo, hi);
+    fcl.run();
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    EXPECT(!weights.is_used());
+    // second run with new input, same packed weights
+    if (is_signed)
+        fill_uniform<int8_t>(src, -128, 127, 31);
+    else
+        fill_uniform<uint8_t>(src, 0, 255, 31);
+    const auto A2 = dense_copy<uint8_t>(src);
+    orc_gemmlowp_fixedpoint(A2.data(), is_signed, K, B.data(), is_signed, N, Cb.data(), want.data(), N, is_signed, batch, N, K,
+                            -in_zp, -w_zp, &mult, &shift, 1, out_zp, lo, hi);
+    fcl.run();
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    size_t inside = 0;
+    for (uint8_t v : want)
+        inside += (is_signed ? (static_cast<int8_t>(v) > lo && static_cast<int8_t>(v) < hi) : (v > lo && v < hi)) ? 1 : 0;
+    EXPECT(inside * 5 > want.size()); // a fair share of the outputs is not clamped: the comparison means something
+    std::printf("       kernel: %s\n", fcl.kernel_name());
+}
+
 static void test_error_paths()
 {
     SECTION("configure() throws on invalid input; run() before configure() throws");
@@ -546,6 +693,7 @@ int main(int argc, char **argv)
             test_tensor_info();
             test_quant_helpers();
             test_validate_tables();
+            test_fully_connected_validate();
             test_error_paths();
         }
         else
@@ -561,6 +709,11 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
             test_convolution(DataType::QASYMM8, true, 32,
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
+            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
+            test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
+            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);
+            test_fully_connected(DataType::QASYMM8, FcCase::AfterConvNchw);
+            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::WeightsReshaped);
         }
     }
     catch (const std::exception &e)

@@ -201,6 +201,41 @@ def test_run_can_be_captured_in_a_hip_graph():
         np.testing.assert_array_equal(Dd.cpu().numpy(), np.roll(want, sum(range(rep + 1)), 0))
     g.close()
 
+@pytest.mark.parametrize("M", [9, 70])
+@pytest.mark.parametrize("k_interleave", [0, 16])
+def test_b_handed_over_transposed_and_with_reordered_k(M, k_interleave):
+    """Fully connected weights arrive as [num_outputs][num_inputs] and, after a convolution in the other data layout,
+    with their K index permuted (CpuTransposeKernel + CpuConvertFullyConnectedWeightsKernel in the reference): both are
+    folded into the packing of B."""
+    import torch
+    rng = np.random.default_rng(48 + M + k_interleave)
+    N, K = 150, 240
+    A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+    Wt = rng.integers(0, 256, size=(N, K), dtype=np.uint8)       # as handed over
+    ldb = K + 8                                                  # with a row stride
+    Wt_padded = np.zeros((N, ldb), dtype=np.uint8)
+    Wt_padded[:, :K] = Wt
+    if k_interleave:
+        k = np.arange(K)
+        src_k = (k % k_interleave) * (K // k_interleave) + k // k_interleave
+        B = Wt[:, src_k].T
+    else:
+        B = Wt.T
+    bias = rng.integers(-4000, 4000, size=N).astype(np.int32)
+    mult, shift = oracle.calculate_quantized_multiplier(0.0009)
+    want = oracle.gemmlowp_fixedpoint(A, np.ascontiguousarray(B), bias, -120, -131, [mult], [shift], 9, 0, 255, np.uint8)
+    for path in paths_for(M):
+        announce("transposed B", M, k_interleave, "path", path)
+        g = capi.Gemm(M, N, K, capi.U8, capi.U8, capi.U8, capi.EPI_FIXEDPOINT, -120, -131,
+                      capi.requant(mult, shift, 9, 0, 255), path=path, ldb=ldb, b_transposed=True,
+                      b_k_interleave=k_interleave)
+        Ad, Bd, Dd = torch.from_numpy(A).cuda(), torch.from_numpy(Wt_padded).cuda(), torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+        g.prepare(Bd, torch.from_numpy(bias).cuda())
+        g.run(Ad, Dd)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(Dd.cpu().numpy(), want)
+        g.close()
+
 def test_requant_extremes_on_device():
     """Accumulators and multipliers at the edges of int32 (saturating SQDMULH, shift 0 / 31, wrap-around adds)
     through the stand-alone output stage."""

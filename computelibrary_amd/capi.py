@@ -22,7 +22,8 @@ EXPORTS = [
 
 class Requant(C.Structure):
     _fields_ = [("per_channel", C.c_int32), ("multiplier", C.c_int32), ("shift", C.c_int32),
-                ("result_offset", C.c_int32), ("min_bound", C.c_int32), ("max_bound", C.c_int32)]
+                ("result_offset", C.c_int32), ("min_bound", C.c_int32), ("max_bound", C.c_int32),
+                ("stage", C.c_int32)]
 
 
 class GemmDesc(C.Structure):
@@ -115,8 +116,11 @@ def dtype_code(x):
     return {"uint8": U8, "int8": S8, "int32": S32, "float32": F32}[name]
 
 
-def requant(mult=0, shift=0, offset=0, lo=-(1 << 31), hi=(1 << 31) - 1, per_channel=False):
-    return Requant(1 if per_channel else 0, int(mult), int(shift), int(offset), int(lo), int(hi))
+STAGE_FIXEDPOINT, STAGE_SCALE = 0, 1
+
+
+def requant(mult=0, shift=0, offset=0, lo=-(1 << 31), hi=(1 << 31) - 1, per_channel=False, stage=STAGE_FIXEDPOINT):
+    return Requant(1 if per_channel else 0, int(mult), int(shift), int(offset), int(lo), int(hi), int(stage))
 
 
 def device_info():

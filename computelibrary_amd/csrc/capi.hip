@@ -257,7 +257,7 @@ struct GemmCore
     int refresh_qparams(hipStream_t s)
     {
         qp_ok = qp_std = false;
-        if (epi != EPI_FIXEDPOINT)
+        if (epi != EPI_FIXEDPOINT || rq.stage != MI355_STAGE_FIXEDPOINT)
             return 0;
         TRY(qp.ensure(sizeof(int32_t) * ((size_t)QP_COUNT * Np + 4)));
         int32_t *flag = qp.as<int32_t>() + (size_t)QP_COUNT * Np;
@@ -286,6 +286,7 @@ struct GemmCore
         p.mult_s              = rq.multiplier;
         p.shift_s             = rq.shift;
         p.result_offset       = rq.result_offset;
+        p.stage               = rq.stage;
         const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
         p.lo                  = rq.min_bound > tlo ? rq.min_bound : tlo;
         p.hi                  = rq.max_bound < thi ? rq.max_bound : thi;
@@ -393,6 +394,10 @@ int check_requant(const mi355_requant &rq, int dst_dtype)
 {
     if (rq.min_bound > rq.max_bound)
         return fail("min_bound > max_bound");
+    if (rq.stage != MI355_STAGE_FIXEDPOINT && rq.stage != MI355_STAGE_SCALE)
+        return fail("unknown output stage %d", rq.stage);
+    if (rq.stage == MI355_STAGE_SCALE && !rq.per_channel && (rq.shift < 0 || rq.shift > 31))
+        return fail("QUANTIZE_DOWN needs a shift in [0, 31] (got %d)", rq.shift);
     const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
     if (rq.max_bound < tlo || rq.min_bound > thi)
         return fail("clamp bounds [%d,%d] do not intersect the destination type's range", rq.min_bound, rq.max_bound);
@@ -637,6 +642,7 @@ int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *s
     const bool   d_host  = !is_device_ptr(dst);
     EpiParams    p{};
     p.mult_s = d.requant.multiplier, p.shift_s = d.requant.shift, p.result_offset = d.requant.result_offset;
+    p.stage  = d.requant.stage;
     const int32_t tlo = d.dst_dtype == MI355_S8 ? -128 : 0, thi = d.dst_dtype == MI355_S8 ? 127 : 255;
     p.lo = d.requant.min_bound > tlo ? d.requant.min_bound : tlo;
     p.hi = d.requant.max_bound < thi ? d.requant.max_bound : thi;

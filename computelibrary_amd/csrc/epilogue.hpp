@@ -28,6 +28,7 @@ struct EpiParams
     int64_t        rowvec_batch_stride;
     int32_t        mult_s, shift_s;
     int32_t        result_offset;
+    int32_t        stage; // 0: QUANTIZE_DOWN_FIXEDPOINT, 1: QUANTIZE_DOWN (integer multiplier, truncating shift)
     int32_t        lo, hi; // clamp range, already intersected with the destination type's range
     float          scale;
     float          act_min, act_max;
@@ -120,6 +121,12 @@ __device__ __forceinline__ int32_t epi_fixedpoint(int32_t acc, int32_t colv, int
                                                   const EpiParams &p)
 {
     const int32_t v = (int32_t)((uint32_t)acc + (uint32_t)colv + (uint32_t)rowv);
+    if (p.stage == 1)
+    {
+        // QUANTIZE_DOWN: offset first, wrap-around multiply, truncating arithmetic shift
+        const int32_t r = (int32_t)(((uint32_t)v + (uint32_t)p.result_offset) * (uint32_t)mult) >> (shift & 31);
+        return clamp_i32(r, p.lo, p.hi);
+    }
     return clamp_i32(requant_fixedpoint(v, mult, shift, p.result_offset), p.lo, p.hi);
 }
 

@@ -66,6 +66,14 @@ mi355_requant make_requant(const GEMMLowpOutputStageInfo &s)
     rq.result_offset = s.gemmlowp_offset;
     rq.min_bound     = s.gemmlowp_min_bound;
     rq.max_bound     = s.gemmlowp_max_bound;
+    rq.stage         = s.type == GEMMLowpOutputStageType::QUANTIZE_DOWN ? MI355_STAGE_SCALE : MI355_STAGE_FIXEDPOINT;
+    if (s.type == GEMMLowpOutputStageType::QUANTIZE_DOWN && s.gemmlowp_min_bound == s.gemmlowp_max_bound)
+    {
+        // equal bounds mean "no bounded activation": only the saturation to the output type remains
+        // (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ScaleKernel.cpp:299-300, tests/validation/reference/GEMMLowp.cpp:95-99)
+        rq.min_bound = std::numeric_limits<int32_t>::lowest();
+        rq.max_bound = std::numeric_limits<int32_t>::max();
+    }
     return rq;
 }
 
@@ -192,9 +200,21 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
                 ARM_COMPUTE_RETURN_ERROR_ON(c->num_dimensions() > 1 || c->dimension(0) != b->dimension(0));
             }
             break;
+        case GEMMLowpOutputStageType::QUANTIZE_DOWN:
+            if (stage.is_quantized_per_channel)
+            {
+                for (size_t j = 0; j < b->dimension(0) && j < stage.gemmlowp_shifts.size(); ++j)
+                    ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.gemmlowp_shifts[j] < 0 || stage.gemmlowp_shifts[j] > 31,
+                                                    "QUANTIZE_DOWN needs shifts in [0, 31]");
+            }
+            else
+                ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.gemmlowp_shift < 0 || stage.gemmlowp_shift > 31,
+                                                "QUANTIZE_DOWN needs a shift in [0, 31]");
+            // the same rules otherwise (CpuGemmLowpOffsetContributionOutputStageKernel.cpp:829-905)
+            [[fallthrough]];
         case GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT:
             ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}),
-                                            "The fixed-point output stage writes QASYMM8 or QASYMM8_SIGNED");
+                                            "The integer output stages write QASYMM8 or QASYMM8_SIGNED");
             ARM_COMPUTE_RETURN_ERROR_ON(stage.gemmlowp_min_bound > stage.gemmlowp_max_bound);
             if (c != nullptr)
             {
@@ -212,8 +232,6 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
                                                 "Per-channel requantization needs a zero rhs offset");
             }
             break;
-        case GEMMLowpOutputStageType::QUANTIZE_DOWN:
-            ARM_COMPUTE_RETURN_ERROR_MSG("QUANTIZE_DOWN (integer multiplier) is not built in this library");
         default:
             ARM_COMPUTE_RETURN_ERROR_MSG("Unsupported output stage");
     }
@@ -262,7 +280,7 @@ void NEGEMMLowpMatrixMultiplyCore::configure(const ITensor *a, const ITensor *b,
     d.act_max  = std::numeric_limits<float>::infinity();
     d.scale    = 1.f;
     d.path     = MI355_PATH_AUTO;
-    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT)
+    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT || stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN)
     {
         d.epilogue = MI355_EPI_FIXEDPOINT;
         d.requant  = make_requant(stage);
@@ -423,8 +441,9 @@ Status NEGEMMLowpOutputStage::validate(const ITensorInfo *input, const ITensorIn
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type != GEMMLowpOutputStageType::QUANTIZE_DOWN &&
                                         info.type != GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT,
                                     "Unsupported output stage type");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type == GEMMLowpOutputStageType::QUANTIZE_DOWN,
-                                    "QUANTIZE_DOWN (integer multiplier) is not built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type == GEMMLowpOutputStageType::QUANTIZE_DOWN &&
+                                        (info.gemmlowp_shift < 0 || info.gemmlowp_shift > 31),
+                                    "QUANTIZE_DOWN needs a shift in [0, 31]");
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::QSYMM16, "QSYMM16 output is not built in this library");
     ARM_COMPUTE_RETURN_ERROR_ON(input->data_type() != DataType::S32 || input->num_channels() != 1);
     ARM_COMPUTE_RETURN_ERROR_ON(info.gemmlowp_min_bound > info.gemmlowp_max_bound);

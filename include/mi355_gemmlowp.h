@@ -64,7 +64,21 @@ typedef enum mi355_path
     MI355_PATH_SKINNY = 3
 } mi355_path;
 
-/* Mirrors the fields of GEMMLowpOutputStageInfo the FIXEDPOINT stage reads
+typedef enum mi355_stage
+{
+    /* QUANTIZE_DOWN_FIXEDPOINT: rounding_shift(sqdmulh(v, multiplier), shift) + result_offset
+     * (src/core/NEON/NEAsymm.h:87-148) */
+    MI355_STAGE_FIXEDPOINT = 0,
+    /* QUANTIZE_DOWN: ((v + result_offset) * multiplier) >> shift, wrap-around multiply, truncating shift, shift in
+     * [0, 31] (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ScaleKernel.cpp:92-180; scalar form in
+     * src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:348-362). The reference's vector lanes for a
+     * signed destination additionally clamp negative results to 0 before narrowing
+     * (CpuGemmLowpOffsetContributionOutputStageKernel.cpp:137-160) while its scalar tail and its test oracle do not:
+     * this library follows the scalar form and the test oracle. */
+    MI355_STAGE_SCALE = 1
+} mi355_stage;
+
+/* Mirrors the fields of GEMMLowpOutputStageInfo the integer output stages read
  * (arm_compute/function_info/GEMMInfo.h:49-82). With per_channel != 0 the per-column
  * multiplier / shift arrays are passed to mi355_gemmlowp_prepare instead. */
 typedef struct mi355_requant
@@ -75,6 +89,7 @@ typedef struct mi355_requant
     int32_t result_offset;
     int32_t min_bound;
     int32_t max_bound;
+    int32_t stage; /* mi355_stage: which of the two integer output stages of GEMMLowpOutputStageType */
 } mi355_requant;
 
 typedef struct mi355_gemm_desc

@@ -33,6 +33,8 @@ def _load():
     lib.orc_rounding_shift_right.argtypes = [C.c_int32, C.c_int32]
     lib.orc_requant_s32.restype = C.c_int32
     lib.orc_requant_s32.argtypes = [C.c_int32] * 4
+    lib.orc_requant_scale_s32.restype = C.c_int32
+    lib.orc_requant_scale_s32.argtypes = [C.c_int32] * 4
     lib.orc_narrow_clamp.restype = C.c_int32
     lib.orc_narrow_clamp.argtypes = [C.c_int32, C.c_int, C.c_int32, C.c_int32]
     lib.orc_calculate_quantized_multiplier.restype = C.c_int
@@ -127,6 +129,32 @@ def gemmlowp_fixedpoint(A, B, bias, a_offset, b_offset, mult, shift, result_offs
                                 C.c_int64(N), _signed(out), M, N, K, C.c_int32(a_offset), C.c_int32(b_offset),
                                 _p(m), _p(s), n, C.c_int32(result_offset), C.c_int32(min_bound),
                                 C.c_int32(max_bound))
+    return out
+
+
+def output_stage_scale(src, bias, mult, shift, result_offset, min_bound, max_bound, dst_dtype):
+    """QUANTIZE_DOWN with an integer multiplier: ((v + bias + result_offset) * mult) >> shift"""
+    src = np.ascontiguousarray(src, dtype=np.int32)
+    M, N = src.shape
+    m, s, n = _qparams(mult, shift)
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.empty((M, N), dtype=dst_dtype)
+    lib.orc_output_stage_scale(_p(src), C.c_int64(N), _p(bias), _p(out), C.c_int64(N), _signed(out), M, N, _p(m), _p(s), n,
+                               C.c_int32(result_offset), C.c_int32(min_bound), C.c_int32(max_bound))
+    return out
+
+
+def gemmlowp_scale(A, B, bias, a_offset, b_offset, mult, shift, result_offset, min_bound, max_bound, dst_dtype):
+    A = np.ascontiguousarray(A)
+    B = np.ascontiguousarray(B)
+    M, K = A.shape
+    _, N = B.shape
+    m, s, n = _qparams(mult, shift)
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.empty((M, N), dtype=dst_dtype)
+    lib.orc_gemmlowp_scale(_p(A), _signed(A), C.c_int64(K), _p(B), _signed(B), C.c_int64(N), _p(bias), _p(out),
+                           C.c_int64(N), _signed(out), M, N, K, C.c_int32(a_offset), C.c_int32(b_offset), _p(m), _p(s), n,
+                           C.c_int32(result_offset), C.c_int32(min_bound), C.c_int32(max_bound))
     return out
 
 
@@ -303,6 +331,17 @@ def ref_quantize_down_fixedpoint(src, bias, mult, shift, result_offset, lo, hi, 
     out = np.empty((M, N), dtype=dst_dtype)
     ref().ref_quantize_down_fixedpoint(_p(src), _p(bias), M, N, _p(m), _p(s), n, C.c_int32(result_offset),
                                        C.c_int32(lo), C.c_int32(hi), _signed(out), _p(out))
+    return out
+
+
+def ref_quantize_down_scale(src, bias, mult, shift, result_offset, lo, hi, dst_dtype):
+    src = np.ascontiguousarray(src, dtype=np.int32)
+    M, N = src.shape
+    m, s, n = _qparams(mult, shift)
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.empty((M, N), dtype=dst_dtype)
+    ref().ref_quantize_down_scale(_p(src), _p(bias), M, N, _p(m), _p(s), n, C.c_int32(result_offset), C.c_int32(lo),
+                                  C.c_int32(hi), _signed(out), _p(out))
     return out
 
 

@@ -204,6 +204,46 @@ void orc_output_stage_fixedpoint(const int32_t *src, int64_t lds, const int32_t 
         }
 }
 
+/* QUANTIZE_DOWN, the integer-multiplier stage: ((v + result_offset) * mult) >> shift with wrap-around arithmetic and a
+ * truncating arithmetic shift (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ScaleKernel.cpp:92-180 and the scalar tail of
+ * src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:348-362; reference test oracle
+ * tests/validation/reference/GEMMLowp.cpp:66-104). shift is in [0, 31]. */
+int32_t orc_requant_scale_s32(int32_t v, int32_t mult, int32_t shift, int32_t result_offset)
+{
+    const uint32_t u = ((uint32_t)v + (uint32_t)result_offset) * (uint32_t)mult;
+    const int32_t  r = (int32_t)u;
+    /* arithmetic shift right, written without relying on the sign behaviour of >> */
+    return r >= 0 ? (r >> shift) : -(int32_t)(((uint32_t)(-(int64_t)r) + ((1u << shift) - 1u)) >> shift);
+}
+
+void orc_output_stage_scale(const int32_t *src, int64_t lds, const int32_t *bias, void *dst, int64_t ldd, int dst_signed,
+                            int M, int N, const int32_t *mult, const int32_t *shift, int n_qparams,
+                            int32_t result_offset, int32_t min_bound, int32_t max_bound)
+{
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j)
+        {
+            int32_t v = src[(int64_t)i * lds + j];
+            if (bias)
+                v = wrap_add(v, bias[j]);
+            const int q = n_qparams > 1 ? j : 0;
+            v           = orc_requant_scale_s32(v, mult[q], shift[q], result_offset);
+            store8(dst, dst_signed, (int64_t)i * ldd + j, orc_narrow_clamp(v, dst_signed, min_bound, max_bound));
+        }
+}
+
+void orc_gemmlowp_scale(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
+                        const int32_t *bias, void *dst, int64_t ldd, int dst_signed, int M, int N, int K,
+                        int32_t a_offset, int32_t b_offset, const int32_t *mult, const int32_t *shift, int n_qparams,
+                        int32_t result_offset, int32_t min_bound, int32_t max_bound)
+{
+    int32_t *t = (int32_t *)malloc(sizeof(int32_t) * (size_t)(M > 0 ? M : 1) * (size_t)(N > 0 ? N : 1));
+    orc_gemmlowp_s32(A, a_signed, lda, B, b_signed, ldb, t, N, M, N, K, a_offset, b_offset);
+    orc_output_stage_scale(t, N, bias, dst, ldd, dst_signed, M, N, mult, shift, n_qparams, result_offset, min_bound,
+                           max_bound);
+    free(t);
+}
+
 /* src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:248-364 (per tensor), :366-461 (per channel) */
 void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
                              const int32_t *bias, void *dst, int64_t ldd, int dst_signed, int M, int N, int K,

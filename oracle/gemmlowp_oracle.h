@@ -53,6 +53,16 @@ void orc_output_stage_fixedpoint(const int32_t *src, int64_t lds, const int32_t 
                                  int dst_signed, int M, int N, const int32_t *mult, const int32_t *shift,
                                  int n_qparams, int32_t result_offset, int32_t min_bound, int32_t max_bound);
 
+/* QUANTIZE_DOWN (integer multiplier): ((v + result_offset) * mult) >> shift, wrap-around, truncating shift, 0 <= shift < 32 */
+int32_t orc_requant_scale_s32(int32_t v, int32_t mult, int32_t shift, int32_t result_offset);
+void orc_output_stage_scale(const int32_t *src, int64_t lds, const int32_t *bias, void *dst, int64_t ldd, int dst_signed,
+                            int M, int N, const int32_t *mult, const int32_t *shift, int n_qparams,
+                            int32_t result_offset, int32_t min_bound, int32_t max_bound);
+void orc_gemmlowp_scale(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
+                        const int32_t *bias, void *dst, int64_t ldd, int dst_signed, int M, int N, int K,
+                        int32_t a_offset, int32_t b_offset, const int32_t *mult, const int32_t *shift, int n_qparams,
+                        int32_t result_offset, int32_t min_bound, int32_t max_bound);
+
 /* GEMM + offset contribution + bias + fixed-point stage in one call */
 void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
                              const int32_t *bias, void *dst, int64_t ldd, int dst_signed, int M, int N, int K,

@@ -109,6 +109,31 @@ extern "C"
         }
     }
 
+    /* tests/validation/reference/GEMMLowp.cpp:66-104,278-307: QUANTIZE_DOWN with an integer multiplier */
+    void ref_quantize_down_scale(const int32_t *in, const int32_t *bias, int M, int N, const int32_t *mult,
+                                 const int32_t *shift, int n_qparams, int32_t result_offset, int32_t lo, int32_t hi,
+                                 int dst_signed, void *out)
+    {
+        const SimpleTensor<int32_t> t = make<int32_t>(TensorShape(N, M), DataType::S32, in);
+        const std::vector<int32_t>  m(mult, mult + n_qparams), s(shift, shift + n_qparams);
+        if (dst_signed)
+        {
+            const SimpleTensor<int8_t> d =
+                bias ? reference::gemmlowp_quantize_down_scale<int32_t, int8_t>(
+                           t, make<int32_t>(TensorShape(N), DataType::S32, bias), result_offset, m, s, lo, hi)
+                     : reference::gemmlowp_quantize_down_scale<int32_t, int8_t>(t, result_offset, m, s, lo, hi);
+            std::memcpy(out, d.data(), d.num_elements());
+        }
+        else
+        {
+            const SimpleTensor<uint8_t> d =
+                bias ? reference::gemmlowp_quantize_down_scale<int32_t, uint8_t>(
+                           t, make<int32_t>(TensorShape(N), DataType::S32, bias), result_offset, m, s, lo, hi)
+                     : reference::gemmlowp_quantize_down_scale<int32_t, uint8_t>(t, result_offset, m, s, lo, hi);
+            std::memcpy(out, d.data(), d.num_elements());
+        }
+    }
+
     /* tests/validation/reference/DequantizationLayer.cpp:69-116 on an S32 tensor, as
      * tests/validation/fixtures/GEMMLowpFixture.h:868-910 uses it for the F32 GEMMLowp reference */
     void ref_dequantize_s32(const int32_t *in, int count, float scale, float *out)

@@ -480,6 +480,66 @@ static void test_output_stage()
     EXPECT(dense_copy<int8_t>(dst) == want);
 }
 
+// QUANTIZE_DOWN (integer multiplier): stand-alone stage without bounds (min == max) and fused into the GEMM
+static void test_quantize_down_scale()
+{
+    SECTION("QUANTIZE_DOWN (integer multiplier): NEGEMMLowpOutputStage and fused NEGEMMLowpMatrixMultiplyCore");
+    {
+        const int M = 9, N = 77;
+        Tensor    src, bias, dst;
+        init_tensor(src, TensorShape(N, M), DataType::S32);
+        init_tensor(bias, TensorShape(N), DataType::S32);
+        init_tensor(dst, TensorShape(N, M), DataType::QASYMM8);
+        GEMMLowpOutputStageInfo os;
+        os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN;
+        os.gemmlowp_multiplier = 5, os.gemmlowp_shift = 9, os.gemmlowp_offset = -700;
+        os.gemmlowp_min_bound = 0, os.gemmlowp_max_bound = 0, os.output_data_type = DataType::QASYMM8;
+        EXPECT(bool(NEGEMMLowpOutputStage::validate(src.info(), bias.info(), dst.info(), os)));
+        GEMMLowpOutputStageInfo bad = os;
+        bad.gemmlowp_shift          = 32;
+        EXPECT(!bool(NEGEMMLowpOutputStage::validate(src.info(), bias.info(), dst.info(), bad)));
+        NEGEMMLowpOutputStage stage;
+        stage.configure(&src, &bias, &dst, os);
+        src.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int32_t>(src, -20000, 30000, 81), fill_uniform<int32_t>(bias, -3000, 3000, 82);
+        stage.run();
+        std::vector<uint8_t> want(M * N);
+        orc_output_stage_scale(reinterpret_cast<const int32_t *>(src.buffer()), N, reinterpret_cast<const int32_t *>(bias.buffer()),
+                               want.data(), N, 0, M, N, &os.gemmlowp_multiplier, &os.gemmlowp_shift, 1, -700,
+                               std::numeric_limits<int32_t>::lowest(), std::numeric_limits<int32_t>::max());
+        EXPECT(dense_copy<uint8_t>(dst) == want);
+    }
+    {
+        const int M = 40, N = 50, K = 96;
+        Tensor    a, b, bias, dst;
+        init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f, 4));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f, -2));
+        init_tensor(bias, TensorShape(N), DataType::S32);
+        init_tensor(dst, TensorShape(N, M), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f, 0));
+        GEMMLowpOutputStageInfo st;
+        st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN;
+        st.gemmlowp_multiplier = 3, st.gemmlowp_shift = 12, st.gemmlowp_offset = 250;
+        st.gemmlowp_min_bound = -100, st.gemmlowp_max_bound = 90, st.output_data_type = DataType::QASYMM8_SIGNED;
+        const GEMMInfo gi(false, false, true, 0, false, false, st);
+        EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), bias.info(), dst.info(), gi)));
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, &bias, &dst, gi);
+        a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(a, -128, 127, 83), fill_uniform<int8_t>(b, -128, 127, 84), fill_uniform<int32_t>(bias, -2000, 2000, 85);
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        const auto Cb = dense_copy<int32_t>(bias);
+        std::vector<int8_t> want(M * N);
+        orc_gemmlowp_scale(A.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 4, -2, &st.gemmlowp_multiplier,
+                           &st.gemmlowp_shift, 1, 250, -100, 90);
+        gemm.run();
+        EXPECT(dense_copy<int8_t>(dst) == want);
+        size_t inside = 0;
+        for (int8_t v : want)
+            inside += (v > -100 && v < 90) ? 1 : 0;
+        EXPECT(inside * 4 > want.size());
+    }
+}
+
 static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act)
 {
     SECTION(per_channel ? "NEGEMMConvolutionLayer NHWC per-channel weights" : "NEGEMMConvolutionLayer NHWC per-tensor weights");
@@ -704,6 +764,7 @@ int main(int argc, char **argv)
             test_gemmlowp_per_channel_and_update();
             test_gemmlowp_f32();
             test_output_stage();
+            test_quantize_down_scale();
             test_convolution(DataType::QASYMM8_SIGNED, true, 64, ActivationLayerInfo());
             test_convolution(DataType::QASYMM8_SIGNED, false, 16, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU));
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());

@@ -129,6 +129,37 @@ def output_stage():
     np.savez_compressed(os.path.join(HERE, "output_stage.npz"), **out)
 
 
+def output_stage_scale():
+    """QUANTIZE_DOWN with an integer multiplier, stand-alone: S32 input + bias through the reference's
+    gemmlowp_quantize_down_scale (tests/validation/reference/GEMMLowp.cpp:66-104), shapes / value ranges of
+    tests/validation/fixtures/GEMMLowpFixture.h (GEMMLowpQuantizeDownInt32ScaleValidationFixture), per tensor and per
+    column, with and without bounds (min == max means none)."""
+    rng = np.random.default_rng(110)
+    out = {}
+    n = 0
+    for signed in (0, 1):
+        lo_t, hi_t = (-128, 127) if signed else (0, 255)
+        for (M, N) in [(1, 1), (7, 15), (13, 33), (5, 128), (3, 1000)]:
+            for variant in range(3):
+                src = rng.integers(-60000, 60001, size=(M, N), dtype=np.int32)
+                bias = rng.integers(-6000, 6001, size=N, dtype=np.int32)
+                per_channel = variant == 2
+                cnt = N if per_channel else 1
+                mult = rng.integers(1, 300, size=cnt).astype(np.int32)
+                shift = rng.integers(4, 17, size=cnt).astype(np.int32)
+                roff = int(rng.integers(-3000, 3000))
+                lo, hi = (0, 0) if variant == 0 else (lo_t + 5, hi_t - 9)
+                with_bias = (n + variant) % 2
+                dst = oracle.ref_quantize_down_scale(src, bias if with_bias else None, mult, shift, roff, lo, hi,
+                                                     np.int8 if signed else np.uint8)
+                out["src%d" % n], out["bias%d" % n], out["dst%d" % n] = src, bias, dst
+                out["mult%d" % n], out["shift%d" % n] = mult, shift
+                out["p%d" % n] = np.array([roff, lo, hi, with_bias], dtype=np.int32)
+                n += 1
+    out["count"] = np.array(n)
+    np.savez_compressed(os.path.join(HERE, "output_stage_scale.npz"), **out)
+
+
 def requant_sweep():
     """The scalar primitive on inputs for which the reference's int arithmetic has no signed overflow."""
     rng = np.random.default_rng(105)
@@ -233,7 +264,8 @@ def conv():
 
 if __name__ == "__main__":
     assert oracle.ref_available(), "build oracle/_ref first (make -C oracle ref)"
-    for fn in (gemmlowp_s32, gemmlowp_batched, fused_fixedpoint, output_stage, requant_sweep, quant_multiplier,
+    for fn in (gemmlowp_s32, gemmlowp_batched, fused_fixedpoint, output_stage, output_stage_scale, requant_sweep,
+               quant_multiplier,
                f32_dequant, im2col, conv):
         fn()
         print("wrote", fn.__name__)

@@ -25,7 +25,7 @@ def announce(*what):
 
 def run_gemm(A, B, epilogue, dst_dtype, a_offset=0, b_offset=0, bias=None, mult=None, shift=None, result_offset=0,
              lo=-(1 << 31), hi=(1 << 31) - 1, scale=1.0, bias_f32=None, act=(-np.inf, np.inf), path=capi.PATH_AUTO,
-             device=False, lda=None, ldd=None):
+             device=False, lda=None, ldd=None, stage=0):
     """A [M][K] or [batch][M][K]; B [K][N] or [batch][K][N]. Returns (numpy result, kernel name)."""
     A3 = A if A.ndim == 3 else A[None]
     batch, M, K = A3.shape
@@ -33,7 +33,7 @@ def run_gemm(A, B, epilogue, dst_dtype, a_offset=0, b_offset=0, bias=None, mult=
     per_channel = mult is not None and np.ndim(mult) > 0 and len(mult) > 1
     rq = capi.requant(0 if per_channel or mult is None else int(np.atleast_1d(mult)[0]),
                       0 if per_channel or shift is None else int(np.atleast_1d(shift)[0]), result_offset, lo, hi,
-                      per_channel)
+                      per_channel, stage)
     dcode = {np.dtype(np.uint8): capi.U8, np.dtype(np.int8): capi.S8, np.dtype(np.int32): capi.S32,
              np.dtype(np.float32): capi.F32}[np.dtype(dst_dtype)]
     lda = lda or K

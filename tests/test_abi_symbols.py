@@ -23,12 +23,29 @@ def test_header_functions_are_exported():
     assert sorted(capi.EXPORTS) == names
 
 
-def test_descriptor_struct_sizes_match_header_layout():
-    # 4 + 4 ints, 6 int64, 2 ints, 6-int requant, 3 floats, 2 ints
-    assert ctypes.sizeof(capi.Requant) == 24
-    assert ctypes.sizeof(capi.GemmDesc) == 32 + 48 + 8 + 24 + 12 + 8 + 4  # + tail padding to 8
-    assert ctypes.sizeof(capi.OutputStageDesc) == 8 + 16 + 4 + 24 + 4
-    assert ctypes.sizeof(capi.ConvDesc) == 21 * 4 + 24 + 8
+def test_descriptor_struct_layouts_match_the_header(tmp_path):
+    """sizeof and the offset of every field, as the C compiler lays out include/mi355_gemmlowp.h, against the ctypes
+    mirrors in computelibrary_amd/capi.py."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    structs = {"mi355_requant": capi.Requant, "mi355_gemm_desc": capi.GemmDesc,
+               "mi355_output_stage_desc": capi.OutputStageDesc, "mi355_conv_desc": capi.ConvDesc}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "mi355_gemmlowp.h"', 'int main(void) {']
+    for cname, ct in structs.items():
+        lines.append('printf("%s %%zu\\n", sizeof(%s));' % (cname, cname))
+        for fname, _ in ct._fields_:
+            lines.append('printf("%s.%s %%zu\\n", offsetof(%s, %s));' % (cname, fname, cname, fname))
+    lines += ['return 0; }']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-I", os.path.join(root, "include"), "-o", str(exe), str(src)])
+    out = dict(l.split() for l in subprocess.check_output([str(exe)], text=True).splitlines())
+    for cname, ct in structs.items():
+        assert int(out[cname]) == ctypes.sizeof(ct), cname
+        for fname, _ in ct._fields_:
+            assert int(out["%s.%s" % (cname, fname)]) == getattr(ct, fname).offset, (cname, fname)
 
 
 def test_create_rejects_bad_descriptors_without_a_gpu():

@@ -264,6 +264,49 @@ def test_output_stage_fixture(golden):
         np.testing.assert_array_equal(out, dst)
 
 
+def test_output_stage_scale_fixture(golden):
+    """QUANTIZE_DOWN (integer multiplier), stand-alone, against the reference oracle's outputs (per-tensor entries)."""
+    g = golden("output_stage_scale.npz")
+    ran = 0
+    for n in range(int(g["count"])):
+        roff, lo, hi, with_bias = (int(x) for x in g["p%d" % n])
+        mult, shift = g["mult%d" % n], g["shift%d" % n]
+        if len(mult) > 1:
+            continue
+        if lo == hi:
+            lo, hi = -(1 << 31), (1 << 31) - 1
+        src, dst = g["src%d" % n], g["dst%d" % n]
+        out = np.zeros_like(dst)
+        announce("scale output stage fixture", n, src.shape, dst.dtype)
+        capi.output_stage(np.ascontiguousarray(src), np.ascontiguousarray(g["bias%d" % n]) if with_bias else None, out,
+                          capi.requant(int(mult[0]), int(shift[0]), roff, lo, hi, stage=capi.STAGE_SCALE))
+        np.testing.assert_array_equal(out, dst)
+        ran += 1
+    assert ran >= 10
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+@pytest.mark.parametrize("M", [7, 200])
+def test_fused_scale_stage_on_every_path(M, per_channel):
+    """GEMM + offset contribution + bias + QUANTIZE_DOWN (integer multiplier) fused, against the oracle whose stage is
+    pinned by the reference's gemmlowp_quantize_down_scale (tests/test_oracle_gemm.py)."""
+    rng = np.random.default_rng(49 + M + int(per_channel))
+    N, K = 170, 256
+    A = rng.integers(0, 256, size=(M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, size=(K, N), dtype=np.uint8)
+    bias = rng.integers(-4000, 4000, size=N).astype(np.int32)
+    cnt = N if per_channel else 1
+    mult = rng.integers(1, 9, size=cnt).astype(np.int32)
+    shift = rng.integers(13, 16, size=cnt).astype(np.int32)
+    b_off = 0 if per_channel else -121
+    want = oracle.gemmlowp_scale(A, B, bias, -130, b_off, mult, shift, 900, 3, 250, np.uint8)
+    assert ((want > 3) & (want < 250)).mean() > 0.2
+    for path in paths_for(M):
+        announce("fused scale stage", M, per_channel, "path", path)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.uint8, -130, b_off, bias, mult, shift, 900, 3, 250, path=path,
+                          device=True, stage=capi.STAGE_SCALE)
+        np.testing.assert_array_equal(got, want)
+
 def test_update_quant_and_rerun():
     """update_quantization_parameters: new offsets / multiplier without re-packing B; run twice gives identical bytes
     (tests/validation/NEON/GEMMLowp.cpp:211-297 MultipleExecutionWithConfigure)."""

@@ -81,6 +81,38 @@ def test_output_stage_fixture(golden):
         np.testing.assert_array_equal(got, dst)
 
 
+def test_output_stage_scale_fixture(golden):
+    """QUANTIZE_DOWN (integer multiplier) against the outputs of the reference's gemmlowp_quantize_down_scale."""
+    g = golden("output_stage_scale.npz")
+    kinds = set()
+    for n in range(int(g["count"])):
+        roff, lo, hi, with_bias = (int(x) for x in g["p%d" % n])
+        dst = g["dst%d" % n]
+        if lo == hi:  # "no bounded activation": only the saturation to the type is left
+            lo, hi = -(1 << 31), (1 << 31) - 1
+        got = oracle.output_stage_scale(g["src%d" % n], g["bias%d" % n] if with_bias else None, g["mult%d" % n],
+                                        g["shift%d" % n], roff, lo, hi, dst.dtype)
+        np.testing.assert_array_equal(got, dst)
+        kinds.add((dst.dtype.name, len(g["mult%d" % n]) > 1, bool(with_bias)))
+        inside = ((dst > np.iinfo(dst.dtype).min) & (dst < np.iinfo(dst.dtype).max)).mean()
+    assert ("uint8", True, True) in kinds or ("uint8", True, False) in kinds
+    assert ("int8", False, True) in kinds and ("int8", False, False) in kinds
+
+
+def test_scale_stage_primitive_properties():
+    """((v + off) * m) >> s: truncating (floor) shift, wrap-around product, agrees with exact integer arithmetic wherever
+    nothing overflows."""
+    rng = np.random.default_rng(111)
+    v = rng.integers(-(1 << 20), 1 << 20, size=5000).astype(np.int64)
+    for m, sft, off in ((1, 0, 0), (3, 9, -40), (255, 16, 1234), (77, 31, -5)):
+        want = ((v + off) * m) >> sft  # python ints: floor division by 2^s
+        got = np.array([oracle.lib.orc_requant_scale_s32(int(x), m, sft, off) for x in v[:500]])
+        np.testing.assert_array_equal(got, want[:500])
+    # wrap-around: the product is taken modulo 2^32 before the shift
+    assert oracle.lib.orc_requant_scale_s32(1 << 30, 4, 0, 0) == 0
+    assert oracle.lib.orc_requant_scale_s32((1 << 30) + 1, 4, 1, 0) == 2
+    assert oracle.lib.orc_requant_scale_s32(-1, 1, 5, 0) == -1  # floor, not round-to-zero
+
 def test_f32_fixture(golden):
     """The reference's test oracle rounds once (float(t)*scale); the NEON order this oracle follows rounds
     acc*scale and offsets*scale separately. Identical when offsets are zero, else equal to ~1 ulp of the

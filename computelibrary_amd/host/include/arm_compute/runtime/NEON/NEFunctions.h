@@ -1,6 +1,7 @@
 #ifndef ACL_MI355_RUNTIME_NEFUNCTIONS_H
 #define ACL_MI355_RUNTIME_NEFUNCTIONS_H
 #include "arm_compute/runtime/NEON/functions/NEFullyConnectedLayer.h"
+#include "arm_compute/runtime/NEON/functions/NEGEMMConv2d.h"
 #include "arm_compute/runtime/NEON/functions/NEGEMMConvolutionLayer.h"
 #include "arm_compute/runtime/NEON/functions/NEGEMMLowpMatrixMultiplyCore.h"
 #include "arm_compute/runtime/NEON/functions/NEGEMMLowpOutputStage.h"

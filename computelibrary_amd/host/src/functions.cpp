@@ -992,4 +992,57 @@ const char *NEFullyConnectedLayer::kernel_name() const
 {
     return _impl->handle ? mi355_gemmlowp_kernel_name(_impl->handle) : "";
 }
+// =====================================================================================================================
+// NEGEMMConv2d
+// =====================================================================================================================
+NEGEMMConv2d::NEGEMMConv2d(const std::shared_ptr<IMemoryManager> &memory_manager)
+    : _conv(std::make_unique<NEGEMMConvolutionLayer>(memory_manager))
+{
+}
+NEGEMMConv2d::~NEGEMMConv2d() = default;
+
+// src/cpu/operators/CpuGemmDirectConv2d.cpp:166-224 of the reference
+Status NEGEMMConv2d::validate(const ITensorInfo *input, const ITensorInfo *weights, const ITensorInfo *biases,
+                              const ITensorInfo *output, const Conv2dInfo &info)
+{
+    ARM_COMPUTE_RETURN_ERROR_ON_NULLPTR(input, weights, output);
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.num_groups > 1, "Grouping (num_groups != 1) is not supported on Cpu");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC, "Data layout supported is NHWC");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.dilation != Size2D(1U, 1U), "Dilation is not supported by NEGEMMConv2d");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.weights_info.weight_format() != WeightFormat::UNSPECIFIED,
+                                    "Fixed-format weights are not built in this library");
+    return NEGEMMConvolutionLayer::validate(input, weights, biases, output, info.conv_info, WeightsInfo(), info.dilation,
+                                            info.act_info, info.enable_fast_math, info.num_groups);
+}
+
+void NEGEMMConv2d::configure(ITensor *input, const ITensor *weights, const ITensor *biases, ITensor *output,
+                             const Conv2dInfo &info)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(input, weights, output);
+    if (output->info()->total_size() != 0)
+        ARM_COMPUTE_ERROR_THROW_ON(validate(input->info(), weights->info(), biases != nullptr ? biases->info() : nullptr,
+                                            output->info(), info));
+    else
+    {
+        ARM_COMPUTE_ERROR_ON_MSG(info.dilation != Size2D(1U, 1U), "Dilation is not supported by NEGEMMConv2d");
+        ARM_COMPUTE_ERROR_ON_MSG(info.num_groups > 1, "Grouping (num_groups != 1) is not supported on Cpu");
+    }
+    _conv->configure(input, weights, biases, output, info.conv_info, WeightsInfo(), info.dilation, info.act_info,
+                     info.enable_fast_math, info.num_groups);
+}
+
+void NEGEMMConv2d::run()
+{
+    _conv->run();
+}
+
+void NEGEMMConv2d::prepare()
+{
+    _conv->prepare();
+}
+
+const char *NEGEMMConv2d::kernel_name() const
+{
+    return _conv->kernel_name();
+}
 } // namespace arm_compute

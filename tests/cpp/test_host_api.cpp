@@ -247,6 +247,27 @@ static void test_fully_connected_validate()
     EXPECT(wf == WeightFormat::UNSPECIFIED);
 }
 
+// accept / reject rules of CpuGemmDirectConv2d::validate (src/cpu/operators/CpuGemmDirectConv2d.cpp:166-224 of the reference)
+static void test_gemm_conv2d_validate()
+{
+    SECTION("NEGEMMConv2d::validate accept / reject");
+    TensorInfo src(TensorShape(16U, 9U, 9U, 2U), 1, DataType::QASYMM8, QuantizationInfo(0.1f, 3));
+    TensorInfo w(TensorShape(16U, 3U, 3U, 8U), 1, DataType::QASYMM8, QuantizationInfo(0.1f, 3));
+    TensorInfo b(TensorShape(8U), 1, DataType::S32), dst(TensorShape(8U, 7U, 7U, 2U), 1, DataType::QASYMM8, QuantizationInfo(0.5f, 1));
+    for (TensorInfo *t : {&src, &w, &dst})
+        t->set_data_layout(DataLayout::NHWC);
+    const PadStrideInfo ps(1, 1, 0, 0);
+    EXPECT(bool(NEGEMMConv2d::validate(&src, &w, &b, &dst, Conv2dInfo(ps, Size2D(1, 1), ActivationLayerInfo(), false, 1))));
+    EXPECT(!bool(NEGEMMConv2d::validate(&src, &w, &b, &dst, Conv2dInfo(ps, Size2D(2, 2), ActivationLayerInfo(), false, 1)))); // dilation
+    EXPECT(!bool(NEGEMMConv2d::validate(&src, &w, &b, &dst, Conv2dInfo(ps, Size2D(1, 1), ActivationLayerInfo(), false, 2)))); // groups
+    TensorInfo src_nchw(src);
+    src_nchw.set_data_layout(DataLayout::NCHW);
+    EXPECT(!bool(NEGEMMConv2d::validate(&src_nchw, &w, &b, &dst, Conv2dInfo(ps, Size2D(1, 1), ActivationLayerInfo(), false, 1))));
+    TensorInfo w_bad(TensorShape(15U, 3U, 3U, 8U), 1, DataType::QASYMM8, QuantizationInfo(0.1f, 3));
+    w_bad.set_data_layout(DataLayout::NHWC);
+    EXPECT(!bool(NEGEMMConv2d::validate(&src, &w_bad, &b, &dst, Conv2dInfo(ps, Size2D(1, 1), ActivationLayerInfo(), false, 1))));
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 // GPU tests
 // ---------------------------------------------------------------------------------------------------------------------
@@ -713,6 +734,45 @@ static void test_fully_connected(DataType dt, FcCase which)
     std::printf("       kernel: %s\n", fcl.kernel_name());
 }
 
+// NEGEMMConv2d: stride 2, asymmetric padding, fused RELU, against the oracle's direct convolution
+static void test_gemm_conv2d()
+{
+    SECTION("NEGEMMConv2d NHWC stride 2, asymmetric padding, RELU");
+    const int batch = 3, H = 17, W = 13, C = 32, OFM = 24, KH = 3, KW = 3;
+    const int in_zp = 5, out_zp = -9;
+    std::vector<float> wscale(OFM);
+    for (int i = 0; i < OFM; ++i)
+        wscale[i] = 0.002f + 0.0007f * i;
+    Tensor src, w, bias, dst;
+    init_tensor(src, TensorShape(C, W, H, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.03f, in_zp));
+    init_tensor(w, TensorShape(C, KW, KH, OFM), DataType::QSYMM8_PER_CHANNEL, QuantizationInfo(wscale));
+    init_tensor(bias, TensorShape(OFM), DataType::S32);
+    init_tensor(dst, TensorShape(), DataType::QASYMM8_SIGNED, QuantizationInfo(0.6f, out_zp));
+    for (Tensor *t : {&src, &w, &dst})
+        t->info()->set_data_layout(DataLayout::NHWC);
+    const PadStrideInfo       ps(2, 2, 1, 0, 0, 1, DimensionRoundingType::FLOOR); // left 1, right 0, top 0, bottom 1
+    const ActivationLayerInfo relu(ActivationLayerInfo::ActivationFunction::RELU);
+    const Conv2dInfo          info(ps, Size2D(1, 1), relu, false, 1);
+    NEGEMMConv2d conv;
+    conv.configure(&src, &w, &bias, &dst, info);
+    const int OW = (W + 1 + 0 - 3) / 2 + 1, OH = (H + 0 + 1 - 3) / 2 + 1;
+    EXPECT(dst.info()->dimension(0) == (size_t)OFM && dst.info()->dimension(1) == (size_t)OW && dst.info()->dimension(2) == (size_t)OH);
+    src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int8_t>(src, -128, 127, 91), fill_uniform<int8_t>(w, -127, 127, 92), fill_uniform<int32_t>(bias, -800, 800, 93);
+    conv.run();
+    GEMMLowpOutputStageInfo st;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(QuantizationInfo(0.03f, in_zp), QuantizationInfo(wscale),
+                                                              QuantizationInfo(0.6f, out_zp), st)));
+    int32_t lo = 0, hi = 0;
+    std::tie(lo, hi) = get_quantized_activation_min_max(relu, DataType::QASYMM8_SIGNED, UniformQuantizationInfo(0.6f, out_zp));
+    std::vector<uint8_t> want(static_cast<size_t>(batch) * OH * OW * OFM);
+    orc_conv_nhwc_direct(src.buffer(), 1, w.buffer(), 1, reinterpret_cast<const int32_t *>(bias.buffer()), want.data(), 1, batch,
+                         H, W, C, OFM, KH, KW, 2, 2, 1, 0, 0, 1, 1, 1, in_zp, 0, st.gemmlowp_multipliers.data(),
+                         st.gemmlowp_shifts.data(), OFM, out_zp, lo, hi);
+    EXPECT(dense_copy<uint8_t>(dst) == want);
+    std::printf("       kernel: %s\n", conv.kernel_name());
+}
+
 static void test_error_paths()
 {
     SECTION("configure() throws on invalid input; run() before configure() throws");
@@ -754,6 +814,7 @@ int main(int argc, char **argv)
             test_quant_helpers();
             test_validate_tables();
             test_fully_connected_validate();
+            test_gemm_conv2d_validate();
             test_error_paths();
         }
         else
@@ -770,6 +831,7 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
             test_convolution(DataType::QASYMM8, true, 32,
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
+            test_gemm_conv2d();
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);

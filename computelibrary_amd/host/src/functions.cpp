@@ -5,6 +5,7 @@
 // Status and never throws, configure() that throws std::runtime_error on invalid input, synchronous run().
 #include "arm_compute/core/utils/quantization/AsymmHelpers.h"
 #include "arm_compute/runtime/NEON/NEFunctions.h"
+#include "arm_compute/runtime/experimental/operators/CpuGEMMLowp.h"
 #include "mi355_gemmlowp.h"
 
 #include <cmath>
@@ -90,6 +91,73 @@ Status check_matrix_layout(const ITensorInfo *t, const char *name)
 const std::set<ActivationLayerInfo::ActivationFunction> fusable_acts = {
     ActivationLayerInfo::ActivationFunction::RELU, ActivationLayerInfo::ActivationFunction::BOUNDED_RELU,
     ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU};
+
+// the C-ABI descriptor of a GEMMLowp on these tensor infos (shapes are x-fastest: a = [K, M, batch], b = [N, K(, batch)],
+// output = [N, M, batch]); per-channel multipliers / shifts are cut to exactly N entries
+void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorInfo *oi, const GEMMInfo &gemm_info,
+                    mi355_gemm_desc &d, std::vector<int32_t> &multipliers, std::vector<int32_t> &shifts)
+{
+    multipliers.clear(), shifts.clear();
+    const GEMMLowpOutputStageInfo stage = gemm_info.gemmlowp_output_stage();
+    d = mi355_gemm_desc{};
+    d.K                = static_cast<int32_t>(ai->dimension(0));
+    d.N                = static_cast<int32_t>(bi->dimension(0));
+    d.M                = static_cast<int32_t>(ai->dimension(1));
+    d.batch            = static_cast<int32_t>(ai->tensor_shape().total_size_upper(2));
+    d.a_dtype          = to_mi355(ai->data_type());
+    d.b_dtype          = to_mi355(bi->data_type());
+    d.dst_dtype        = to_mi355(oi->data_type());
+    d.lda              = ai->strides_in_bytes()[1];
+    d.ldb              = bi->strides_in_bytes()[1];
+    d.ldd              = oi->strides_in_bytes()[1] / oi->element_size();
+    d.a_batch_stride   = ai->strides_in_bytes()[2];
+    d.b_batch_stride   = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
+    if (gemm_info.depth_output_gemm3d() != 0)
+        d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
+    else
+        d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
+    d.a_offset = ai->quantization_info().uniform().offset;
+    d.b_offset = is_data_type_quantized_per_channel(bi->data_type()) ? 0 : bi->quantization_info().uniform().offset;
+    d.act_min  = -std::numeric_limits<float>::infinity();
+    d.act_max  = std::numeric_limits<float>::infinity();
+    d.scale    = 1.f;
+    d.path     = MI355_PATH_AUTO;
+    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT || stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN)
+    {
+        d.epilogue = MI355_EPI_FIXEDPOINT;
+        d.requant  = make_requant(stage);
+        if (stage.is_quantized_per_channel)
+        {
+            multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.N);
+            shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.N);
+        }
+    }
+    else if (oi->data_type() == DataType::F32)
+    {
+        d.epilogue = MI355_EPI_F32;
+        d.scale    = ai->quantization_info().uniform().scale * bi->quantization_info().uniform().scale;
+        const ActivationLayerInfo act = gemm_info.activation_info();
+        if (act.enabled())
+        {
+            switch (act.activation())
+            {
+                case ActivationLayerInfo::ActivationFunction::RELU:
+                    d.act_min = 0.f;
+                    break;
+                case ActivationLayerInfo::ActivationFunction::BOUNDED_RELU:
+                    d.act_min = 0.f, d.act_max = act.a();
+                    break;
+                case ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU:
+                    d.act_min = act.b(), d.act_max = act.a();
+                    break;
+                default:
+                    ARM_COMPUTE_ERROR("Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
+            }
+        }
+    }
+    else
+        d.epilogue = MI355_EPI_S32;
+}
 } // namespace
 
 // =====================================================================================================================
@@ -254,67 +322,8 @@ void NEGEMMLowpMatrixMultiplyCore::configure(const ITensor *a, const ITensor *b,
     s.is_prepared = false;
     s.b_constant  = gemm_info.reshape_b_only_on_first_run(); // NEGEMMLowpMatrixMultiplyCore.cpp:77-81 of the reference
 
-    const ITensorInfo *ai = a->info(), *bi = b->info(), *oi = output->info();
-    const GEMMLowpOutputStageInfo stage = gemm_info.gemmlowp_output_stage();
+    fill_gemm_desc(a->info(), b->info(), output->info(), gemm_info, s.desc, s.multipliers, s.shifts);
     mi355_gemm_desc &d = s.desc;
-    d                  = mi355_gemm_desc{};
-    d.K                = static_cast<int32_t>(ai->dimension(0));
-    d.N                = static_cast<int32_t>(bi->dimension(0));
-    d.M                = static_cast<int32_t>(ai->dimension(1));
-    d.batch            = static_cast<int32_t>(ai->tensor_shape().total_size_upper(2));
-    d.a_dtype          = to_mi355(ai->data_type());
-    d.b_dtype          = to_mi355(bi->data_type());
-    d.dst_dtype        = to_mi355(oi->data_type());
-    d.lda              = ai->strides_in_bytes()[1];
-    d.ldb              = bi->strides_in_bytes()[1];
-    d.ldd              = oi->strides_in_bytes()[1] / oi->element_size();
-    d.a_batch_stride   = ai->strides_in_bytes()[2];
-    d.b_batch_stride   = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
-    if (gemm_info.depth_output_gemm3d() != 0)
-        d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
-    else
-        d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
-    d.a_offset = ai->quantization_info().uniform().offset;
-    d.b_offset = is_data_type_quantized_per_channel(bi->data_type()) ? 0 : bi->quantization_info().uniform().offset;
-    d.act_min  = -std::numeric_limits<float>::infinity();
-    d.act_max  = std::numeric_limits<float>::infinity();
-    d.scale    = 1.f;
-    d.path     = MI355_PATH_AUTO;
-    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT || stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN)
-    {
-        d.epilogue = MI355_EPI_FIXEDPOINT;
-        d.requant  = make_requant(stage);
-        if (stage.is_quantized_per_channel)
-        {
-            s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.N);
-            s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.N);
-        }
-    }
-    else if (oi->data_type() == DataType::F32)
-    {
-        d.epilogue = MI355_EPI_F32;
-        d.scale    = ai->quantization_info().uniform().scale * bi->quantization_info().uniform().scale;
-        const ActivationLayerInfo act = gemm_info.activation_info();
-        if (act.enabled())
-        {
-            switch (act.activation())
-            {
-                case ActivationLayerInfo::ActivationFunction::RELU:
-                    d.act_min = 0.f;
-                    break;
-                case ActivationLayerInfo::ActivationFunction::BOUNDED_RELU:
-                    d.act_min = 0.f, d.act_max = act.a();
-                    break;
-                case ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU:
-                    d.act_min = act.b(), d.act_max = act.a();
-                    break;
-                default:
-                    ARM_COMPUTE_ERROR("Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
-            }
-        }
-    }
-    else
-        d.epilogue = MI355_EPI_S32;
     check_abi(mi355_gemmlowp_create(&d, &s.handle), "NEGEMMLowpMatrixMultiplyCore::configure");
 }
 
@@ -1045,4 +1054,134 @@ const char *NEGEMMConv2d::kernel_name() const
 {
     return _conv->kernel_name();
 }
+// =====================================================================================================================
+// experimental::op::CpuGEMMLowp
+// =====================================================================================================================
+namespace experimental
+{
+namespace op
+{
+struct CpuGEMMLowp::Impl
+{
+    mi355_gemm_desc      desc{};
+    mi355_gemm_handle   *handle{nullptr};
+    ActivationLayerInfo  act_info{};
+    bool                 is_prepared{false};
+    bool                 b_constant{true};
+    bool                 has_bias{false};
+    std::vector<int32_t> multipliers, shifts;
+
+    ~Impl()
+    {
+        if (handle)
+            mi355_gemmlowp_destroy(handle);
+    }
+};
+
+CpuGEMMLowp::CpuGEMMLowp() : _impl(std::make_unique<Impl>()) {}
+CpuGEMMLowp::~CpuGEMMLowp() = default;
+
+MemoryRequirements CpuGEMMLowp::workspace() const
+{
+    return {}; // packed B, column sums and staging buffers live in device memory owned by the handle
+}
+
+Status CpuGEMMLowp::validate(const ITensorInfo *a, const ITensorInfo *b, const ITensorInfo *c, const ITensorInfo *output,
+                             const GEMMInfo &gemm_info)
+{
+    return NEGEMMLowpMatrixMultiplyCore::validate(a, b, c, output, gemm_info);
+}
+
+void CpuGEMMLowp::configure(const ITensorInfo *a, const ITensorInfo *b, const ITensorInfo *c, ITensorInfo *output,
+                            const GEMMInfo &gemm_info)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(a, b, output);
+    ARM_COMPUTE_ERROR_THROW_ON(validate(a, b, c, output, gemm_info));
+    Impl &s = *_impl;
+    if (s.handle)
+    {
+        mi355_gemmlowp_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.act_info    = gemm_info.activation_info();
+    s.is_prepared = false;
+    s.b_constant  = gemm_info.reshape_b_only_on_first_run(); // CpuGEMMLowp.cpp:60-66 of the reference
+    s.has_bias    = c != nullptr;
+    fill_gemm_desc(a, b, output, gemm_info, s.desc, s.multipliers, s.shifts);
+    check_abi(mi355_gemmlowp_create(&s.desc, &s.handle), "CpuGEMMLowp::configure");
+}
+
+void CpuGEMMLowp::update_quantization_parameters(const QuantizationInfo &a, const QuantizationInfo &b,
+                                                 const QuantizationInfo &c, const DataType data_type,
+                                                 const bool is_prepared, const bool negated_offsets)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "update_quantization_parameters() before configure()");
+    ARM_COMPUTE_ERROR_ON_MSG(s.desc.epilogue != MI355_EPI_FIXEDPOINT || s.desc.requant.per_channel,
+                             "only a per-tensor fixed-point output stage can be updated in place");
+    int32_t                       lo = get_min_max(data_type).first, hi = get_min_max(data_type).second;
+    const UniformQuantizationInfo uo = c.uniform();
+    if (fusable_acts.count(s.act_info.activation()) != 0)
+        std::tie(lo, hi) = get_quantized_activation_min_max(s.act_info, data_type, uo);
+    GEMMLowpOutputStageInfo out;
+    out.type                     = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+    out.gemmlowp_offset          = uo.offset;
+    out.gemmlowp_min_bound       = lo;
+    out.gemmlowp_max_bound       = hi;
+    out.is_quantized_per_channel = false;
+    out.output_data_type         = data_type;
+    ARM_COMPUTE_ERROR_THROW_ON(quantization::calculate_quantized_multipliers(a, b, c, out));
+    s.desc.a_offset = negated_offsets ? -a.uniform().offset : a.uniform().offset;
+    s.desc.b_offset = negated_offsets ? -b.uniform().offset : b.uniform().offset;
+    s.desc.requant  = make_requant(out);
+    check_abi(mi355_gemmlowp_update_quant(s.handle, s.desc.a_offset, s.desc.b_offset, &s.desc.requant, s.desc.scale, nullptr),
+              "CpuGEMMLowp::update_quantization_parameters");
+    s.is_prepared = s.is_prepared && is_prepared;
+}
+
+void CpuGEMMLowp::prepare(ITensorPack &tensors)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "CpuGEMMLowp::prepare() before configure()");
+    if (s.is_prepared)
+        return;
+    const ITensor *b = tensors.get_const_tensor(ACL_SRC_1);
+    ARM_COMPUTE_ERROR_ON_MSG(b == nullptr || b->buffer() == nullptr, "matrix B (ACL_SRC_1) is missing or has no memory");
+    const int32_t *bias = nullptr;
+    if (s.desc.epilogue == MI355_EPI_FIXEDPOINT && s.has_bias)
+    {
+        const ITensor *c = tensors.get_const_tensor(ACL_SRC_2);
+        ARM_COMPUTE_ERROR_ON_MSG(c == nullptr || c->buffer() == nullptr, "bias (ACL_SRC_2) is missing or has no memory");
+        bias = reinterpret_cast<const int32_t *>(first_element(c));
+    }
+    check_abi(mi355_gemmlowp_prepare(s.handle, first_element(b), bias, s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                     s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "CpuGEMMLowp::prepare");
+    if (s.b_constant)
+    {
+        b->mark_as_unused();
+        s.is_prepared = true;
+    }
+}
+
+void CpuGEMMLowp::run(ITensorPack &tensors)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "CpuGEMMLowp::run() before configure()");
+    const ITensor *a   = tensors.get_const_tensor(ACL_SRC_0);
+    ITensor       *dst = tensors.get_tensor(ACL_DST);
+    ARM_COMPUTE_ERROR_ON_MSG(a == nullptr || dst == nullptr || a->buffer() == nullptr || dst->buffer() == nullptr,
+                             "ACL_SRC_0 / ACL_DST missing or without memory");
+    prepare(tensors);
+    const float *bias_f32 = nullptr;
+    if (s.desc.epilogue == MI355_EPI_F32 && s.has_bias)
+    {
+        const ITensor *c = tensors.get_const_tensor(ACL_SRC_2);
+        ARM_COMPUTE_ERROR_ON_MSG(c == nullptr || c->buffer() == nullptr, "bias (ACL_SRC_2) is missing or has no memory");
+        bias_f32 = reinterpret_cast<const float *>(first_element(c));
+    }
+    check_abi(mi355_gemmlowp_run(s.handle, first_element(a), bias_f32, first_element(dst), nullptr), "CpuGEMMLowp::run");
+}
+} // namespace op
+} // namespace experimental
 } // namespace arm_compute

@@ -5,6 +5,7 @@
 //   test_host_api --gpu   : configure / prepare / run on the device, host buffers and imported device buffers
 #include "arm_compute/core/utils/quantization/AsymmHelpers.h"
 #include "arm_compute/runtime/NEON/NEFunctions.h"
+#include "arm_compute/runtime/experimental/operators/CpuGEMMLowp.h"
 #include "arm_compute/runtime/Tensor.h"
 #include "gemmlowp_oracle.h"
 
@@ -773,6 +774,59 @@ static void test_gemm_conv2d()
     std::printf("       kernel: %s\n", conv.kernel_name());
 }
 
+// experimental::op::CpuGEMMLowp: configured on infos, run on an ITensorPack, re-quantised without re-packing B
+static void test_stateless_operator()
+{
+    SECTION("experimental::op::CpuGEMMLowp on an ITensorPack, update_quantization_parameters with negated offsets");
+    const int M = 45, N = 70, K = 160;
+    const QuantizationInfo aq(0.02f, 7), bq(0.004f, -3), oq(0.05f, 11);
+    TensorInfo ai(TensorShape(K, M), 1, DataType::QASYMM8_SIGNED, aq), bi(TensorShape(N, K), 1, DataType::QASYMM8_SIGNED, bq);
+    TensorInfo ci(TensorShape(N), 1, DataType::S32), oi(TensorShape(N, M), 1, DataType::QASYMM8_SIGNED, oq);
+    GEMMLowpOutputStageInfo st;
+    st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT, st.output_data_type = DataType::QASYMM8_SIGNED;
+    st.gemmlowp_offset = 11, st.gemmlowp_min_bound = -128, st.gemmlowp_max_bound = 127;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(aq, bq, oq, st)));
+    const GEMMInfo gi(false, false, true, 0, false, false, st);
+    EXPECT(bool(experimental::op::CpuGEMMLowp::validate(&ai, &bi, &ci, &oi, gi)));
+    experimental::op::CpuGEMMLowp op;
+    op.configure(&ai, &bi, &ci, &oi, gi);
+    EXPECT(op.workspace().empty());
+    Tensor a, b, c, dst;
+    a.allocator()->init(ai), b.allocator()->init(bi), c.allocator()->init(ci), dst.allocator()->init(oi);
+    a.allocator()->allocate(), b.allocator()->allocate(), c.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int8_t>(a, -128, 127, 101), fill_uniform<int8_t>(b, -128, 127, 102), fill_uniform<int32_t>(c, -3000, 3000, 103);
+    ITensorPack pack{{ACL_SRC_0, &a}, {ACL_SRC_1, &b}, {ACL_SRC_2, &c}, {ACL_DST, &dst}};
+    EXPECT(pack.size() == 4 && pack.get_const_tensor(ACL_SRC_1) == &b && pack.get_tensor(ACL_DST) == &dst);
+    op.run(pack);
+    const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+    const auto Cb = dense_copy<int32_t>(c);
+    std::vector<int8_t> want(M * N);
+    orc_gemmlowp_fixedpoint(A.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 7, -3, &st.gemmlowp_multiplier,
+                            &st.gemmlowp_shift, 1, 11, -128, 127);
+    EXPECT(dense_copy<int8_t>(dst) == want);
+    EXPECT(!b.is_used());
+    // a different pack (other activations, other destination), same packed weights
+    Tensor a2, dst2;
+    a2.allocator()->init(ai), dst2.allocator()->init(oi);
+    a2.allocator()->allocate(), dst2.allocator()->allocate();
+    fill_uniform<int8_t>(a2, -128, 127, 104);
+    ITensorPack pack2{{ACL_SRC_0, &a2}, {ACL_SRC_1, &b}, {ACL_SRC_2, &c}, {ACL_DST, &dst2}};
+    op.run(pack2);
+    const auto A2 = dense_copy<int8_t>(a2);
+    orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 7, -3, &st.gemmlowp_multiplier,
+                            &st.gemmlowp_shift, 1, 11, -128, 127);
+    EXPECT(dense_copy<int8_t>(dst2) == want);
+    // new quantization, offsets negated as a convolution / fully connected caller would ask
+    const QuantizationInfo aq2(0.03f, -4), bq2(0.006f, 2), oq2(0.08f, -6);
+    op.update_quantization_parameters(aq2, bq2, oq2, DataType::QASYMM8_SIGNED, true, true);
+    op.run(pack2);
+    GEMMLowpOutputStageInfo st2;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(aq2, bq2, oq2, st2)));
+    orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 4, -2, &st2.gemmlowp_multiplier,
+                            &st2.gemmlowp_shift, 1, -6, -128, 127);
+    EXPECT(dense_copy<int8_t>(dst2) == want);
+}
+
 static void test_error_paths()
 {
     SECTION("configure() throws on invalid input; run() before configure() throws");
@@ -832,6 +886,7 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, true, 32,
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
             test_gemm_conv2d();
+            test_stateless_operator();
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);

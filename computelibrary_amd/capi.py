@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355gemmlowp.so")
 U8, S8, S32, F32 = 0, 1, 2, 3
 EPI_S32, EPI_FIXEDPOINT, EPI_F32 = 0, 1, 2
 PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
+GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
 
 EXPORTS = [
     "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_run",
@@ -34,7 +35,7 @@ class GemmDesc(C.Structure):
                 ("a_offset", C.c_int32), ("b_offset", C.c_int32), ("requant", Requant),
                 ("scale", C.c_float), ("act_min", C.c_float), ("act_max", C.c_float),
                 ("path", C.c_int32), ("b_transposed", C.c_int32), ("b_k_interleave", C.c_int32),
-                ("reserved", C.c_int32)]
+                ("flags", C.c_int32)]
 
 
 class OutputStageDesc(C.Structure):
@@ -134,12 +135,12 @@ class Gemm:
 
     def __init__(self, M, N, K, a_dtype, b_dtype, dst_dtype, epilogue, a_offset=0, b_offset=0, rq=None, scale=1.0,
                  act_min=-np.inf, act_max=np.inf, batch=1, b_batched=False, lda=None, ldb=None, ldd=None,
-                 path=PATH_AUTO, b_transposed=False, b_k_interleave=0):
+                 path=PATH_AUTO, b_transposed=False, b_k_interleave=0, flags=0):
         lda, ldb, ldd = lda or K, ldb or (K if b_transposed else N), ldd or N
         b_rows = N if b_transposed else K
         self.desc = GemmDesc(M, N, K, batch, a_dtype, b_dtype, dst_dtype, epilogue, lda, ldb, ldd, M * lda,
                              b_rows * ldb if b_batched else 0, M * ldd, a_offset, b_offset, rq or requant(), scale,
-                             act_min, act_max, path, 1 if b_transposed else 0, b_k_interleave, 0)
+                             act_min, act_max, path, 1 if b_transposed else 0, b_k_interleave, flags)
         self._h = C.c_void_p()
         _check(lib().mi355_gemmlowp_create(C.byref(self.desc), C.byref(self._h)))
 

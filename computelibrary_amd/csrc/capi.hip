@@ -138,6 +138,7 @@ struct GemmCore
     int32_t a_offset = 0, b_offset = 0; // as given (added convention)
     mi355_requant rq{};
     float   scale = 1.f, act_min = -INFINITY, act_max = INFINITY;
+    bool    accumulate = false, act_twice = false;
     int     path = MI355_PATH_AUTO, cfg_idx = 0, dma_idx = -1;
     int     Kp = 0, Np = 0;
     bool    b_shared = true; // one B for all batches
@@ -295,6 +296,8 @@ struct GemmCore
         p.act_max             = act_max;
         p.has_offsets         = (a_offset != 0 || b_offset != 0) ? 1 : 0;
         p.dst_signed          = dst_dtype == MI355_S8;
+        p.accumulate          = accumulate ? 1 : 0;
+        p.act_twice           = act_twice ? 1 : 0;
     }
 
     // A, D and bias_f32 are device pointers here
@@ -483,6 +486,10 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
         default:
             return fail("unknown epilogue %d", d.epilogue);
     }
+    if ((d.flags & ~(MI355_GEMM_ACCUMULATE | MI355_GEMM_ACT_TWICE)) != 0)
+        return fail("unknown flag bits 0x%x", d.flags);
+    if ((d.flags & MI355_GEMM_ACCUMULATE) && d.epilogue == MI355_EPI_FIXEDPOINT)
+        return fail("accumulation is only possible into an S32 or F32 destination");
     if (d.batch > 1 && (d.a_batch_stride < (int64_t)(d.M - 1) * d.lda + d.K || d.d_batch_stride < (int64_t)(d.M - 1) * d.ldd + d.N))
         return fail("batch stride smaller than one matrix");
     if (d.batch > 1 && d.b_batch_stride != 0 &&
@@ -499,6 +506,7 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
     c.a_offset = d.a_offset, c.b_offset = d.b_offset;
     c.rq = d.requant, c.scale = d.scale, c.act_min = d.act_min, c.act_max = d.act_max;
     c.path     = d.path;
+    c.accumulate = (d.flags & MI355_GEMM_ACCUMULATE) != 0, c.act_twice = (d.flags & MI355_GEMM_ACT_TWICE) != 0;
     c.b_shared = d.batch == 1 || d.b_batch_stride == 0;
     if (c.choose_kernel())
     {
@@ -590,8 +598,8 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     {
         TRY(h->stageD.ensure(d_elems * esz));
         Dd = h->stageD.p;
-        if (d.ldd != d.N || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
-            HIP_TRY(hipMemcpyAsync(Dd, D, d_elems * esz, hipMemcpyHostToDevice, s)); // keep the caller's padding
+        if (c.accumulate || d.ldd != d.N || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
+            HIP_TRY(hipMemcpyAsync(Dd, D, d_elems * esz, hipMemcpyHostToDevice, s)); // previous values / padding
     }
     TRY(c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, Dd, d.ldd, d.d_batch_stride, (const float *)bfd, s));
     if (d_host)

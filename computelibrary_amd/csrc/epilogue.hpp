@@ -41,6 +41,8 @@ struct EpiParams
     const int32_t *qp;
     int64_t        qp_stride;
     int32_t        qp_std; // every column: multiplier >= 2^30, shift in [2, 31]; |result_offset| < 2^28 (see std_requant)
+    int32_t        accumulate; // EPI_S32 / EPI_F32: add the destination's previous contents (GEMMInfo::accumulate)
+    int32_t        act_twice;  // EPI_F32: the activation clamp is also applied before the offset term is added
 };
 
 // Per-column constants of the branch-free requantisation used by the pipelined kernel's epilogue, valid for
@@ -130,17 +132,24 @@ __device__ __forceinline__ int32_t epi_fixedpoint(int32_t acc, int32_t colv, int
     return clamp_i32(requant_fixedpoint(v, mult, shift, p.result_offset), p.lo, p.hi);
 }
 
-// float(acc)*scale (+bias) then + float(offset terms)*scale, two separate roundings and no fused multiply-add, in the
-// order of src/core/NEON/kernels/arm_gemm/quantized.cpp:1000-1012 followed by
-// src/cpu/kernels/gemmlowp/generic/neon/fp32.cpp:31-54
-__device__ __forceinline__ float epi_f32(int32_t acc, int32_t off, float bias, bool has_bias, const EpiParams &p)
+// float(acc)*scale (+bias) (+ previous destination value) then + float(offset terms)*scale, separate roundings and no
+// fused multiply-add, in the order of src/core/NEON/kernels/arm_gemm/quantized.cpp:1000-1017 followed by
+// src/cpu/kernels/gemmlowp/generic/neon/fp32.cpp:31-54. The reference clamps twice when an activation the assembly
+// GEMM understands is set: inside the dequantising merge (quantized.cpp:1015, before the offset term exists) and again
+// as the post-op (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:326-332); act_twice reproduces the first one.
+__device__ __forceinline__ float epi_f32(int32_t acc, int32_t off, float bias, bool has_bias, const EpiParams &p,
+                                         float prev = 0.f)
 {
 #pragma clang fp contract(off) // the multiply and the add must round separately, as the two NEON instructions do
     float r = (float)acc * p.scale;
     if (has_bias)
         r = r + bias;
+    if (p.accumulate)
+        r = r + prev;
     if (p.has_offsets)
     {
+        if (p.act_twice)
+            r = fminf(fmaxf(r, p.act_min), p.act_max);
         const float scaled = (float)off * p.scale;
         r                  = r + scaled;
     }

@@ -399,7 +399,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
                 epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
         }
     }
-    else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store)
+    else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store && !g.epi.accumulate)
     {
         // the ring is free beyond the last barrier: 32 x (FN*128 + 16) bytes per wave
         if constexpr (EPI != EPI_FIXEDPOINT)

@@ -149,12 +149,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
                 const int32_t rv  = p.rowvec ? p.rowvec[i] : 0;
                 const int64_t idx = (int64_t)i * g.ldd + j;
                 if (EPI == EPI_S32)
-                    ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc[n][r] + (uint32_t)cv[n] + (uint32_t)rv);
+                    ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc[n][r] + (uint32_t)cv[n] + (uint32_t)rv +
+                                                      (p.accumulate ? (uint32_t)((int32_t *)g.D)[idx] : 0u));
                 else if (EPI == EPI_FIXEDPOINT)
                     ((int8_t *)g.D)[idx] = (int8_t)epi_fixedpoint(acc[n][r], cv[n], rv, mu[n], sh[n], p);
                 else
                     ((float *)g.D)[idx] = epi_f32(acc[n][r], (int32_t)((uint32_t)cv[n] + (uint32_t)rv), bf[n],
-                                                  p.bias_f32 != nullptr, p);
+                                                  p.bias_f32 != nullptr, p, p.accumulate ? ((float *)g.D)[idx] : 0.f);
             }
         }
     }

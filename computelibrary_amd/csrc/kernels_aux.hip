@@ -450,13 +450,14 @@ __global__ __launch_bounds__(256) void simple_gemm_kernel(GemmArgs g, uint8_t fl
     const int32_t    rv  = p.rowvec ? p.rowvec[(int64_t)bz * p.rowvec_batch_stride + i] : 0;
     const int64_t    idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j;
     if (EPI == EPI_S32)
-        ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc + (uint32_t)cv + (uint32_t)rv);
+        ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc + (uint32_t)cv + (uint32_t)rv +
+                                          (p.accumulate ? (uint32_t)((int32_t *)g.D)[idx] : 0u));
     else if (EPI == EPI_FIXEDPOINT)
         ((int8_t *)g.D)[idx] =
             (int8_t)epi_fixedpoint(acc, cv, rv, p.mult ? p.mult[j] : p.mult_s, p.shift ? p.shift[j] : p.shift_s, p);
     else
         ((float *)g.D)[idx] = epi_f32(acc, (int32_t)((uint32_t)cv + (uint32_t)rv), p.bias_f32 ? p.bias_f32[j] : 0.f,
-                                      p.bias_f32 != nullptr, p);
+                                      p.bias_f32 != nullptr, p, p.accumulate ? ((float *)g.D)[idx] : 0.f);
 }
 
 int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s)

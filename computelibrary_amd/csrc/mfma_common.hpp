@@ -98,12 +98,13 @@ __device__ __forceinline__ void epilogue_store(const v16i (&acc)[FM][FN], const 
                     const int32_t a   = acc[fm][fn][r];
                     const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j;
                     if (EPI == EPI_S32)
-                        ((int32_t *)D)[idx] = (int32_t)((uint32_t)a + (uint32_t)cv + (uint32_t)rv);
+                        ((int32_t *)D)[idx] = (int32_t)((uint32_t)a + (uint32_t)cv + (uint32_t)rv +
+                                                        (p.accumulate ? (uint32_t)((int32_t *)D)[idx] : 0u));
                     else if (EPI == EPI_FIXEDPOINT)
                         ((int8_t *)D)[idx] = (int8_t)epi_fixedpoint(a, cv, rv, mu, sh, p);
                     else
-                        ((float *)D)[idx] =
-                            epi_f32(a, (int32_t)((uint32_t)cv + (uint32_t)rv), bf, p.bias_f32 != nullptr, p);
+                        ((float *)D)[idx] = epi_f32(a, (int32_t)((uint32_t)cv + (uint32_t)rv), bf, p.bias_f32 != nullptr,
+                                                    p, p.accumulate ? ((float *)D)[idx] : 0.f);
                 }
             }
         }
@@ -178,10 +179,23 @@ __device__ __forceinline__ void epilogue_store_t(const v16i (&acc)[FM][FN], cons
                 }
                 else if (EPI == EPI_S32)
                 {
-                    v4i o;
+                    v4i o, prev = {0, 0, 0, 0};
+                    if (p.accumulate)
+                    {
+                        if (vec)
+                            prev = *(const v4i *)((int32_t *)D + idx);
+                        else
+                        {
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                if (j0 + t < g.N)
+                                    prev[t] = ((int32_t *)D)[idx + t];
+                        }
+                    }
 #pragma unroll
                     for (int t = 0; t < 4; ++t)
-                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
+                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm] +
+                                         (uint32_t)prev[t]);
                     if (vec)
                         *(v4i *)((int32_t *)D + idx) = o;
                     else
@@ -195,11 +209,23 @@ __device__ __forceinline__ void epilogue_store_t(const v16i (&acc)[FM][FN], cons
                 else
                 {
                     typedef float v4f __attribute__((ext_vector_type(4)));
-                    v4f o;
+                    v4f o, prev = {0.f, 0.f, 0.f, 0.f};
+                    if (p.accumulate)
+                    {
+                        if (vec)
+                            prev = *(const v4f *)((float *)D + idx);
+                        else
+                        {
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                if (j0 + t < g.N)
+                                    prev[t] = ((float *)D)[idx + t];
+                        }
+                    }
 #pragma unroll
                     for (int t = 0; t < 4; ++t)
                         o[t] = epi_f32(acc[fm][fn][4 * q + t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv[fm]), bf[t],
-                                       p.bias_f32 != nullptr, p);
+                                       p.bias_f32 != nullptr, p, prev[t]);
                     if (vec)
                         *(v4f *)((float *)D + idx) = o;
                     else

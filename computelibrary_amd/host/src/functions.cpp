@@ -102,15 +102,16 @@ void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorI
     d = mi355_gemm_desc{};
     d.K                = static_cast<int32_t>(ai->dimension(0));
     d.N                = static_cast<int32_t>(bi->dimension(0));
-    d.M                = static_cast<int32_t>(ai->dimension(1));
-    d.batch            = static_cast<int32_t>(ai->tensor_shape().total_size_upper(2));
+    const bool a3d     = gemm_info.reinterpret_input_as_3d(); // [K, W, H, batch]: M = W * H
+    d.M                = static_cast<int32_t>(a3d ? ai->dimension(1) * ai->dimension(2) : ai->dimension(1));
+    d.batch            = static_cast<int32_t>(ai->tensor_shape().total_size_upper(a3d ? 3 : 2));
     d.a_dtype          = to_mi355(ai->data_type());
     d.b_dtype          = to_mi355(bi->data_type());
     d.dst_dtype        = to_mi355(oi->data_type());
     d.lda              = ai->strides_in_bytes()[1];
     d.ldb              = bi->strides_in_bytes()[1];
     d.ldd              = oi->strides_in_bytes()[1] / oi->element_size();
-    d.a_batch_stride   = ai->strides_in_bytes()[2];
+    d.a_batch_stride   = ai->strides_in_bytes()[a3d ? 3 : 2];
     d.b_batch_stride   = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
     if (gemm_info.depth_output_gemm3d() != 0)
         d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
@@ -122,6 +123,7 @@ void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorI
     d.act_max  = std::numeric_limits<float>::infinity();
     d.scale    = 1.f;
     d.path     = MI355_PATH_AUTO;
+    d.flags    = gemm_info.accumulate() ? MI355_GEMM_ACCUMULATE : 0;
     if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT || stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN)
     {
         d.epilogue = MI355_EPI_FIXEDPOINT;
@@ -153,6 +155,11 @@ void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorI
                 default:
                     ARM_COMPUTE_ERROR("Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
             }
+            // the reference's assembly GEMM takes these three when the lower bound is 0 and clamps inside its merge
+            // step, before the offset term is added; the CpuActivation post-op then clamps again
+            // (src/core/utils/AssemblyUtils.cpp:32-62, src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:326-332)
+            if (act.b() == 0.f)
+                d.flags |= MI355_GEMM_ACT_TWICE;
         }
     }
     else
@@ -228,16 +235,26 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
     {
         ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.type != GEMMLowpOutputStageType::NONE,
                                         "Accumulation is not supported for output QASYMM8/QASYMM8_SIGNED");
-        ARM_COMPUTE_RETURN_ERROR_MSG("Accumulation into the destination is not built in this library");
     }
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.reinterpret_input_as_3d(),
-                                    "reinterpret_input_as_3d is not built in this library");
+    // [K, W, H, batch] read as W*H rows per batch: the rows of consecutive planes must be evenly spaced
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.reinterpret_input_as_3d() &&
+                                        a->strides_in_bytes()[2] != a->dimension(1) * a->strides_in_bytes()[1],
+                                    "reinterpret_input_as_3d needs planes without padding between them");
 
     // shapes
     ARM_COMPUTE_RETURN_ERROR_ON(b->dimension(0) != output->dimension(0));
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.reinterpret_input_as_3d() && gemm_info.depth_output_gemm3d() == 0,
+                                    "reinterpret_input_as_3d is only built together with a 3D output");
     if (gemm_info.depth_output_gemm3d() != 0)
     {
-        ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1) * output->dimension(2));
+        if (gemm_info.reinterpret_input_as_3d())
+        {
+            ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1));
+            ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(2) != output->dimension(2));
+            ARM_COMPUTE_RETURN_ERROR_ON(a->tensor_shape().total_size_upper(3) != output->tensor_shape().total_size_upper(3));
+        }
+        else
+            ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1) * output->dimension(2));
         ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->strides_in_bytes()[2] !=
                                             output->dimension(1) * output->strides_in_bytes()[1],
                                         "GEMM3D output planes must be contiguous (no y padding)");
@@ -247,10 +264,11 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
         ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1));
         ARM_COMPUTE_RETURN_ERROR_ON(a->tensor_shape().total_size_upper(2) != output->tensor_shape().total_size_upper(2));
     }
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(b->num_dimensions() > 2 &&
-                                        b->tensor_shape().total_size_upper(2) != a->tensor_shape().total_size_upper(2),
+    const size_t a_batch_dim = gemm_info.reinterpret_input_as_3d() ? 3 : 2;
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(b->num_dimensions() > 2 && b->tensor_shape().total_size_upper(2) !=
+                                                                   a->tensor_shape().total_size_upper(a_batch_dim),
                                     "Batched B must have as many matrices as A");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(a->num_dimensions() > 3 || b->num_dimensions() > 3,
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(a->num_dimensions() > a_batch_dim + 1 || b->num_dimensions() > 3,
                                     "More than one batch dimension is not supported");
     ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(a, "a"));
     ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(b, "b"));

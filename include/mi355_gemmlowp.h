@@ -92,6 +92,21 @@ typedef struct mi355_requant
     int32_t stage; /* mi355_stage: which of the two integer output stages of GEMMLowpOutputStageType */
 } mi355_requant;
 
+/* mi355_gemm_desc::flags */
+enum mi355_gemm_flags
+{
+    /* S32 / F32 destinations only: the result is added to what the destination holds (GEMMInfo::accumulate,
+     * src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:393-401; int32 adds wrap as they do in the GEMM's own
+     * accumulators, the float add sits between the bias and the offset term, src/core/NEON/kernels/arm_gemm/
+     * quantized.cpp:1007-1014). */
+    MI355_GEMM_ACCUMULATE = 1,
+    /* F32 destination: the activation clamp [act_min, act_max] is applied to float(acc)*scale (+bias) (+previous)
+     * AND again after the offset term, as the reference does when the activation is one its assembly GEMM fuses
+     * (quantized.cpp:1015 inside the merge, then the CpuActivation post-op,
+     * src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:326-332). Without the bit: once, at the end. */
+    MI355_GEMM_ACT_TWICE = 2
+};
+
 typedef struct mi355_gemm_desc
 {
     int32_t       M, N, K, batch;
@@ -112,7 +127,7 @@ typedef struct mi355_gemm_desc
                                        over. Replaces CpuConvertFullyConnectedWeights
                                        (src/cpu/kernels/CpuConvertFullyConnectedWeightsKernel.cpp:60-66,118-121; f is its
                                        _factor2). 0 or 1: none. Must divide K. */
-    int32_t       reserved;
+    int32_t       flags;            /* MI355_GEMM_* bits (enum mi355_gemm_flags) */
 } mi355_gemm_desc;
 
 typedef struct mi355_gemm_handle mi355_gemm_handle;

@@ -158,16 +158,18 @@ def gemmlowp_scale(A, B, bias, a_offset, b_offset, mult, shift, result_offset, m
     return out
 
 
-def gemmlowp_f32(A, B, bias, a_offset, b_offset, scale, act_min=-np.inf, act_max=np.inf):
+def gemmlowp_f32(A, B, bias, a_offset, b_offset, scale, act_min=-np.inf, act_max=np.inf, prev=None, act_twice=False):
+    """prev: previous destination values to accumulate into (GEMMInfo::accumulate), or None"""
     A = np.ascontiguousarray(A)
     B = np.ascontiguousarray(B)
     M, K = A.shape
     _, N = B.shape
     bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
-    out = np.empty((M, N), dtype=np.float32)
+    out = np.empty((M, N), dtype=np.float32) if prev is None else np.array(prev, dtype=np.float32, order="C")
+    assert out.shape == (M, N)
     lib.orc_gemmlowp_f32(_p(A), _signed(A), C.c_int64(K), _p(B), _signed(B), C.c_int64(N), _p(bias), _p(out),
                          C.c_int64(N), M, N, K, C.c_int32(a_offset), C.c_int32(b_offset), C.c_float(scale),
-                         C.c_float(act_min), C.c_float(act_max))
+                         C.c_float(act_min), C.c_float(act_max), 1 if prev is not None else 0, 1 if act_twice else 0)
     return out
 
 

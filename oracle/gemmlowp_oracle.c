@@ -257,14 +257,16 @@ void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const voi
     free(t);
 }
 
-/* src/core/NEON/kernels/arm_gemm/quantized.cpp:977-1030 (float(acc)*scale + bias, clamp) followed by
- * src/cpu/kernels/gemmlowp/generic/neon/impl.h:95-155 + fp32.cpp:31-54 (+= float(offset terms)*scale).
- * The activation clamp of the first step is only active when the operator fuses it; the function
- * object runs it as a post-op after the offsets (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:326-332,806-810),
- * which is what act_min/act_max model here. */
+/* src/core/NEON/kernels/arm_gemm/quantized.cpp:977-1030 (float(acc)*scale, + bias, + previous destination value when
+ * accumulating, clamp) followed by src/cpu/kernels/gemmlowp/generic/neon/impl.h:95-155 + fp32.cpp:31-54
+ * (+= float(offset terms)*scale) and the CpuActivation post-op
+ * (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:326-332,806-810). The first clamp only exists for the
+ * activations the assembly GEMM takes (src/core/utils/AssemblyUtils.cpp:32-62: RELU, BOUNDED_RELU and LU_BOUNDED_RELU
+ * with lower bound 0): act_twice says whether it does. It only matters when an offset term follows it.
+ * accumulate: dst holds the previous values on entry (GEMMInfo::accumulate). */
 void orc_gemmlowp_f32(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
                       const float *bias, float *dst, int64_t ldd, int M, int N, int K, int32_t a_offset,
-                      int32_t b_offset, float scale, float act_min, float act_max)
+                      int32_t b_offset, float scale, float act_min, float act_max, int accumulate, int act_twice)
 {
     int32_t *acc    = (int32_t *)malloc(sizeof(int32_t) * (size_t)(M > 0 ? M : 1) * (size_t)(N > 0 ? N : 1));
     int32_t *rowsum = (int32_t *)malloc(sizeof(int32_t) * (size_t)(M > 0 ? M : 1));
@@ -276,8 +278,17 @@ void orc_gemmlowp_f32(const void *A, int a_signed, int64_t lda, const void *B, i
             volatile float r = (float)acc[(int64_t)i * N + j] * scale; /* volatile: forbid FMA contraction */
             if (bias)
                 r = r + bias[j];
+            if (accumulate)
+                r = r + dst[(int64_t)i * ldd + j];
             if (a_offset != 0 || b_offset != 0)
             {
+                if (act_twice)
+                {
+                    if (r < act_min)
+                        r = act_min;
+                    if (r > act_max)
+                        r = act_max;
+                }
                 /* each term is only formed when its offset is non-zero, exactly like the four branches of
                  * neon_run_offset_contribution_float; the integer sum is identical either way */
                 const int32_t  off    = offset_term(a_offset, b_offset, K, colsum[j], rowsum[i]);

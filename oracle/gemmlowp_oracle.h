@@ -22,6 +22,8 @@
  * exists to confirm that no fused multiply-add is emitted there, so with non-zero offsets the
  * last-bit behaviour of that one function is "parity unpinned" (the reference's own test
  * oracle, one rounding, is also exported by oracle/_ref and both agree to 1e-6 relative).
+ * Its act_twice clamp (an activation together with non-zero offsets on the F32 path) follows the
+ * source order too; none of the reference's tests runs that combination: "parity unpinned".
  */
 #ifndef ORACLE_GEMMLOWP_ORACLE_H
 #define ORACLE_GEMMLOWP_ORACLE_H
@@ -69,10 +71,11 @@ void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const voi
                              int32_t a_offset, int32_t b_offset, const int32_t *mult, const int32_t *shift,
                              int n_qparams, int32_t result_offset, int32_t min_bound, int32_t max_bound);
 
-/* GEMM with F32 dequantised output: float(acc)*scale (+bias) then + float(offset terms)*scale, then clamp */
+/* GEMM with F32 dequantised output: float(acc)*scale (+bias) (+ previous dst when accumulate) (clamp when act_twice)
+ * then + float(offset terms)*scale, then clamp */
 void orc_gemmlowp_f32(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
                       const float *bias, float *dst, int64_t ldd, int M, int N, int K, int32_t a_offset,
-                      int32_t b_offset, float scale, float act_min, float act_max);
+                      int32_t b_offset, float scale, float act_min, float act_max, int accumulate, int act_twice);
 
 /* ---- convolution lowering ------------------------------------------------------------------ */
 /* NHWC src [batch][H][W][C] -> patch matrix [batch*OH*OW][KH*KW*C], K ordered (ky, kx, c) */

@@ -169,6 +169,13 @@ static void test_validate_tables()
     GEMMInfo acc;
     acc.set_accumulate(true);
     EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o8, acc)));
+    // the reference's accumulation validate test (tests/validation/NEON/GEMMLowp.cpp:135-163): S32 yes, quantized no
+    EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o32, acc)));
+    GEMMInfo acc_fused(false, false, true, 0, false, false, st);
+    acc_fused.set_accumulate(true);
+    st.gemmlowp_min_bound = 0, st.gemmlowp_max_bound = 255;
+    acc_fused.set_gemmlowp_output_stage(st);
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o8, acc_fused)));
     EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(nullptr, &b, nullptr, &o32)));
 
     SECTION("NEGEMMLowpOutputStage::validate");
@@ -387,6 +394,82 @@ static void test_gemmlowp_s32_batched()
     }
 }
 
+// GEMMInfo::accumulate (the fixture of tests/validation/fixtures/GEMMLowpFixture.h:187-193,469-483: the destination is
+// filled first and the product is added to it) and a [K, W, H, batch] input read as W*H rows with a 3D output
+static void test_gemmlowp_accumulate_and_3d()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore accumulate into S32 / F32; reinterpret_input_as_3d + depth_output_gemm3d");
+    const int M = 23, N = 37, K = 40;
+    {
+        Tensor a, b, dst;
+        init_tensor(a, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(1.f / 255, 3));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8, QuantizationInfo(1.f / 255, -9));
+        init_tensor(dst, TensorShape(N, M), DataType::S32);
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<uint8_t>(a, 0, 255, 1), fill_uniform<uint8_t>(b, 0, 255, 2);
+        fill_uniform<int32_t>(dst, -100000, 100000, 3);
+        const auto prev = dense_copy<int32_t>(dst);
+        GEMMInfo   info;
+        info.set_accumulate(true);
+        EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), nullptr, dst.info(), info)));
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, info);
+        gemm.run();
+        const auto A = dense_copy<uint8_t>(a), B = dense_copy<uint8_t>(b);
+        std::vector<int32_t> want(M * N);
+        orc_gemmlowp_s32(A.data(), 0, K, B.data(), 0, N, want.data(), N, M, N, K, 3, -9);
+        for (int i = 0; i < M * N; ++i)
+            want[i] += prev[i];
+        EXPECT(dense_copy<int32_t>(dst) == want);
+    }
+    {
+        Tensor a, b, dst;
+        init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(0.02f, 0));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(0.005f, 0));
+        init_tensor(dst, TensorShape(N, M), DataType::F32);
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(a, -128, 127, 4), fill_uniform<int8_t>(b, -128, 127, 5);
+        std::mt19937                    rng(6);
+        std::normal_distribution<float> nd(0.f, 2.f);
+        for (int i = 0; i < M * N; ++i)
+            reinterpret_cast<float *>(dst.buffer())[i] = nd(rng);
+        auto     want = dense_copy<float>(dst);
+        GEMMInfo info(false, false, true);
+        info.set_accumulate(true);
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, info);
+        gemm.run();
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        orc_gemmlowp_f32(A.data(), 1, K, B.data(), 1, N, nullptr, want.data(), N, M, N, K, 0, 0, 0.02f * 0.005f, -INFINITY,
+                         INFINITY, 1, 0);
+        EXPECT(dense_copy<float>(dst) == want);
+    }
+    {
+        // a = [K, W, H, batch] -> M = W*H rows per batch; dst = [N, W, H, batch]
+        const int W = 5, H = 4, batch = 2;
+        Tensor    a, b, dst;
+        init_tensor(a, TensorShape(K, W, H, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.1f, 2));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(0.2f, -1));
+        init_tensor(dst, TensorShape(N, W, H, batch), DataType::S32);
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(a, -128, 127, 7), fill_uniform<int8_t>(b, -128, 127, 8);
+        GEMMInfo info(false, false, true, H /* depth_output_gemm3d */, true /* reinterpret_input_as_3d */);
+        EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), nullptr, dst.info(), info)));
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, info);
+        gemm.run();
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        std::vector<int32_t> want(batch * W * H * N);
+        orc_gemmlowp_s32(A.data(), 1, K, B.data(), 1, N, want.data(), N, batch * W * H, N, K, 2, -1);
+        EXPECT(dense_copy<int32_t>(dst) == want);
+        // a 3D input without a 3D output is not built
+        Tensor flat;
+        init_tensor(flat, TensorShape(N, W * H, batch), DataType::S32);
+        EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), nullptr, flat.info(),
+                                                            GEMMInfo(false, false, true, 0, true))));
+    }
+}
+
 static void test_gemmlowp_per_channel_and_update()
 {
     SECTION("NEGEMMLowpMatrixMultiplyCore per-channel QSYMM8_PER_CHANNEL rhs");
@@ -470,7 +553,7 @@ static void test_gemmlowp_f32()
     const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
     std::vector<float> want(M * N);
     orc_gemmlowp_f32(A.data(), 1, K, B.data(), 1, N, reinterpret_cast<const float *>(bias.buffer()), want.data(), N, M, N, K, 3,
-                     -2, 0.02f * 0.005f, 0.f, INFINITY);
+                     -2, 0.02f * 0.005f, 0.f, INFINITY, 0, 1);
     const auto got = dense_copy<float>(dst);
     bool       ok  = true;
     for (size_t i = 0; i < want.size(); ++i)
@@ -876,6 +959,7 @@ int main(int argc, char **argv)
             test_gemmlowp_fused_u8(false);
             test_gemmlowp_fused_u8(true);
             test_gemmlowp_s32_batched();
+            test_gemmlowp_accumulate_and_3d();
             test_gemmlowp_per_channel_and_update();
             test_gemmlowp_f32();
             test_output_stage();

@@ -25,8 +25,9 @@ def announce(*what):
 
 def run_gemm(A, B, epilogue, dst_dtype, a_offset=0, b_offset=0, bias=None, mult=None, shift=None, result_offset=0,
              lo=-(1 << 31), hi=(1 << 31) - 1, scale=1.0, bias_f32=None, act=(-np.inf, np.inf), path=capi.PATH_AUTO,
-             device=False, lda=None, ldd=None, stage=0):
-    """A [M][K] or [batch][M][K]; B [K][N] or [batch][K][N]. Returns (numpy result, kernel name)."""
+             device=False, lda=None, ldd=None, stage=0, prev=None, flags=0):
+    """A [M][K] or [batch][M][K]; B [K][N] or [batch][K][N]. prev: what the destination holds before the call (for
+    GEMM_ACCUMULATE). Returns (numpy result, kernel name)."""
     A3 = A if A.ndim == 3 else A[None]
     batch, M, K = A3.shape
     N = B.shape[-1]
@@ -39,11 +40,13 @@ def run_gemm(A, B, epilogue, dst_dtype, a_offset=0, b_offset=0, bias=None, mult=
     lda = lda or K
     ldd = ldd or N
     g = capi.Gemm(M, N, K, CODE[A.dtype], CODE[B.dtype], dcode, epilogue, a_offset, b_offset, rq, scale, act[0],
-                  act[1], batch=batch, b_batched=(B.ndim == 3), lda=lda, ldd=ldd, path=path)
+                  act[1], batch=batch, b_batched=(B.ndim == 3), lda=lda, ldd=ldd, path=path, flags=flags)
     name = g.kernel_name
     Ah = np.zeros((batch, M, lda), dtype=A.dtype)
     Ah[:, :, :K] = A3
     Dh = np.full((batch, M, ldd), 77, dtype=dst_dtype)
+    if prev is not None:
+        Dh[:, :, :N] = prev if prev.ndim == 3 else prev[None]
     mult_a = None if not per_channel else np.ascontiguousarray(mult, dtype=np.int32)
     shift_a = None if not per_channel else np.ascontiguousarray(shift, dtype=np.int32)
     bias_a = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)

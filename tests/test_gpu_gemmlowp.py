@@ -236,6 +236,61 @@ def test_b_handed_over_transposed_and_with_reordered_k(M, k_interleave):
         np.testing.assert_array_equal(Dd.cpu().numpy(), want)
         g.close()
 
+@pytest.mark.parametrize("device", [False, True])
+@pytest.mark.parametrize("M,N,K,ldd,path", [(200, 136, 192, None, capi.PATH_MFMA), (70, 61, 100, 67, capi.PATH_MFMA),
+                                            (8, 136, 192, None, capi.PATH_SKINNY), (9, 20, 33, None, capi.PATH_SIMPLE),
+                                            (96, 130, 64, 131, capi.PATH_MFMA)])
+def test_accumulate_into_s32_and_f32(M, N, K, ldd, path, device):
+    """GEMMInfo::accumulate: dst += result. S32 adds wrap (the destination is the GEMM's own accumulator in the
+    reference, tests/validation/fixtures/GEMMLowpFixture.h:469-483 only uses values that cannot overflow); F32 adds the
+    previous value between the bias and the offset term (src/core/NEON/kernels/arm_gemm/quantized.cpp:1007-1014)."""
+    rng = np.random.default_rng(zlib.crc32(("acc %d %d %d" % (M, N, K)).encode()))
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    prev_i = rng.integers(-(1 << 31), (1 << 31) - 1, size=(M, N), dtype=np.int64).astype(np.int32)
+    announce("accumulate S32", M, N, K, ldd, path, device)
+    got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, 5, -3, path=path, device=device, ldd=ldd, prev=prev_i,
+                      flags=capi.GEMM_ACCUMULATE)
+    want = (oracle.gemmlowp_s32(A, B, 5, -3).astype(np.int64) + prev_i).astype(np.int32)  # wraps
+    assert np.array_equal(got, want)
+    prev_f = rng.normal(0.0, 3.0, size=(M, N)).astype(np.float32)
+    bias = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+    for offs, act, twice in [((0, 0), (-np.inf, np.inf), False), ((5, -3), (0.0, 6.0), True), ((5, -3), (0.0, np.inf), False)]:
+        announce("accumulate F32", M, N, K, ldd, path, device, offs, act, twice)
+        flags = capi.GEMM_ACCUMULATE | (capi.GEMM_ACT_TWICE if twice else 0)
+        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, offs[0], offs[1], scale=1e-3, bias_f32=bias, act=act, path=path,
+                          device=device, ldd=ldd, prev=prev_f, flags=flags)
+        want = oracle.gemmlowp_f32(A, B, bias, offs[0], offs[1], 1e-3, act[0], act[1], prev=prev_f, act_twice=twice)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))  # same float operations in the same order
+
+
+@pytest.mark.parametrize("M", [8, 150])
+def test_f32_activation_clamps_before_and_after_the_offset_term(M):
+    """With an activation its assembly GEMM fuses, the reference clamps float(acc)*scale+bias, adds the offset term and
+    clamps again (quantized.cpp:1015, then CpuGemmLowpMatrixMultiplyCore.cpp:326-332): GEMM_ACT_TWICE. The two differ
+    from a single clamp wherever the first clamp moved the value and the offset term moves it back inside."""
+    rng = np.random.default_rng(77 + M)
+    N, K = 96, 128
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    once = oracle.gemmlowp_f32(A, B, None, 40, 25, 1e-3, 0.0, 6.0)
+    twice = oracle.gemmlowp_f32(A, B, None, 40, 25, 1e-3, 0.0, 6.0, act_twice=True)
+    assert (once != twice).mean() > 0.05  # the case tells the two apart
+    announce("act twice", M)
+    got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, 40, 25, scale=1e-3, act=(0.0, 6.0), flags=capi.GEMM_ACT_TWICE)
+    assert np.array_equal(got.view(np.uint32), twice.view(np.uint32))
+    got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, 40, 25, scale=1e-3, act=(0.0, 6.0))
+    assert np.array_equal(got.view(np.uint32), once.view(np.uint32))
+
+
+def test_accumulate_is_rejected_with_an_output_stage():
+    with pytest.raises(capi.Mi355Error, match="accumulation"):
+        capi.Gemm(16, 16, 16, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, rq=capi.requant(1 << 30, 1, 0, -128, 127),
+                  flags=capi.GEMM_ACCUMULATE)
+    with pytest.raises(capi.Mi355Error, match="flag"):
+        capi.Gemm(16, 16, 16, capi.S8, capi.S8, capi.S32, capi.EPI_S32, flags=64)
+
+
 def test_requant_extremes_on_device():
     """Accumulators and multipliers at the edges of int32 (saturating SQDMULH, shift 0 / 31, wrap-around adds)
     through the stand-alone output stage."""

@@ -145,6 +145,31 @@ def test_f32_bias_and_activation():
     np.testing.assert_array_equal(got, want.astype(np.float32))
 
 
+def test_f32_accumulate_and_double_clamp_against_numpy_float32():
+    """numpy float32 arithmetic rounds every operation separately, like the NEON instructions of
+    src/core/NEON/kernels/arm_gemm/quantized.cpp:1000-1017 and src/cpu/kernels/gemmlowp/generic/neon/fp32.cpp:31-54:
+    ((acc*s + bias) + prev) -> clamp -> + off*s -> clamp, written out independently of the C oracle."""
+    rng = np.random.default_rng(14)
+    A = rng.integers(-128, 128, size=(12, 64), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(64, 20), dtype=np.int8)
+    bias = rng.normal(0, 3, size=20).astype(np.float32)
+    prev = rng.normal(0, 5, size=(12, 20)).astype(np.float32)
+    s = np.float32(1e-3)
+    acc = (A.astype(np.int32) @ B.astype(np.int32))
+    off = exact_t(A, B, 30, 20).astype(np.int64) - acc
+    lo, hi = np.float32(0), np.float32(6)
+    r = (acc.astype(np.float32) * s + bias) + prev
+    want_twice = np.clip(np.clip(r, lo, hi) + off.astype(np.float32) * s, lo, hi)
+    want_once = np.clip(r + off.astype(np.float32) * s, lo, hi)
+    got_twice = oracle.gemmlowp_f32(A, B, bias, 30, 20, float(s), 0.0, 6.0, prev=prev, act_twice=True)
+    got_once = oracle.gemmlowp_f32(A, B, bias, 30, 20, float(s), 0.0, 6.0, prev=prev)
+    np.testing.assert_array_equal(got_twice, want_twice)
+    np.testing.assert_array_equal(got_once, want_once)
+    assert (want_once != want_twice).any()
+    # without accumulation the previous contents must not matter
+    np.testing.assert_array_equal(oracle.gemmlowp_f32(A, B, bias, 0, 0, float(s)), acc.astype(np.float32) * s + bias)
+
+
 @pytest.mark.skipif(not oracle.ref_available(), reason="oracle/_ref not built (needs the reference checkout)")
 def test_fused_against_live_reference_config1_shape():
     """BASELINE config 1 at full size (256^3, QASYMM8, both zero-point conventions) through the reference's code."""

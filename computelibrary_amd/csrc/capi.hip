@@ -635,12 +635,26 @@ int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *s
     const mi355_output_stage_desc &d = *desc;
     if (d.M < 1 || d.N < 1 || d.ld_src < d.N || d.ld_dst < d.N)
         return fail("bad output-stage shape");
-    if (!is_8bit(d.dst_dtype))
-        return fail("output stage writes QASYMM8 or QASYMM8_SIGNED");
+    const bool s16 = d.dst_dtype == MI355_S16;
+    if (!is_8bit(d.dst_dtype) && !s16)
+        return fail("output stage writes QASYMM8, QASYMM8_SIGNED or QSYMM16");
     if (d.requant.per_channel)
         return fail("the stand-alone output stage is per-tensor");
-    if (check_requant(d.requant, d.dst_dtype))
+    if (s16)
+    {
+        if (d.requant.stage != MI355_STAGE_FIXEDPOINT || d.requant.result_offset != 0)
+            return fail("the QSYMM16 output stage is QUANTIZE_DOWN_FIXEDPOINT without a result offset");
+        if (d.requant.min_bound > d.requant.max_bound)
+            return fail("min_bound > max_bound");
+        // the reference narrows the bounds to int16 with a plain cast: only bounds that survive it are meaningful
+        const bool whole = d.requant.min_bound <= -32768 && d.requant.max_bound >= 32767;
+        if (!whole && (d.requant.min_bound < -32768 || d.requant.max_bound > 32767))
+            return fail("QSYMM16 clamp bounds [%d,%d] are partly outside the int16 range", d.requant.min_bound,
+                        d.requant.max_bound);
+    }
+    else if (check_requant(d.requant, d.dst_dtype))
         return 1;
+    const size_t desz = s16 ? 2 : 1;
     hipStream_t s = (hipStream_t)stream;
     DevBuf      sSrc, sBias, sDst;
     const void *srcd, *biasd;
@@ -651,7 +665,7 @@ int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *s
     EpiParams    p{};
     p.mult_s = d.requant.multiplier, p.shift_s = d.requant.shift, p.result_offset = d.requant.result_offset;
     p.stage  = d.requant.stage;
-    const int32_t tlo = d.dst_dtype == MI355_S8 ? -128 : 0, thi = d.dst_dtype == MI355_S8 ? 127 : 255;
+    const int32_t tlo = s16 ? -32768 : d.dst_dtype == MI355_S8 ? -128 : 0, thi = s16 ? 32767 : d.dst_dtype == MI355_S8 ? 127 : 255;
     p.lo = d.requant.min_bound > tlo ? d.requant.min_bound : tlo;
     p.hi = d.requant.max_bound < thi ? d.requant.max_bound : thi;
     auto body = [&]() -> int
@@ -660,14 +674,17 @@ int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *s
         TRY(to_device(bias, sizeof(int32_t) * d.N, sBias, s, &biasd));
         if (d_host)
         {
-            TRY(sDst.ensure(d_elems));
+            TRY(sDst.ensure(d_elems * desz));
             Dd = sDst.p;
             if (d.ld_dst != d.N)
-                HIP_TRY(hipMemcpyAsync(Dd, dst, d_elems, hipMemcpyHostToDevice, s));
+                HIP_TRY(hipMemcpyAsync(Dd, dst, d_elems * desz, hipMemcpyHostToDevice, s));
         }
-        HIP_TRY(output_stage_launch((const int32_t *)srcd, d.ld_src, (const int32_t *)biasd, Dd, d.ld_dst, d.M, d.N, p, s));
+        if (s16)
+            HIP_TRY(output_stage_s16_launch((const int32_t *)srcd, d.ld_src, (const int32_t *)biasd, Dd, d.ld_dst, d.M, d.N, p, s));
+        else
+            HIP_TRY(output_stage_launch((const int32_t *)srcd, d.ld_src, (const int32_t *)biasd, Dd, d.ld_dst, d.M, d.N, p, s));
         if (d_host)
-            HIP_TRY(hipMemcpyAsync(dst, Dd, d_elems, hipMemcpyDeviceToHost, s));
+            HIP_TRY(hipMemcpyAsync(dst, Dd, d_elems * desz, hipMemcpyDeviceToHost, s));
         if (d_host || srcd != src || biasd != bias)
             HIP_TRY(hipStreamSynchronize(s));
         return 0;

@@ -113,6 +113,26 @@ __device__ __forceinline__ int32_t requant_fixedpoint(int32_t v, int32_t mult, i
     return (int32_t)((uint32_t)r + (uint32_t)result_offset);
 }
 
+// SQRDMULH: (a * b + 2^30) >> 31, saturating the single overflowing case (vqrdmulhq_n_s32, src/core/NEON/NESymm.h:62-69)
+__device__ __forceinline__ int32_t sqrdmulh(int32_t a, int32_t b)
+{
+    if (a == INT32_MIN && b == INT32_MIN)
+        return INT32_MAX;
+    return (int32_t)(((int64_t)a * (int64_t)b + ((int64_t)1 << 30)) >> 31);
+}
+
+// int32 -> QSYMM16 (finalize_quantization_int16, src/core/NEON/NESymm.h:54-85): no result offset; [lo, hi] already
+// intersected with the int16 range
+__device__ __forceinline__ int32_t requant_fixedpoint_s16(int32_t v, int32_t mult, int32_t shift, int32_t lo, int32_t hi)
+{
+    int32_t r;
+    if (shift < 0)
+        r = sqrdmulh((-shift >= 32) ? 0 : (int32_t)((uint32_t)v << (-shift)), mult);
+    else
+        r = rounding_shift_right(sqrdmulh(v, mult), shift);
+    return min(max(r, lo), hi);
+}
+
 __device__ __forceinline__ int32_t clamp_i32(int32_t v, int32_t lo, int32_t hi)
 {
     return min(max(v, lo), hi);

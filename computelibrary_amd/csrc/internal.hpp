@@ -115,6 +115,8 @@ int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t
                      int32_t b_off, hipStream_t s);
 int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                         int N, const EpiParams &epi, hipStream_t s);
+int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
+                            int N, const EpiParams &epi, hipStream_t s);
 int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);
 // one thread per output; A dense [M][lda] (unflipped or flipped per flip_a), Bp packed
 int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s);

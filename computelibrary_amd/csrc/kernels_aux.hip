@@ -361,6 +361,53 @@ __global__ __launch_bounds__(256) void output_stage_kernel(const int32_t *__rest
     }
 }
 
+// CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel
+// (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel.cpp:76-200): 4 B read + 2 B written per element
+template <bool VEC4>
+__global__ __launch_bounds__(256) void output_stage_s16_kernel(const int32_t *__restrict__ src, int64_t ld_src,
+                                                               const int32_t *__restrict__ bias, int16_t *__restrict__ dst,
+                                                               int64_t ld_dst, int M, int N, EpiParams p)
+{
+    const int     per_row = VEC4 ? N / 4 : N;
+    const int64_t idx     = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)M * per_row)
+        return;
+    const int i = (int)(idx / per_row), q = (int)(idx % per_row);
+    if (VEC4)
+    {
+        typedef short v4s __attribute__((ext_vector_type(4)));
+        const int j = q * 4;
+        v4i       v = *(const v4i *)(src + (int64_t)i * ld_src + j);
+        v4i       b = {0, 0, 0, 0};
+        if (bias)
+            b = *(const v4i *)(bias + j);
+        v4s o;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            o[t] = (short)requant_fixedpoint_s16((int32_t)((uint32_t)v[t] + (uint32_t)b[t]), p.mult_s, p.shift_s, p.lo, p.hi);
+        *(v4s *)(dst + (int64_t)i * ld_dst + j) = o;
+    }
+    else
+        dst[(int64_t)i * ld_dst + q] = (int16_t)requant_fixedpoint_s16(
+            (int32_t)((uint32_t)src[(int64_t)i * ld_src + q] + (uint32_t)(bias ? bias[q] : 0)), p.mult_s, p.shift_s, p.lo, p.hi);
+}
+
+int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
+                            int N, const EpiParams &epi, hipStream_t s)
+{
+    if (M <= 0 || N <= 0)
+        return 0;
+    const bool vec = (N % 4 == 0) && (ld_src % 4 == 0) && (ld_dst % 4 == 0) && (((uintptr_t)src & 15) == 0) &&
+                     (((uintptr_t)dst & 7) == 0) && (bias == nullptr || ((uintptr_t)bias & 15) == 0);
+    const int64_t total = (int64_t)M * (vec ? N / 4 : N);
+    const dim3    grid((unsigned)((total + 255) / 256)), block(256);
+    if (vec)
+        output_stage_s16_kernel<true><<<grid, block, 0, s>>>(src, ld_src, bias, (int16_t *)dst, ld_dst, M, N, epi);
+    else
+        output_stage_s16_kernel<false><<<grid, block, 0, s>>>(src, ld_src, bias, (int16_t *)dst, ld_dst, M, N, epi);
+    return launch_status();
+}
+
 int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                         int N, const EpiParams &epi, hipStream_t s)
 {

@@ -30,6 +30,8 @@ int to_mi355(DataType dt)
         case DataType::QSYMM8_PER_CHANNEL:
         case DataType::S8:
             return MI355_S8;
+        case DataType::QSYMM16:
+            return MI355_S16;
         case DataType::S32:
             return MI355_S32;
         case DataType::F32:
@@ -471,7 +473,17 @@ Status NEGEMMLowpOutputStage::validate(const ITensorInfo *input, const ITensorIn
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.type == GEMMLowpOutputStageType::QUANTIZE_DOWN &&
                                         (info.gemmlowp_shift < 0 || info.gemmlowp_shift > 31),
                                     "QUANTIZE_DOWN needs a shift in [0, 31]");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::QSYMM16, "QSYMM16 output is not built in this library");
+    // QSYMM16 only has a fixed-point kernel (src/cpu/operators/CpuGemmLowpOutputStage.cpp:73-80,91-107)
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::QSYMM16 &&
+                                        info.type != GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT,
+                                    "Unsupported output data type.");
+    if (output->data_type() == DataType::QSYMM16)
+    {
+        // the int16 kernel narrows the bounds with a plain cast: accept what survives it
+        const bool whole = info.gemmlowp_min_bound <= -32768 && info.gemmlowp_max_bound >= 32767;
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(!whole && (info.gemmlowp_min_bound < -32768 || info.gemmlowp_max_bound > 32767),
+                                        "QSYMM16 bounds partly outside the int16 range");
+    }
     ARM_COMPUTE_RETURN_ERROR_ON(input->data_type() != DataType::S32 || input->num_channels() != 1);
     ARM_COMPUTE_RETURN_ERROR_ON(info.gemmlowp_min_bound > info.gemmlowp_max_bound);
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.is_quantized_per_channel, "The stand-alone output stage is per-tensor");
@@ -517,8 +529,19 @@ void NEGEMMLowpOutputStage::configure(const ITensor *input, const ITensor *bias,
     s.desc.ld_src    = ii->strides_in_bytes()[1] / ii->element_size();
     s.desc.ld_dst    = oi->strides_in_bytes()[1] / oi->element_size();
     s.desc.dst_dtype = to_mi355(oi->data_type());
-    s.desc.requant   = make_requant(info);
-    s.configured     = true;
+    if (oi->data_type() == DataType::QSYMM16)
+    {
+        // no result offset on this path: the reference's int16 kernel is not given one (CpuGemmLowpOutputStage.cpp:73-80)
+        s.desc.requant            = mi355_requant{};
+        s.desc.requant.multiplier = info.gemmlowp_multiplier;
+        s.desc.requant.shift      = info.gemmlowp_shift;
+        s.desc.requant.min_bound  = info.gemmlowp_min_bound;
+        s.desc.requant.max_bound  = info.gemmlowp_max_bound;
+        s.desc.requant.stage      = MI355_STAGE_FIXEDPOINT;
+    }
+    else
+        s.desc.requant = make_requant(info);
+    s.configured = true;
 }
 
 void NEGEMMLowpOutputStage::run()

@@ -43,7 +43,8 @@ typedef enum mi355_dtype
     MI355_U8  = 0, /* QASYMM8 */
     MI355_S8  = 1, /* QASYMM8_SIGNED, QSYMM8, QSYMM8_PER_CHANNEL */
     MI355_S32 = 2,
-    MI355_F32 = 3
+    MI355_F32 = 3,
+    MI355_S16 = 4 /* QSYMM16: only as the destination of mi355_output_stage_run */
 } mi355_dtype;
 
 /* What happens to the int32 accumulators. Replaces the choice the reference makes between
@@ -161,12 +162,16 @@ const char *mi355_gemmlowp_kernel_name(const mi355_gemm_handle *h);
 /* Stand-alone output stage on an int32 matrix. Replaces CpuGemmLowpOutputStage::run ->
  * CpuGemmLowpQuantizeDownInt32To{Int8,Uint8}ScaleByFixedPointKernel
  * (src/cpu/operators/CpuGemmLowpOutputStage.cpp:163-167,
- *  src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt8ScaleByFixedPointKernel.cpp:79-181). Stateless. */
+ *  src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt8ScaleByFixedPointKernel.cpp:79-181). Stateless.
+ * With dst_dtype MI355_S16 it replaces CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel
+ * (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel.cpp:76-200, arithmetic in
+ *  src/core/NEON/NESymm.h:54-85): the multiply is the ROUNDING doubling high multiply there, there is no result offset
+ *  (it must be 0), ld_dst counts int16 elements, and the bounds are either the whole int16 range or inside it. */
 typedef struct mi355_output_stage_desc
 {
     int32_t       M, N;
     int64_t       ld_src, ld_dst;
-    int32_t       dst_dtype; /* MI355_U8 or MI355_S8 */
+    int32_t       dst_dtype; /* MI355_U8, MI355_S8, or MI355_S16 (FIXEDPOINT only) */
     mi355_requant requant;   /* per-tensor */
 } mi355_output_stage_desc;
 

@@ -35,6 +35,10 @@ def _load():
     lib.orc_requant_s32.argtypes = [C.c_int32] * 4
     lib.orc_requant_scale_s32.restype = C.c_int32
     lib.orc_requant_scale_s32.argtypes = [C.c_int32] * 4
+    lib.orc_sqrdmulh_s32.restype = C.c_int32
+    lib.orc_sqrdmulh_s32.argtypes = [C.c_int32, C.c_int32]
+    lib.orc_requant_fixedpoint_s16.restype = C.c_int16
+    lib.orc_requant_fixedpoint_s16.argtypes = [C.c_int32] * 5
     lib.orc_narrow_clamp.restype = C.c_int32
     lib.orc_narrow_clamp.argtypes = [C.c_int32, C.c_int, C.c_int32, C.c_int32]
     lib.orc_calculate_quantized_multiplier.restype = C.c_int
@@ -141,6 +145,17 @@ def output_stage_scale(src, bias, mult, shift, result_offset, min_bound, max_bou
     out = np.empty((M, N), dtype=dst_dtype)
     lib.orc_output_stage_scale(_p(src), C.c_int64(N), _p(bias), _p(out), C.c_int64(N), _signed(out), M, N, _p(m), _p(s), n,
                                C.c_int32(result_offset), C.c_int32(min_bound), C.c_int32(max_bound))
+    return out
+
+
+def output_stage_fixedpoint_s16(src, bias, mult, shift, min_bound=-32768, max_bound=32767):
+    """int32 -> QSYMM16 (rounding doubling high multiply, rounding shift, no offset)"""
+    src = np.ascontiguousarray(src, dtype=np.int32)
+    M, N = src.shape
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.empty((M, N), dtype=np.int16)
+    lib.orc_output_stage_fixedpoint_s16(_p(src), C.c_int64(N), _p(bias), _p(out), C.c_int64(N), M, N, C.c_int32(mult),
+                                        C.c_int32(shift), C.c_int32(min_bound), C.c_int32(max_bound))
     return out
 
 
@@ -344,6 +359,16 @@ def ref_quantize_down_scale(src, bias, mult, shift, result_offset, lo, hi, dst_d
     out = np.empty((M, N), dtype=dst_dtype)
     ref().ref_quantize_down_scale(_p(src), _p(bias), M, N, _p(m), _p(s), n, C.c_int32(result_offset), C.c_int32(lo),
                                   C.c_int32(hi), _signed(out), _p(out))
+    return out
+
+
+def ref_quantize_down_fixedpoint_s16(src, bias, mult, shift, lo, hi):
+    src = np.ascontiguousarray(src, dtype=np.int32)
+    M, N = src.shape
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    out = np.empty((M, N), dtype=np.int16)
+    ref().ref_quantize_down_fixedpoint_s16(_p(src), _p(bias), M, N, C.c_int32(mult), C.c_int32(shift), C.c_int32(lo),
+                                           C.c_int32(hi), _p(out))
     return out
 
 

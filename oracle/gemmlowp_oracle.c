@@ -257,6 +257,53 @@ void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const voi
     free(t);
 }
 
+/* SQRDMULH, the rounding doubling multiply returning the high half: sat((2*a*b + 2^31) >> 32) = sat((a*b + 2^30) >> 31).
+ * Only a == b == INT32_MIN saturates. (Arm ARM, SQRDMULH; used as vqrdmulhq_n_s32 in src/core/NEON/NESymm.h:62-69 and
+ * written out as (in_64 + (1 << 30)) >> 31 in its scalar twin, NESymm.h:105-114.) */
+int32_t orc_sqrdmulh_s32(int32_t a, int32_t b)
+{
+    if (a == INT32_MIN && b == INT32_MIN)
+        return INT32_MAX;
+    return (int32_t)(((int64_t)a * (int64_t)b + ((int64_t)1 << 30)) >> 31);
+}
+
+/* src/core/NEON/NESymm.h:54-85 (the vector lanes: the left shift wraps in int32 as vmulq_n_s32 does, the right shift
+ * is vrshlq_s32, i.e. round half up, exact): int32 -> int16, no offset; bounded == !(min <= -32768 && max >= 32767)
+ * (src/cpu/kernels/CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel.cpp:205). */
+int16_t orc_requant_fixedpoint_s16(int32_t v, int32_t mult, int32_t shift, int32_t min_bound, int32_t max_bound)
+{
+    int32_t r;
+    if (shift < 0)
+        r = orc_sqrdmulh_s32(-shift >= 32 ? 0 : wrap_mul(v, (int32_t)((uint32_t)1 << (-shift))), mult);
+    else
+        r = orc_rounding_shift_right(orc_sqrdmulh_s32(v, mult), shift);
+    if (r < -32768)
+        r = -32768;
+    if (r > 32767)
+        r = 32767;
+    if (!(min_bound <= -32768 && max_bound >= 32767))
+    {
+        if (r < min_bound)
+            r = min_bound;
+        if (r > max_bound)
+            r = max_bound;
+    }
+    return (int16_t)r;
+}
+
+/* CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel::run_internal (.cpp:76-200): bias add wraps */
+void orc_output_stage_fixedpoint_s16(const int32_t *src, int64_t ld_src, const int32_t *bias, int16_t *dst,
+                                     int64_t ld_dst, int M, int N, int32_t mult, int32_t shift, int32_t min_bound,
+                                     int32_t max_bound)
+{
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j)
+        {
+            const int32_t v = (int32_t)((uint32_t)src[(int64_t)i * ld_src + j] + (uint32_t)(bias ? bias[j] : 0));
+            dst[(int64_t)i * ld_dst + j] = orc_requant_fixedpoint_s16(v, mult, shift, min_bound, max_bound);
+        }
+}
+
 /* src/core/NEON/kernels/arm_gemm/quantized.cpp:977-1030 (float(acc)*scale, + bias, + previous destination value when
  * accumulating, clamp) followed by src/cpu/kernels/gemmlowp/generic/neon/impl.h:95-155 + fp32.cpp:31-54
  * (+= float(offset terms)*scale) and the CpuActivation post-op

@@ -109,6 +109,20 @@ extern "C"
         }
     }
 
+    /* the same template with a 16-bit destination (tests/validation/reference/GEMMLowp.cpp:110-157,423-437); note that it
+     * multiplies with the non-rounding SQDMULH model whereas the NEON int16 kernel uses the rounding one */
+    void ref_quantize_down_fixedpoint_s16(const int32_t *in, const int32_t *bias, int M, int N, int32_t mult, int32_t shift,
+                                          int32_t lo, int32_t hi, int16_t *out)
+    {
+        const SimpleTensor<int32_t> t = make<int32_t>(TensorShape(N, M), DataType::S32, in);
+        const std::vector<int32_t>  m(1, mult), s(1, shift);
+        const SimpleTensor<int16_t> d =
+            bias ? reference::gemmlowp_quantize_down_scale_by_fixedpoint<int32_t, int16_t>(
+                       t, make<int32_t>(TensorShape(N), DataType::S32, bias), m, s, 0, lo, hi)
+                 : reference::gemmlowp_quantize_down_scale_by_fixedpoint<int32_t, int16_t>(t, m, s, 0, lo, hi);
+        std::memcpy(out, d.data(), sizeof(int16_t) * d.num_elements());
+    }
+
     /* tests/validation/reference/GEMMLowp.cpp:66-104,278-307: QUANTIZE_DOWN with an integer multiplier */
     void ref_quantize_down_scale(const int32_t *in, const int32_t *bias, int M, int N, const int32_t *mult,
                                  const int32_t *shift, int n_qparams, int32_t result_offset, int32_t lo, int32_t hi,

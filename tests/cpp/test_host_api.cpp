@@ -583,6 +583,29 @@ static void test_output_stage()
     orc_output_stage_fixedpoint(reinterpret_cast<const int32_t *>(src.buffer()), N, reinterpret_cast<const int32_t *>(bias.buffer()),
                                 want.data(), N, 1, M, N, &os.gemmlowp_multiplier, &os.gemmlowp_shift, 1, -3, -100, 120);
     EXPECT(dense_copy<int8_t>(dst) == want);
+
+    SECTION("NEGEMMLowpOutputStage S32 -> QSYMM16 (rounding multiply, offset ignored)");
+    Tensor dst16;
+    os.gemmlowp_offset    = 9; // the int16 kernel is not given the offset (src/cpu/operators/CpuGemmLowpOutputStage.cpp:73-80)
+    os.gemmlowp_min_bound = -30000, os.gemmlowp_max_bound = 32767, os.output_data_type = DataType::QSYMM16;
+    os.gemmlowp_multiplier = 2000000000, os.gemmlowp_shift = 1;
+    NEGEMMLowpOutputStage stage16;
+    stage16.configure(&src, &bias, &dst16, os);
+    EXPECT(dst16.info()->data_type() == DataType::QSYMM16);
+    dst16.allocator()->allocate();
+    fill_uniform<int32_t>(src, -100000, 100000, 73);
+    stage16.run();
+    std::vector<int16_t> want16(M * N);
+    orc_output_stage_fixedpoint_s16(reinterpret_cast<const int32_t *>(src.buffer()), N,
+                                    reinterpret_cast<const int32_t *>(bias.buffer()), want16.data(), N, M, N, 2000000000, 1,
+                                    -30000, 32767);
+    EXPECT(dense_copy<int16_t>(dst16) == want16);
+    int lo_hits = 0, hi_hits = 0;
+    for (int16_t v : want16)
+        lo_hits += v == -30000, hi_hits += v == 32767;
+    EXPECT(lo_hits > 0 && hi_hits > 0 && lo_hits + hi_hits < M * N / 2); // both bounds bite, most values are inside
+    os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN;
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(src.info(), bias.info(), dst16.info(), os)));
 }
 
 // QUANTIZE_DOWN (integer multiplier): stand-alone stage without bounds (min == max) and fused into the GEMM

@@ -319,6 +319,40 @@ def test_output_stage_fixture(golden):
         np.testing.assert_array_equal(out, dst)
 
 
+@pytest.mark.parametrize("device", [False, True])
+@pytest.mark.parametrize("N,ld_dst", [(64, None), (37, None), (64, 68), (40, 41)])
+def test_output_stage_to_qsymm16(N, ld_dst, device):
+    """int32 -> QSYMM16 (CpuGemmLowpQuantizeDownInt32ToInt16ScaleByFixedPointKernel): rounding high multiply, no offset"""
+    import torch
+    rng = np.random.default_rng(160 + N)
+    M = 50
+    src = np.concatenate([rng.integers(-(1 << 31), 1 << 31, size=(M // 2, N)),
+                          rng.integers(-(1 << 18), 1 << 18, size=(M - M // 2, N))]).astype(np.int32)
+    bias = rng.integers(-5000, 5000, size=N).astype(np.int32)
+    ld = ld_dst or N
+    for mult, shift, lo, hi in [(1518500250, 3, -32768, 32767), ((1 << 31) - 1, 0, -(1 << 31), (1 << 31) - 1),
+                                (1 << 30, -2, -100, 20000), (1073741825, 17, 0, 32767), (-(1 << 30), 5, -32768, 32767)]:
+        for b in (bias, None):
+            announce("output stage s16", N, ld_dst, device, mult, shift, lo, hi, b is not None)
+            want = oracle.output_stage_fixedpoint_s16(src, b, mult, shift, lo, hi)
+            dst = np.full((M, ld), 77, dtype=np.int16)
+            rq = capi.requant(mult, shift, 0, lo, hi)
+            if device:
+                sd, dd = torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda()
+                bd = None if b is None else torch.from_numpy(b).cuda()
+                capi.output_stage(sd, bd, dd, rq, ld_dst=ld)
+                torch.cuda.synchronize()
+                dst = dd.cpu().numpy()
+            else:
+                capi.output_stage(src, b, dst, rq, ld_dst=ld)
+            assert np.array_equal(dst[:, :N], want)
+            assert (dst[:, N:] == 77).all()
+    with pytest.raises(capi.Mi355Error, match="result offset"):
+        capi.output_stage(src, None, np.zeros((M, N), dtype=np.int16), capi.requant(1 << 30, 1, 5, -32768, 32767))
+    with pytest.raises(capi.Mi355Error, match="int16 range"):
+        capi.output_stage(src, None, np.zeros((M, N), dtype=np.int16), capi.requant(1 << 30, 1, 0, -40000, 100))
+
+
 def test_output_stage_scale_fixture(golden):
     """QUANTIZE_DOWN (integer multiplier), stand-alone, against the reference oracle's outputs (per-tensor entries)."""
     g = golden("output_stage_scale.npz")

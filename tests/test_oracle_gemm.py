@@ -145,6 +145,55 @@ def test_f32_bias_and_activation():
     np.testing.assert_array_equal(got, want.astype(np.float32))
 
 
+def _sqrdmulh_model(a, b):
+    """Arm ARM, SQRDMULH (vector, 32-bit): SInt sat((2 * a * b + (1 << 31)) >> 32), with Python integers"""
+    r = (2 * a * b + (1 << 31)) >> 32
+    return max(-(1 << 31), min((1 << 31) - 1, r))
+
+
+def _requant_s16_model(v, mult, shift, lo, hi):
+    """src/core/NEON/NESymm.h:54-85 lane by lane with Python integers (the int32 left shift wraps)"""
+    wrap = lambda x: ((x + (1 << 31)) % (1 << 32)) - (1 << 31)
+    if shift < 0:
+        r = _sqrdmulh_model(wrap(v * (1 << -shift)), mult)
+    else:
+        r = _sqrdmulh_model(v, mult)
+        if shift > 0:
+            r = (r + (1 << (shift - 1))) >> shift  # SRSHL by -shift: round half up, no overflow in big integers
+    r = max(-32768, min(32767, r))
+    if not (lo <= -32768 and hi >= 32767):
+        r = max(lo, min(hi, r))
+    return r
+
+
+def test_requant_s16_against_big_integer_model_and_reference_within_one():
+    rng = np.random.default_rng(16)
+    edge = [0, 1, -1, 2, -2, (1 << 31) - 1, -(1 << 31), 1 << 30, -(1 << 30), 12345678, -87654321]
+    for a in edge:
+        for b in edge:
+            assert oracle.lib.orc_sqrdmulh_s32(a, b) == _sqrdmulh_model(a, b), (a, b)
+    vals = np.concatenate([np.array(edge, dtype=np.int64), rng.integers(-(1 << 31), 1 << 31, size=300),
+                           rng.integers(-(1 << 17), 1 << 17, size=300)])
+    for mult in [1 << 30, (1 << 31) - 1, 1518500250, 1073741825, 0, -(1 << 30)]:
+        for shift in [-3, -1, 0, 1, 2, 7, 15, 31]:
+            for lo, hi in [(-32768, 32767), (-(1 << 31), (1 << 31) - 1), (-100, 20000), (0, 32767)]:
+                for v in vals[::7]:
+                    got = oracle.lib.orc_requant_fixedpoint_s16(int(v), mult, shift, lo, hi)
+                    assert got == _requant_s16_model(int(v), mult, shift, lo, hi), (v, mult, shift, lo, hi)
+    # rounding vs truncating high multiply: a value where they differ, hand-checked:
+    # 3 * 1518500250 = 4555500750; (x + 2^30) >> 31 = 2 (2.121 rounds to 2); 5 * 1518500250 -> 3.535 -> 4, truncating gives 3
+    assert oracle.lib.orc_sqrdmulh_s32(5, 1518500250) == 4 and oracle.lib.orc_sqdmulh(5, 1518500250) == 3
+    if oracle.ref_available():
+        # the reference's portable oracle multiplies without rounding: never more than 1 apart, and not always equal
+        src = rng.integers(-(1 << 20), 1 << 20, size=(9, 40)).astype(np.int32)
+        bias = rng.integers(-1000, 1000, size=40).astype(np.int32)
+        for mult, shift in [(1518500250, 4), (1 << 30, 0), (2000000000, 9)]:
+            want = oracle.ref_quantize_down_fixedpoint_s16(src, bias, mult, shift, -(1 << 31), (1 << 31) - 1)
+            got = oracle.output_stage_fixedpoint_s16(src, bias, mult, shift)
+            d = got.astype(np.int32) - want.astype(np.int32)
+            assert np.abs(d).max() <= 1 and (d >= 0).all()
+
+
 def test_f32_accumulate_and_double_clamp_against_numpy_float32():
     """numpy float32 arithmetic rounds every operation separately, like the NEON instructions of
     src/core/NEON/kernels/arm_gemm/quantized.cpp:1000-1017 and src/cpu/kernels/gemmlowp/generic/neon/fp32.cpp:31-54:

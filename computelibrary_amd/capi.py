@@ -12,6 +12,7 @@ U8, S8, S32, F32, S16 = 0, 1, 2, 3, 4
 EPI_S32, EPI_FIXEDPOINT, EPI_F32 = 0, 1, 2
 PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
 GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
+NHWC, NCHW = 0, 1
 
 EXPORTS = [
     "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_run",
@@ -48,7 +49,7 @@ class ConvDesc(C.Structure):
                 ("batch", "H", "W", "C", "OFM", "KH", "KW", "stride_x", "stride_y", "pad_left", "pad_top",
                  "pad_right", "pad_bottom", "dilation_x", "dilation_y", "src_dtype", "weights_dtype", "dst_dtype",
                  "src_offset", "weights_offset", "pad_value")] + [("requant", Requant), ("path", C.c_int32),
-                                                                  ("reserved", C.c_int32)]
+                                                                  ("layout", C.c_int32)]
 
 
 _lib = None
@@ -177,10 +178,10 @@ def output_stage(src, bias, dst, rq, stream=None, ld_src=None, ld_dst=None):
 
 
 def conv_desc(batch, H, W, Cc, OFM, KH, KW, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), src_dtype=S8,
-              weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0):
+              weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0, layout=0):
     return ConvDesc(batch, H, W, Cc, OFM, KH, KW, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0],
                     dilation[1], src_dtype, weights_dtype, dst_dtype, src_offset, weights_offset, pad_value,
-                    rq or requant(), path, 0)
+                    rq or requant(), path, layout)
 
 
 class Conv:

@@ -422,6 +422,7 @@ struct mi355_conv_handle
     ConvGeom        geom;
     bool            implicit = false;
     DevBuf          stageSrc, stageW, stageDst, stageBias, stageMult, stageShift, cols;
+    DevBuf          nhwcSrc, nhwcW, nhwcDst; // MI355_NCHW: the tensors in the kernels' layout
 };
 
 extern "C"
@@ -735,6 +736,8 @@ static int conv_check(const mi355_conv_desc &d)
         return fail("negative padding");
     if (!is_8bit(d.src_dtype) || !is_8bit(d.weights_dtype) || !is_8bit(d.dst_dtype))
         return fail("convolution tensors must be 8-bit");
+    if (d.layout != MI355_NHWC && d.layout != MI355_NCHW)
+        return fail("unknown layout %d", d.layout);
     return 0;
 }
 
@@ -788,6 +791,13 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t 
     GemmCore   &c = h->core;
     const void *wd, *biasd, *multd, *shiftd;
     TRY(to_device(weights, (size_t)c.N * c.K, h->stageW, s, &wd));
+    if (h->d.layout == MI355_NCHW)
+    {
+        // [OFM][C][KH*KW] -> [OFM][KH*KW][C]
+        TRY(h->nhwcW.ensure((size_t)c.N * c.K));
+        HIP_TRY(transpose_bytes_launch(wd, h->nhwcW.p, c.N, h->d.C, h->d.KH * h->d.KW, s));
+        wd = h->nhwcW.p;
+    }
     TRY(to_device(bias, sizeof(int32_t) * c.N, h->stageBias, s, &biasd));
     TRY(to_device(c.rq.per_channel ? mult : nullptr, sizeof(int32_t) * c.N, h->stageMult, s, &multd));
     TRY(to_device(c.rq.per_channel ? shift : nullptr, sizeof(int32_t) * c.N, h->stageShift, s, &shiftd));
@@ -855,6 +865,17 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         TRY(h->stageDst.ensure(dst_bytes));
         Dd = h->stageDst.p;
     }
+    const bool nchw   = d.layout == MI355_NCHW;
+    void      *Dfinal = Dd;
+    if (nchw)
+    {
+        // every image [C][H*W] -> [H*W][C]; the kernels write [OH*OW][OFM] per image into a buffer of their own
+        TRY(h->nhwcSrc.ensure(src_bytes));
+        TRY(h->nhwcDst.ensure(dst_bytes));
+        HIP_TRY(transpose_bytes_launch(srcd, h->nhwcSrc.p, d.batch, d.C, d.H * d.W, s));
+        srcd = h->nhwcSrc.p;
+        Dd   = h->nhwcDst.p;
+    }
     if (h->implicit && (((uintptr_t)srcd) & 15) == 0)
     {
         GemmArgs g{};
@@ -877,12 +898,17 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         HIP_TRY(im2col_nhwc_launch(srcd, h->cols.p, d.batch, g2, ldc, s));
         TRY(c.run_dense(h->cols.as<int8_t>(), ldc, 0, Dd, c.N, 0, nullptr, s));
     }
+    if (nchw)
+    {
+        HIP_TRY(transpose_bytes_launch(Dd, Dfinal, d.batch, h->geom.OH * h->geom.OW, c.N, s));
+        Dd = Dfinal;
+    }
     if (d_host)
     {
         HIP_TRY(hipMemcpyAsync(dst, Dd, dst_bytes, hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
     }
-    else if (srcd != src)
+    else if (!is_device_ptr(src))
         HIP_TRY(hipStreamSynchronize(s));
     return 0;
 }
@@ -894,6 +920,7 @@ void mi355_conv_destroy(mi355_conv_handle *h)
     h->core.release();
     h->stageSrc.release(), h->stageW.release(), h->stageDst.release(), h->stageBias.release();
     h->stageMult.release(), h->stageShift.release(), h->cols.release();
+    h->nhwcSrc.release(), h->nhwcW.release(), h->nhwcDst.release();
     delete h;
 }
 
@@ -908,6 +935,8 @@ int mi355_im2col_nhwc_run(const mi355_conv_desc *desc, const void *src, void *ds
         return fail("null argument");
     const mi355_conv_desc &d = *desc;
     TRY(conv_check(d));
+    if (d.layout != MI355_NHWC)
+        return fail("mi355_im2col_nhwc_run lowers NHWC tensors only");
     ConvGeom g{};
     conv_geom(d, g);
     g.pad_word      = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;

@@ -117,6 +117,8 @@ int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias,
                         int N, const EpiParams &epi, hipStream_t s);
 int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                             int N, const EpiParams &epi, hipStream_t s);
+// [batch][R][C] bytes -> [batch][C][R]
+int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
 int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);
 // one thread per output; A dense [M][lda] (unflipped or flipped per flip_a), Bp packed
 int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s);

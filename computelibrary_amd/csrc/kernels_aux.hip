@@ -478,6 +478,38 @@ int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g,
     return launch_status();
 }
 
+// ---- byte-matrix transpose: [batch][R][C] -> [batch][C][R] ---------------------------------------------------------
+// The NCHW <-> NHWC conversions around the NHWC convolution kernel (one image is a C x HW byte matrix) and of NCHW
+// weights ([OFM][C][KH*KW] -> [OFM][KH*KW][C]). 64 x 64 tiles through LDS so that reads and writes both run along rows.
+__global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                              int R, int C)
+{
+    __shared__ uint8_t tile[64][65];
+    const int64_t      base = (int64_t)blockIdx.z * R * C;
+    const int          r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int          tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll 4
+    for (int y = ty; y < 64; y += 4)
+        if (r0 + y < R && c0 + tx < C)
+            tile[y][tx] = src[base + (int64_t)(r0 + y) * C + c0 + tx];
+    __syncthreads();
+#pragma unroll 4
+    for (int y = ty; y < 64; y += 4)
+        if (c0 + y < C && r0 + tx < R)
+            dst[base + (int64_t)(c0 + y) * R + r0 + tx] = tile[tx][y];
+}
+
+int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s)
+{
+    if (batch <= 0 || R <= 0 || C <= 0)
+        return 0;
+    if (batch > 65535 || (R + 63) / 64 > 65535)
+        return (int)hipErrorInvalidValue;
+    const dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)batch), block(256);
+    transpose_bytes_kernel<<<grid, block, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, R, C);
+    return launch_status();
+}
+
 // ---- one thread per output: the plainest possible statement of the path, for cross-checking only ----------------------
 template <int EPI>
 __global__ __launch_bounds__(256) void simple_gemm_kernel(GemmArgs g, uint8_t flip)

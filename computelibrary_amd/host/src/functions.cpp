@@ -6,6 +6,7 @@
 #include "arm_compute/core/utils/quantization/AsymmHelpers.h"
 #include "arm_compute/runtime/NEON/NEFunctions.h"
 #include "arm_compute/runtime/experimental/operators/CpuGEMMLowp.h"
+#include "arm_compute/runtime/experimental/operators/CpuGemmConv2d.h"
 #include "mi355_gemmlowp.h"
 
 #include <cmath>
@@ -419,12 +420,13 @@ void NEGEMMLowpMatrixMultiplyCore::run()
         const int32_t bo = is_data_type_quantized_per_channel(s.b->info()->data_type())
                                ? 0
                                : s.b->info()->quantization_info().uniform().offset;
-        if (ao != s.desc.a_offset || bo != s.desc.b_offset)
+        // ... and so is the dequantisation scale of the F32 path (:776-784)
+        const float sc = s.desc.epilogue == MI355_EPI_F32 ? s.a->info()->quantization_info().uniform().scale *
+                                                                s.b->info()->quantization_info().uniform().scale
+                                                          : s.desc.scale;
+        if (ao != s.desc.a_offset || bo != s.desc.b_offset || sc != s.desc.scale)
         {
-            s.desc.a_offset = ao, s.desc.b_offset = bo;
-            if (s.desc.epilogue == MI355_EPI_F32)
-                s.desc.scale = s.a->info()->quantization_info().uniform().scale *
-                               s.b->info()->quantization_info().uniform().scale;
+            s.desc.a_offset = ao, s.desc.b_offset = bo, s.desc.scale = sc;
             check_abi(mi355_gemmlowp_update_quant(s.handle, ao, bo, nullptr, s.desc.scale, nullptr),
                       "NEGEMMLowpMatrixMultiplyCore::run");
         }
@@ -585,6 +587,13 @@ NEGEMMConvolutionLayer::~NEGEMMConvolutionLayer() = default;
 
 namespace
 {
+// positions of width / height / channels in a 4D tensor shape (get_data_layout_dimension_index of the reference)
+struct ConvDims
+{
+    size_t w, h, c;
+    explicit ConvDims(DataLayout l) : w(l == DataLayout::NHWC ? 1 : 0), h(l == DataLayout::NHWC ? 2 : 1), c(l == DataLayout::NHWC ? 0 : 2) {}
+};
+
 // requantisation of a quantized convolution, as CpuGemmConv2d::configure_mm derives it
 // (src/cpu/operators/CpuGemmConv2d.cpp:266-313 of the reference)
 Status conv_output_stage(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *dst,
@@ -625,10 +634,12 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
                                     "Weights must be QASYMM8, QASYMM8_SIGNED or QSYMM8_PER_CHANNEL");
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != weights->data_layout(), "Mismatching data layouts");
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(num_groups > 1, "Grouping (num_groups != 1) is not supported");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC, "Only the NHWC layout is built in this library");
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC && input->data_layout() != DataLayout::NCHW,
+                                    "Unknown data layout");
+    const ConvDims dm(input->data_layout());
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_type() == DataType::QASYMM8_SIGNED && weights->data_type() == DataType::QASYMM8,
                                     "QASYMM8_SIGNED input with QASYMM8 weights is not supported");
-    ARM_COMPUTE_RETURN_ERROR_ON(weights->dimension(0) != input->dimension(0)); // channels
+    ARM_COMPUTE_RETURN_ERROR_ON(weights->dimension(dm.c) != input->dimension(dm.c)); // channels
     ARM_COMPUTE_RETURN_ERROR_ON(weights->num_dimensions() > 4);
     ARM_COMPUTE_RETURN_ERROR_ON(input->num_dimensions() > 4);
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() != input->data_type(),
@@ -646,13 +657,14 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
         ARM_COMPUTE_RETURN_ERROR_ON_MSG(fusable_acts.count(act_info.activation()) == 0,
                                         "Only RELU, BOUNDED_RELU and LU_BOUNDED_RELU can be fused");
     unsigned int conv_w = 0, conv_h = 0;
-    std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(input->dimension(1)), static_cast<int>(input->dimension(2)),
-                                                 static_cast<int>(weights->dimension(1)), static_cast<int>(weights->dimension(2)),
+    std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(input->dimension(dm.w)), static_cast<int>(input->dimension(dm.h)),
+                                                 static_cast<int>(weights->dimension(dm.w)), static_cast<int>(weights->dimension(dm.h)),
                                                  conv_info, dilation);
     if (output->total_size() != 0)
     {
-        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(0) != weights->dimension(3));
-        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(1) != conv_w || output->dimension(2) != conv_h);
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_layout() != input->data_layout(), "Mismatching data layouts");
+        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(dm.c) != weights->dimension(3));
+        ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(dm.w) != conv_w || output->dimension(dm.h) != conv_h);
         ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(3) != input->dimension(3));
     }
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->has_padding() || weights->has_padding() || output->has_padding(),
@@ -675,51 +687,49 @@ Status NEGEMMConvolutionLayer::has_opt_impl(WeightFormat &expected_weight_format
     ARM_COMPUTE_RETURN_ERROR_MSG("No fixed-format kernel available");
 }
 
-void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weights, const ITensor *biases,
-                                       ITensor *output, const PadStrideInfo &conv_info, const WeightsInfo &weights_info,
-                                       const Size2D &dilation, const ActivationLayerInfo &act_info,
-                                       bool enable_fast_math, unsigned int num_groups)
+namespace
 {
-    ARM_COMPUTE_ERROR_ON_NULLPTR(input, weights, output);
-    const ITensorInfo *ii = input->info(), *wi = weights->info();
-    if (output->info()->total_size() == 0 && output->info()->is_resizable())
-    {
-        unsigned int conv_w = 0, conv_h = 0;
-        std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(ii->dimension(1)), static_cast<int>(ii->dimension(2)),
-                                                     static_cast<int>(wi->dimension(1)), static_cast<int>(wi->dimension(2)),
-                                                     conv_info, dilation);
-        const QuantizationInfo keep = output->info()->quantization_info();
-        output->info()->set_tensor_shape(TensorShape(wi->dimension(3), conv_w, conv_h, ii->dimension(3)));
-        output->info()->set_num_channels(1);
-        output->info()->set_data_type(ii->data_type());
-        output->info()->set_data_layout(ii->data_layout());
-        output->info()->set_quantization_info(keep.empty() ? ii->quantization_info() : keep);
-    }
-    ARM_COMPUTE_ERROR_THROW_ON(validate(ii, wi, biases != nullptr ? biases->info() : nullptr, output->info(), conv_info,
-                                        weights_info, dilation, act_info, enable_fast_math, num_groups));
-    Impl &s = *_impl;
-    if (s.handle)
-    {
-        mi355_conv_destroy(s.handle);
-        s.handle = nullptr;
-    }
-    s.src = input, s.weights = weights, s.biases = biases, s.dst = output, s.act = act_info;
-    s.is_prepared = false;
+// an uninitialised output takes the convolved shape, the input's type, layout and (unless it already has one) quantization
+void conv_auto_init_output(const ITensorInfo *ii, const ITensorInfo *wi, ITensorInfo *oi, const PadStrideInfo &conv_info,
+                           const Size2D &dilation)
+{
+    if (oi->total_size() != 0 || !oi->is_resizable())
+        return;
+    const ConvDims dm(ii->data_layout());
+    unsigned int   conv_w = 0, conv_h = 0;
+    std::tie(conv_w, conv_h) = scaled_dimensions(static_cast<int>(ii->dimension(dm.w)), static_cast<int>(ii->dimension(dm.h)),
+                                                 static_cast<int>(wi->dimension(dm.w)), static_cast<int>(wi->dimension(dm.h)),
+                                                 conv_info, dilation);
+    const QuantizationInfo keep = oi->quantization_info();
+    TensorShape            shape;
+    shape.set(dm.c, wi->dimension(3)), shape.set(dm.w, conv_w), shape.set(dm.h, conv_h), shape.set(3, ii->dimension(3));
+    oi->set_tensor_shape(shape);
+    oi->set_num_channels(1);
+    oi->set_data_type(ii->data_type());
+    oi->set_data_layout(ii->data_layout());
+    oi->set_quantization_info(keep.empty() ? ii->quantization_info() : keep);
+}
 
+// the C-ABI descriptor of a (validated) convolution on these tensor infos
+void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, const PadStrideInfo &conv_info,
+                    const Size2D &dilation, const ActivationLayerInfo &act_info, mi355_conv_desc &d,
+                    std::vector<int32_t> &multipliers, std::vector<int32_t> &shifts)
+{
     GEMMLowpOutputStageInfo stage;
-    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, output->info(), act_info, stage));
-    mi355_conv_desc &d = s.desc;
-    d                  = mi355_conv_desc{};
-    d.C = static_cast<int32_t>(ii->dimension(0)), d.W = static_cast<int32_t>(ii->dimension(1));
-    d.H = static_cast<int32_t>(ii->dimension(2)), d.batch = static_cast<int32_t>(ii->tensor_shape().total_size_upper(3));
-    d.KW = static_cast<int32_t>(wi->dimension(1)), d.KH = static_cast<int32_t>(wi->dimension(2));
+    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, oi, act_info, stage));
+    const ConvDims dm(ii->data_layout());
+    d        = mi355_conv_desc{};
+    d.layout = ii->data_layout() == DataLayout::NHWC ? MI355_NHWC : MI355_NCHW;
+    d.C = static_cast<int32_t>(ii->dimension(dm.c)), d.W = static_cast<int32_t>(ii->dimension(dm.w));
+    d.H = static_cast<int32_t>(ii->dimension(dm.h)), d.batch = static_cast<int32_t>(ii->tensor_shape().total_size_upper(3));
+    d.KW = static_cast<int32_t>(wi->dimension(dm.w)), d.KH = static_cast<int32_t>(wi->dimension(dm.h));
     d.OFM      = static_cast<int32_t>(wi->dimension(3));
     d.stride_x = conv_info.stride().first, d.stride_y = conv_info.stride().second;
     d.pad_left = conv_info.pad_left(), d.pad_top = conv_info.pad_top();
     d.pad_right = conv_info.pad_right(), d.pad_bottom = conv_info.pad_bottom();
     d.dilation_x = static_cast<int32_t>(dilation.x()), d.dilation_y = static_cast<int32_t>(dilation.y());
     d.src_dtype = to_mi355(ii->data_type()), d.weights_dtype = to_mi355(wi->data_type());
-    d.dst_dtype = to_mi355(output->info()->data_type());
+    d.dst_dtype = to_mi355(oi->data_type());
     // the GEMM adds its offsets: hand it the negated zero points (CpuGemmConv2d.cpp:266-280 of the reference);
     // im2col pads with the un-negated input zero point (src/cpu/kernels/directconv2d/impl.h:333-334)
     const int32_t in_zp = ii->quantization_info().uniform().offset;
@@ -731,12 +741,53 @@ void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weig
     d.path      = 0;
     if (stage.is_quantized_per_channel)
     {
-        s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
-        s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.OFM);
+        multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
+        shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.OFM);
     }
     else
-        s.multipliers.clear(), s.shifts.clear();
-    check_abi(mi355_conv_create(&d, &s.handle), "NEGEMMConvolutionLayer::configure");
+        multipliers.clear(), shifts.clear();
+}
+
+// new quantization of src / weights / dst into an existing descriptor
+void refresh_conv_quant(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, const ActivationLayerInfo &act,
+                        mi355_conv_desc &d, std::vector<int32_t> &multipliers, std::vector<int32_t> &shifts)
+{
+    GEMMLowpOutputStageInfo stage;
+    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, oi, act, stage));
+    const int32_t in_zp = ii->quantization_info().uniform().offset;
+    d.src_offset        = -in_zp;
+    d.pad_value         = in_zp;
+    d.weights_offset =
+        is_data_type_quantized_per_channel(wi->data_type()) ? 0 : -wi->quantization_info().uniform().offset;
+    d.requant = make_requant(stage);
+    if (stage.is_quantized_per_channel)
+    {
+        multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
+        shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.OFM);
+    }
+}
+} // namespace
+
+void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weights, const ITensor *biases,
+                                       ITensor *output, const PadStrideInfo &conv_info, const WeightsInfo &weights_info,
+                                       const Size2D &dilation, const ActivationLayerInfo &act_info,
+                                       bool enable_fast_math, unsigned int num_groups)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(input, weights, output);
+    const ITensorInfo *ii = input->info(), *wi = weights->info();
+    conv_auto_init_output(ii, wi, output->info(), conv_info, dilation);
+    ARM_COMPUTE_ERROR_THROW_ON(validate(ii, wi, biases != nullptr ? biases->info() : nullptr, output->info(), conv_info,
+                                        weights_info, dilation, act_info, enable_fast_math, num_groups));
+    Impl &s = *_impl;
+    if (s.handle)
+    {
+        mi355_conv_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.src = input, s.weights = weights, s.biases = biases, s.dst = output, s.act = act_info;
+    s.is_prepared = false;
+    fill_conv_desc(ii, wi, output->info(), conv_info, dilation, act_info, s.desc, s.multipliers, s.shifts);
+    check_abi(mi355_conv_create(&s.desc, &s.handle), "NEGEMMConvolutionLayer::configure");
 }
 
 void NEGEMMConvolutionLayer::prepare()
@@ -759,20 +810,7 @@ void NEGEMMConvolutionLayer::update_quantization_parameters()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "update_quantization_parameters() before configure()");
-    GEMMLowpOutputStageInfo stage;
-    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(s.src->info(), s.weights->info(), s.dst->info(), s.act, stage));
-    const int32_t in_zp   = s.src->info()->quantization_info().uniform().offset;
-    s.desc.src_offset     = -in_zp;
-    s.desc.pad_value      = in_zp;
-    s.desc.weights_offset = is_data_type_quantized_per_channel(s.weights->info()->data_type())
-                                ? 0
-                                : -s.weights->info()->quantization_info().uniform().offset;
-    s.desc.requant = make_requant(stage);
-    if (stage.is_quantized_per_channel)
-    {
-        s.multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + s.desc.OFM);
-        s.shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + s.desc.OFM);
-    }
+    refresh_conv_quant(s.src->info(), s.weights->info(), s.dst->info(), s.act, s.desc, s.multipliers, s.shifts);
     check_abi(mi355_conv_update_quant(s.handle, s.desc.src_offset, s.desc.weights_offset, s.desc.pad_value,
                                       &s.desc.requant, s.multipliers.empty() ? nullptr : s.multipliers.data(),
                                       s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
@@ -1222,6 +1260,119 @@ void CpuGEMMLowp::run(ITensorPack &tensors)
         bias_f32 = reinterpret_cast<const float *>(first_element(c));
     }
     check_abi(mi355_gemmlowp_run(s.handle, first_element(a), bias_f32, first_element(dst), nullptr), "CpuGEMMLowp::run");
+}
+
+// =====================================================================================================================
+// experimental::op::CpuGemmConv2d
+// =====================================================================================================================
+struct CpuGemmConv2d::Impl
+{
+    mi355_conv_desc      desc{};
+    mi355_conv_handle   *handle{nullptr};
+    ActivationLayerInfo  act{};
+    bool                 is_prepared{false};
+    bool                 has_bias{false};
+    std::vector<int32_t> multipliers, shifts;
+
+    ~Impl()
+    {
+        if (handle)
+            mi355_conv_destroy(handle);
+    }
+};
+
+CpuGemmConv2d::CpuGemmConv2d() : _impl(std::make_unique<Impl>()) {}
+CpuGemmConv2d::~CpuGemmConv2d() = default;
+
+MemoryRequirements CpuGemmConv2d::workspace() const
+{
+    return {}; // packed weights, the lowered patch matrix (when one is needed) and staging buffers belong to the handle
+}
+
+Status CpuGemmConv2d::validate(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *biases,
+                               const ITensorInfo *output, const PadStrideInfo &conv_info, const WeightsInfo &weights_info,
+                               const Size2D &dilation, const ActivationLayerInfo &act_info, bool enable_fast_math,
+                               unsigned int num_groups)
+{
+    return NEGEMMConvolutionLayer::validate(src, weights, biases, output, conv_info, weights_info, dilation, act_info,
+                                            enable_fast_math, num_groups);
+}
+
+Status CpuGemmConv2d::has_opt_impl(arm_compute::WeightFormat &expected_weight_format, const ITensorInfo *src,
+                                   const ITensorInfo *weights, const ITensorInfo *biases, const ITensorInfo *output,
+                                   const PadStrideInfo &conv_info, const WeightsInfo &weights_info, const Size2D &dilation,
+                                   const ActivationLayerInfo &act_info, bool enable_fast_math)
+{
+    return NEGEMMConvolutionLayer::has_opt_impl(expected_weight_format, src, weights, biases, output, conv_info,
+                                                weights_info, dilation, act_info, enable_fast_math);
+}
+
+void CpuGemmConv2d::configure(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *biases,
+                              ITensorInfo *dst, const PadStrideInfo &conv_info, const WeightsInfo &weights_info,
+                              const Size2D &dilation, const ActivationLayerInfo &act_info, bool enable_fast_math,
+                              unsigned int num_groups)
+{
+    ARM_COMPUTE_ERROR_ON_NULLPTR(src, weights, dst);
+    conv_auto_init_output(src, weights, dst, conv_info, dilation);
+    ARM_COMPUTE_ERROR_THROW_ON(
+        validate(src, weights, biases, dst, conv_info, weights_info, dilation, act_info, enable_fast_math, num_groups));
+    Impl &s = *_impl;
+    if (s.handle)
+    {
+        mi355_conv_destroy(s.handle);
+        s.handle = nullptr;
+    }
+    s.act = act_info, s.is_prepared = false, s.has_bias = biases != nullptr;
+    fill_conv_desc(src, weights, dst, conv_info, dilation, act_info, s.desc, s.multipliers, s.shifts);
+    check_abi(mi355_conv_create(&s.desc, &s.handle), "CpuGemmConv2d::configure");
+}
+
+void CpuGemmConv2d::prepare(ITensorPack &tensors)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "CpuGemmConv2d::prepare() before configure()");
+    if (s.is_prepared)
+        return;
+    const ITensor *w = tensors.get_const_tensor(ACL_SRC_1);
+    ARM_COMPUTE_ERROR_ON_MSG(w == nullptr || w->buffer() == nullptr, "weights (ACL_SRC_1) are missing or have no memory");
+    const int32_t *bias = nullptr;
+    if (s.has_bias)
+    {
+        const ITensor *b = tensors.get_const_tensor(ACL_SRC_2);
+        ARM_COMPUTE_ERROR_ON_MSG(b == nullptr || b->buffer() == nullptr, "biases (ACL_SRC_2) are missing or have no memory");
+        bias = reinterpret_cast<const int32_t *>(first_element(b));
+    }
+    check_abi(mi355_conv_prepare(s.handle, first_element(w), bias, s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                 s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "CpuGemmConv2d::prepare");
+    w->mark_as_unused();
+    s.is_prepared = true;
+}
+
+void CpuGemmConv2d::update_quantization_parameters(ITensorPack &tensors)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "update_quantization_parameters() before configure()");
+    const ITensor *src = tensors.get_const_tensor(ACL_SRC_0), *w = tensors.get_const_tensor(ACL_SRC_1);
+    const ITensor *dst = tensors.get_const_tensor(ACL_DST);
+    ARM_COMPUTE_ERROR_ON_MSG(src == nullptr || w == nullptr || dst == nullptr, "ACL_SRC_0 / ACL_SRC_1 / ACL_DST missing");
+    refresh_conv_quant(src->info(), w->info(), dst->info(), s.act, s.desc, s.multipliers, s.shifts);
+    check_abi(mi355_conv_update_quant(s.handle, s.desc.src_offset, s.desc.weights_offset, s.desc.pad_value, &s.desc.requant,
+                                      s.multipliers.empty() ? nullptr : s.multipliers.data(),
+                                      s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
+              "CpuGemmConv2d::update_quantization_parameters");
+}
+
+void CpuGemmConv2d::run(ITensorPack &tensors)
+{
+    Impl &s = *_impl;
+    ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "CpuGemmConv2d::run() before configure()");
+    const ITensor *src = tensors.get_const_tensor(ACL_SRC_0);
+    ITensor       *dst = tensors.get_tensor(ACL_DST);
+    ARM_COMPUTE_ERROR_ON_MSG(src == nullptr || dst == nullptr || src->buffer() == nullptr || dst->buffer() == nullptr,
+                             "ACL_SRC_0 / ACL_DST missing or without memory");
+    prepare(tensors);
+    check_abi(mi355_conv_run(s.handle, first_element(src), first_element(dst), nullptr), "CpuGemmConv2d::run");
 }
 } // namespace op
 } // namespace experimental

@@ -178,6 +178,15 @@ typedef struct mi355_output_stage_desc
 int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *src, const int32_t *bias, void *dst,
                            void *stream);
 
+typedef enum mi355_conv_layout
+{
+    MI355_NHWC = 0, /* src [batch][H][W][C], weights [OFM][KH][KW][C], dst [batch][OH][OW][OFM] */
+    /* src [batch][C][H][W], weights [OFM][C][KH][KW], dst [batch][OFM][OH][OW]: the reference's other layout
+     * (im2col over channel planes + CpuCol2ImKernel, src/cpu/operators/CpuGemmConv2d.cpp:556-621; same integers).
+     * Converted to and from NHWC on the device around the same kernels: one extra pass over src and dst. */
+    MI355_NCHW = 1
+} mi355_conv_layout;
+
 /* Quantized NHWC convolution lowered to GEMM. Replaces CpuGemmConv2d::{configure,prepare,run}
  * (src/cpu/operators/CpuGemmConv2d.cpp:461-651, :1011-1101, :923-1008): CpuIm2ColKernel + CpuWeightsReshapeKernel
  * + CpuGemmLowpMatrixMultiplyCore. src is [batch][H][W][C], weights [OFM][KH][KW][C], dst [batch][OH][OW][OFM].
@@ -193,7 +202,7 @@ typedef struct mi355_conv_desc
     int32_t       pad_value;
     mi355_requant requant;
     int32_t       path; /* 0 auto (implicit GEMM where the shape allows), 1 force explicit im2col + GEMM */
-    int32_t       reserved;
+    int32_t       layout; /* mi355_conv_layout of src, weights and dst */
 } mi355_conv_desc;
 
 typedef struct mi355_conv_handle mi355_conv_handle;

@@ -6,6 +6,7 @@
 #include "arm_compute/core/utils/quantization/AsymmHelpers.h"
 #include "arm_compute/runtime/NEON/NEFunctions.h"
 #include "arm_compute/runtime/experimental/operators/CpuGEMMLowp.h"
+#include "arm_compute/runtime/experimental/operators/CpuGemmConv2d.h"
 #include "arm_compute/runtime/Tensor.h"
 #include "gemmlowp_oracle.h"
 
@@ -467,6 +468,48 @@ static void test_gemmlowp_accumulate_and_3d()
         init_tensor(flat, TensorShape(N, W * H, batch), DataType::S32);
         EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), nullptr, flat.info(),
                                                             GEMMInfo(false, false, true, 0, true))));
+    }
+}
+
+// dynamic quantization info: offsets (and the F32 path's scale) are read again on every run
+// (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:668-674,758-784; the fixture sets it after configure,
+// tests/validation/fixtures/GEMMLowpFixture.h:171-185)
+static void test_gemmlowp_dynamic_qinfo()
+{
+    SECTION("NEGEMMLowpMatrixMultiplyCore with dynamic quantization info (S32 and F32 destinations)");
+    const int M = 19, N = 33, K = 48;
+    for (int f32 = 0; f32 < 2; ++f32)
+    {
+        Tensor a, b, dst;
+        init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f, 0, true));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f, 0, true));
+        init_tensor(dst, TensorShape(N, M), f32 ? DataType::F32 : DataType::S32);
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(a, -128, 127, 90 + f32), fill_uniform<int8_t>(b, -128, 127, 92 + f32);
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, GEMMInfo(false, false, true));
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        const struct { float sa, sb; int ao, bo; } steps[] = {{0.5f, 0.25f, 0, 0}, {0.02f, 0.005f, 7, -4}, {0.1f, 0.005f, 7, -4},
+                                                              {0.1f, 0.3f, -11, 0}};
+        for (const auto &st : steps)
+        {
+            a.info()->set_quantization_info(QuantizationInfo(st.sa, st.ao, true));
+            b.info()->set_quantization_info(QuantizationInfo(st.sb, st.bo, true));
+            gemm.run();
+            if (f32)
+            {
+                std::vector<float> want(M * N);
+                orc_gemmlowp_f32(A.data(), 1, K, B.data(), 1, N, nullptr, want.data(), N, M, N, K, st.ao, st.bo, st.sa * st.sb,
+                                 -INFINITY, INFINITY, 0, 0);
+                EXPECT(dense_copy<float>(dst) == want);
+            }
+            else
+            {
+                std::vector<int32_t> want(M * N);
+                orc_gemmlowp_s32(A.data(), 1, K, B.data(), 1, N, want.data(), N, M, N, K, st.ao, st.bo);
+                EXPECT(dense_copy<int32_t>(dst) == want);
+            }
+        }
     }
 }
 
@@ -933,6 +976,99 @@ static void test_stateless_operator()
     EXPECT(dense_copy<int8_t>(dst2) == want);
 }
 
+// the channel-planar layout through NEGEMMConvolutionLayer and the stateless operator on an ITensorPack: both against
+// the oracle's direct convolution of the same data in NHWC order
+static void test_convolution_nchw_and_stateless()
+{
+    SECTION("NEGEMMConvolutionLayer NCHW; experimental::op::CpuGemmConv2d on an ITensorPack");
+    const int batch = 2, H = 10, W = 7, C = 16, OFM = 20, KH = 3, KW = 2, in_zp = 3, out_zp = -4;
+    std::mt19937 rng(140);
+    std::uniform_int_distribution<int> u8(-128, 127), uw(-127, 127), ub(-400, 400);
+    std::uniform_real_distribution<float> us(0.0005f, 0.05f);
+    std::vector<int8_t> src_nhwc(batch * H * W * C), w_nhwc(OFM * KH * KW * C);
+    std::vector<int32_t> biasv(OFM);
+    std::vector<float> wscale(OFM);
+    for (auto &v : src_nhwc) v = (int8_t)u8(rng);
+    for (auto &v : w_nhwc) v = (int8_t)uw(rng);
+    for (auto &v : biasv) v = ub(rng);
+    for (auto &v : wscale) v = us(rng);
+    const PadStrideInfo psi(2, 1, 1, 0, 2, 1, DimensionRoundingType::FLOOR); // stride (2,1), pad l1 r0 t2 b1
+    int OH = 0, OW = 0;
+    orc_conv_out_dims(H, W, KH, KW, 2, 1, 1, 2, 0, 1, 1, 1, &OH, &OW);
+    const QuantizationInfo iq(0.02f, in_zp), wq(wscale), oq(0.7f, out_zp);
+    GEMMLowpOutputStageInfo st;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(iq, wq, oq, st)));
+    std::vector<int8_t> want(batch * OH * OW * OFM);
+    auto expect = [&](const GEMMLowpOutputStageInfo &stage, int ozp)
+    {
+        orc_conv_nhwc_direct(src_nhwc.data(), 1, w_nhwc.data(), 1, biasv.data(), want.data(), 1, batch, H, W, C, OFM, KH, KW, 2,
+                             1, 1, 2, 0, 1, 1, 1, in_zp, 0, stage.gemmlowp_multipliers.data(), stage.gemmlowp_shifts.data(), OFM,
+                             ozp, -128, 127);
+    };
+    expect(st, out_zp);
+    {
+        Tensor src, w, bias, dst;
+        init_tensor(src, TensorShape(W, H, C, batch), DataType::QASYMM8_SIGNED, iq);
+        init_tensor(w, TensorShape(KW, KH, C, OFM), DataType::QSYMM8_PER_CHANNEL, wq);
+        init_tensor(bias, TensorShape(OFM), DataType::S32);
+        init_tensor(dst, TensorShape(), DataType::QASYMM8_SIGNED, oq);
+        for (Tensor *t : {&src, &w, &dst})
+            t->info()->set_data_layout(DataLayout::NCHW);
+        NEGEMMConvolutionLayer conv;
+        conv.configure(&src, &w, &bias, &dst, psi);
+        EXPECT(dst.info()->dimension(0) == (size_t)OW && dst.info()->dimension(1) == (size_t)OH &&
+               dst.info()->dimension(2) == (size_t)OFM && dst.info()->dimension(3) == (size_t)batch);
+        src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+        for (int n = 0; n < batch; ++n)
+            for (int c = 0; c < C; ++c)
+                for (int y = 0; y < H; ++y)
+                    for (int x = 0; x < W; ++x)
+                        reinterpret_cast<int8_t *>(src.buffer())[((n * C + c) * H + y) * W + x] = src_nhwc[((n * H + y) * W + x) * C + c];
+        for (int o = 0; o < OFM; ++o)
+            for (int c = 0; c < C; ++c)
+                for (int t = 0; t < KH * KW; ++t)
+                    reinterpret_cast<int8_t *>(w.buffer())[(o * C + c) * KH * KW + t] = w_nhwc[(o * KH * KW + t) * C + c];
+        std::memcpy(bias.buffer(), biasv.data(), sizeof(int32_t) * OFM);
+        conv.run();
+        bool ok = true;
+        for (int n = 0; n < batch; ++n)
+            for (int o = 0; o < OFM; ++o)
+                for (int p = 0; p < OH * OW; ++p)
+                    ok = ok && reinterpret_cast<const int8_t *>(dst.buffer())[(n * OFM + o) * OH * OW + p] == want[(n * OH * OW + p) * OFM + o];
+        EXPECT(ok);
+        std::printf("       kernel: %s\n", conv.kernel_name());
+    }
+    {
+        TensorInfo si(TensorShape(C, W, H, batch), 1, DataType::QASYMM8_SIGNED, iq), wi(TensorShape(C, KW, KH, OFM), 1, DataType::QSYMM8_PER_CHANNEL, wq);
+        TensorInfo bi(TensorShape(OFM), 1, DataType::S32), di(TensorShape(), 1, DataType::QASYMM8_SIGNED, oq);
+        si.set_data_layout(DataLayout::NHWC), wi.set_data_layout(DataLayout::NHWC), di.set_data_layout(DataLayout::NHWC);
+        experimental::op::CpuGemmConv2d op;
+        op.configure(&si, &wi, &bi, &di, psi);
+        EXPECT(di.dimension(0) == (size_t)OFM && di.dimension(1) == (size_t)OW && di.dimension(2) == (size_t)OH);
+        EXPECT(bool(experimental::op::CpuGemmConv2d::validate(&si, &wi, &bi, &di, psi)));
+        EXPECT(op.workspace().empty());
+        Tensor src, w, bias, dst;
+        src.allocator()->init(si), w.allocator()->init(wi), bias.allocator()->init(bi), dst.allocator()->init(di);
+        src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+        std::memcpy(src.buffer(), src_nhwc.data(), src_nhwc.size());
+        std::memcpy(w.buffer(), w_nhwc.data(), w_nhwc.size());
+        std::memcpy(bias.buffer(), biasv.data(), sizeof(int32_t) * OFM);
+        ITensorPack pack{{ACL_SRC_0, &src}, {ACL_SRC_1, &w}, {ACL_SRC_2, &bias}, {ACL_DST, &dst}};
+        op.run(pack);
+        EXPECT(dense_copy<int8_t>(dst) == want);
+        EXPECT(!w.is_used());
+        // the output's quantization changes after configure: re-derived from the pack's tensors, weights stay packed
+        const QuantizationInfo oq2(1.3f, out_zp + 7);
+        dst.info()->set_quantization_info(oq2);
+        op.update_quantization_parameters(pack);
+        op.run(pack);
+        GEMMLowpOutputStageInfo st2;
+        EXPECT(bool(quantization::calculate_quantized_multipliers(iq, wq, oq2, st2)));
+        expect(st2, out_zp + 7);
+        EXPECT(dense_copy<int8_t>(dst) == want);
+    }
+}
+
 static void test_error_paths()
 {
     SECTION("configure() throws on invalid input; run() before configure() throws");
@@ -983,6 +1119,7 @@ int main(int argc, char **argv)
             test_gemmlowp_fused_u8(true);
             test_gemmlowp_s32_batched();
             test_gemmlowp_accumulate_and_3d();
+            test_gemmlowp_dynamic_qinfo();
             test_gemmlowp_per_channel_and_update();
             test_gemmlowp_f32();
             test_output_stage();
@@ -994,6 +1131,7 @@ int main(int argc, char **argv)
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
             test_gemm_conv2d();
             test_stateless_operator();
+            test_convolution_nchw_and_stateless();
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);

@@ -11,20 +11,24 @@ CODE = {np.dtype(np.uint8): capi.U8, np.dtype(np.int8): capi.S8}
 
 
 def run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dilation=(1, 1), path=0,
-             device=True):
+             device=True, layout=capi.NHWC):
+    """src [batch][H][W][C], w [OFM][KH][KW][C]; with layout NCHW they are handed over (and the result comes back)
+    channel-planar, and the NHWC view of the result is returned"""
     B_, H, W, C = src.shape
     OFM, KH, KW, _ = w.shape
+    if layout == capi.NCHW:
+        src, w = np.ascontiguousarray(src.transpose(0, 3, 1, 2)), np.ascontiguousarray(w.transpose(0, 3, 1, 2))
     pc = len(np.atleast_1d(mult)) > 1
     rq = capi.requant(0 if pc else int(np.atleast_1d(mult)[0]), 0 if pc else int(np.atleast_1d(shift)[0]), out_zp, lo,
                       hi, pc)
     d = capi.conv_desc(B_, H, W, C, OFM, KH, KW, stride, pad, dilation, CODE[src.dtype], CODE[w.dtype],
-                       CODE[src.dtype], -in_zp, -w_zp, in_zp, rq, path)
+                       CODE[src.dtype], -in_zp, -w_zp, in_zp, rq, path, layout)
     cv = capi.Conv(d)
     OH, OW = cv.out_dims()
     m = np.ascontiguousarray(mult, dtype=np.int32) if pc else None
     s = np.ascontiguousarray(shift, dtype=np.int32) if pc else None
     b = np.ascontiguousarray(bias, dtype=np.int32)
-    out = np.zeros((B_, OH, OW, OFM), dtype=src.dtype)
+    out = np.zeros((B_, OH, OW, OFM) if layout == capi.NHWC else (B_, OFM, OH, OW), dtype=src.dtype)
     if device:
         import torch
         sd, wd, od = to_dev(src), to_dev(w), to_dev(out)
@@ -38,6 +42,8 @@ def run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad
         cv.run(np.ascontiguousarray(src), out)
     name = cv.kernel_name
     cv.close()
+    if layout == capi.NCHW:
+        out = out.transpose(0, 2, 3, 1)
     return out, name
 
 
@@ -100,3 +106,24 @@ def test_conv_seeded_strides_dilation_uint8():
             got, _ = run_conv(src, w, bias, zp, 0, mult, shift, -5 if dt == np.int8 else 9, lo, hi, stride, pad, dil,
                               path=path)
             np.testing.assert_array_equal(got, want)
+        # the channel-planar layout gives the same integers (the reference's NCHW im2col only orders K differently)
+        for device in (True, False):
+            announce("conv seeded NCHW", shape, wshape, stride, pad, dil, "device", device)
+            got, _ = run_conv(src, w, bias, zp, 0, mult, shift, -5 if dt == np.int8 else 9, lo, hi, stride, pad, dil,
+                              device=device, layout=capi.NCHW)
+            np.testing.assert_array_equal(got, want)
+
+
+def test_conv_nchw_fixture(golden):
+    """The reference oracle's outputs (tests/golden/conv_nhwc.npz) with every tensor handed over channel-planar"""
+    g = golden("conv_nhwc.npz")
+    for n in range(int(g["count"])):
+        sx, sy, pl, pt, pr, pb, in_zp, w_zp, out_zp, pc = (int(x) for x in g["p%d" % n])
+        src, w, bias, want = g["src%d" % n], g["w%d" % n], g["bias%d" % n], g["dst%d" % n]
+        in_scale, out_scale = g["scales%d" % n]
+        mult, shift = oracle.calculate_quantized_multipliers(in_scale, g["wscale%d" % n], out_scale)
+        lo, hi = (-128, 127) if src.dtype == np.int8 else (0, 255)
+        announce("conv NCHW fixture", n, src.shape, w.shape)
+        got, _ = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, (sx, sy), (pl, pt, pr, pb),
+                          layout=capi.NCHW)
+        np.testing.assert_array_equal(got, want)

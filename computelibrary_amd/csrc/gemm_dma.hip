@@ -10,9 +10,13 @@
 // one contiguous segment per row. The loads are issued from inline assembly with hand-placed s_waitcnt vmcnt(n): the
 // compiler cannot tell which stage a direct-to-LDS load writes and would force vmcnt(0) before every LDS read.
 //
-// Roles: a block has 8 consumer waves and 4 producer waves (3 waves per SIMD). The producers do nothing but issue the
-// direct-to-LDS loads: such a load occupies its wave for as long as the texture addresser takes to accept it (about 18
-// clocks per 1 KiB on this part), which would otherwise stall the wave's matrix instructions.
+// Roles: a block has 8 consumer waves and 4 producer waves (3 waves per SIMD). The producers do nothing but issue
+// direct-to-LDS loads: such a load occupies its wave for as long as the texture addresser takes to accept it (about 23
+// clocks per 1 KiB for the whole compute unit, i.e. about 90 for a wave that shares it with three others), which
+// would otherwise stall the wave's matrix instructions. A K step needs (BM + BN) * BK / 1024 of them - for the
+// 256 x 128 x 128 tile 48, as many clocks as the step's matrix instructions take - so the addresser must not idle while
+// the producers wait in a barrier: for dense tiles the consumers stage the (edge-free, zero-padded) B panel themselves
+// in their operand-read slot, and the producers only the A panel.
 //
 // LDS -> matrix cores: the consumers form two groups of four (one wave of each group per SIMD) that run half a K step
 // apart ("ping-pong"): while one group streams its 16 matrix instructions for a K step out of registers, the other
@@ -215,6 +219,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     constexpr int KK    = BK / 32;
     constexpr int STAGE = (BM + BN) * BK;
     static_assert((AU + BU) % NP == 0, "staging shape");
+    // Dense tiles: inside the K loop the consumers stage the B panel themselves (CBU units per wave and K step, issued
+    // while their operand reads are in flight) and the producers only the A panel. The block's direct-to-LDS loads then
+    // come from all 12 waves instead of 4 and keep flowing while the producers sit in a barrier.
+    constexpr bool CDMA = !CONV && (BU % NW == 0) && (AU % NP == 0) && (AU / NP) % 2 == 0;
+    constexpr int  CBU  = CDMA ? BU / NW : 0;   // B units per consumer wave per stage
+    constexpr int  PLP  = CDMA ? AU / NP : LPP; // loads per producer wave per stage inside the loop
     static_assert(TM % 32 == 0 && TN % 32 == 0 && FM >= 1 && FN >= 1, "wave tile");
     static_assert(NS >= 3 && (NS - 2) * LPP < 64, "ring depth / vmcnt range");
     static_assert(NW * 32 * (FN * 128 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
@@ -256,12 +266,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
             // consumer groups wait for all of them. Ring slot of stage kt-1: free since barrier 2kt.
             const bool more = kt + NS - 1 < nk;
             if (more)
-                prod.template issue<0, LPP / 2>(kt + NS - 1, (kt + NS - 1) % NS);
+                prod.template issue<0, PLP / 2>(kt + NS - 1, (kt + NS - 1) % NS);
             block_barrier(); // barrier 2kt+1
             if (more)
-                prod.template issue<LPP / 2, LPP>(kt + NS - 1, (kt + NS - 1) % NS);
+                prod.template issue<PLP / 2, PLP>(kt + NS - 1, (kt + NS - 1) % NS);
             if (more)
-                wait_vmcnt<(NS - 2) * LPP>(); // stage kt+1 complete
+                wait_vmcnt<(NS - 2) * PLP>(); // this wave's part of stage kt+1 complete
             else
                 wait_vmcnt<0>();
             block_barrier(); // barrier 2kt+2
@@ -330,6 +340,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         b_sw[f]       = swz<CPR>(row);
     }
 
+    // this wave's share of the B panel (CDMA): units wave + i*NW, which all have the lane -> column map of unit `wave`
+    const int8_t  *cb_base = g.Bp + (int64_t)bz * g.bp_batch_stride + (int64_t)n0 * g.Kp + (int64_t)wave * RPU * g.Kp;
+    const uint32_t cb_lane = (uint32_t)(lane / CPR) * (uint32_t)g.Kp +
+                             (uint32_t)(((lane % CPR) ^ swz<CPR>(wave * RPU + lane / CPR)) * 16);
+    const uint32_t cb_lds  = lds0 + (uint32_t)(AU + wave) * 1024u;
+
     block_barrier(); // barrier 0: stage 0 is in LDS
     if (group == 1)
         block_barrier(); // group 1 runs one slot behind group 0
@@ -349,6 +365,15 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
             for (int f = 0; f < FN; ++f)
                 fb[kk][f] = *(const v4i *)(s + b_rd[f] + (((kk * 2 + lh) ^ b_sw[f]) << 4));
         }
+        if (CDMA && kt + NS - 1 < nk)
+        {
+            // stage kt+NS-1 goes into the ring slot of stage kt-1, whose last reader finished before barrier 2kt
+            const int st = kt + NS - 1;
+#pragma unroll
+            for (int i = 0; i < CBU; ++i)
+                dma16s(cb_base + (int64_t)st * BK + (int64_t)i * NW * RPU * g.Kp, cb_lane,
+                       cb_lds + (uint32_t)(st % NS) * STAGE + (uint32_t)(i * NW) * 1024u);
+        }
         if (FLIP_A)
         {
 #pragma unroll
@@ -358,6 +383,15 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
                     fa[kk][f] ^= (int)0x80808080;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // the units this wave issued one K step ago (stage kt+NS-2) have to be in LDS before the barrier that opens
+        // that stage to its first reader; only the CBU just issued may still be in flight
+        if (CDMA)
+        {
+            if (kt + NS - 1 < nk)
+                wait_vmcnt<CBU>();
+            else
+                wait_vmcnt<0>();
+        }
         __builtin_amdgcn_sched_barrier(0);
         block_barrier();
 
@@ -372,6 +406,8 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         __builtin_amdgcn_sched_barrier(0);
         block_barrier();
     }
+    if (CDMA)
+        wait_vmcnt<0>();
     if (group == 0)
         block_barrier(); // barrier 2nk+1; every operand read of every wave is complete beyond this point
 

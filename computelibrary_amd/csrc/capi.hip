@@ -738,6 +738,13 @@ static int conv_check(const mi355_conv_desc &d)
         return fail("convolution tensors must be 8-bit");
     if (d.layout != MI355_NHWC && d.layout != MI355_NCHW)
         return fail("unknown layout %d", d.layout);
+    if ((d.src_pixel_stride != 0 && d.src_pixel_stride < d.C) || (d.weights_pixel_stride != 0 && d.weights_pixel_stride < d.C) ||
+        (d.dst_pixel_stride != 0 && d.dst_pixel_stride < d.OFM))
+        return fail("pixel stride smaller than the pixel");
+    if (d.layout != MI355_NHWC && ((d.src_pixel_stride != 0 && d.src_pixel_stride != d.C) ||
+                                   (d.weights_pixel_stride != 0 && d.weights_pixel_stride != d.C) ||
+                                   (d.dst_pixel_stride != 0 && d.dst_pixel_stride != d.OFM)))
+        return fail("pixel strides are an NHWC notion");
     return 0;
 }
 
@@ -790,7 +797,16 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t 
     hipStream_t s = (hipStream_t)stream;
     GemmCore   &c = h->core;
     const void *wd, *biasd, *multd, *shiftd;
-    TRY(to_device(weights, (size_t)c.N * c.K, h->stageW, s, &wd));
+    const int64_t wps   = h->d.weights_pixel_stride;
+    const int64_t wtaps = (int64_t)c.N * h->d.KH * h->d.KW;
+    const bool    w_pad = wps != 0 && wps != h->d.C;
+    TRY(to_device(weights, w_pad ? (size_t)((wtaps - 1) * wps + h->d.C) : (size_t)c.N * c.K, h->stageW, s, &wd));
+    if (w_pad)
+    {
+        TRY(h->nhwcW.ensure((size_t)c.N * c.K));
+        HIP_TRY(restride_launch(wd, h->nhwcW.p, wtaps, h->d.C, wps, h->d.C, s));
+        wd = h->nhwcW.p;
+    }
     if (h->d.layout == MI355_NCHW)
     {
         // [OFM][C][KH*KW] -> [OFM][KH*KW][C]
@@ -855,15 +871,33 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     const mi355_conv_desc &d = h->d;
     if (!c.prepared)
         return fail("run before prepare");
-    const size_t src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N;
-    const void  *srcd;
-    TRY(to_device(src, src_bytes, h->stageSrc, s, &srcd));
+    const size_t  src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N;
+    const int64_t pixels    = (int64_t)d.batch * d.H * d.W;
+    const bool    s_pad     = d.src_pixel_stride != 0 && d.src_pixel_stride != d.C;
+    const bool    d_pad     = d.dst_pixel_stride != 0 && d.dst_pixel_stride != d.OFM;
+    const size_t  dst_ext   = d_pad ? (size_t)((int64_t)(c.M - 1) * d.dst_pixel_stride + c.N) : dst_bytes;
+    const void   *srcd;
+    TRY(to_device(src, s_pad ? (size_t)((pixels - 1) * d.src_pixel_stride + d.C) : src_bytes, h->stageSrc, s, &srcd));
+    if (s_pad)
+    {
+        TRY(h->nhwcSrc.ensure(src_bytes));
+        HIP_TRY(restride_launch(srcd, h->nhwcSrc.p, pixels, d.C, d.src_pixel_stride, d.C, s));
+        srcd = h->nhwcSrc.p;
+    }
     const bool d_host = !is_device_ptr(dst);
     void      *Dd     = dst;
     if (d_host)
     {
-        TRY(h->stageDst.ensure(dst_bytes));
+        TRY(h->stageDst.ensure(dst_ext));
         Dd = h->stageDst.p;
+        if (d_pad)
+            HIP_TRY(hipMemcpyAsync(Dd, dst, dst_ext, hipMemcpyHostToDevice, s)); // keep the caller's padding bytes
+    }
+    void *Dpadded = Dd;
+    if (d_pad)
+    {
+        TRY(h->nhwcDst.ensure(dst_bytes));
+        Dd = h->nhwcDst.p;
     }
     const bool nchw   = d.layout == MI355_NCHW;
     void      *Dfinal = Dd;
@@ -903,9 +937,14 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         HIP_TRY(transpose_bytes_launch(Dd, Dfinal, d.batch, h->geom.OH * h->geom.OW, c.N, s));
         Dd = Dfinal;
     }
+    if (d_pad)
+    {
+        HIP_TRY(restride_launch(Dd, Dpadded, c.M, c.N, c.N, d.dst_pixel_stride, s));
+        Dd = Dpadded;
+    }
     if (d_host)
     {
-        HIP_TRY(hipMemcpyAsync(dst, Dd, dst_bytes, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipMemcpyAsync(dst, Dd, dst_ext, hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
     }
     else if (!is_device_ptr(src))

@@ -119,6 +119,9 @@ int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *b
                             int N, const EpiParams &epi, hipStream_t s);
 // [batch][R][C] bytes -> [batch][C][R]
 int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
+// dst[s * dst_stride + c] = src[s * src_stride + c] for s < segments, c < seg (bytes)
+int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64_t src_stride, int64_t dst_stride,
+                    hipStream_t s);
 int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);
 // one thread per output; A dense [M][lda] (unflipped or flipped per flip_a), Bp packed
 int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s);

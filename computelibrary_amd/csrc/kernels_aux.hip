@@ -510,6 +510,32 @@ int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, 
     return launch_status();
 }
 
+// ---- segment gather / scatter: dst[s * dst_stride + c] = src[s * src_stride + c], c < seg ------------------------------
+// Tensors that carry padding along the channel dimension (pixels seg bytes long, src_stride apart) to dense and back.
+__global__ __launch_bounds__(256) void restride_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                       int64_t segments, int seg, int64_t src_stride, int64_t dst_stride)
+{
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= segments * seg)
+        return;
+    const int64_t sgm = idx / seg;
+    const int     c   = (int)(idx - sgm * seg);
+    dst[sgm * dst_stride + c] = src[sgm * src_stride + c];
+}
+
+int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64_t src_stride, int64_t dst_stride,
+                    hipStream_t s)
+{
+    if (segments <= 0 || seg <= 0)
+        return 0;
+    const int64_t total = segments * seg;
+    if ((total + 255) / 256 > 0x7FFFFFFF)
+        return (int)hipErrorInvalidValue;
+    restride_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)src, (uint8_t *)dst,
+                                                                                 segments, seg, src_stride, dst_stride);
+    return launch_status();
+}
+
 // ---- one thread per output: the plainest possible statement of the path, for cross-checking only ----------------------
 template <int EPI>
 __global__ __launch_bounds__(256) void simple_gemm_kernel(GemmArgs g, uint8_t flip)

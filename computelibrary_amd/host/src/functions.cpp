@@ -348,10 +348,39 @@ void NEGEMMLowpMatrixMultiplyCore::configure(const ITensor *a, const ITensor *b,
     check_abi(mi355_gemmlowp_create(&d, &s.handle), "NEGEMMLowpMatrixMultiplyCore::configure");
 }
 
+namespace
+{
+// Padding may be added to a tensor between configure() and the first run (the reference's fixtures do exactly that:
+// tests/validation/fixtures/GEMMLowpFixture.h:300-304) and the reference reads strides when it runs. The strides are
+// part of the descriptor here: when they have changed, the handle is made again (nothing is packed yet in that flow).
+bool gemm_strides_changed(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorInfo *oi, const GEMMInfo &info,
+                          mi355_gemm_desc &d)
+{
+    mi355_gemm_desc       now;
+    std::vector<int32_t> m, sh;
+    fill_gemm_desc(ai, bi, oi, info, now, m, sh);
+    const bool changed = now.lda != d.lda || now.ldb != d.ldb || now.ldd != d.ldd || now.a_batch_stride != d.a_batch_stride ||
+                         now.b_batch_stride != d.b_batch_stride || now.d_batch_stride != d.d_batch_stride;
+    if (changed)
+        d.lda = now.lda, d.ldb = now.ldb, d.ldd = now.ldd, d.a_batch_stride = now.a_batch_stride,
+        d.b_batch_stride = now.b_batch_stride, d.d_batch_stride = now.d_batch_stride;
+    return changed;
+}
+} // namespace
+
 void NEGEMMLowpMatrixMultiplyCore::prepare()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMLowpMatrixMultiplyCore::prepare() before configure()");
+    if (gemm_strides_changed(s.a->info(), s.b->info(), s.output->info(), s.info, s.desc))
+    {
+        ARM_COMPUTE_ERROR_THROW_ON(validate(s.a->info(), s.b->info(), s.c != nullptr ? s.c->info() : nullptr,
+                                            s.output->info(), s.info));
+        mi355_gemmlowp_destroy(s.handle);
+        s.handle = nullptr;
+        check_abi(mi355_gemmlowp_create(&s.desc, &s.handle), "NEGEMMLowpMatrixMultiplyCore::prepare");
+        s.is_prepared = false;
+    }
     if (s.is_prepared)
         return;
     ARM_COMPUTE_ERROR_ON_MSG(s.b->buffer() == nullptr, "matrix B has no memory");
@@ -667,8 +696,20 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
         ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(dm.w) != conv_w || output->dimension(dm.h) != conv_h);
         ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(3) != input->dimension(3));
     }
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->has_padding() || weights->has_padding() || output->has_padding(),
-                                    "Padded tensors are not supported by the convolution of this library");
+    // padding along the channel dimension of NHWC tensors (what the reference's fixtures add: add_padding_x,
+    // tests/validation/Helpers.cpp:335-357) is taken as a pixel stride; anything else has to be dense
+    for (const ITensorInfo *t : {input, weights, output})
+    {
+        if (t->total_size() == 0)
+            continue;
+        if (input->data_layout() == DataLayout::NHWC)
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->strides_in_bytes()[2] != t->dimension(1) * t->strides_in_bytes()[1] ||
+                                                (t->num_dimensions() > 3 &&
+                                                 t->strides_in_bytes()[3] != t->dimension(2) * t->strides_in_bytes()[2]),
+                                            "Only padding along the channel dimension is supported by this convolution");
+        else
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->has_padding(), "Padded NCHW tensors are not supported by this convolution");
+    }
     GEMMLowpOutputStageInfo stage;
     ARM_COMPUTE_RETURN_ON_ERROR(conv_output_stage(input, weights, output, act_info, stage));
     return Status{};
@@ -739,6 +780,12 @@ void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorI
     d.pad_value = in_zp;
     d.requant   = make_requant(stage);
     d.path      = 0;
+    if (d.layout == MI355_NHWC)
+    {
+        d.src_pixel_stride     = static_cast<int64_t>(ii->strides_in_bytes()[1]);
+        d.weights_pixel_stride = static_cast<int64_t>(wi->strides_in_bytes()[1]);
+        d.dst_pixel_stride     = static_cast<int64_t>(oi->strides_in_bytes()[1]);
+    }
     if (stage.is_quantized_per_channel)
     {
         multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
@@ -790,10 +837,32 @@ void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weig
     check_abi(mi355_conv_create(&s.desc, &s.handle), "NEGEMMConvolutionLayer::configure");
 }
 
+namespace
+{
+// see gemm_strides_changed: the same for the convolution's pixel strides
+bool conv_strides_changed(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, mi355_conv_desc &d)
+{
+    if (d.layout != MI355_NHWC)
+        return false;
+    const int64_t sp = static_cast<int64_t>(ii->strides_in_bytes()[1]), wp = static_cast<int64_t>(wi->strides_in_bytes()[1]);
+    const int64_t dp = static_cast<int64_t>(oi->strides_in_bytes()[1]);
+    const bool    changed = sp != d.src_pixel_stride || wp != d.weights_pixel_stride || dp != d.dst_pixel_stride;
+    d.src_pixel_stride = sp, d.weights_pixel_stride = wp, d.dst_pixel_stride = dp;
+    return changed;
+}
+} // namespace
+
 void NEGEMMConvolutionLayer::prepare()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMConvolutionLayer::prepare() before configure()");
+    if (conv_strides_changed(s.src->info(), s.weights->info(), s.dst->info(), s.desc))
+    {
+        mi355_conv_destroy(s.handle);
+        s.handle = nullptr;
+        check_abi(mi355_conv_create(&s.desc, &s.handle), "NEGEMMConvolutionLayer::prepare");
+        s.is_prepared = false;
+    }
     if (s.is_prepared)
         return;
     ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");

@@ -203,6 +203,12 @@ typedef struct mi355_conv_desc
     mi355_requant requant;
     int32_t       path; /* 0 auto (implicit GEMM where the shape allows), 1 force explicit im2col + GEMM */
     int32_t       layout; /* mi355_conv_layout of src, weights and dst */
+    /* NHWC only: bytes from one pixel (one tap of the weights) to the next when the tensors carry padding along the
+     * channel dimension, as the reference's own fixtures give them (add_padding_x, tests/validation/Helpers.cpp:335-357;
+     * ITensorInfo::strides_in_bytes()[1]). Rows, planes and batches must follow without further gaps. 0 = dense (C, C,
+     * OFM). The pointers passed to prepare / run address the first element. Padded tensors are gathered into dense
+     * device buffers first (one extra pass) and the result is scattered into dst, leaving its padding untouched. */
+    int64_t       src_pixel_stride, weights_pixel_stride, dst_pixel_stride;
 } mi355_conv_desc;
 
 typedef struct mi355_conv_handle mi355_conv_handle;

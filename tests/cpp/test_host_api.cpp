@@ -341,17 +341,23 @@ static void test_gemmlowp_fused_u8(bool padded)
     SECTION(padded ? "NEGEMMLowpMatrixMultiplyCore fused QASYMM8 (x-padded tensors)" : "NEGEMMLowpMatrixMultiplyCore fused QASYMM8");
     const int   M = 72, N = 33, K = 52;
     Tensor      a, b, bias, dst;
-    const PaddingSize pad = padded ? PaddingSize(0, 5, 0, 3) : PaddingSize(0);
-    init_tensor(a, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(1.f / 255, -9), pad);
-    init_tensor(b, TensorShape(N, K), DataType::QASYMM8, QuantizationInfo(1.f / 255, 1), pad);
+    init_tensor(a, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(1.f / 255, -9));
+    init_tensor(b, TensorShape(N, K), DataType::QASYMM8, QuantizationInfo(1.f / 255, 1));
     init_tensor(bias, TensorShape(N), DataType::S32);
-    init_tensor(dst, TensorShape(N, M), DataType::QASYMM8, QuantizationInfo(0.3f, 10), pad);
+    init_tensor(dst, TensorShape(N, M), DataType::QASYMM8, QuantizationInfo(0.3f, 10));
     GEMMLowpOutputStageInfo st;
     st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
     st.gemmlowp_multiplier = 1518500250, st.gemmlowp_shift = 8, st.gemmlowp_offset = 10;
     st.gemmlowp_min_bound = 0, st.gemmlowp_max_bound = 255, st.output_data_type = DataType::QASYMM8;
     NEGEMMLowpMatrixMultiplyCore gemm;
     gemm.configure(&a, &b, &bias, &dst, GEMMInfo(false, false, true, 0, false, false, st));
+    if (padded)
+    {
+        // the order of the reference's fixture: configure, then add_padding_x, then allocate
+        // (tests/validation/fixtures/GEMMLowpFixture.h:289-310)
+        a.info()->extend_padding(PaddingSize(0, 5, 0, 3)), b.info()->extend_padding(PaddingSize(0, 11, 0, 2));
+        dst.info()->extend_padding(PaddingSize(0, 1, 0, 16)), bias.info()->extend_padding(PaddingSize(0, 3, 0, 4));
+    }
     a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
     fill_uniform<uint8_t>(a, 0, 255, 1), fill_uniform<uint8_t>(b, 0, 255, 2), fill_uniform<int32_t>(bias, -1000, 1000, 3);
     const auto A = dense_copy<uint8_t>(a), B = dense_copy<uint8_t>(b);
@@ -711,9 +717,12 @@ static void test_quantize_down_scale()
     }
 }
 
-static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act)
+// padded: src / weights / dst carry padding along x (the channels), as the reference's fixture adds it with
+// add_padding_x (tests/validation/fixtures/ConvolutionLayerFixture.h:464-469)
+static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act, bool padded = false)
 {
-    SECTION(per_channel ? "NEGEMMConvolutionLayer NHWC per-channel weights" : "NEGEMMConvolutionLayer NHWC per-tensor weights");
+    SECTION(padded ? "NEGEMMConvolutionLayer NHWC, tensors padded along x"
+                   : per_channel ? "NEGEMMConvolutionLayer NHWC per-channel weights" : "NEGEMMConvolutionLayer NHWC per-tensor weights");
     const bool is_signed = dt == DataType::QASYMM8_SIGNED;
     const int  batch = 2, H = 9, W = 8, OFM = 24, KH = 3, KW = 3;
     const int  in_zp = is_signed ? -1 : 127, out_zp = is_signed ? -5 : 9, w_zp = (per_channel || is_signed) ? 0 : 120;
@@ -733,6 +742,14 @@ static void test_convolution(DataType dt, bool per_channel, int C, const Activat
     NEGEMMConvolutionLayer conv;
     conv.configure(&src, &w, &bias, &dst, PadStrideInfo(1, 1, 1, 1), WeightsInfo(), Size2D(1, 1), act);
     EXPECT(dst.info()->dimension(0) == (size_t)OFM && dst.info()->dimension(1) == (size_t)W && dst.info()->dimension(2) == (size_t)H);
+    if (padded)
+    {
+        // after configure and before allocation, like the fixture: PaddingSize(top, right, bottom, left)
+        src.info()->extend_padding(PaddingSize(0, 7, 0, 3));
+        w.info()->extend_padding(PaddingSize(0, 16, 0, 1));
+        bias.info()->extend_padding(PaddingSize(0, 2, 0, 5));
+        dst.info()->extend_padding(PaddingSize(0, 4, 0, 9));
+    }
     src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
     if (is_signed)
         fill_uniform<int8_t>(src, -128, 127, 82);
@@ -754,10 +771,11 @@ static void test_convolution(DataType dt, bool per_channel, int C, const Activat
     if (act.enabled())
         std::tie(lo, hi) = get_quantized_activation_min_max(act, dt, UniformQuantizationInfo(0.9f, out_zp));
     std::vector<uint8_t> want(batch * H * W * OFM);
-    orc_conv_nhwc_direct(src.buffer(), is_signed, w.buffer(), (per_channel || is_signed) ? 1 : 0,
-                         reinterpret_cast<const int32_t *>(bias.buffer()), want.data(), is_signed, batch, H, W, C, OFM, KH, KW,
-                         1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp, st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(),
-                         per_channel ? OFM : 1, out_zp, lo, hi);
+    const auto src_d = dense_copy<uint8_t>(src), w_d = dense_copy<uint8_t>(w);
+    const auto bias_d = dense_copy<int32_t>(bias);
+    orc_conv_nhwc_direct(src_d.data(), is_signed, w_d.data(), (per_channel || is_signed) ? 1 : 0, bias_d.data(), want.data(),
+                         is_signed, batch, H, W, C, OFM, KH, KW, 1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp,
+                         st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(), per_channel ? OFM : 1, out_zp, lo, hi);
     EXPECT(dense_copy<uint8_t>(dst) == want);
     std::printf("       kernel: %s\n", conv.kernel_name());
 
@@ -771,10 +789,9 @@ static void test_convolution(DataType dt, bool per_channel, int C, const Activat
     lo = is_signed ? -128 : 0, hi = is_signed ? 127 : 255;
     if (act.enabled())
         std::tie(lo, hi) = get_quantized_activation_min_max(act, dt, UniformQuantizationInfo(1.7f, out_zp + 2));
-    orc_conv_nhwc_direct(src.buffer(), is_signed, w.buffer(), (per_channel || is_signed) ? 1 : 0,
-                         reinterpret_cast<const int32_t *>(bias.buffer()), want.data(), is_signed, batch, H, W, C, OFM, KH, KW,
-                         1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp, st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(),
-                         per_channel ? OFM : 1, out_zp + 2, lo, hi);
+    orc_conv_nhwc_direct(src_d.data(), is_signed, w_d.data(), (per_channel || is_signed) ? 1 : 0, bias_d.data(), want.data(),
+                         is_signed, batch, H, W, C, OFM, KH, KW, 1, 1, 1, 1, 1, 1, 1, 1, in_zp, w_zp,
+                         st.gemmlowp_multipliers.data(), st.gemmlowp_shifts.data(), per_channel ? OFM : 1, out_zp + 2, lo, hi);
     EXPECT(dense_copy<uint8_t>(dst) == want);
 }
 
@@ -1129,6 +1146,8 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
             test_convolution(DataType::QASYMM8, true, 32,
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
+            test_convolution(DataType::QASYMM8_SIGNED, true, 32, ActivationLayerInfo(), true);
+            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), true);
             test_gemm_conv2d();
             test_stateless_operator();
             test_convolution_nchw_and_stateless();

@@ -127,3 +127,48 @@ def test_conv_nchw_fixture(golden):
         got, _ = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, (sx, sy), (pl, pt, pr, pb),
                           layout=capi.NCHW)
         np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("device", [True, False])
+def test_conv_tensors_padded_along_channels(device):
+    """src, weights and dst with padding between pixels, as the reference's convolution fixture hands them over
+    (add_padding_x, tests/validation/Helpers.cpp:335-357): same result, padding bytes of dst untouched."""
+    import torch
+    rng = np.random.default_rng(61)
+    for (B_, H, W, C, OFM, KH, KW, sp, wp, dp) in [(2, 9, 8, 16, 24, 3, 3, 16 + 5, 16 + 9, 24 + 3),
+                                                   (1, 7, 7, 6, 10, 3, 2, 6 + 16, 6 + 1, 10 + 7),
+                                                   (2, 6, 6, 32, 32, 1, 1, 32 + 2, 32, 32 + 16)]:
+        src = rng.integers(-128, 128, size=(B_, H, W, C), dtype=np.int8)
+        w = rng.integers(-127, 128, size=(OFM, KH, KW, C), dtype=np.int8)
+        bias = rng.integers(-500, 500, size=OFM, dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multipliers(0.02, rng.uniform(0.01, 1, OFM), 1.1)
+        pad = (1, 1, 1, 1) if KH == 3 else (0, 0, 0, 0)
+        want = oracle.conv_nhwc_direct(src, w, bias, 4, 0, mult, shift, -5, -128, 127, (1, 1), pad, (1, 1))
+        OH, OW = want.shape[1], want.shape[2]
+        src_p = np.full((B_, H, W, sp), 99, dtype=np.int8)
+        src_p[..., :C] = src
+        w_p = np.full((OFM, KH, KW, wp), 77, dtype=np.int8)
+        w_p[..., :C] = w
+        dst_p = np.full((B_, OH, OW, dp), 55, dtype=np.int8)
+        rq = capi.requant(0, 0, -5, -128, 127, True)
+        d = capi.conv_desc(B_, H, W, C, OFM, KH, KW, (1, 1), pad, (1, 1), capi.S8, capi.S8, capi.S8, -4, 0, 4, rq, 0,
+                           capi.NHWC, (sp, wp, dp))
+        cv = capi.Conv(d)
+        announce("conv padded", (B_, H, W, C, OFM, KH, KW), (sp, wp, dp), "device", device)
+        m, sh = np.ascontiguousarray(mult, dtype=np.int32), np.ascontiguousarray(shift, dtype=np.int32)
+        if device:
+            sd, wd, od = to_dev(src_p), to_dev(w_p), to_dev(dst_p)
+            keep = [to_dev(bias), to_dev(m), to_dev(sh)]
+            cv.prepare(wd, *keep)
+            cv.run(sd, od)
+            torch.cuda.synchronize()
+            got = od.cpu().numpy()
+        else:
+            cv.prepare(w_p, bias, m, sh)
+            got = dst_p.copy()
+            cv.run(src_p, got)
+        cv.close()
+        np.testing.assert_array_equal(got[..., :OFM], want)
+        assert (got[..., OFM:] == 55).all(), "padding bytes of the destination were overwritten"
+    with pytest.raises(capi.Mi355Error, match="pixel stride"):
+        capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 1, 1, pixel_strides=(8, 0, 0)))

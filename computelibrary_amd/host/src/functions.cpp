@@ -580,6 +580,9 @@ void NEGEMMLowpOutputStage::run()
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(!s.configured, "NEGEMMLowpOutputStage::run() before configure()");
     ARM_COMPUTE_ERROR_ON_MSG(s.src->buffer() == nullptr || s.dst->buffer() == nullptr, "tensor without memory");
+    // strides are read when running, as the reference does: its fixtures pad the tensors after configure()
+    s.desc.ld_src = s.src->info()->strides_in_bytes()[1] / s.src->info()->element_size();
+    s.desc.ld_dst = s.dst->info()->strides_in_bytes()[1] / s.dst->info()->element_size();
     check_abi(mi355_output_stage_run(&s.desc, reinterpret_cast<const int32_t *>(first_element(s.src)),
                                      s.bias ? reinterpret_cast<const int32_t *>(first_element(s.bias)) : nullptr,
                                      first_element(s.dst), nullptr),
@@ -910,6 +913,7 @@ struct NEFullyConnectedLayer::Impl
     mi355_gemm_handle *handle{nullptr};
     bool               is_prepared{false};
     bool               dynamic_weights{false};
+    FullyConnectedLayerInfo fc_info{};
 
     ~Impl()
     {
@@ -973,6 +977,18 @@ Status fc_geometry(const ITensorInfo *src, const ITensorInfo *weights, const ITe
         g.k_interleave     = fc_info.weights_trained_layout == DataLayout::NCHW ? chans : plane;
     }
     return Status{};
+}
+
+// row strides of the three matrices; true when they differ from what d held
+bool fc_strides(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, const FcGeometry &g, mi355_gemm_desc &d)
+{
+    // flattening an unpadded tensor is the identity on its bytes; a row that is a whole GEMM row keeps its own stride
+    const int64_t lda = ii->dimension(0) == g.K ? static_cast<int64_t>(ii->strides_in_bytes()[1]) : static_cast<int64_t>(g.K);
+    const int64_t ldb = static_cast<int64_t>(wi->strides_in_bytes()[1] / wi->element_size());
+    const int64_t ldd = static_cast<int64_t>(g.M > 1 ? oi->strides_in_bytes()[1] / oi->element_size() : g.N);
+    const bool    changed = lda != d.lda || ldb != d.ldb || ldd != d.ldd;
+    d.lda = lda, d.ldb = ldb, d.ldd = ldd;
+    return changed;
 }
 
 Status fc_output_stage(const ITensorInfo *src, const ITensorInfo *weights, const ITensorInfo *dst,
@@ -1046,7 +1062,14 @@ Status NEFullyConnectedLayer::validate(const ITensorInfo *input, const ITensorIn
         ARM_COMPUTE_RETURN_ERROR_ON(biases->dimension(0) != g.N);
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->dimension(0) != g.N, "The output's first dimension must be the number of outputs");
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->tensor_shape().total_size() != g.M * g.N, "Mismatching number of batches");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->has_padding(), "A padded input cannot be flattened in place");
+    // a padded input is fine as long as one row of it is one row of the GEMM (nothing to flatten across the padding)
+    if (input->has_padding())
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->dimension(0) != g.K, "A padded input cannot be flattened in place");
+        for (size_t i = 2; i < input->num_dimensions(); ++i)
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->strides_in_bytes()[i] != input->dimension(i - 1) * input->strides_in_bytes()[i - 1],
+                                            "Padding between the rows' planes is not supported");
+    }
     ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(weights, "weights"));
     ARM_COMPUTE_RETURN_ON_ERROR(check_matrix_layout(output, "output"));
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(g.M > 1 && output->num_dimensions() > 2 && output->has_padding(),
@@ -1081,9 +1104,7 @@ void NEFullyConnectedLayer::configure(const ITensor *input, const ITensor *weigh
     d.M = static_cast<int32_t>(g.M), d.N = static_cast<int32_t>(g.N), d.K = static_cast<int32_t>(g.K), d.batch = 1;
     d.a_dtype = to_mi355(ii->data_type()), d.b_dtype = to_mi355(wi->data_type()), d.dst_dtype = to_mi355(oi->data_type());
     d.epilogue = MI355_EPI_FIXEDPOINT;
-    d.lda      = static_cast<int64_t>(g.K); // flattening an unpadded tensor is the identity on its bytes
-    d.ldb      = static_cast<int64_t>(wi->strides_in_bytes()[1] / wi->element_size());
-    d.ldd      = static_cast<int64_t>(g.M > 1 ? oi->strides_in_bytes()[1] / oi->element_size() : g.N);
+    fc_strides(ii, wi, oi, g, d);
     d.a_batch_stride = d.b_batch_stride = d.d_batch_stride = 0;
     // the GEMM adds its offsets: negated zero points (CpuFullyConnected.cpp:98-103,166-171 of the reference)
     d.a_offset       = -ii->quantization_info().uniform().offset;
@@ -1099,7 +1120,7 @@ void NEFullyConnectedLayer::configure(const ITensor *input, const ITensor *weigh
     Impl      &s    = *_impl;
     const bool keep = fc_info.retain_internal_weights && s.handle != nullptr && s.is_prepared && s.desc.M == d.M &&
                       s.desc.N == d.N && s.desc.K == d.K && s.desc.b_dtype == d.b_dtype;
-    s.src = input, s.weights = weights, s.biases = biases, s.dst = output;
+    s.src = input, s.weights = weights, s.biases = biases, s.dst = output, s.fc_info = fc_info;
     s.dynamic_weights = !wi->are_values_constant() && !g.weights_reshaped;
     if (keep)
     {
@@ -1123,6 +1144,20 @@ void NEFullyConnectedLayer::prepare()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEFullyConnectedLayer::prepare() before configure()");
+    {
+        // padding added after configure() (see gemm_strides_changed)
+        FcGeometry g;
+        ARM_COMPUTE_ERROR_THROW_ON(fc_geometry(s.src->info(), s.weights->info(), s.dst->info(), s.fc_info, g));
+        if (fc_strides(s.src->info(), s.weights->info(), s.dst->info(), g, s.desc))
+        {
+            ARM_COMPUTE_ERROR_THROW_ON(validate(s.src->info(), s.weights->info(), s.biases != nullptr ? s.biases->info() : nullptr,
+                                                s.dst->info(), s.fc_info));
+            mi355_gemmlowp_destroy(s.handle);
+            s.handle = nullptr;
+            check_abi(mi355_gemmlowp_create(&s.desc, &s.handle), "NEFullyConnectedLayer::prepare");
+            s.is_prepared = false;
+        }
+    }
     if (s.is_prepared && !s.dynamic_weights)
         return;
     ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");

@@ -625,11 +625,14 @@ static void test_output_stage()
     NEGEMMLowpOutputStage stage;
     stage.configure(&src, &bias, &dst, os);
     EXPECT(dst.info()->data_type() == DataType::QASYMM8_SIGNED && dst.info()->dimension(0) == (size_t)N);
+    // padding after configure, before allocation, as the reference's fixture does
+    src.info()->extend_padding(PaddingSize(0, 3, 0, 2)), dst.info()->extend_padding(PaddingSize(0, 9, 0, 5));
     src.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
     fill_uniform<int32_t>(src, -6000, 6000, 71), fill_uniform<int32_t>(bias, -6000, 6000, 72);
     stage.run();
     std::vector<int8_t> want(M * N);
-    orc_output_stage_fixedpoint(reinterpret_cast<const int32_t *>(src.buffer()), N, reinterpret_cast<const int32_t *>(bias.buffer()),
+    const auto src_d = dense_copy<int32_t>(src);
+    orc_output_stage_fixedpoint(src_d.data(), N, reinterpret_cast<const int32_t *>(bias.buffer()),
                                 want.data(), N, 1, M, N, &os.gemmlowp_multiplier, &os.gemmlowp_shift, 1, -3, -100, 120);
     EXPECT(dense_copy<int8_t>(dst) == want);
 
@@ -645,9 +648,9 @@ static void test_output_stage()
     fill_uniform<int32_t>(src, -100000, 100000, 73);
     stage16.run();
     std::vector<int16_t> want16(M * N);
-    orc_output_stage_fixedpoint_s16(reinterpret_cast<const int32_t *>(src.buffer()), N,
-                                    reinterpret_cast<const int32_t *>(bias.buffer()), want16.data(), N, M, N, 2000000000, 1,
-                                    -30000, 32767);
+    const auto src_d2 = dense_copy<int32_t>(src);
+    orc_output_stage_fixedpoint_s16(src_d2.data(), N, reinterpret_cast<const int32_t *>(bias.buffer()), want16.data(), N, M, N,
+                                    2000000000, 1, -30000, 32767);
     EXPECT(dense_copy<int16_t>(dst16) == want16);
     int lo_hits = 0, hi_hits = 0;
     for (int16_t v : want16)
@@ -847,6 +850,12 @@ static void test_fully_connected(DataType dt, FcCase which)
     EXPECT(bool(NEFullyConnectedLayer::validate(src.info(), weights.info(), bias.info(), dst.info(), fc)));
     NEFullyConnectedLayer fcl;
     fcl.configure(&src, &weights, &bias, &dst, fc);
+    // the reference's fixture pads every tensor along x after configure()
+    // (tests/validation/fixtures/FullyConnectedLayerFixture.h:232-240); an input that has to be flattened stays dense here
+    weights.info()->extend_padding(PaddingSize(0, 6, 0, 1)), bias.info()->extend_padding(PaddingSize(0, 2, 0, 2));
+    dst.info()->extend_padding(PaddingSize(0, 3, 0, 7));
+    if (which == FcCase::AfterFc || which == FcCase::WeightsReshaped)
+        src.info()->extend_padding(PaddingSize(0, 4, 0, 12));
     src.allocator()->allocate(), weights.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
     if (is_signed)
         fill_uniform<int8_t>(src, -128, 127, 21), fill_uniform<int8_t>(weights, -128, 127, 22);

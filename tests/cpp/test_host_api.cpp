@@ -519,6 +519,81 @@ static void test_gemmlowp_dynamic_qinfo()
     }
 }
 
+// The shapes and offsets of the reference's small datasets, through the function classes with padded tensors:
+// tests/datasets/SmallGEMMLowpDataset.h:42-65 (S32 output, 2D and 3D), tests/datasets/GEMMLowpFusedOffsetOutputDataset.h:
+// 120-165 (fused fixed-point output; batched B that changes between runs)
+static void test_reference_small_datasets()
+{
+    SECTION("the reference's SmallGEMMLowp / FusedOffsetOutput / BatchedMatMul dataset shapes");
+    struct Cfg { int K, M, N, batch, depth3d, ao, bo; };
+    const Cfg s32_cfgs[] = {{21, 1, 1, 1, 0, 0, 0},    {21, 13, 33, 1, 0, 0, 0},  {31, 3, 72, 1, 0, -2, 13}, {52, 13, 33, 1, 0, 0, 4},
+                            {52, 26, 33, 1, 0, -2, 0}, {31, 27, 23, 1, 0, 5, 13}, {38, 43, 21, 1, 0, -3, -2}, {32, 72, 17, 1, 0, -9, 1},
+                            {21, 14, 34, 1, 7, 0, 0},  {31, 1, 3, 1, 1, -2, 13}};
+    unsigned seed = 500;
+    for (const Cfg &c : s32_cfgs)
+    {
+        Tensor a, b, dst;
+        init_tensor(a, TensorShape(c.K, c.M), DataType::QASYMM8, QuantizationInfo(1.f / 255, c.ao));
+        init_tensor(b, TensorShape(c.N, c.K), DataType::QASYMM8, QuantizationInfo(1.f / 255, c.bo));
+        init_tensor(dst, c.depth3d ? TensorShape(c.N, c.depth3d, c.M / c.depth3d) : TensorShape(c.N, c.M), DataType::S32);
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, GEMMInfo(false, false, false, c.depth3d));
+        a.info()->extend_padding(PaddingSize(0, 1 + seed % 16, 0, 1 + seed % 7)), b.info()->extend_padding(PaddingSize(0, 3, 0, 16));
+        if (!c.depth3d)
+            dst.info()->extend_padding(PaddingSize(0, 5, 0, 2));
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<uint8_t>(a, 0, 255, seed++), fill_uniform<uint8_t>(b, 0, 255, seed++);
+        gemm.run();
+        const auto A = dense_copy<uint8_t>(a), B = dense_copy<uint8_t>(b);
+        std::vector<int32_t> want(c.M * c.N);
+        orc_gemmlowp_s32(A.data(), 0, c.K, B.data(), 0, c.N, want.data(), c.N, c.M, c.N, c.K, c.ao, c.bo);
+        EXPECT(dense_copy<int32_t>(dst) == want);
+    }
+    const Cfg fused_cfgs[] = {{21, 13, 1, 1, 0, 3, -7},   {52, 13, 33, 1, 0, -12, 5},  {31, 27, 23, 1, 0, 0, 9},    {32, 72, 16, 1, 0, -1, 0},
+                              {21, 1, 43, 1, 0, 6, 6},    {31, 3, 72, 1, 0, -20, 11},  {32, 72, 17, 1, 0, 2, -3},
+                              {4, 3, 2, 1, 0, 1, 1},      {12, 15, 7, 1, 0, -5, 2},    {59, 17, 36, 1, 0, 7, -8},   {2, 4, 5, 3, 0, -3, 4},
+                              {15, 7, 29, 3, 0, 10, -2},  {56, 17, 5, 32, 0, -9, 9},   {13, 256, 19, 32, 0, 4, -6}};
+    for (const Cfg &c : fused_cfgs)
+        for (int sgn = 0; sgn < 2; ++sgn)
+        {
+            const DataType dt = sgn ? DataType::QASYMM8_SIGNED : DataType::QASYMM8;
+            const int      ao = c.ao + (sgn ? 0 : -128), bo = c.bo + (sgn ? 0 : -128); // zero-mean products for both types
+            Tensor         a, b, bias, dst;
+            init_tensor(a, c.batch > 1 ? TensorShape(c.K, c.M, c.batch) : TensorShape(c.K, c.M), dt, QuantizationInfo(0.05f, ao));
+            init_tensor(b, c.batch > 1 ? TensorShape(c.N, c.K, c.batch) : TensorShape(c.N, c.K), dt, QuantizationInfo(0.02f, bo));
+            init_tensor(bias, TensorShape(c.N), DataType::S32);
+            init_tensor(dst, c.batch > 1 ? TensorShape(c.N, c.M, c.batch) : TensorShape(c.N, c.M), dt, QuantizationInfo(1.f, sgn ? -3 : 120));
+            GEMMLowpOutputStageInfo st;
+            st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT, st.output_data_type = dt;
+            st.gemmlowp_offset = sgn ? -3 : 120, st.gemmlowp_min_bound = sgn ? -128 : 0, st.gemmlowp_max_bound = sgn ? 127 : 255;
+            // products of K terms of magnitude ~74*74: bring one standard deviation to about 60 output steps
+            EXPECT(bool(quantization::calculate_quantized_multiplier(60.f / (5476.f * std::sqrt((float)c.K)), &st.gemmlowp_multiplier,
+                                                                     &st.gemmlowp_shift)));
+            NEGEMMLowpMatrixMultiplyCore gemm;
+            gemm.configure(&a, &b, &bias, &dst, GEMMInfo(false, false, c.batch == 1 /* batched B changes */, 0, false, false, st));
+            a.info()->extend_padding(PaddingSize(0, 2, 0, 9)), dst.info()->extend_padding(PaddingSize(0, 8, 0, 1));
+            a.allocator()->allocate(), b.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+            for (int rep = 0; rep < (c.batch > 1 ? 2 : 1); ++rep)
+            {
+                if (sgn)
+                    fill_uniform<int8_t>(a, -128, 127, seed++), fill_uniform<int8_t>(b, -128, 127, seed++);
+                else
+                    fill_uniform<uint8_t>(a, 0, 255, seed++), fill_uniform<uint8_t>(b, 0, 255, seed++);
+                fill_uniform<int32_t>(bias, -2000, 2000, seed++);
+                gemm.run();
+                const auto A = dense_copy<uint8_t>(a), B = dense_copy<uint8_t>(b);
+                const auto Cb = dense_copy<int32_t>(bias);
+                std::vector<uint8_t> want((size_t)c.batch * c.M * c.N);
+                for (int z = 0; z < c.batch; ++z)
+                    orc_gemmlowp_fixedpoint(A.data() + (size_t)z * c.M * c.K, sgn, c.K, B.data() + (size_t)z * c.K * c.N, sgn, c.N,
+                                            Cb.data(), want.data() + (size_t)z * c.M * c.N, c.N, sgn, c.M, c.N, c.K,
+                                            ao, bo, &st.gemmlowp_multiplier,
+                                            &st.gemmlowp_shift, 1, st.gemmlowp_offset, st.gemmlowp_min_bound, st.gemmlowp_max_bound);
+                EXPECT(dense_copy<uint8_t>(dst) == want);
+            }
+        }
+}
+
 static void test_gemmlowp_per_channel_and_update()
 {
     SECTION("NEGEMMLowpMatrixMultiplyCore per-channel QSYMM8_PER_CHANNEL rhs");
@@ -1144,6 +1219,7 @@ int main(int argc, char **argv)
             test_gemmlowp_fused_u8(false);
             test_gemmlowp_fused_u8(true);
             test_gemmlowp_s32_batched();
+            test_reference_small_datasets();
             test_gemmlowp_accumulate_and_3d();
             test_gemmlowp_dynamic_qinfo();
             test_gemmlowp_per_channel_and_update();

@@ -172,3 +172,44 @@ def test_conv_tensors_padded_along_channels(device):
         assert (got[..., OFM:] == 55).all(), "padding bytes of the destination were overwritten"
     with pytest.raises(capi.Mi355Error, match="pixel stride"):
         capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 1, 1, pixel_strides=(8, 0, 0)))
+
+
+def test_conv_random_geometry_sweep():
+    """40 seeded geometries: kernel sizes, strides, asymmetric padding, dilation, channel counts on and off the implicit
+    loader's 16-byte granularity, both layouts, both signs, per-tensor and per-channel weights"""
+    rng = np.random.default_rng(777)
+    done = 0
+    while done < 40:
+        B_ = int(rng.integers(1, 4))
+        H, W = int(rng.integers(3, 15)), int(rng.integers(3, 15))
+        C = int(rng.choice([3, 8, 16, 16, 32, 48, 64, 20]))
+        OFM = int(rng.choice([1, 7, 16, 24, 64, 65]))
+        KH, KW = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        stride = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pad = tuple(int(x) for x in rng.integers(0, 3, size=4))
+        if H + pad[1] + pad[3] < dil[1] * (KH - 1) + 1 or W + pad[0] + pad[2] < dil[0] * (KW - 1) + 1:
+            continue
+        dt = np.int8 if rng.integers(2) else np.uint8
+        per_channel = bool(rng.integers(2))
+        w_dt = np.int8 if (per_channel or dt == np.int8) else np.uint8
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=(B_, H, W, C)).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + (1 if w_dt == np.int8 else 0), np.iinfo(w_dt).max + 1,
+                         size=(OFM, KH, KW, C)).astype(w_dt)
+        bias = rng.integers(-800, 800, size=OFM, dtype=np.int32)
+        in_zp = int(rng.integers(-10, 10)) if dt == np.int8 else int(rng.integers(100, 150))
+        w_zp = 0 if (per_channel or w_dt == np.int8) else int(rng.integers(100, 150))
+        out_zp = -5 if dt == np.int8 else 9
+        reals = rng.uniform(0.2, 2.0, size=OFM if per_channel else 1) * 60.0 / (74.0 * 74.0 * np.sqrt(KH * KW * C))
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi = (-128, 127) if dt == np.int8 else (0, 255)
+        want = oracle.conv_nhwc_direct(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dil)
+        layout = capi.NCHW if rng.integers(3) == 0 else capi.NHWC
+        path = int(rng.integers(2))
+        device = bool(rng.integers(2))
+        announce("conv sweep", done, src.shape, w.shape, stride, pad, dil, dt.__name__, "pc", per_channel, "layout", layout,
+                 "path", path, "dev", device)
+        got, _ = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dil, path=path, device=device,
+                          layout=layout)
+        np.testing.assert_array_equal(got, want, err_msg="case %d" % done)
+        done += 1

@@ -99,6 +99,52 @@ def test_seeded_against_oracle_all_sign_combinations(a_dt, b_dt):
             np.testing.assert_array_equal(got, want_q)
 
 
+def test_random_shape_sweep_against_oracle():
+    """60 seeded cases over ragged shapes, every epilogue, both operand signs, aligned and unaligned row strides, and
+    K around the pipelined kernel's ring depth (1 to 6 steps of 128, with and without a tail)"""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        M = int(rng.choice([1, 3, 8, 16, 17, 63, 64, 65, 127, 129, 255, 257, 300]))
+        N = int(rng.choice([1, 4, 15, 16, 33, 64, 100, 128, 129, 255, 256, 260]))
+        K = int(rng.choice([16, 32, 100, 127, 128, 129, 240, 256, 272, 384, 400, 512, 640, 700, 768]))
+        a_dt = np.int8 if rng.integers(2) else np.uint8
+        b_dt = np.int8 if (a_dt == np.int8 or rng.integers(2)) else np.uint8
+        lda = K + int(rng.choice([0, 0, 16, 4, 3]))
+        ldd = N + int(rng.choice([0, 0, 16, 4, 1]))
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(np.iinfo(b_dt).min, np.iinfo(b_dt).max + 1, size=(K, N)).astype(b_dt)
+        epi = int(rng.integers(3))
+        device = bool(rng.integers(2))
+        path = capi.PATH_AUTO if rng.integers(4) else capi.PATH_MFMA
+        announce("sweep", case, (M, N, K), a_dt.__name__, b_dt.__name__, "lda", lda, "ldd", ldd, "epi", epi, "dev", device,
+                 "path", path)
+        if epi == 0:
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=path, device=device, lda=lda, ldd=ldd)
+            want = oracle.gemmlowp_s32(A, B, ao, bo)
+        elif epi == 1:
+            per_channel = bool(rng.integers(2)) and b_dt == np.int8
+            bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+            reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N if per_channel else 1)) * 128.0 / np.sqrt(K)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            dt = a_dt
+            lo, hi = (-128, 127) if dt == np.int8 else (0, 255)
+            off = -7 if dt == np.int8 else 121
+            bo_eff = 0 if per_channel else bo
+            got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, dt, ao, bo_eff, bias, mult, shift, off, lo, hi, path=path,
+                              device=device, lda=lda, ldd=ldd)
+            want = oracle.gemmlowp_fixedpoint(A, B, bias, ao, bo_eff, mult, shift, off, lo, hi, dt)
+        else:
+            if a_dt != np.int8 or b_dt != np.int8:
+                A, B = A.view(np.int8), B.view(np.int8)
+            bias = rng.normal(0.0, 1.0, size=N).astype(np.float32) if rng.integers(2) else None
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=bias, path=path, device=device,
+                              lda=lda, ldd=ldd)
+            want = oracle.gemmlowp_f32(A, B, bias, ao, bo, 3e-4)
+            got, want = got.view(np.uint32), want.view(np.uint32)
+        assert np.array_equal(got, want), "case %d" % case
+
+
 @pytest.mark.parametrize("K,lda", [(1000, 1000), (1001, 1001), (998, 1000), (64, 80), (17, 17), (1, 1)])
 def test_row_strides_and_k_tails(K, lda):
     """A rows that are not 16-byte aligned (dword-aligned: direct loads with a guarded tail; otherwise the padded

@@ -52,7 +52,9 @@ class ConvDesc(C.Structure):
                                                                   ("layout", C.c_int32),
                                                                   ("src_pixel_stride", C.c_int64),
                                                                   ("weights_pixel_stride", C.c_int64),
-                                                                  ("dst_pixel_stride", C.c_int64)]
+                                                                  ("dst_pixel_stride", C.c_int64),
+                                                                  ("scale", C.c_float), ("act_min", C.c_float),
+                                                                  ("act_max", C.c_float), ("flags", C.c_int32)]
 
 
 _lib = None
@@ -181,10 +183,12 @@ def output_stage(src, bias, dst, rq, stream=None, ld_src=None, ld_dst=None):
 
 
 def conv_desc(batch, H, W, Cc, OFM, KH, KW, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), src_dtype=S8,
-              weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0, layout=0, pixel_strides=(0, 0, 0)):
+              weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0, layout=0, pixel_strides=(0, 0, 0), scale=1.0,
+              act=(-np.inf, np.inf), flags=0):
     return ConvDesc(batch, H, W, Cc, OFM, KH, KW, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0],
                     dilation[1], src_dtype, weights_dtype, dst_dtype, src_offset, weights_offset, pad_value,
-                    rq or requant(), path, layout, pixel_strides[0], pixel_strides[1], pixel_strides[2])
+                    rq or requant(), path, layout, pixel_strides[0], pixel_strides[1], pixel_strides[2], scale,
+                    act[0], act[1], flags)
 
 
 class Conv:

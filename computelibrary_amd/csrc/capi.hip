@@ -423,6 +423,8 @@ struct mi355_conv_handle
     bool            implicit = false;
     DevBuf          stageSrc, stageW, stageDst, stageBias, stageMult, stageShift, cols;
     DevBuf          nhwcSrc, nhwcW, nhwcDst; // MI355_NCHW: the tensors in the kernels' layout
+    DevBuf          biasF;                   // F32 destination: the float bias
+    bool            has_bias_f32 = false;
 };
 
 extern "C"
@@ -734,12 +736,19 @@ static int conv_check(const mi355_conv_desc &d)
         return fail("stride and dilation must be >= 1");
     if (d.pad_left < 0 || d.pad_top < 0 || d.pad_right < 0 || d.pad_bottom < 0)
         return fail("negative padding");
-    if (!is_8bit(d.src_dtype) || !is_8bit(d.weights_dtype) || !is_8bit(d.dst_dtype))
-        return fail("convolution tensors must be 8-bit");
+    if (!is_8bit(d.src_dtype) || !is_8bit(d.weights_dtype) || (!is_8bit(d.dst_dtype) && d.dst_dtype != MI355_F32))
+        return fail("convolution source and weights must be 8-bit, the destination 8-bit or F32");
+    if (d.dst_dtype == MI355_F32)
+    {
+        if (d.layout != MI355_NHWC || (d.dst_pixel_stride != 0 && d.dst_pixel_stride != (int64_t)d.OFM * 4))
+            return fail("the F32 destination of a convolution must be dense NHWC");
+        if ((d.flags & ~MI355_GEMM_ACT_TWICE) != 0)
+            return fail("unknown flag bits 0x%x", d.flags);
+    }
     if (d.layout != MI355_NHWC && d.layout != MI355_NCHW)
         return fail("unknown layout %d", d.layout);
     if ((d.src_pixel_stride != 0 && d.src_pixel_stride < d.C) || (d.weights_pixel_stride != 0 && d.weights_pixel_stride < d.C) ||
-        (d.dst_pixel_stride != 0 && d.dst_pixel_stride < d.OFM))
+        (d.dst_pixel_stride != 0 && d.dst_pixel_stride < (int64_t)d.OFM * (d.dst_dtype == MI355_F32 ? 4 : 1)))
         return fail("pixel stride smaller than the pixel");
     if (d.layout != MI355_NHWC && ((d.src_pixel_stride != 0 && d.src_pixel_stride != d.C) ||
                                    (d.weights_pixel_stride != 0 && d.weights_pixel_stride != d.C) ||
@@ -754,7 +763,9 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         return fail("null argument");
     const mi355_conv_desc &d = *desc;
     TRY(conv_check(d));
-    TRY(check_requant(d.requant, d.dst_dtype));
+    const bool f32 = d.dst_dtype == MI355_F32;
+    if (!f32)
+        TRY(check_requant(d.requant, d.dst_dtype));
     mi355_conv_handle *h = new (std::nothrow) mi355_conv_handle();
     if (!h)
         return fail("out of host memory");
@@ -769,17 +780,24 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         return fail("convolution too large");
     }
     c.M = (int)M64, c.N = d.OFM, c.K = (int)K64, c.batch = 1;
-    c.epi = EPI_FIXEDPOINT, c.dst_dtype = d.dst_dtype;
+    c.epi = f32 ? EPI_F32 : EPI_FIXEDPOINT, c.dst_dtype = d.dst_dtype;
     c.flip_a = d.src_dtype == MI355_U8, c.flip_b = d.weights_dtype == MI355_U8;
     c.a_offset = d.src_offset, c.b_offset = d.weights_offset;
     c.rq = d.requant, c.path = MI355_PATH_MFMA, c.b_shared = true;
+    if (f32)
+    {
+        c.rq    = mi355_requant{};
+        c.scale = d.scale, c.act_min = d.act_min, c.act_max = d.act_max;
+        c.act_twice = (d.flags & MI355_GEMM_ACT_TWICE) != 0;
+    }
     if (c.choose_kernel())
     {
         delete h;
         return 1;
     }
     // the on-the-fly loader moves 16-byte pieces of one tap: needs C % 16 == 0; it has no row sums: needs b_off == 0
-    h->implicit      = d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(d, h->geom);
+    // (the F32 epilogue only exists on the dense kernels: that destination always takes the explicit lowering)
+    h->implicit      = !f32 && d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(d, h->geom);
     h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
     if (h->implicit)
         c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
@@ -789,7 +807,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     return 0;
 }
 
-int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t *bias, const int32_t *mult,
+int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const void *bias, const int32_t *mult,
                        const int32_t *shift, void *stream)
 {
     if (!h || !weights)
@@ -797,6 +815,18 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t 
     hipStream_t s = (hipStream_t)stream;
     GemmCore   &c = h->core;
     const void *wd, *biasd, *multd, *shiftd;
+    const bool  f32 = c.epi == EPI_F32;
+    if (f32)
+    {
+        // the float bias is an argument of every launch: keep a device copy of the caller's values
+        h->has_bias_f32 = bias != nullptr;
+        if (bias)
+        {
+            TRY(h->biasF.ensure(sizeof(float) * (size_t)c.N));
+            HIP_TRY(hipMemcpyAsync(h->biasF.p, bias, sizeof(float) * (size_t)c.N, hipMemcpyDefault, s));
+        }
+        bias = nullptr;
+    }
     const int64_t wps   = h->d.weights_pixel_stride;
     const int64_t wtaps = (int64_t)c.N * h->d.KH * h->d.KW;
     const bool    w_pad = wps != 0 && wps != h->d.C;
@@ -834,6 +864,8 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
         return fail("null argument");
     hipStream_t s = (hipStream_t)stream;
     GemmCore   &c = h->core;
+    if (c.epi == EPI_F32)
+        return fail("the F32 destination has no requantisation to update: create a new handle for new scales");
     TRY(check_requant(*requant, c.dst_dtype));
     if ((requant->per_channel != 0) != (c.rq.per_channel != 0))
         return fail("update cannot switch between per-tensor and per-channel requantisation");
@@ -871,10 +903,11 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     const mi355_conv_desc &d = h->d;
     if (!c.prepared)
         return fail("run before prepare");
-    const size_t  src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N;
+    const size_t  desz      = c.epi == EPI_F32 ? 4 : 1;
+    const size_t  src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N * desz;
     const int64_t pixels    = (int64_t)d.batch * d.H * d.W;
     const bool    s_pad     = d.src_pixel_stride != 0 && d.src_pixel_stride != d.C;
-    const bool    d_pad     = d.dst_pixel_stride != 0 && d.dst_pixel_stride != d.OFM;
+    const bool    d_pad     = d.dst_pixel_stride != 0 && d.dst_pixel_stride != (int64_t)d.OFM * (int64_t)desz;
     const size_t  dst_ext   = d_pad ? (size_t)((int64_t)(c.M - 1) * d.dst_pixel_stride + c.N) : dst_bytes;
     const void   *srcd;
     TRY(to_device(src, s_pad ? (size_t)((pixels - 1) * d.src_pixel_stride + d.C) : src_bytes, h->stageSrc, s, &srcd));
@@ -930,7 +963,7 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         const int ldc = round_up(c.K, 16);
         TRY(h->cols.ensure((size_t)c.M * ldc));
         HIP_TRY(im2col_nhwc_launch(srcd, h->cols.p, d.batch, g2, ldc, s));
-        TRY(c.run_dense(h->cols.as<int8_t>(), ldc, 0, Dd, c.N, 0, nullptr, s));
+        TRY(c.run_dense(h->cols.as<int8_t>(), ldc, 0, Dd, c.N, 0, h->has_bias_f32 ? h->biasF.as<float>() : nullptr, s));
     }
     if (nchw)
     {
@@ -959,7 +992,7 @@ void mi355_conv_destroy(mi355_conv_handle *h)
     h->core.release();
     h->stageSrc.release(), h->stageW.release(), h->stageDst.release(), h->stageBias.release();
     h->stageMult.release(), h->stageShift.release(), h->cols.release();
-    h->nhwcSrc.release(), h->nhwcW.release(), h->nhwcDst.release();
+    h->nhwcSrc.release(), h->nhwcW.release(), h->nhwcDst.release(), h->biasF.release();
     delete h;
 }
 

@@ -674,11 +674,20 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
     ARM_COMPUTE_RETURN_ERROR_ON(weights->dimension(dm.c) != input->dimension(dm.c)); // channels
     ARM_COMPUTE_RETURN_ERROR_ON(weights->num_dimensions() > 4);
     ARM_COMPUTE_RETURN_ERROR_ON(input->num_dimensions() > 4);
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() != input->data_type(),
-                                    "Output must have the input's data type (the F32 destination is not built)");
+    // QASYMM8_SIGNED in, F32 out: the dequantising path (src/cpu/operators/CpuGemmConv2d.cpp:156-159,763-770 of the reference)
+    const bool dequant = input->data_type() == DataType::QASYMM8_SIGNED && output->data_type() == DataType::F32;
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() != input->data_type() && !dequant,
+                                    "Output must have the input's data type, or be F32 for a QASYMM8_SIGNED input");
+    if (dequant)
+    {
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights->data_type() != DataType::QASYMM8_SIGNED,
+                                        "The F32 destination needs QASYMM8_SIGNED weights");
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC || output->has_padding(),
+                                        "The F32 destination is built for dense NHWC tensors");
+    }
     if (biases != nullptr)
     {
-        ARM_COMPUTE_RETURN_ERROR_ON(biases->data_type() != DataType::S32);
+        ARM_COMPUTE_RETURN_ERROR_ON(biases->data_type() != (dequant ? DataType::F32 : DataType::S32));
         ARM_COMPUTE_RETURN_ERROR_ON(biases->dimension(0) != weights->dimension(3));
         ARM_COMPUTE_RETURN_ERROR_ON(biases->num_dimensions() > 1);
     }
@@ -713,8 +722,11 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
         else
             ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->has_padding(), "Padded NCHW tensors are not supported by this convolution");
     }
-    GEMMLowpOutputStageInfo stage;
-    ARM_COMPUTE_RETURN_ON_ERROR(conv_output_stage(input, weights, output, act_info, stage));
+    if (!dequant)
+    {
+        GEMMLowpOutputStageInfo stage;
+        ARM_COMPUTE_RETURN_ON_ERROR(conv_output_stage(input, weights, output, act_info, stage));
+    }
     return Status{};
 }
 
@@ -759,8 +771,10 @@ void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorI
                     const Size2D &dilation, const ActivationLayerInfo &act_info, mi355_conv_desc &d,
                     std::vector<int32_t> &multipliers, std::vector<int32_t> &shifts)
 {
+    const bool              dequant = oi->data_type() == DataType::F32;
     GEMMLowpOutputStageInfo stage;
-    ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, oi, act_info, stage));
+    if (!dequant)
+        ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, oi, act_info, stage));
     const ConvDims dm(ii->data_layout());
     d        = mi355_conv_desc{};
     d.layout = ii->data_layout() == DataLayout::NHWC ? MI355_NHWC : MI355_NCHW;
@@ -781,8 +795,34 @@ void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorI
     d.weights_offset =
         is_data_type_quantized_per_channel(wi->data_type()) ? 0 : -wi->quantization_info().uniform().offset;
     d.pad_value = in_zp;
-    d.requant   = make_requant(stage);
     d.path      = 0;
+    d.act_min   = -std::numeric_limits<float>::infinity();
+    d.act_max   = std::numeric_limits<float>::infinity();
+    d.scale     = 1.f;
+    if (dequant)
+    {
+        // the GEMM's dequantisation scale and fused activation, as for NEGEMMLowpMatrixMultiplyCore with an F32 output
+        d.scale = ii->quantization_info().uniform().scale * wi->quantization_info().uniform().scale;
+        if (act_info.enabled())
+        {
+            switch (act_info.activation())
+            {
+                case ActivationLayerInfo::ActivationFunction::RELU:
+                    d.act_min = 0.f;
+                    break;
+                case ActivationLayerInfo::ActivationFunction::BOUNDED_RELU:
+                    d.act_min = 0.f, d.act_max = act_info.a();
+                    break;
+                default: // LU_BOUNDED_RELU (validate() admits no other)
+                    d.act_min = act_info.b(), d.act_max = act_info.a();
+                    break;
+            }
+            if (act_info.b() == 0.f)
+                d.flags |= MI355_GEMM_ACT_TWICE;
+        }
+    }
+    else
+        d.requant = make_requant(stage);
     if (d.layout == MI355_NHWC)
     {
         d.src_pixel_stride     = static_cast<int64_t>(ii->strides_in_bytes()[1]);
@@ -802,6 +842,8 @@ void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorI
 void refresh_conv_quant(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, const ActivationLayerInfo &act,
                         mi355_conv_desc &d, std::vector<int32_t> &multipliers, std::vector<int32_t> &shifts)
 {
+    ARM_COMPUTE_ERROR_ON_MSG(oi->data_type() == DataType::F32,
+                             "A convolution with an F32 destination has to be configured again for new quantization");
     GEMMLowpOutputStageInfo stage;
     ARM_COMPUTE_ERROR_THROW_ON(conv_output_stage(ii, wi, oi, act, stage));
     const int32_t in_zp = ii->quantization_info().uniform().offset;
@@ -869,8 +911,7 @@ void NEGEMMConvolutionLayer::prepare()
     if (s.is_prepared)
         return;
     ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");
-    check_abi(mi355_conv_prepare(s.handle, first_element(s.weights),
-                                 s.biases ? reinterpret_cast<const int32_t *>(first_element(s.biases)) : nullptr,
+    check_abi(mi355_conv_prepare(s.handle, first_element(s.weights), s.biases ? first_element(s.biases) : nullptr,
                                  s.multipliers.empty() ? nullptr : s.multipliers.data(),
                                  s.shifts.empty() ? nullptr : s.shifts.data(), nullptr),
               "NEGEMMConvolutionLayer::prepare");

@@ -209,12 +209,19 @@ typedef struct mi355_conv_desc
      * OFM). The pointers passed to prepare / run address the first element. Padded tensors are gathered into dense
      * device buffers first (one extra pass) and the result is scattered into dst, leaving its padding untouched. */
     int64_t       src_pixel_stride, weights_pixel_stride, dst_pixel_stride;
+    /* dst_dtype MI355_F32 only - the dequantising convolution (CpuGemmConv2d with a QASYMM8_SIGNED input and an F32
+     * destination, src/cpu/operators/CpuGemmConv2d.cpp:297-305,391-393): no requantisation, dst = float(acc) * scale
+     * (+ float bias) + float(offset terms) * scale, clamped to [act_min, act_max] as MI355_EPI_F32 does; flags takes
+     * MI355_GEMM_ACT_TWICE. Dense NHWC only; the bias passed to mi355_conv_prepare is then OFM floats. */
+    float         scale, act_min, act_max;
+    int32_t       flags;
 } mi355_conv_desc;
 
 typedef struct mi355_conv_handle mi355_conv_handle;
 
 int  mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out);
-int  mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const int32_t *bias, const int32_t *mult,
+/* bias: OFM int32 (8-bit destinations) or OFM floats (F32 destination), or NULL */
+int  mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const void *bias, const int32_t *mult,
                         const int32_t *shift, void *stream);
 /* Replaces CpuGemmConv2d::update_quantization_parameters (:858-908): new offsets, pad value and requantisation without
  * touching the packed weights. mult / shift (OFM int32 each) are read only when requant->per_channel. */

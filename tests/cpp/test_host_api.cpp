@@ -1170,6 +1170,49 @@ static void test_convolution_nchw_and_stateless()
     }
 }
 
+// QASYMM8_SIGNED convolution with an F32 destination and a fused RELU (the dequantising path of CpuGemmConv2d)
+static void test_convolution_f32_destination()
+{
+    SECTION("NEGEMMConvolutionLayer QASYMM8_SIGNED -> F32 with F32 bias and RELU");
+    const int batch = 2, H = 8, W = 9, C = 16, OFM = 12, KH = 3, KW = 3, in_zp = 5, w_zp = -2;
+    Tensor src, w, bias, dst;
+    init_tensor(src, TensorShape(C, W, H, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.02f, in_zp));
+    init_tensor(w, TensorShape(C, KW, KH, OFM), DataType::QASYMM8_SIGNED, QuantizationInfo(0.005f, w_zp));
+    init_tensor(bias, TensorShape(OFM), DataType::F32);
+    init_tensor(dst, TensorShape(OFM, W, H, batch), DataType::F32);
+    for (Tensor *t : {&src, &w, &dst})
+        t->info()->set_data_layout(DataLayout::NHWC);
+    const ActivationLayerInfo relu(ActivationLayerInfo::ActivationFunction::RELU);
+    EXPECT(bool(NEGEMMConvolutionLayer::validate(src.info(), w.info(), bias.info(), dst.info(), PadStrideInfo(1, 1, 1, 1), WeightsInfo(),
+                                                 Size2D(1, 1), relu)));
+    NEGEMMConvolutionLayer conv;
+    conv.configure(&src, &w, &bias, &dst, PadStrideInfo(1, 1, 1, 1), WeightsInfo(), Size2D(1, 1), relu);
+    src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+    fill_uniform<int8_t>(src, -128, 127, 151), fill_uniform<int8_t>(w, -127, 127, 152);
+    std::mt19937                    rng(153);
+    std::normal_distribution<float> nd(0.f, 2.f);
+    for (int j = 0; j < OFM; ++j)
+        reinterpret_cast<float *>(bias.buffer())[j] = nd(rng);
+    conv.run();
+    const int K = KH * KW * C, M = batch * H * W;
+    std::vector<uint8_t> cols((size_t)M * K);
+    orc_im2col_nhwc(src.buffer(), cols.data(), batch, H, W, C, KH, KW, 1, 1, 1, 1, 1, 1, 1, 1, (uint8_t)in_zp);
+    std::vector<int8_t> Bm((size_t)K * OFM); // weights [OFM][K] -> B [K][OFM]
+    for (int o = 0; o < OFM; ++o)
+        for (int k = 0; k < K; ++k)
+            Bm[(size_t)k * OFM + o] = reinterpret_cast<const int8_t *>(w.buffer())[(size_t)o * K + k];
+    std::vector<float> want((size_t)M * OFM);
+    orc_gemmlowp_f32(cols.data(), 1, K, Bm.data(), 1, OFM, reinterpret_cast<const float *>(bias.buffer()), want.data(), OFM, M, OFM,
+                     K, -in_zp, -w_zp, 0.02f * 0.005f, 0.f, INFINITY, 0, 1);
+    EXPECT(dense_copy<float>(dst) == want);
+    std::printf("       kernel: %s\n", conv.kernel_name());
+    // an F32 destination with per-channel or unsigned weights has no kernel
+    Tensor wpc;
+    init_tensor(wpc, TensorShape(C, KW, KH, OFM), DataType::QSYMM8_PER_CHANNEL, QuantizationInfo(std::vector<float>(OFM, 0.01f)));
+    wpc.info()->set_data_layout(DataLayout::NHWC);
+    EXPECT(!bool(NEGEMMConvolutionLayer::validate(src.info(), wpc.info(), bias.info(), dst.info(), PadStrideInfo(1, 1, 1, 1))));
+}
+
 static void test_error_paths()
 {
     SECTION("configure() throws on invalid input; run() before configure() throws");
@@ -1236,6 +1279,7 @@ int main(int argc, char **argv)
             test_gemm_conv2d();
             test_stateless_operator();
             test_convolution_nchw_and_stateless();
+            test_convolution_f32_destination();
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);

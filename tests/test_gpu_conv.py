@@ -213,3 +213,39 @@ def test_conv_random_geometry_sweep():
                           layout=layout)
         np.testing.assert_array_equal(got, want, err_msg="case %d" % done)
         done += 1
+
+
+@pytest.mark.parametrize("device", [True, False])
+def test_conv_with_f32_destination(device):
+    """QASYMM8_SIGNED input and weights, F32 destination (src/cpu/operators/CpuGemmConv2d.cpp:297-305 of the reference):
+    the im2col matrix through the dequantising GEMM; checked against the oracle's im2col + F32 GEMM, identical bits"""
+    import torch
+    rng = np.random.default_rng(91)
+    for (B_, H, W, C, OFM, KH, KW, stride, pad, in_zp, w_zp, act, twice) in [
+            (2, 9, 8, 16, 24, 3, 3, (1, 1), (1, 1, 1, 1), 4, 0, (-np.inf, np.inf), False),
+            (1, 7, 6, 5, 9, 3, 2, (2, 1), (0, 1, 1, 0), -3, 6, (0.0, np.inf), True),
+            (3, 5, 5, 32, 64, 1, 1, (1, 1), (0, 0, 0, 0), 0, 0, (0.0, 6.0), True)]:
+        src = rng.integers(-128, 128, size=(B_, H, W, C), dtype=np.int8)
+        w = rng.integers(-127, 128, size=(OFM, KH, KW, C), dtype=np.int8)
+        bias = rng.normal(0.0, 2.0, size=OFM).astype(np.float32)
+        scale = float(np.float32(0.02) * np.float32(0.005))
+        cols = oracle.im2col_nhwc(src, KH, KW, stride, pad, (1, 1), in_zp)
+        want = oracle.gemmlowp_f32(cols, oracle.weights_reshape(w), bias, -in_zp, -w_zp, scale, act[0], act[1],
+                                   act_twice=twice)
+        d = capi.conv_desc(B_, H, W, C, OFM, KH, KW, stride, pad, (1, 1), capi.S8, capi.S8, capi.F32, -in_zp, -w_zp, in_zp,
+                           scale=scale, act=act, flags=capi.GEMM_ACT_TWICE if twice else 0)
+        cv = capi.Conv(d)
+        OH, OW = cv.out_dims()
+        out = np.zeros((B_, OH, OW, OFM), dtype=np.float32)
+        announce("conv f32", (B_, H, W, C, OFM, KH, KW), stride, pad, in_zp, w_zp, act, "device", device, cv.kernel_name)
+        if device:
+            sd, wd, od, bd = to_dev(src), to_dev(w), to_dev(out), to_dev(bias)
+            cv.prepare(wd, bd)
+            cv.run(sd, od)
+            torch.cuda.synchronize()
+            out = od.cpu().numpy()
+        else:
+            cv.prepare(w, bias)
+            cv.run(src, out)
+        cv.close()
+        assert np.array_equal(out.reshape(-1, OFM).view(np.uint32), want.view(np.uint32))

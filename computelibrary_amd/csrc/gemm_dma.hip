@@ -237,7 +237,10 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     int tm, tn, bz;
-    tile_coords_batched(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, bz, tm, tn);
+    if (g.tile_magic_ok)
+        tile_coords_batched_fast(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, g.magic_tiles, g.magic_group, bz, tm, tn);
+    else
+        tile_coords_batched(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, bz, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = (g.K + BK - 1) / BK;
 
@@ -508,6 +511,16 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
             return (int)e;
     }
     GemmArgs a       = args;
+    // reciprocals for the tile map: floor(2^32 / d) + 1 gives x / d exactly while x * d < 2^32; the 4-wide groups are
+    // split with a 16-bit reciprocal of 3
+    const int64_t nblocks = (int64_t)args.tiles_m * args.tiles_n * batch;
+    const int64_t d_tiles = (int64_t)args.tiles_m * args.tiles_n, d_group = 4 * (int64_t)args.tiles_n;
+    a.tile_magic_ok       = (nblocks * d_tiles < ((int64_t)1 << 32) && d_tiles * d_group < ((int64_t)1 << 32) && d_group < 65536 &&
+                       d_tiles > 1 && d_group > 1)
+                                ? 1
+                                : 0;
+    a.magic_tiles = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_tiles) + 1u : 0u;
+    a.magic_group = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_group) + 1u : 0u;
     void    *kargs[] = {&a};
     dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block(c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);

@@ -46,6 +46,10 @@ struct GemmArgs
     ConvGeom      conv;
     const int8_t *fill16; // 16 readable bytes: what a staged 16-byte column reads where A has no data (zeros / pad value)
     const int8_t *a_end;  // dense A: one past the last byte of the last row of the last batch (no 16-byte read may cross it)
+    // floor(2^32 / d) + 1 for d = tiles_m * tiles_n and d = 4 * tiles_n (see fast_div), valid for every tile id of the
+    // launch; tile_magic_ok == 0: divide
+    uint32_t magic_tiles, magic_group;
+    int32_t  tile_magic_ok;
 };
 
 struct MfmaConfig

@@ -56,6 +56,27 @@ __device__ __forceinline__ void tile_coords_batched(int bid, int nblocks, int ti
     tn                = in_grp / gsize;
 }
 
+// The same map with the two run-time divisors replaced by multiplications with host-computed reciprocals (every wave of
+// every block walks this dependent scalar chain before it can do anything else) and the group size, 1 to 4, by shifts.
+__device__ __forceinline__ void tile_coords_batched_fast(int bid, int nblocks, int tiles_m, int tiles_n, uint32_t magic_tiles,
+                                                         uint32_t magic_group, int &bz, int &tm, int &tn)
+{
+    int l = bid;
+    if ((nblocks & 7) == 0)
+        l = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+    const int tpb = tiles_m * tiles_n;
+    bz            = nblocks == tpb ? 0 : (int)__umulhi((uint32_t)l, magic_tiles);
+    l -= bz * tpb;
+    const int per_grp = 4 * tiles_n;
+    const int grp     = (int)__umulhi((uint32_t)l, magic_group);
+    const int first   = grp * 4;
+    const int gsize   = min(tiles_m - first, 4);
+    const int in_grp  = l - grp * per_grp;
+    // in_grp < 4 * tiles_n: x / 3 == (x * 0xAAAB) >> 17 holds for x < 2^16
+    tn = gsize == 4 ? in_grp >> 2 : gsize == 2 ? in_grp >> 1 : gsize == 1 ? in_grp : (int)(((uint32_t)in_grp * 0xAAABu) >> 17);
+    tm = first + in_grp - tn * gsize;
+}
+
 // Accumulator (fm, fn, r) of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 block.
 // (row0, col0) is the wave's top-left output coordinate.
 template <int EPI, int FM, int FN>

@@ -215,8 +215,8 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     constexpr int AU = BM / RPU, BU = BN / RPU; // staging units of the A and the B part of a stage
     constexpr int LPP = (AU + BU) / NP;         // loads per producer wave per stage: unit u belongs to producer u % NP
     constexpr int TM = BM / 2 / GWM, TN = BN / GWN;
-    constexpr int FM = TM / 32, FN = TN / 32;
-    constexpr int KK    = BK / 32;
+    constexpr int RS = TM / 16, QS = TN / 16; // 16 x 16 accumulator blocks of a wave: row slots x column slots
+    constexpr int KK    = BK / 64;            // matrix instructions along K per stage (each covers 64)
     constexpr int STAGE = (BM + BN) * BK;
     static_assert((AU + BU) % NP == 0, "staging shape");
     // Dense tiles: inside the K loop the consumers stage the B panel themselves (CBU units per wave and K step, issued
@@ -225,9 +225,9 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     constexpr bool CDMA = !CONV && (BU % NW == 0) && (AU % NP == 0) && (AU / NP) % 2 == 0;
     constexpr int  CBU  = CDMA ? BU / NW : 0;   // B units per consumer wave per stage
     constexpr int  PLP  = CDMA ? AU / NP : LPP; // loads per producer wave per stage inside the loop
-    static_assert(TM % 32 == 0 && TN % 32 == 0 && FM >= 1 && FN >= 1, "wave tile");
+    static_assert(TM % 16 == 0 && TN % 16 == 0 && RS >= 1 && QS >= 1 && BK % 64 == 0, "wave tile");
     static_assert(NS >= 3 && (NS - 2) * LPP < 64, "ring depth / vmcnt range");
-    static_assert(NW * 32 * (FN * 128 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
+    static_assert(NW * 16 * (QS * 64 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
@@ -316,29 +316,27 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         }
     }
 
-    v16i acc[FM][FN];
+    v4i acc[RS][QS];
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+    for (int i = 0; i < RS; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[i][j][r] = 0;
+        for (int j = 0; j < QS; ++j)
+            acc[i][j] = (v4i){0, 0, 0, 0};
 
-    // operand read addresses: lane -> (row lane%32, 16-byte column lane/32) of a 32 x 32 operand block
-    const int lr = lane & 31, lh = lane >> 5;
-    int       a_rd[FM], b_rd[FN], a_sw[FM], b_sw[FN];
+    // operand read addresses: lane -> (row lane%16, 16-byte column lane/16) of a 16 row x 64 byte operand block
+    const int lr = lane & 15, lh = lane >> 4;
+    int       a_rd[RS], b_rd[QS], a_sw[RS], b_sw[QS];
 #pragma unroll
-    for (int f = 0; f < FM; ++f)
+    for (int f = 0; f < RS; ++f)
     {
-        const int row = row_w + f * 32 + lr;
+        const int row = row_w + f * 16 + lr;
         a_rd[f]       = row * BK;
         a_sw[f]       = swz<CPR>(row);
     }
 #pragma unroll
-    for (int f = 0; f < FN; ++f)
+    for (int f = 0; f < QS; ++f)
     {
-        const int row = col_w + f * 32 + lr;
+        const int row = col_w + f * 16 + lr;
         b_rd[f]       = BM * BK + row * BK;
         b_sw[f]       = swz<CPR>(row);
     }
@@ -353,7 +351,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     if (group == 1)
         block_barrier(); // group 1 runs one slot behind group 0
 
-    v4i fa[KK][FM], fb[KK][FN];
+    v4i fa[KK][RS], fb[KK][QS];
     for (int kt = 0; kt < nk; ++kt)
     {
         // ---- load slot: operands of K step kt from LDS into registers ----
@@ -362,11 +360,11 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         for (int kk = 0; kk < KK; ++kk)
         {
 #pragma unroll
-            for (int f = 0; f < FM; ++f)
-                fa[kk][f] = *(const v4i *)(s + a_rd[f] + (((kk * 2 + lh) ^ a_sw[f]) << 4));
+            for (int f = 0; f < RS; ++f)
+                fa[kk][f] = *(const v4i *)(s + a_rd[f] + (((kk * 4 + lh) ^ a_sw[f]) << 4));
 #pragma unroll
-            for (int f = 0; f < FN; ++f)
-                fb[kk][f] = *(const v4i *)(s + b_rd[f] + (((kk * 2 + lh) ^ b_sw[f]) << 4));
+            for (int f = 0; f < QS; ++f)
+                fb[kk][f] = *(const v4i *)(s + b_rd[f] + (((kk * 4 + lh) ^ b_sw[f]) << 4));
         }
         if (CDMA && kt + NS - 1 < nk)
         {
@@ -382,7 +380,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-                for (int f = 0; f < FM; ++f)
+                for (int f = 0; f < RS; ++f)
                     fa[kk][f] ^= (int)0x80808080;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -402,10 +400,10 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < RS; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < QS; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         block_barrier();
     }
@@ -429,23 +427,23 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         {
             char *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
             if (g.epi.vec_store16 && g.epi.qp_std)
-                epilogue_store_staged<true, FM, FN, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                epilogue_store_staged<true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
                                                                 [] { __syncthreads(); });
             else if (g.epi.vec_store16)
-                epilogue_store_staged<false, FM, FN, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                epilogue_store_staged<false, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
                                                                  [] { __syncthreads(); });
             else
-                epilogue_store_fast<FM, FN, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+                epilogue_store_fast<RS, QS, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
         }
     }
     else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store && !g.epi.accumulate)
     {
-        // the ring is free beyond the last barrier: 32 x (FN*128 + 16) bytes per wave
+        // the ring is free beyond the last barrier: 16 x (QS*64 + 16) bytes per wave
         if constexpr (EPI != EPI_FIXEDPOINT)
-            epilogue_store_wave32<EPI, FM, FN>(acc, g, smem + wave * 32 * (FN * 128 + 16), m0 + row_w, n0 + col_w, lane, bz);
+            epilogue_store_wave32<EPI, RS, QS>(acc, g, smem + wave * 16 * (QS * 64 + 16), m0 + row_w, n0 + col_w, lane, bz);
     }
     else
-        epilogue_store_t<EPI, FM, FN>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
+        epilogue_store_t<EPI, RS, QS>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
 }
 
 // ---- instantiation table -------------------------------------------------------------------------------------------

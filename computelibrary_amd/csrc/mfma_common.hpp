@@ -131,187 +131,62 @@ __device__ __forceinline__ void epilogue_store(const v16i (&acc)[FM][FN], const 
         }
     }
 }
-// Transposed accumulators (the B panel was the first matrix operand): accumulator (fm, fn, r) of lane l holds output
-// row l%32 of row block fm and output column 8*(r/4) + 4*(l/32) + r%4 of column block fn, i.e. every register quad is
-// 4 consecutive columns of one row: per-column parameters are read as 16-byte vectors and 4 results leave in one store.
-template <int EPI, int FM, int FN>
-__device__ __forceinline__ void epilogue_store_t(const v16i (&acc)[FM][FN], const GemmArgs &g, int row0, int col0,
+// Accumulators of the pipelined kernel: 16 x 16 blocks produced by v_mfma_i32_16x16x64_i8 with the B panel as the first
+// matrix operand, i.e. transposed. A wave's sub-tile is RS row slots of 16 rows by QS column slots of 16 columns; lane l
+// holds, for every (rs, qs), output row rs*16 + l%16 and the 4 consecutive output columns qs*16 + 4*(l/16) + {0..3}
+// in the 4 registers of acc[rs][qs]: per-column parameters are read as 16-byte vectors and 4 results leave in one store.
+// (row0, col0) is the wave's top-left output coordinate.
+template <int EPI, int RS, int QS>
+__device__ __forceinline__ void epilogue_store_t(const v4i (&acc)[RS][QS], const GemmArgs &g, int row0, int col0,
                                                  int lane, int bz)
 {
-    const int        lr = lane & 31, lh = lane >> 5;
+    const int        lr = lane & 15, lh = lane >> 4;
     const EpiParams &p      = g.epi;
     const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
     const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
     char            *D      = (char *)g.D;
-    int32_t          rv[FM];
+    int32_t          rv[RS];
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
+    for (int rs = 0; rs < RS; ++rs)
     {
-        const int i = row0 + fm * 32 + lr;
-        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+        const int i = row0 + rs * 16 + lr;
+        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
     }
 #pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
+    for (int qs = 0; qs < QS; ++qs)
     {
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
+        const int j0 = col0 + qs * 16 + 4 * lh; // first of 4 consecutive columns; inside the padded vectors
+        const v4i cv = *(const v4i *)(colvec + j0);
+        v4i       mu = {p.mult_s, p.mult_s, p.mult_s, p.mult_s};
+        v4i       sh = {p.shift_s, p.shift_s, p.shift_s, p.shift_s};
+        float     bf[4] = {0.f, 0.f, 0.f, 0.f};
+        if (EPI == EPI_FIXEDPOINT && p.mult)
         {
-            const int j0 = col0 + fn * 32 + 8 * q + 4 * lh; // first of 4 consecutive columns; inside the padded vectors
-            const v4i cv = *(const v4i *)(colvec + j0);
-            v4i       mu = {p.mult_s, p.mult_s, p.mult_s, p.mult_s};
-            v4i       sh = {p.shift_s, p.shift_s, p.shift_s, p.shift_s};
-            float     bf[4] = {0.f, 0.f, 0.f, 0.f};
-            if (EPI == EPI_FIXEDPOINT && p.mult)
-            {
-                mu = *(const v4i *)(p.mult + j0);
-                sh = *(const v4i *)(p.shift + j0);
-            }
-            if (EPI == EPI_F32 && p.bias_f32)
-            {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (j0 + t < g.N)
-                        bf[t] = p.bias_f32[j0 + t];
-            }
-#pragma unroll
-            for (int fm = 0; fm < FM; ++fm)
-            {
-                const int i = row0 + fm * 32 + lr;
-                if (i >= g.M || j0 >= g.N)
-                    continue;
-                const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
-                const bool    vec = p.vec_store && (j0 + 3 < g.N);
-                if (EPI == EPI_FIXEDPOINT)
-                {
-                    uint32_t packed = 0;
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        packed |= ((uint32_t)epi_fixedpoint(acc[fm][fn][4 * q + t], cv[t], rv[fm], mu[t], sh[t], p) & 0xFFu)
-                                  << (8 * t);
-                    if (vec)
-                        *(uint32_t *)(D + idx) = packed;
-                    else
-                    {
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (j0 + t < g.N)
-                                D[idx + t] = (char)(packed >> (8 * t));
-                    }
-                }
-                else if (EPI == EPI_S32)
-                {
-                    v4i o, prev = {0, 0, 0, 0};
-                    if (p.accumulate)
-                    {
-                        if (vec)
-                            prev = *(const v4i *)((int32_t *)D + idx);
-                        else
-                        {
-#pragma unroll
-                            for (int t = 0; t < 4; ++t)
-                                if (j0 + t < g.N)
-                                    prev[t] = ((int32_t *)D)[idx + t];
-                        }
-                    }
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm] +
-                                         (uint32_t)prev[t]);
-                    if (vec)
-                        *(v4i *)((int32_t *)D + idx) = o;
-                    else
-                    {
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (j0 + t < g.N)
-                                ((int32_t *)D)[idx + t] = o[t];
-                    }
-                }
-                else
-                {
-                    typedef float v4f __attribute__((ext_vector_type(4)));
-                    v4f o, prev = {0.f, 0.f, 0.f, 0.f};
-                    if (p.accumulate)
-                    {
-                        if (vec)
-                            prev = *(const v4f *)((float *)D + idx);
-                        else
-                        {
-#pragma unroll
-                            for (int t = 0; t < 4; ++t)
-                                if (j0 + t < g.N)
-                                    prev[t] = ((float *)D)[idx + t];
-                        }
-                    }
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = epi_f32(acc[fm][fn][4 * q + t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv[fm]), bf[t],
-                                       p.bias_f32 != nullptr, p, prev[t]);
-                    if (vec)
-                        *(v4f *)((float *)D + idx) = o;
-                    else
-                    {
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (j0 + t < g.N)
-                                ((float *)D)[idx + t] = o[t];
-                    }
-                }
-            }
+            mu = *(const v4i *)(p.mult + j0);
+            sh = *(const v4i *)(p.shift + j0);
         }
-    }
-}
-// FIXEDPOINT epilogue of the pipelined kernel for multipliers >= 0. The block's per-column constants were staged in LDS
-// as par[6][BN]: row 0 the folded offset/bias vector, rows 1..5 the QP_* vectors; col_in_tile is the wave's first
-// column inside the block tile. Same accumulator layout as epilogue_store_t.
-template <int FM, int FN, int BN>
-__device__ __forceinline__ void epilogue_store_fast(const v16i (&acc)[FM][FN], const GemmArgs &g, const int32_t *par,
-                                                    int row0, int col0, int col_in_tile, int lane, int bz)
-{
-    const int        lr = lane & 31, lh = lane >> 5;
-    const EpiParams &p      = g.epi;
-    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
-    char            *D      = (char *)g.D;
-    int32_t          rv[FM];
-#pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
-    {
-        const int i = row0 + fm * 32 + lr;
-        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
-    }
-#pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
-    {
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
+        if (EPI == EPI_F32 && p.bias_f32)
         {
-            const int c  = col_in_tile + fn * 32 + 8 * q + 4 * lh;
-            const int j0 = col0 + fn * 32 + 8 * q + 4 * lh;
-            const v4i cv = *(const v4i *)(par + 0 * BN + c);
-            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
-            const v4i cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
-            const v4i ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
-            const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
-            const v4i rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
 #pragma unroll
-            for (int fm = 0; fm < FM; ++fm)
+            for (int t = 0; t < 4; ++t)
+                if (j0 + t < g.N)
+                    bf[t] = p.bias_f32[j0 + t];
+        }
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
+        {
+            const int i = row0 + rs * 16 + lr;
+            if (i >= g.M || j0 >= g.N)
+                continue;
+            const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
+            const bool    vec = p.vec_store && (j0 + 3 < g.N);
+            if (EPI == EPI_FIXEDPOINT)
             {
-                const int i = row0 + fm * 32 + lr;
-                int32_t   o[4];
+                uint32_t packed = 0;
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                {
-                    const int32_t v = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
-                    o[t]            = fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
-                }
-                // low bytes of o[0..3] -> one dword
-                const uint32_t p01    = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
-                const uint32_t p23    = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
-                const uint32_t packed = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
-                if (i >= g.M || j0 >= g.N)
-                    continue;
-                const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
-                if (p.vec_store && (j0 + 3 < g.N))
+                    packed |= ((uint32_t)epi_fixedpoint(acc[rs][qs][t], cv[t], rv[rs], mu[t], sh[t], p) & 0xFFu) << (8 * t);
+                if (vec)
                     *(uint32_t *)(D + idx) = packed;
                 else
                 {
@@ -321,64 +196,177 @@ __device__ __forceinline__ void epilogue_store_fast(const v16i (&acc)[FM][FN], c
                             D[idx + t] = (char)(packed >> (8 * t));
                 }
             }
+            else if (EPI == EPI_S32)
+            {
+                v4i o, prev = {0, 0, 0, 0};
+                if (p.accumulate)
+                {
+                    if (vec)
+                        prev = *(const v4i *)((int32_t *)D + idx);
+                    else
+                    {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (j0 + t < g.N)
+                                prev[t] = ((int32_t *)D)[idx + t];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv[rs] + (uint32_t)prev[t]);
+                if (vec)
+                    *(v4i *)((int32_t *)D + idx) = o;
+                else
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (j0 + t < g.N)
+                            ((int32_t *)D)[idx + t] = o[t];
+                }
+            }
+            else
+            {
+                typedef float v4f __attribute__((ext_vector_type(4)));
+                v4f o, prev = {0.f, 0.f, 0.f, 0.f};
+                if (p.accumulate)
+                {
+                    if (vec)
+                        prev = *(const v4f *)((float *)D + idx);
+                    else
+                    {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (j0 + t < g.N)
+                                prev[t] = ((float *)D)[idx + t];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    o[t] = epi_f32(acc[rs][qs][t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv[rs]), bf[t], p.bias_f32 != nullptr, p,
+                                   prev[t]);
+                if (vec)
+                    *(v4f *)((float *)D + idx) = o;
+                else
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (j0 + t < g.N)
+                            ((float *)D)[idx + t] = o[t];
+                }
+            }
+        }
+    }
+}
+// FIXEDPOINT epilogue of the pipelined kernel for multipliers >= 0. The block's per-column constants were staged in LDS
+// as par[6][BN]: row 0 the folded offset/bias vector, rows 1..5 the QP_* vectors; col_in_tile is the wave's first
+// column inside the block tile. Same accumulator layout as epilogue_store_t.
+template <int RS, int QS, int BN>
+__device__ __forceinline__ void epilogue_store_fast(const v4i (&acc)[RS][QS], const GemmArgs &g, const int32_t *par,
+                                                    int row0, int col0, int col_in_tile, int lane, int bz)
+{
+    const int        lr = lane & 15, lh = lane >> 4;
+    const EpiParams &p      = g.epi;
+    const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
+    char            *D      = (char *)g.D;
+    int32_t          rv[RS];
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs)
+    {
+        const int i = row0 + rs * 16 + lr;
+        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+    }
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs)
+    {
+        const int c  = col_in_tile + qs * 16 + 4 * lh;
+        const int j0 = col0 + qs * 16 + 4 * lh;
+        const v4i cv = *(const v4i *)(par + 0 * BN + c);
+        const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
+        const v4i cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
+        const v4i ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
+        const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
+        const v4i rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
+        {
+            const int i = row0 + rs * 16 + lr;
+            int32_t   o[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+            {
+                const int32_t v = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv[rs]);
+                o[t]            = fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
+            }
+            // low bytes of o[0..3] -> one dword
+            const uint32_t p01    = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
+            const uint32_t p23    = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
+            const uint32_t packed = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+            if (i >= g.M || j0 >= g.N)
+                continue;
+            const int64_t idx = (int64_t)bz * g.d_batch_stride + (int64_t)i * g.ldd + j0;
+            if (p.vec_store && (j0 + 3 < g.N))
+                *(uint32_t *)(D + idx) = packed;
+            else
+            {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (j0 + t < g.N)
+                        D[idx + t] = (char)(packed >> (8 * t));
+            }
         }
     }
 }
 // The same arithmetic as epilogue_store_fast, but the packed 8-bit results of the whole BM x BN block tile are first
-// laid out in LDS (row pitch BN + 16 bytes) and then written with 16 bytes per lane, BN/16 lanes per output row, so a
-// wave instruction writes whole rows of the tile instead of 8-byte pieces of 32 different rows. All NW consumer waves
-// of the block call this together; `barrier` is executed once between the two phases by every wave of the block.
-// Requires p.vec_store16. stage must not overlap par.
-template <bool STD, int FM, int FN, int BM, int BN, int NW, typename Barrier>
-__device__ __forceinline__ void epilogue_store_staged(const v16i (&acc)[FM][FN], const GemmArgs &g, const int32_t *par,
+// laid out in LDS (row pitch BN + 16 bytes: the 64 dword writes of a wave instruction - 16 rows by 4 dwords - then hit
+// 64 different banks) and then written with 16 bytes per lane, BN/16 lanes per output row, so a wave instruction writes
+// whole rows of the tile instead of 16-byte pieces of 16 different rows. All NW consumer waves of the block call this
+// together; `barrier` is executed once between the two phases by every wave of the block. Requires p.vec_store16.
+// stage must not overlap par.
+template <bool STD, int RS, int QS, int BM, int BN, int NW, typename Barrier>
+__device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], const GemmArgs &g, const int32_t *par,
                                                       char *stage, int m0, int n0, int row_in_tile, int col_in_tile,
                                                       int wave, int lane, int bz, Barrier barrier)
 {
     constexpr int    PITCH = BN + 16;
-    const int        lr = lane & 31, lh = lane >> 5;
+    const int        lr = lane & 15, lh = lane >> 4;
     const EpiParams &p      = g.epi;
     const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
-    int32_t          rv[FM];
+    int32_t          rv[RS];
     const int32_t    off2p1 = 2 * p.result_offset + 1;
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
+    for (int rs = 0; rs < RS; ++rs)
     {
-        const int i = m0 + row_in_tile + fm * 32 + lr;
-        rv[fm]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+        const int i = m0 + row_in_tile + rs * 16 + lr;
+        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
     }
 #pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
+    for (int qs = 0; qs < QS; ++qs)
     {
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
+        const int c  = col_in_tile + qs * 16 + 4 * lh;
+        const v4i cv = *(const v4i *)(par + 0 * BN + c);
+        const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
+        const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
+        v4i       cm = {0, 0, 0, 0}, ls = cm, rm = cm;
+        if (!STD)
         {
-            const int c  = col_in_tile + fn * 32 + 8 * q + 4 * lh;
-            const v4i cv = *(const v4i *)(par + 0 * BN + c);
-            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BN + c);
-            const v4i r1 = *(const v4i *)(par + (1 + QP_RSM1) * BN + c);
-            v4i       cm = {0, 0, 0, 0}, ls = cm, rm = cm;
-            if (!STD)
-            {
-                cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
-                ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
-                rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
-            }
+            cm = *(const v4i *)(par + (1 + QP_CMASK) * BN + c);
+            ls = *(const v4i *)(par + (1 + QP_LS) * BN + c);
+            rm = *(const v4i *)(par + (1 + QP_RMASK) * BN + c);
+        }
 #pragma unroll
-            for (int fm = 0; fm < FM; ++fm)
-            {
-                int32_t o[4];
+        for (int rs = 0; rs < RS; ++rs)
+        {
+            int32_t o[4];
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                {
-                    const int32_t v = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv[fm]);
-                    o[t] = STD ? std_requant(v, s2[t], r1[t], off2p1, p.lo, p.hi)
-                               : fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
-                }
-                const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
-                const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
-                *(uint32_t *)(stage + (row_in_tile + fm * 32 + lr) * PITCH + c) =
-                    __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+            for (int t = 0; t < 4; ++t)
+            {
+                const int32_t v = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv[rs]);
+                o[t] = STD ? std_requant(v, s2[t], r1[t], off2p1, p.lo, p.hi)
+                           : fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
             }
+            const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
+            const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
+            *(uint32_t *)(stage + (row_in_tile + rs * 16 + lr) * PITCH + c) = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
         }
     }
     barrier();
@@ -404,62 +392,59 @@ __device__ __forceinline__ void epilogue_store_staged(const v16i (&acc)[FM][FN],
         }
     }
 }
-// S32 / F32 results of one wave's (FM*32) x (FN*32) sub-tile, 32 rows at a time through a wave-private LDS area
-// (32 rows, pitch FN*128 + 16 bytes) so that they leave as 16 bytes per lane along whole row segments of FN*128 bytes
-// instead of 32-byte pieces of 32 different rows. Needs no synchronisation with other waves. Requires p.vec_store.
-template <int EPI, int FM, int FN>
-__device__ __forceinline__ void epilogue_store_wave32(const v16i (&acc)[FM][FN], const GemmArgs &g, char *stage, int row0,
+// S32 / F32 results of one wave's (RS*16) x (QS*16) sub-tile, 16 rows at a time through a wave-private LDS area
+// (16 rows, pitch QS*64 + 16 bytes) so that they leave as 16 bytes per lane along whole row segments of QS*64 bytes
+// instead of 16-byte pieces of 16 different rows. Needs no synchronisation with other waves. Requires p.vec_store.
+template <int EPI, int RS, int QS>
+__device__ __forceinline__ void epilogue_store_wave32(const v4i (&acc)[RS][QS], const GemmArgs &g, char *stage, int row0,
                                                       int col0, int lane, int bz)
 {
     static_assert(EPI == EPI_S32 || EPI == EPI_F32, "32-bit outputs only");
-    constexpr int    PITCH = FN * 128 + 16;
-    constexpr int    LPR   = FN * 8;   // lanes per output row segment
+    constexpr int    PITCH = QS * 64 + 16;
+    constexpr int    LPR   = QS * 4;   // lanes per output row segment
     constexpr int    RPI   = 64 / LPR; // rows per wave instruction
-    const int        lr = lane & 31, lh = lane >> 5;
+    static_assert(LPR <= 64 && 16 % RPI == 0, "wave tile width");
+    const int        lr = lane & 15, lh = lane >> 4;
     const EpiParams &p      = g.epi;
     const int32_t   *colvec = p.colvec + (int64_t)bz * p.colvec_batch_stride;
     const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
     char            *D      = (char *)g.D + (int64_t)bz * g.d_batch_stride * 4;
     const int        rr = lane / LPR, cc = lane % LPR;
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
+    for (int rs = 0; rs < RS; ++rs)
     {
-        const int     i  = row0 + fm * 32 + lr;
+        const int     i  = row0 + rs * 16 + lr;
         const int32_t rv = (rowvec && i < g.M) ? rowvec[i] : 0;
 #pragma unroll
-        for (int fn = 0; fn < FN; ++fn)
+        for (int qs = 0; qs < QS; ++qs)
         {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
+            const int c  = qs * 16 + 4 * lh;
+            const int j0 = col0 + c; // inside the padded vectors
+            const v4i cv = *(const v4i *)(colvec + j0);
+            v4i       o;
+            if (EPI == EPI_S32)
             {
-                const int c  = fn * 32 + 8 * q + 4 * lh;
-                const int j0 = col0 + c; // inside the padded vectors
-                const v4i cv = *(const v4i *)(colvec + j0);
-                v4i       o;
-                if (EPI == EPI_S32)
-                {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = (int32_t)((uint32_t)acc[fm][fn][4 * q + t] + (uint32_t)cv[t] + (uint32_t)rv);
-                }
-                else
-                {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                    {
-                        const float bf = (p.bias_f32 && j0 + t < g.N) ? p.bias_f32[j0 + t] : 0.f;
-                        o[t] = __float_as_int(epi_f32(acc[fm][fn][4 * q + t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bf,
-                                                      p.bias_f32 != nullptr, p));
-                    }
-                }
-                *(v4i *)(stage + lr * PITCH + c * 4) = o;
+                for (int t = 0; t < 4; ++t)
+                    o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv);
             }
+            else
+            {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                {
+                    const float bf = (p.bias_f32 && j0 + t < g.N) ? p.bias_f32[j0 + t] : 0.f;
+                    o[t] = __float_as_int(epi_f32(acc[rs][qs][t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bf,
+                                                  p.bias_f32 != nullptr, p));
+                }
+            }
+            *(v4i *)(stage + lr * PITCH + c * 4) = o;
         }
 #pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it)
+        for (int it = 0; it < 16 / RPI; ++it)
         {
             const int r  = it * RPI + rr;
-            const int gi = row0 + fm * 32 + r, j0 = col0 + cc * 4;
+            const int gi = row0 + rs * 16 + r, j0 = col0 + cc * 4;
             if (gi >= g.M || j0 >= g.N)
                 continue;
             const v4i     val = *(const v4i *)(stage + r * PITCH + cc * 16);

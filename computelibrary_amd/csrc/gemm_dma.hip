@@ -19,13 +19,18 @@
 // in their operand-read slot, and the producers only the A panel.
 //
 // LDS -> matrix cores: the consumers form two groups of four (one wave of each group per SIMD) that run half a K step
-// apart ("ping-pong"): while one group streams its 16 matrix instructions for a K step out of registers, the other
+// apart ("ping-pong"): while one group streams its 32 matrix instructions for a K step out of registers, the other
 // group reads its operands for the next step from LDS. Two workgroup barriers per K step keep the groups in
 // anti-phase; group 1 takes one extra barrier before the loop and group 0 one after it, so every wave executes the
 // same number of barriers.
 //
+// The matrix instruction is v_mfma_i32_16x16x64_i8, not the 32x32x32 one: both do the same multiply-accumulates per
+// clock, but the longer K per instruction halves the accumulator updates per multiply, and under this part's power limit
+// (random operands) that is worth about 10 % of the kernel's time. Operand traffic is the same: it is set by the wave's
+// 64 x 64 sub-tile, 4 + 4 operand blocks of 16 rows x 64 bytes per 64 of K.
+//
 // Accumulators are kept transposed (the B panel is fed as the first matrix operand), so each lane ends up with 4
-// consecutive output columns per register quad: the epilogue reads the per-column parameters as 16-byte vectors and
+// consecutive output columns per accumulator block: the epilogue reads the per-column parameters as 16-byte vectors and
 // packs 4 int8 results into one dword. Those dwords go to LDS first (the ring is free by then) and leave as whole
 // 128-byte tile rows, 16 bytes per lane; where the destination is not 16-byte aligned they are stored directly.
 #include "mfma_common.hpp"

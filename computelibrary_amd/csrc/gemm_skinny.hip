@@ -20,10 +20,15 @@ namespace mi355
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 
-template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL>
+// Row pitch of the staged copy of A (STAGE_A): 1 KiB of a row's K slice + 64 bytes, which spreads the 8 rows an
+// operand read touches over the LDS banks
+constexpr int SK_A_PITCH = 1024 + 64;
+
+template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 {
     __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][SK_A_PITCH]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -74,26 +79,70 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
         acc[n] = (v4i){0, 0, 0, 0};
     const v4i zero4 = {0, 0, 0, 0};
     int       kb    = kb0;
-    // whole steps inside the wave's range and inside K: straight-line loads, all in flight together
-    for (; kb + SK_UNROLL <= kb1 && (kb + SK_UNROLL) * 64 <= g.K; kb += SK_UNROLL)
+
+    // STAGE_A (M <= 8, every wave's K slice at most 1 KiB per row, K a multiple of 64, 16-byte aligned rows): the wave
+    // copies its slice of A into LDS once, with all 64 lanes per load, and takes the operand blocks from there.
+    // Loading them from global memory inside the stream costs one half-empty load instruction (rows 8..15 are padding)
+    // per B load and 16 % of the kernel's time, although A never leaves the L2.
+    char *a_lds = a_stage + wave * 8 * SK_A_PITCH;
+    v4i   ta[STAGE_A ? 8 : 1];
+    if (STAGE_A)
     {
-        v4i fa[SK_UNROLL], fb[SK_UNROLL][NG];
+        // branch-free (a branch per row would put a full wait behind every load): rows past M re-read row M-1 into
+        // staging rows nobody reads, lanes past the slice re-read its first 16 bytes into the unused end of the pitch
+        const int slice = max(kb1 - kb0, 0) * 64; // bytes per row, <= 1024
+        const int col   = lane * 16 < slice ? lane * 16 : 0;
+        const int8_t *src = g.A + (int64_t)min(kb0, KB - 1) * 64 + col;
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            ta[r] = *(const v4i *)(src + (int64_t)min(r, g.M - 1) * g.lda);
+    }
+    const char *a_frag = a_lds + arow * SK_A_PITCH + akc; // this lane's piece of the operand block of k block kb0
+    // whole steps inside the wave's range and inside K: straight-line loads, all in flight together; the loads of the
+    // next step directly follow the matrix instructions of this one. (Issuing the first step's loads before the wave
+    // waits for its slice of A measured 1 % slower: the 8 + 8 registers of both are then live together.)
+    v4i  fb[SK_UNROLL][NG];
+    auto whole_step = [&](int k) { return k + SK_UNROLL <= kb1 && (k + SK_UNROLL) * 64 <= g.K; };
+    auto load_b     = [&](int k)
+    {
 #pragma unroll
         for (int u = 0; u < SK_UNROLL; ++u)
-        {
-            fa[u] = zero4;
 #pragma unroll
             for (int n = 0; n < NG; ++n)
-                fb[u][n] = __builtin_nontemporal_load((const v4i *)(b_ptr[n] + (int64_t)(kb + u) * 1024));
+                fb[u][n] = __builtin_nontemporal_load((const v4i *)(b_ptr[n] + (int64_t)(k + u) * 1024));
+    };
+    if (STAGE_A)
+    {
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+        {
+            if (FLIP_A)
+                ta[r] ^= (int)0x80808080;
+            *(v4i *)(a_lds + r * SK_A_PITCH + lane * 16) = ta[r];
         }
+    }
+    bool more = whole_step(kb);
+    if (more)
+        load_b(kb);
+    while (more)
+    {
+        v4i fa[SK_UNROLL];
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; ++u)
+            fa[u] = zero4;
         if (a_live)
         {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u)
             {
-                fa[u] = *(const v4i *)(a_ptr + (int64_t)(kb + u) * 64);
-                if (FLIP_A)
-                    fa[u] ^= (int)0x80808080;
+                if (STAGE_A)
+                    fa[u] = *(const v4i *)(a_frag + (kb + u - kb0) * 64);
+                else
+                {
+                    fa[u] = *(const v4i *)(a_ptr + (int64_t)(kb + u) * 64);
+                    if (FLIP_A)
+                        fa[u] ^= (int)0x80808080;
+                }
             }
         }
 #pragma unroll
@@ -101,6 +150,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 #pragma unroll
             for (int n = 0; n < NG; ++n)
                 acc[n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u][n], acc[n], 0, 0, 0);
+        kb += SK_UNROLL;
+        more = whole_step(kb);
+        if (more)
+            load_b(kb);
     }
     // remaining k blocks one at a time, with the guarded loads of the K tail
     for (; kb < kb1; ++kb)
@@ -110,7 +163,12 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
         for (int n = 0; n < NG; ++n)
             fb[n] = *(const v4i *)(b_ptr[n] + (int64_t)kb * 1024);
         const int rem = g.K - (kb * 64 + akc);
-        if (a_live && rem > 0)
+        if (STAGE_A)
+        {
+            if (a_live)
+                fa = *(const v4i *)(a_frag + (kb - kb0) * 64);
+        }
+        else if (a_live && rem > 0)
         {
             fa = rem >= 16 ? *(const v4i *)(a_ptr + (int64_t)kb * 64) : load16_partial(a_ptr + (int64_t)kb * 64, rem);
             if (FLIP_A)
@@ -161,12 +219,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     }
 }
 
-template <int NG, int WAVES, int UNROLL>
+template <int NG, int WAVES, int UNROLL, bool STAGE_A>
 static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
 {
-    const int  groups = (a.N + 15) / 16;
-    const dim3 grid((groups + NG - 1) / NG), block(WAVES * 64);
-#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL><<<grid, block, 0, s>>>(a)
+    const int    groups = (a.N + 15) / 16;
+    const dim3   grid((groups + NG - 1) / NG), block(WAVES * 64);
+    const size_t lds = STAGE_A ? (size_t)WAVES * 8 * SK_A_PITCH : 0;
+#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A><<<grid, block, lds, s>>>(a)
     if (epi == EPI_S32)
         flip_a ? MI355_SK(EPI_S32, true) : MI355_SK(EPI_S32, false);
     else if (epi == EPI_FIXEDPOINT)
@@ -188,6 +247,12 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     static const char *force  = getenv("MI355_SKINNY_WAVES");
     const int          groups = (args.N + 15) / 16;
     const int          waves  = force ? atoi(force) : (groups >= 512 ? 4 : 8);
-    return waves == 4 ? skinny_launch_v<1, 4, 8>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8>(epi, flip_a, args, s);
+    // A goes through LDS when a wave's K slice fits 1 KiB per row and nothing about it needs guarding
+    const int  per   = ((int)(args.Kp / 64) + waves - 1) / waves;
+    const bool stage = args.M <= 8 && per <= 16 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
+                       ((uintptr_t)args.A & 15) == 0 && getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    if (stage)
+        return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, s);
+    return waves == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);
 }
 } // namespace mi355

@@ -165,7 +165,9 @@ struct GemmCore
         Kp = round_up(K, PACK_K_ALIGN);
         Np = round_up(N, PACK_N_ALIGN);
         if (path == MI355_PATH_AUTO)
-            path = (M <= SKINNY_MAX_M && batch == 1) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
+            // measured: up to 32 rows the streaming kernel always wins; up to 64 rows only while N is small enough
+            // that the pipelined kernel would leave most compute units without a tile
+            path = (batch == 1 && (M <= 32 || (M <= SKINNY_MAX_M && N < 8192))) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
         if (path == MI355_PATH_SKINNY && (M > SKINNY_MAX_M || batch != 1))
             return fail("skinny path needs M <= %d and batch == 1", SKINNY_MAX_M);
         if (path == MI355_PATH_SIMPLE)
@@ -193,12 +195,41 @@ struct GemmCore
                 (void)env;
                 return best;
             };
+            // The pipelined kernel's tile is chosen with a small cost model in clocks per compute unit, from what was
+            // measured on the device: a K step costs the largest of its direct-to-LDS stream (about 44 bytes per
+            // clock and compute unit), its matrix instructions (4096 multiply-accumulates per clock) and the two
+            // barrier-separated slots of the consumer groups (about 1000 clocks per 128 bytes of K, whatever the tile);
+            // every tile adds a fixed start-up plus an epilogue proportional to its outputs, which co-resident
+            // workgroups overlap. Ties go to the deeper ring (more loads in flight when B comes from HBM).
+            auto pick_dma = [&]() -> int
+            {
+                int    best = -1, best_lds = 0;
+                double best_cost = 0;
+                for (int i = 0; i < DMA_AUTO_CONFIGS; ++i)
+                {
+                    const MfmaConfig c = dma_config(i);
+                    if ((N <= 64 && c.BN > 64) || Kp % c.BK != 0)
+                        continue;
+                    const double tiles   = (double)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN) * batch;
+                    const double per_cu  = std::ceil(tiles / cus);
+                    const int    occ_lds = (160 * 1024) / c.lds_bytes, occ_wav = 32 / c.waves;
+                    const double occ     = std::max(1, std::min(occ_lds, occ_wav));
+                    const double nk      = (double)((K + c.BK - 1) / c.BK);
+                    const double step    = std::max({(double)(c.BM + c.BN) * c.BK / 44.0, (double)c.BM * c.BN * c.BK / 4096.0,
+                                                     1000.0 * c.BK / 128.0});
+                    const double fixed   = 6000.0 + (double)c.BM * c.BN / 4.4;
+                    const double cost    = per_cu * nk * step + std::ceil(per_cu / occ) * fixed;
+                    if (best < 0 || cost < best_cost || (cost == best_cost && c.lds_bytes > best_lds))
+                        best = i, best_cost = cost, best_lds = c.lds_bytes;
+                }
+                return best;
+            };
             cfg_idx = pick(mfma_num_configs(), mfma_config, nullptr);
-            dma_idx = pick(DMA_AUTO_CONFIGS, dma_config, nullptr);
+            dma_idx = pick_dma();
             const char *f1 = getenv("MI355_GEMM_CFG"), *f2 = getenv("MI355_DMA_CFG");
             if (f1 && atoi(f1) >= 0 && atoi(f1) < mfma_num_configs())
                 cfg_idx = atoi(f1);
-            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs())
+            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs() && Kp % dma_config(atoi(f2)).BK == 0)
                 dma_idx = atoi(f2);
             if (getenv("MI355_NO_DMA") || K < 16)
                 dma_idx = -1;

@@ -83,9 +83,10 @@ struct PanelProducer
     static constexpr int LPA   = (AU + NP - 1) / NP; // at most this many of them are A units
     static constexpr int STAGE = (BM + BN) * BK;
     static_assert((AU + BU) % NP == 0, "staging shape");
-    // swz(row) of row = u*RPU + r depends on u only through (4u) & (CPR-1): constant for CPR <= 4, the parity of u for
-    // CPR == 8 - and u = pw + i*NP keeps its parity when NP is even
-    static_assert(CPR <= 4 || (CPR == 8 && NP % 2 == 0), "every unit of a producer wave must share the lane -> column map");
+    // swz(row) of row = u*RPU + r depends on u only through (u*RPU) & (CPR-1): constant for CPR <= 4, the parity of u
+    // for CPR == 8 and u mod 4 for CPR == 16 - and u = pw + i*NP keeps those when NP is a multiple of 2 and 4
+    static_assert(CPR <= 4 || (CPR == 8 && NP % 2 == 0) || (CPR == 16 && NP % 4 == 0),
+                  "every unit of a producer wave must share the lane -> column map");
 
     const int8_t *a_base, *b_base, *fill16, *a_end; // wave-uniform
     uint32_t      lane_a, lane_b; // dense A: (l / CPR) * lda + column bytes; B: (l / CPR) * Kp + column bytes
@@ -389,12 +390,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
                     fa[kk][f] ^= (int)0x80808080;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        // the units this wave issued one K step ago (stage kt+NS-2) have to be in LDS before the barrier that opens
-        // that stage to its first reader; only the CBU just issued may still be in flight
+        // this wave's units of stage kt+1 have to be in LDS before the barrier that opens that stage to its first
+        // reader; the NS-2 younger stages (the last of them just issued) may still be in flight
         if (CDMA)
         {
             if (kt + NS - 1 < nk)
-                wait_vmcnt<CBU>();
+                wait_vmcnt<(NS - 2) * CBU>();
             else
                 wait_vmcnt<0>();
         }
@@ -479,6 +480,8 @@ static const DmaEntry g_dma[] = {
     MI355_DCFG("pp_128x128x128_s3", 128, 128, 128, 2, 2, 3),
     MI355_DCFG("pp_128x64x128_s3", 128, 64, 128, 2, 2, 3),
     MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
+    MI355_DCFG("pp_64x64x128_s6", 64, 64, 128, 1, 2, 6),
+    MI355_DCFG("pp_128x64x256_s3", 128, 64, 256, 2, 2, 3),
     MI355_DCFG("pp_256x128x64_s4", 256, 128, 64, 2, 2, 4),
 };
 
@@ -488,7 +491,10 @@ int dma_num_configs()
 }
 MfmaConfig dma_config(int idx)
 {
-    return g_dma[idx].cfg;
+    MfmaConfig c = g_dma[idx].cfg;
+    c.waves      = g_dma[idx].threads / 64;
+    c.lds_bytes  = g_dma[idx].lds_bytes;
+    return c;
 }
 
 int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s)

@@ -1,4 +1,4 @@
-// K3: bandwidth-bound GEMM for M <= 16 (decode-shaped: one token batch against a large weight matrix).
+// K3: bandwidth-bound GEMM for M <= 64 (decode-shaped: one token batch against a large weight matrix).
 //
 // The reference has no dedicated kernel above M == 1 (GemvPretransposed, src/core/NEON/kernels/arm_gemm/gemm_qint8.cpp:75-79)
 // and otherwise runs its hybrid kernels; here the whole run is one streaming pass over B at HBM speed.
@@ -6,9 +6,9 @@
 // B is packed at prepare time into 1 KiB blocks of 16 columns x 64 k in matrix-core operand order
 // (Bs[Np/16][Kp/64][64 lanes][16 bytes]), so every wave-wide load is one contiguous, fully coalesced 1 KiB read and a
 // column group's K range is one contiguous stream. A block owns NG groups of 16 output columns; its WAVES waves split
-// the k blocks, each keeping UNROLL steps of loads in flight, multiply with v_mfma_i32_16x16x64_i8 (A rows padded to 16
-// with zeros; A itself is tiny and stays in L2), reduce the partial 16 x 16 accumulators through LDS, and wave 0 applies
-// the fused offset / requantisation epilogue. The kernel lives on memory-level parallelism: every block of the grid
+// the k blocks, each keeping UNROLL steps of loads in flight, multiply with v_mfma_i32_16x16x64_i8 (MR blocks of 16 A
+// rows, padded with zeros; A itself is tiny and stays in L2), reduce the partial 16 x 16 accumulators through LDS, and
+// wave r applies the fused offset / requantisation epilogue to row block r. The kernel lives on memory-level parallelism: every block of the grid
 // should be resident at once, so the register footprint is kept small (the K tail has its own one-step loop) and the
 // number of waves per block is chosen from the number of column groups.
 #include "internal.hpp"
@@ -24,9 +24,10 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 // operand read touches over the LDS banks
 constexpr int SK_A_PITCH = 1024 + 64;
 
-template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A>
+template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A, int MR>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 {
+    static_assert(MR >= 1 && MR <= SK_WAVES && (!STAGE_A || MR == 1), "row blocks");
     __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
     extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][SK_A_PITCH]
 
@@ -36,8 +37,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     const int KB   = (int)(g.Kp / 64);
     const int NGT  = (int)((g.N + 15) / 16);
 
-    // wave 0 applies the epilogue to column ng0*16 + (lane%16) + 16*n: fetch its per-column constants now, so that
-    // their latency is hidden behind the B stream instead of following it
+    // waves 0..MR-1 apply the epilogue to column ng0*16 + (lane%16) + 16*n: fetch its per-column constants now, so
+    // that their latency is hidden behind the B stream instead of following it
     const EpiParams &p = g.epi;
     int32_t          cv[NG], mu[NG], sh[NG];
     float            bf[NG];
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     {
         const int j = min((ng0 + n) * 16 + (lane & 15), g.N - 1);
         cv[n] = 0, mu[n] = p.mult_s, sh[n] = p.shift_s, bf[n] = 0.f;
-        if (wave == 0)
+        if (wave < MR)
         {
             cv[n] = p.colvec[j];
             if (EPI == EPI_FIXEDPOINT && p.mult)
@@ -66,17 +67,25 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 
     const int   arow   = lane & 15;
     const int   akc    = (lane >> 4) * 16;
-    const bool  a_live = arow < g.M;
-    const int8_t *__restrict__ a_ptr = g.A + (int64_t)min(arow, g.M - 1) * g.lda + akc;
+    bool          a_live[MR];
+    const int8_t *a_ptr[MR]; // rows past M re-read row M-1 and multiply as zeros
+#pragma unroll
+    for (int rb = 0; rb < MR; ++rb)
+    {
+        a_live[rb] = rb * 16 + arow < g.M;
+        a_ptr[rb]  = g.A + (int64_t)min(rb * 16 + arow, g.M - 1) * g.lda + akc;
+    }
     const int8_t *b_ptr[NG];
 #pragma unroll
     for (int n = 0; n < NG; ++n)
         b_ptr[n] = g.Bp + ((int64_t)min(ng0 + n, NGT - 1) * KB * 64 + lane) * 16;
 
-    v4i acc[NG];
+    v4i acc[MR][NG];
 #pragma unroll
-    for (int n = 0; n < NG; ++n)
-        acc[n] = (v4i){0, 0, 0, 0};
+    for (int rb = 0; rb < MR; ++rb)
+#pragma unroll
+        for (int n = 0; n < NG; ++n)
+            acc[rb][n] = (v4i){0, 0, 0, 0};
     const v4i zero4 = {0, 0, 0, 0};
     int       kb    = kb0;
 
@@ -121,77 +130,156 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
             *(v4i *)(a_lds + r * SK_A_PITCH + lane * 16) = ta[r];
         }
     }
-    bool more = whole_step(kb);
-    if (more)
-        load_b(kb);
-    while (more)
+    if constexpr (MR == 1)
     {
-        v4i fa[SK_UNROLL];
+        bool more = whole_step(kb);
+        if (more)
+            load_b(kb);
+        while (more)
+        {
+            v4i fa[SK_UNROLL];
 #pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u)
-            fa[u] = zero4;
-        if (a_live)
+            for (int u = 0; u < SK_UNROLL; ++u)
+                fa[u] = zero4;
+            if (a_live[0])
+            {
+#pragma unroll
+                for (int u = 0; u < SK_UNROLL; ++u)
+                {
+                    if (STAGE_A)
+                        fa[u] = *(const v4i *)(a_frag + (kb + u - kb0) * 64);
+                    else
+                    {
+                        fa[u] = *(const v4i *)(a_ptr[0] + (int64_t)(kb + u) * 64);
+                        if (FLIP_A)
+                            fa[u] ^= (int)0x80808080;
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+                for (int n = 0; n < NG; ++n)
+                    acc[0][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u][n], acc[0][n], 0, 0, 0);
+            kb += SK_UNROLL;
+            more = whole_step(kb);
+            if (more)
+                load_b(kb);
+        }
+    }
+    else
+    {
+        // Several row blocks: the operand blocks of A come from the L2 with every step, so a wave would wait a full
+        // memory latency per step. Two register sets instead: the loads of step s+1 (B and A, branch-free - rows past
+        // M re-read row M-1 and are zeroed afterwards) are issued before the matrix instructions of step s.
+        v4i  fa[SK_UNROLL][MR], fb2[SK_UNROLL][NG], fa2[SK_UNROLL][MR];
+        auto load_ab = [&](v4i(&b)[SK_UNROLL][NG], v4i(&a)[SK_UNROLL][MR], int k)
         {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u)
             {
-                if (STAGE_A)
-                    fa[u] = *(const v4i *)(a_frag + (kb + u - kb0) * 64);
-                else
-                {
-                    fa[u] = *(const v4i *)(a_ptr + (int64_t)(kb + u) * 64);
-                    if (FLIP_A)
-                        fa[u] ^= (int)0x80808080;
-                }
+#pragma unroll
+                for (int n = 0; n < NG; ++n)
+                    b[u][n] = __builtin_nontemporal_load((const v4i *)(b_ptr[n] + (int64_t)(k + u) * 1024));
+#pragma unroll
+                for (int rb = 0; rb < MR; ++rb)
+                    a[u][rb] = *(const v4i *)(a_ptr[rb] + (int64_t)(k + u) * 64);
             }
-        }
+        };
+        auto multiply = [&](v4i(&b)[SK_UNROLL][NG], v4i(&a)[SK_UNROLL][MR])
+        {
 #pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u)
+            for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-            for (int n = 0; n < NG; ++n)
-                acc[n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u][n], acc[n], 0, 0, 0);
-        kb += SK_UNROLL;
-        more = whole_step(kb);
+                for (int rb = 0; rb < MR; ++rb)
+                {
+                    if (FLIP_A)
+                        a[u][rb] ^= (int)0x80808080;
+                    if (!a_live[rb])
+                        a[u][rb] = zero4;
+#pragma unroll
+                    for (int n = 0; n < NG; ++n)
+                        acc[rb][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][rb], b[u][n], acc[rb][n], 0, 0, 0);
+                }
+        };
+        bool more = whole_step(kb);
         if (more)
-            load_b(kb);
+            load_ab(fb, fa, kb);
+        while (more)
+        {
+            const bool more2 = whole_step(kb + SK_UNROLL);
+            if (more2)
+                load_ab(fb2, fa2, kb + SK_UNROLL);
+            multiply(fb, fa);
+            kb += SK_UNROLL;
+            if (!more2)
+                break;
+            more = whole_step(kb + SK_UNROLL);
+            if (more)
+                load_ab(fb, fa, kb + SK_UNROLL);
+            multiply(fb2, fa2);
+            kb += SK_UNROLL;
+        }
     }
     // remaining k blocks one at a time, with the guarded loads of the K tail
     for (; kb < kb1; ++kb)
     {
-        v4i fa = zero4, fb[NG];
+        v4i fa[MR], fb[NG];
 #pragma unroll
         for (int n = 0; n < NG; ++n)
             fb[n] = *(const v4i *)(b_ptr[n] + (int64_t)kb * 1024);
         const int rem = g.K - (kb * 64 + akc);
-        if (STAGE_A)
+#pragma unroll
+        for (int rb = 0; rb < MR; ++rb)
         {
-            if (a_live)
-                fa = *(const v4i *)(a_frag + (kb - kb0) * 64);
-        }
-        else if (a_live && rem > 0)
-        {
-            fa = rem >= 16 ? *(const v4i *)(a_ptr + (int64_t)kb * 64) : load16_partial(a_ptr + (int64_t)kb * 64, rem);
-            if (FLIP_A)
-                fa ^= (int)0x80808080;
+            fa[rb] = zero4;
+            if (STAGE_A)
+            {
+                if (a_live[rb])
+                    fa[rb] = *(const v4i *)(a_frag + (kb - kb0) * 64);
+            }
+            else if (a_live[rb] && rem > 0)
+            {
+                fa[rb] = rem >= 16 ? *(const v4i *)(a_ptr[rb] + (int64_t)kb * 64)
+                                   : load16_partial(a_ptr[rb] + (int64_t)kb * 64, rem);
+                if (FLIP_A)
+                    fa[rb] ^= (int)0x80808080;
+            }
         }
 #pragma unroll
-        for (int n = 0; n < NG; ++n)
-            acc[n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb[n], acc[n], 0, 0, 0);
+        for (int rb = 0; rb < MR; ++rb)
+#pragma unroll
+            for (int n = 0; n < NG; ++n)
+                acc[rb][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb], fb[n], acc[rb][n], 0, 0, 0);
     }
 
+    // one row block at a time through the same LDS: wave rb sums and finishes row block rb
+    v4i sum[NG];
 #pragma unroll
     for (int n = 0; n < NG; ++n)
-        *(v4i *)&red[wave][n][lane][0] = acc[n];
-    __syncthreads();
-    if (wave != 0)
-        return;
+        sum[n] = (v4i){0, 0, 0, 0};
 #pragma unroll
-    for (int w = 1; w < SK_WAVES; ++w)
+    for (int rb = 0; rb < MR; ++rb)
+    {
+        if (rb > 0)
+            __syncthreads();
 #pragma unroll
         for (int n = 0; n < NG; ++n)
-            acc[n] += *(const v4i *)&red[w][n][lane][0];
+            *(v4i *)&red[wave][n][lane][0] = acc[rb][n];
+        __syncthreads();
+        if (wave == rb)
+        {
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+#pragma unroll
+                for (int n = 0; n < NG; ++n)
+                    sum[n] += *(const v4i *)&red[w][n][lane][0];
+        }
+    }
+    if (wave >= MR)
+        return;
 
-    // accumulator r of lane l is row 4*(l/16) + r, column l%16
+    // accumulator r of lane l is row 16*rb + 4*(l/16) + r, column l%16
 #pragma unroll
     for (int n = 0; n < NG; ++n)
     {
@@ -201,31 +289,31 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 #pragma unroll
         for (int r = 0; r < 4; ++r)
         {
-            const int i = 4 * (lane >> 4) + r;
+            const int i = 16 * wave + 4 * (lane >> 4) + r;
             if (i < g.M)
             {
                 const int32_t rv  = p.rowvec ? p.rowvec[i] : 0;
                 const int64_t idx = (int64_t)i * g.ldd + j;
                 if (EPI == EPI_S32)
-                    ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)acc[n][r] + (uint32_t)cv[n] + (uint32_t)rv +
+                    ((int32_t *)g.D)[idx] = (int32_t)((uint32_t)sum[n][r] + (uint32_t)cv[n] + (uint32_t)rv +
                                                       (p.accumulate ? (uint32_t)((int32_t *)g.D)[idx] : 0u));
                 else if (EPI == EPI_FIXEDPOINT)
-                    ((int8_t *)g.D)[idx] = (int8_t)epi_fixedpoint(acc[n][r], cv[n], rv, mu[n], sh[n], p);
+                    ((int8_t *)g.D)[idx] = (int8_t)epi_fixedpoint(sum[n][r], cv[n], rv, mu[n], sh[n], p);
                 else
-                    ((float *)g.D)[idx] = epi_f32(acc[n][r], (int32_t)((uint32_t)cv[n] + (uint32_t)rv), bf[n],
+                    ((float *)g.D)[idx] = epi_f32(sum[n][r], (int32_t)((uint32_t)cv[n] + (uint32_t)rv), bf[n],
                                                   p.bias_f32 != nullptr, p, p.accumulate ? ((float *)g.D)[idx] : 0.f);
             }
         }
     }
 }
 
-template <int NG, int WAVES, int UNROLL, bool STAGE_A>
+template <int NG, int WAVES, int UNROLL, bool STAGE_A, int MR = 1>
 static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
 {
     const int    groups = (a.N + 15) / 16;
     const dim3   grid((groups + NG - 1) / NG), block(WAVES * 64);
     const size_t lds = STAGE_A ? (size_t)WAVES * 8 * SK_A_PITCH : 0;
-#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A><<<grid, block, lds, s>>>(a)
+#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR><<<grid, block, lds, s>>>(a)
     if (epi == EPI_S32)
         flip_a ? MI355_SK(EPI_S32, true) : MI355_SK(EPI_S32, false);
     else if (epi == EPI_FIXEDPOINT)
@@ -251,6 +339,26 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     const int  per   = ((int)(args.Kp / 64) + waves - 1) / waves;
     const bool stage = args.M <= 8 && per <= 16 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
                        ((uintptr_t)args.A & 15) == 0 && getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    if (args.M > 16)
+    {
+        // More than one block of 16 rows: A (L2 resident) is re-read once per block of the grid, which costs as much as
+        // the B stream unless a block covers several column groups - as many as still leave a few hundred blocks.
+        static const char *force_ng = getenv("MI355_SKINNY_NG");
+        const int          mr       = args.M > 32 ? 4 : 2;
+        int                ng       = groups >= 1024 ? 4 : (groups >= 512 ? 2 : 1);
+        if (force_ng)
+            ng = atoi(force_ng);
+        ng = ng >= 4 && mr == 4 ? 4 : (ng >= 2 ? 2 : 1);
+        const int blocks = (groups + ng - 1) / ng;
+        const int w      = force ? atoi(force) : (blocks >= 320 ? 4 : 8);
+#define MI355_SKV(NG_, MR_)                                                                          \
+    (w == 4 ? skinny_launch_v<NG_, 4, 2, false, MR_>(epi, flip_a, args, s)                           \
+            : skinny_launch_v<NG_, 8, 2, false, MR_>(epi, flip_a, args, s))
+        if (mr == 2)
+            return ng == 2 ? MI355_SKV(2, 2) : MI355_SKV(1, 2);
+        return ng == 4 ? MI355_SKV(4, 4) : (ng == 2 ? MI355_SKV(2, 4) : MI355_SKV(1, 4));
+#undef MI355_SKV
+    }
     if (stage)
         return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, s);
     return waves == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);

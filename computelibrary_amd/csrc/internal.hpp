@@ -56,6 +56,7 @@ struct MfmaConfig
 {
     const char *name;
     int         BM, BN, BK;
+    int         waves = 0, lds_bytes = 0; // per workgroup (filled in for the pipelined kernel's configurations)
 };
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
@@ -93,10 +94,10 @@ int         mfma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const Gemm
 int         dma_num_configs();
 MfmaConfig  dma_config(int idx);
 int         dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
-constexpr int DMA_AUTO_CONFIGS = 4; // the first entries are the ones the heuristic picks from; the rest are experiments
+constexpr int DMA_AUTO_CONFIGS = 6; // the first entries are the ones the heuristic picks from; the rest are experiments
 
-// gemm_skinny.hip — M <= 16, B packed in matrix-core operand order (see pack_b_skinny)
-constexpr int SKINNY_MAX_M = 16;
+// gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
+constexpr int SKINNY_MAX_M = 64;
 int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
 
 // kernels_aux.hip

@@ -59,7 +59,7 @@ def test_create_rejects_bad_descriptors_without_a_gpu():
     with __import__("pytest").raises(capi.Mi355Error):
         capi.Gemm(4, 4, 4, capi.U8, capi.U8, capi.S32, capi.EPI_S32, lda=2)
     with __import__("pytest").raises(capi.Mi355Error):
-        capi.Gemm(40, 4, 4, capi.U8, capi.U8, capi.S32, capi.EPI_S32, path=capi.PATH_SKINNY)
+        capi.Gemm(80, 4, 4, capi.U8, capi.U8, capi.S32, capi.EPI_S32, path=capi.PATH_SKINNY)
     g = capi.Gemm(4, 4, 4, capi.U8, capi.U8, capi.U8, capi.EPI_FIXEDPOINT, rq=rq)
     assert g.kernel_name.startswith("skinny")
     g.close()

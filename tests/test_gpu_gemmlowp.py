@@ -15,7 +15,7 @@ PATHS = [capi.PATH_SIMPLE, capi.PATH_MFMA, capi.PATH_SKINNY]
 
 
 def paths_for(M, batch=1):
-    return [p for p in PATHS if p != capi.PATH_SKINNY or (M <= 16 and batch == 1)]
+    return [p for p in PATHS if p != capi.PATH_SKINNY or (M <= 64 and batch == 1)]
 
 
 def test_device_is_gfx950():
@@ -143,6 +143,65 @@ def test_random_shape_sweep_against_oracle():
             want = oracle.gemmlowp_f32(A, B, bias, ao, bo, 3e-4)
             got, want = got.view(np.uint32), want.view(np.uint32)
         assert np.array_equal(got, want), "case %d" % case
+
+
+PIPELINED_CONFIGS = ["pp_256x128x128_s3", "pp_128x128x128_s3", "pp_128x64x128_s3", "pp_64x64x128_s3", "pp_64x64x128_s6",
+                     "pp_128x64x256_s3", "pp_256x128x64_s4"]
+
+
+@pytest.mark.parametrize("cfg", range(len(PIPELINED_CONFIGS)))
+def test_every_pipelined_configuration(cfg, monkeypatch):
+    """Each tile / ring-depth configuration of the pipelined kernel, forced through the environment override, on K of
+    one to nine steps with and without a tail (the 256-byte-step configuration needs a packed K that is a multiple of
+    256 and is otherwise replaced by the automatic choice)."""
+    monkeypatch.setenv("MI355_DMA_CFG", str(cfg))
+    rng = np.random.default_rng(70 + cfg)
+    for (M, N, K) in [(300, 200, 512), (70, 129, 100), (257, 64, 1100), (129, 300, 250), (64, 65, 2048)]:
+        A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+        announce("pipelined config", cfg, (M, N, K))
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_MFMA, device=True)
+        kp = -(-K // 128) * 128
+        if cfg != 5 or kp % 256 == 0:
+            assert name == PIPELINED_CONFIGS[cfg], name
+        np.testing.assert_array_equal(got, oracle.gemmlowp_s32(A, B, ao, bo))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, 0, bias, mult, shift, -7, -128, 127, path=capi.PATH_MFMA,
+                          device=True)
+        np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, -7, -128, 127, np.int8))
+        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, path=capi.PATH_MFMA, device=True)
+        np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
+
+
+@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 63, 64])
+def test_skinny_kernel_with_several_row_blocks(M):
+    """17 to 64 rows run as 2 or 4 blocks of 16 rows in the streaming kernel; N picks 1, 2 or 4 column groups per
+    workgroup and 4 or 8 waves; K covers whole steps only, a tail of whole 64-byte blocks, and a ragged tail."""
+    rng = np.random.default_rng(900 + M)
+    for (N, K) in [(100, 200), (4100, 1024), (8200, 333), (16400, 448), (21000, 192)]:
+        a_dt = np.int8 if (N // 100) % 2 else np.uint8
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+        announce("skinny row blocks", (M, N, K), a_dt.__name__)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_SKINNY, device=True)
+        assert name.startswith("skinny"), name
+        np.testing.assert_array_equal(got, oracle.gemmlowp_s32(A, B, ao, bo))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, 0, bias, mult, shift, off, lo, hi, path=capi.PATH_SKINNY,
+                          device=True)
+        np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
+        if a_dt == np.int8:
+            biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, path=capi.PATH_SKINNY,
+                              device=True)
+            np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
 
 
 @pytest.mark.parametrize("K,lda", [(1000, 1000), (1001, 1001), (998, 1000), (64, 80), (17, 17), (1, 1)])

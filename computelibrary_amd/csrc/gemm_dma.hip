@@ -231,6 +231,9 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     constexpr bool CDMA = !CONV && (BU % NW == 0) && (AU % NP == 0) && (AU / NP) % 2 == 0;
     constexpr int  CBU  = CDMA ? BU / NW : 0;   // B units per consumer wave per stage
     constexpr int  PLP  = CDMA ? AU / NP : LPP; // loads per producer wave per stage inside the loop
+    // Small wave tiles: a slot of matrix instructions is much shorter than a slot of operand reads, so running the two
+    // consumer groups one slot apart only serialises their reads; both groups then read and multiply in the same slots.
+    constexpr bool INPHASE = RS * QS * KK <= 16;
     static_assert(TM % 16 == 0 && TN % 16 == 0 && RS >= 1 && QS >= 1 && BK % 64 == 0, "wave tile");
     static_assert(NS >= 3 && (NS - 2) * LPP < 64, "ring depth / vmcnt range");
     static_assert(NW * 16 * (QS * 64 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
@@ -354,7 +357,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     const uint32_t cb_lds  = lds0 + (uint32_t)(AU + wave) * 1024u;
 
     block_barrier(); // barrier 0: stage 0 is in LDS
-    if (group == 1)
+    if (group == 1 && !INPHASE)
         block_barrier(); // group 1 runs one slot behind group 0
 
     v4i fa[KK][RS], fb[KK][QS];
@@ -415,7 +418,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     }
     if (CDMA)
         wait_vmcnt<0>();
-    if (group == 0)
+    if (group == 0 || INPHASE)
         block_barrier(); // barrier 2nk+1; every operand read of every wave is complete beyond this point
 
     if (fast)

@@ -25,7 +25,7 @@ INT8_DENSE_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix rate (5.0 PO
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM-side bytes of one launch of the config-2 kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the
 # same counters read for a plain copy (profiles/gemm_kernels_hbm_traffic_and_lds_counters.txt holds the runs)
-CFG2_MEASURED_TRAFFIC_BYTES = int((33137.7 * (262144.0 / 131086.8) + 8192.0) * 1024)  # 76.2 MB: 67.8 read + 8.4 written
+CFG2_MEASURED_TRAFFIC_BYTES = int((33131.3 * (262144.0 / 131086.8) + 8192.0) * 1024)  # 76.2 MB: 67.8 read + 8.4 written
 
 
 def quantized_multipliers(scales):

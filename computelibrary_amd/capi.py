@@ -8,7 +8,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libmi355gemmlowp.so")
 
-U8, S8, S32, F32, S16 = 0, 1, 2, 3, 4
+U8, S8, S32, F32, S16, F16 = 0, 1, 2, 3, 4, 5
 EPI_S32, EPI_FIXEDPOINT, EPI_F32 = 0, 1, 2
 PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
 GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
@@ -120,7 +120,7 @@ def ptr(x):
 
 def dtype_code(x):
     name = str(x.dtype).replace("torch.", "")
-    return {"uint8": U8, "int8": S8, "int32": S32, "float32": F32, "int16": S16}[name]
+    return {"uint8": U8, "int8": S8, "int32": S32, "float32": F32, "int16": S16, "float16": F16}[name]
 
 
 STAGE_FIXEDPOINT, STAGE_SCALE = 0, 1

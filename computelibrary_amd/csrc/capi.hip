@@ -444,6 +444,7 @@ struct mi355_gemm_handle
     mi355_gemm_desc d;
     GemmCore        core;
     DevBuf          stageA, stageB, stageD, stageBiasF, stageBias, stageMult, stageShift;
+    DevBuf          wsF32; // MI355_F16 destination: the dense F32 matrix the kernels write
 };
 
 struct mi355_conv_handle
@@ -514,8 +515,8 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
                 return 1;
             break;
         case MI355_EPI_F32:
-            if (d.dst_dtype != MI355_F32)
-                return fail("F32 epilogue needs an F32 destination");
+            if (d.dst_dtype != MI355_F32 && d.dst_dtype != MI355_F16)
+                return fail("F32 epilogue needs an F32 or F16 destination");
             break;
         default:
             return fail("unknown epilogue %d", d.epilogue);
@@ -620,7 +621,8 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     const mi355_gemm_desc &d = h->d;
     if (bias_f32 && c.epi != EPI_F32)
         return fail("float bias is only valid with the F32 epilogue");
-    const size_t esz     = d.dst_dtype == MI355_S32 || d.dst_dtype == MI355_F32 ? 4 : 1;
+    const bool   f16     = d.dst_dtype == MI355_F16;
+    const size_t esz     = d.dst_dtype == MI355_S32 || d.dst_dtype == MI355_F32 ? 4 : (f16 ? 2 : 1);
     const size_t a_bytes = (size_t)(d.batch - 1) * d.a_batch_stride + (size_t)(d.M - 1) * d.lda + d.K;
     const size_t d_elems = (size_t)(d.batch - 1) * d.d_batch_stride + (size_t)(d.M - 1) * d.ldd + d.N;
     const void  *Ad, *bfd;
@@ -635,7 +637,24 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
         if (c.accumulate || d.ldd != d.N || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
             HIP_TRY(hipMemcpyAsync(Dd, D, d_elems * esz, hipMemcpyHostToDevice, s)); // previous values / padding
     }
-    TRY(c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, Dd, d.ldd, d.d_batch_stride, (const float *)bfd, s));
+    if (f16)
+    {
+        // the kernels write a dense F32 matrix, which is rounded into the half destination afterwards. Accumulating:
+        // the addition (and the activation, which has to follow it) happens in that second step, on halfs.
+        TRY(h->wsF32.ensure(sizeof(float) * (size_t)d.batch * d.M * d.N));
+        float      *ws  = h->wsF32.as<float>();
+        const bool  acc = c.accumulate, twice = c.act_twice;
+        const float lo = c.act_min, hi = c.act_max;
+        if (acc)
+            c.accumulate = false, c.act_twice = false, c.act_min = -INFINITY, c.act_max = INFINITY;
+        const int rc = c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, ws, d.N, (int64_t)d.M * d.N, (const float *)bfd, s);
+        c.accumulate = acc, c.act_twice = twice, c.act_min = lo, c.act_max = hi;
+        if (rc)
+            return rc;
+        HIP_TRY(f32_to_f16_launch(ws, Dd, d.batch, d.M, d.N, d.ldd, d.d_batch_stride, acc, lo, hi, s));
+    }
+    else
+        TRY(c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, Dd, d.ldd, d.d_batch_stride, (const float *)bfd, s));
     if (d_host)
     {
         HIP_TRY(hipMemcpyAsync(D, Dd, d_elems * esz, hipMemcpyDeviceToHost, s));
@@ -652,7 +671,7 @@ void mi355_gemmlowp_destroy(mi355_gemm_handle *h)
         return;
     h->core.release();
     h->stageA.release(), h->stageB.release(), h->stageD.release(), h->stageBiasF.release(), h->stageBias.release();
-    h->stageMult.release(), h->stageShift.release();
+    h->stageMult.release(), h->stageShift.release(), h->wsF32.release();
     delete h;
 }
 

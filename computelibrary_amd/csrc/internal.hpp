@@ -125,6 +125,10 @@ int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *b
 // [batch][R][C] bytes -> [batch][C][R]
 int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
 // dst[s * dst_stride + c] = src[s * src_stride + c] for s < segments, c < seg (bytes)
+// dense F32 [batch][M][N] -> F16 destination (row stride ldh, batch stride, in elements), optionally added to its
+// previous contents in half arithmetic and clamped
+int f32_to_f16_launch(const float *dense_f32, void *half_matrix, int batch, int M, int N, int64_t ldh,
+                      int64_t h_batch_stride, bool accumulate, float act_min, float act_max, hipStream_t s);
 int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64_t src_stride, int64_t dst_stride,
                     hipStream_t s);
 int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);

@@ -536,6 +536,45 @@ int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64
     return launch_status();
 }
 
+// ---- F16 destinations: [batch][M][N] halfs with row / batch strides <- the dense F32 matrix the GEMM kernels write --------
+// Conversion to half rounds to nearest even (the reference's host-side half type is configured the same way,
+// support/Half.h:33-34). Accumulating: the rounded half is added to the previous half as the reference's test oracle
+// adds halfs (both widened, one float addition, rounded again; tests/validation/fixtures/GEMMLowpFixture.h:912-918),
+// and the activation clamp follows the addition.
+__global__ __launch_bounds__(256) void f32_to_f16_kernel(const float *__restrict__ f, _Float16 *__restrict__ h,
+                                                         int64_t total, int M, int N, int64_t ldh, int64_t h_batch_stride,
+                                                         int accumulate, float act_min, float act_max)
+{
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total)
+        return;
+    const int64_t row = idx / N;
+    const int     j   = (int)(idx - row * N);
+    const int64_t bz  = row / M;
+    const int     i   = (int)(row - bz * M);
+    const int64_t hi  = bz * h_batch_stride + (int64_t)i * ldh + j;
+    _Float16      v   = (_Float16)f[idx];
+    if (accumulate)
+    {
+        const float sum = (float)h[hi] + (float)v;
+        v               = (_Float16)fminf(fmaxf(sum, act_min), act_max);
+    }
+    h[hi] = v;
+}
+
+int f32_to_f16_launch(const float *dense_f32, void *half_matrix, int batch, int M, int N, int64_t ldh,
+                      int64_t h_batch_stride, bool accumulate, float act_min, float act_max, hipStream_t s)
+{
+    const int64_t total = (int64_t)batch * M * N;
+    if (total <= 0)
+        return 0;
+    if ((total + 255) / 256 > 0x7FFFFFFF)
+        return (int)hipErrorInvalidValue;
+    f32_to_f16_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>(
+        dense_f32, (_Float16 *)half_matrix, total, M, N, ldh, h_batch_stride, accumulate ? 1 : 0, act_min, act_max);
+    return launch_status();
+}
+
 // ---- one thread per output: the plainest possible statement of the path, for cross-checking only ----------------------
 template <int EPI>
 __global__ __launch_bounds__(256) void simple_gemm_kernel(GemmArgs g, uint8_t flip)

@@ -37,6 +37,8 @@ int to_mi355(DataType dt)
             return MI355_S32;
         case DataType::F32:
             return MI355_F32;
+        case DataType::F16:
+            return MI355_F16;
         default:
             return -1;
     }
@@ -137,7 +139,7 @@ void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorI
             shifts.assign(stage.gemmlowp_shifts.begin(), stage.gemmlowp_shifts.begin() + d.N);
         }
     }
-    else if (oi->data_type() == DataType::F32)
+    else if (oi->data_type() == DataType::F32 || oi->data_type() == DataType::F16)
     {
         d.epilogue = MI355_EPI_F32;
         d.scale    = ai->quantization_info().uniform().scale * bi->quantization_info().uniform().scale;
@@ -216,10 +218,14 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
                                                                 DataType::QSYMM8, DataType::QSYMM8_PER_CHANNEL}) ||
                                         b->num_channels() != 1,
                                     "Matrix B must be QASYMM8, QASYMM8_SIGNED, QSYMM8 or QSYMM8_PER_CHANNEL");
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::F16, "F16 output is not built in this library");
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::S32, DataType::QASYMM8,
-                                                                     DataType::QASYMM8_SIGNED, DataType::F32}),
-                                    "Output must be S32, QASYMM8, QASYMM8_SIGNED or F32");
+                                                                     DataType::QASYMM8_SIGNED, DataType::F32, DataType::F16}),
+                                    "Output must be S32, QASYMM8, QASYMM8_SIGNED, F32 or F16");
+    // the half leg of the dequantising GEMM is exercised by the reference with signed operands only
+    // (tests/validation/NEON/GEMMLowp.cpp:598-607)
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->data_type() == DataType::F16 &&
+                                        (a->data_type() != DataType::QASYMM8_SIGNED || b->data_type() != DataType::QASYMM8_SIGNED),
+                                    "An F16 output needs QASYMM8_SIGNED operands");
     const GEMMLowpOutputStageInfo stage = gemm_info.gemmlowp_output_stage();
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(c != nullptr && output->data_type() != DataType::F32 &&
                                         stage.type == GEMMLowpOutputStageType::NONE,
@@ -281,7 +287,7 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
     switch (stage.type)
     {
         case GEMMLowpOutputStageType::NONE:
-            ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::S32, DataType::F32}),
+            ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::S32, DataType::F32, DataType::F16}),
                                             "A quantized output needs an output stage");
             if (c != nullptr)
             {

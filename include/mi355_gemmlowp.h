@@ -44,7 +44,8 @@ typedef enum mi355_dtype
     MI355_S8  = 1, /* QASYMM8_SIGNED, QSYMM8, QSYMM8_PER_CHANNEL */
     MI355_S32 = 2,
     MI355_F32 = 3,
-    MI355_S16 = 4 /* QSYMM16: only as the destination of mi355_output_stage_run */
+    MI355_S16 = 4, /* QSYMM16: only as the destination of mi355_output_stage_run */
+    MI355_F16 = 5  /* IEEE half: only as the destination of mi355_gemmlowp_run with MI355_EPI_F32 */
 } mi355_dtype;
 
 /* What happens to the int32 accumulators. Replaces the choice the reference makes between
@@ -54,7 +55,12 @@ typedef enum mi355_epilogue
 {
     MI355_EPI_S32        = 0, /* dst = acc + offset contribution                       (int32) */
     MI355_EPI_FIXEDPOINT = 1, /* + bias, QUANTIZE_DOWN_FIXEDPOINT, clamp               (uint8 / int8) */
-    MI355_EPI_F32        = 2  /* float(acc)*scale (+ f32 bias) + float(offsets)*scale, activation clamp (float) */
+    MI355_EPI_F32        = 2  /* float(acc)*scale (+ f32 bias) + float(offsets)*scale, activation clamp (float).
+                               * With an MI355_F16 destination the same float result is rounded to half, nearest even
+                               * (the F16 leg of the dequantising GEMMLowp: src/cpu/operators/
+                               * CpuGemmLowpMatrixMultiplyCore.cpp:305-309,374-375 and
+                               * src/cpu/kernels/gemmlowp/generic/neon/fp16.cpp:32-70; with MI355_GEMM_ACCUMULATE the
+                               * previous half values are widened, added in float, and the sum rounded once). */
 } mi355_epilogue;
 
 typedef enum mi355_path

@@ -27,6 +27,10 @@ def _load():
     if not os.path.exists(_LIB_PATH):
         build(with_ref=False)
     lib = C.CDLL(_LIB_PATH)
+    lib.orc_f32_to_f16.restype = C.c_uint16
+    lib.orc_f32_to_f16.argtypes = [C.c_float]
+    lib.orc_f16_to_f32.restype = C.c_float
+    lib.orc_f16_to_f32.argtypes = [C.c_uint16]
     lib.orc_sqdmulh.restype = C.c_int32
     lib.orc_sqdmulh.argtypes = [C.c_int32, C.c_int32]
     lib.orc_rounding_shift_right.restype = C.c_int32
@@ -186,6 +190,31 @@ def gemmlowp_f32(A, B, bias, a_offset, b_offset, scale, act_min=-np.inf, act_max
                          C.c_int64(N), M, N, K, C.c_int32(a_offset), C.c_int32(b_offset), C.c_float(scale),
                          C.c_float(act_min), C.c_float(act_max), 1 if prev is not None else 0, 1 if act_twice else 0)
     return out
+
+
+def gemmlowp_f16(A, B, bias, a_offset, b_offset, scale, act_min=-np.inf, act_max=np.inf, prev=None, act_twice=False):
+    """F16 destination: the float result (previous half values widened when accumulating) rounded to half once"""
+    A = np.ascontiguousarray(A)
+    B = np.ascontiguousarray(B)
+    M, K = A.shape
+    _, N = B.shape
+    bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    out = np.empty((M, N), dtype=np.float16) if prev is None else np.array(prev, dtype=np.float16, order="C")
+    assert out.shape == (M, N)
+    lib.orc_gemmlowp_f16(_p(A), _signed(A), C.c_int64(K), _p(B), _signed(B), C.c_int64(N), _p(bias), _p(out),
+                         C.c_int64(N), M, N, K, C.c_int32(a_offset), C.c_int32(b_offset), C.c_float(scale),
+                         C.c_float(act_min), C.c_float(act_max), 1 if prev is not None else 0, 1 if act_twice else 0)
+    return out
+
+
+def f32_to_f16_bits(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    return np.array([lib.orc_f32_to_f16(C.c_float(v)) for v in x.ravel()], dtype=np.uint16).reshape(x.shape)
+
+
+def f16_bits_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    return np.array([lib.orc_f16_to_f32(int(v)) for v in h.ravel()], dtype=np.float32).reshape(h.shape)
 
 
 def conv_out_dims(H, W, KH, KW, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1)):
@@ -376,6 +405,14 @@ def ref_dequantize_s32(src, scale):
     src = np.ascontiguousarray(src, dtype=np.int32)
     out = np.empty(src.shape, dtype=np.float32)
     ref().ref_dequantize_s32(_p(src), int(src.size), C.c_float(scale), _p(out))
+    return out
+
+
+def ref_dequantize_s32_f16(src, scale, prev=None):
+    src = np.ascontiguousarray(src, dtype=np.int32)
+    out = np.empty(src.shape, dtype=np.float16)
+    prev = None if prev is None else np.ascontiguousarray(prev, dtype=np.float16)
+    ref().ref_dequantize_s32_f16(_p(src), int(src.size), C.c_float(scale), _p(prev), _p(out))
     return out
 
 

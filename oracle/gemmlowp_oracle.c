@@ -354,6 +354,96 @@ void orc_gemmlowp_f32(const void *A, int a_signed, int64_t lda, const void *B, i
     free(colsum);
 }
 
+/* float -> IEEE half, round to nearest, ties to even: how the reference's host-side half type converts
+ * (support/Half.h:33-34 sets HALF_ROUND_STYLE 1 and HALF_ROUND_TIES_TO_EVEN 1 for include/half/half.hpp) and what
+ * vcvt_f16_f32 does in src/cpu/kernels/gemmlowp/generic/neon/fp16.cpp:52-55. Returns the 16 bits. */
+uint16_t orc_f32_to_f16(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, sizeof(x));
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t mag  = x & 0x7FFFFFFFu;
+    if (mag >= 0x7F800000u) /* infinity / NaN */
+        return (uint16_t)(sign | 0x7C00u | (mag > 0x7F800000u ? 0x0200u | ((mag >> 13) & 0x03FFu) : 0u));
+    if (mag >= 0x477FF000u) /* rounds to a magnitude >= 65520: overflows to infinity */
+        return (uint16_t)(sign | 0x7C00u);
+    if (mag < 0x33000001u) /* at most half of the smallest subnormal (2^-25): rounds to zero */
+        return (uint16_t)sign;
+    const int      e    = (int)(mag >> 23) - 127;       /* unbiased exponent, -25 .. 15 */
+    const uint32_t man  = (mag & 0x007FFFFFu) | 0x00800000u; /* 24-bit significand with the leading one */
+    /* shift so that the result keeps 11 significant bits (normal) or fewer (subnormal, e < -14) */
+    const int      sh   = e < -14 ? 13 + (-14 - e) : 13;
+    uint32_t       q    = man >> sh;
+    const uint32_t rem  = man & ((1u << sh) - 1u), half = 1u << (sh - 1);
+    if (rem > half || (rem == half && (q & 1u)))
+        ++q;
+    /* q carries the leading one for normals: (e+15) << 10 added to q - 0x400; a carry out of the significand bumps
+     * the exponent by itself. Subnormals: exponent field 0, q is the fraction (a carry makes the smallest normal). */
+    const uint32_t h = e < -14 ? q : (((uint32_t)(e + 15) << 10) + (q - 0x400u));
+    return (uint16_t)(sign | h);
+}
+
+float orc_f16_to_f32(uint16_t h)
+{
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t ex   = (h >> 10) & 0x1Fu, fr = h & 0x3FFu;
+    uint32_t       x;
+    if (ex == 0x1Fu)
+        x = sign | 0x7F800000u | (fr << 13);
+    else if (ex != 0)
+        x = sign | ((ex + 112u) << 23) | (fr << 13);
+    else if (fr == 0)
+        x = sign;
+    else
+    {
+        int      e = -1;
+        uint32_t m = fr;
+        do
+        {
+            ++e;
+            m <<= 1;
+        } while ((m & 0x400u) == 0);
+        x = sign | ((uint32_t)(112 - e) << 23) | ((m & 0x3FFu) << 13);
+    }
+    float f;
+    memcpy(&f, &x, sizeof(f));
+    return f;
+}
+
+/* GEMMLowp with an F16 destination (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:305-309,374-375; test
+ * tests/validation/NEON/GEMMLowp.cpp:598-621; reference values tests/validation/fixtures/GEMMLowpFixture.h:908-920 =
+ * half(float(s32) * scale), to which the previous half values are added IN HALF when accumulating: both operands
+ * widened, one float addition, rounded again). Here: the float result of orc_gemmlowp_f32 rounded to half; when
+ * accumulating, that half is added to the previous half the fixture's way and the activation clamp, which must follow
+ * the addition, is applied to the sum (the clamp ahead of the offset term that act_twice stands for is then skipped).
+ * Without offsets this is the fixture's value bit for bit; with offsets the float value underneath differs by the
+ * rounding order of orc_gemmlowp_f32 (<= 1e-5 relative), which rarely crosses a half rounding boundary (the NEON kernels
+ * themselves add in half precision and are only held to a 0.2 relative tolerance by that test). */
+void orc_gemmlowp_f16(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
+                      const float *bias, uint16_t *dst, int64_t ldd, int M, int N, int K, int32_t a_offset,
+                      int32_t b_offset, float scale, float act_min, float act_max, int accumulate, int act_twice)
+{
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)(M > 0 ? M : 1) * (size_t)(N > 0 ? N : 1));
+    orc_gemmlowp_f32(A, a_signed, lda, B, b_signed, ldb, bias, tmp, N, M, N, K, a_offset, b_offset, scale,
+                     accumulate ? -INFINITY : act_min, accumulate ? INFINITY : act_max, 0, accumulate ? 0 : act_twice);
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j)
+        {
+            uint16_t h = orc_f32_to_f16(tmp[(int64_t)i * N + j]);
+            if (accumulate)
+            {
+                volatile float sum = orc_f16_to_f32(dst[(int64_t)i * ldd + j]) + orc_f16_to_f32(h);
+                if (sum < act_min)
+                    sum = act_min;
+                if (sum > act_max)
+                    sum = act_max;
+                h = orc_f32_to_f16(sum);
+            }
+            dst[(int64_t)i * ldd + j] = h;
+        }
+    free(tmp);
+}
+
 /* src/core/Utils.cpp:288-332 (FLOOR rounding, the default of PadStrideInfo) */
 void orc_conv_out_dims(int H, int W, int KH, int KW, int stride_x, int stride_y, int pad_left, int pad_top,
                        int pad_right, int pad_bottom, int dil_x, int dil_y, int *OH, int *OW)

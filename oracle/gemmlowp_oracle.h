@@ -26,6 +26,9 @@
  * test oracle uses the non-rounding multiply for every output type and no NEON test covers the
  * int16 kernel, so it is pinned by the architectural definition of SQRDMULH (big-integer model in
  * tests/test_oracle_gemm.py) and to within 1 of oracle/_ref: "parity unpinned" beyond that.
+ * orc_f32_to_f16 / orc_gemmlowp_f16: the conversion is pinned against numpy's IEEE conversion (every half, every
+ * midpoint, the thresholds) and the function against the reference's half dequantization + half addition in
+ * oracle/_ref (identical bits without offsets; with offsets the float underneath is orc_gemmlowp_f32's).
  * Its act_twice clamp (an activation together with non-zero offsets on the F32 path) follows the
  * source order too; none of the reference's tests runs that combination: "parity unpinned".
  */
@@ -87,6 +90,11 @@ void orc_gemmlowp_fixedpoint(const void *A, int a_signed, int64_t lda, const voi
 void orc_gemmlowp_f32(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
                       const float *bias, float *dst, int64_t ldd, int M, int N, int K, int32_t a_offset,
                       int32_t b_offset, float scale, float act_min, float act_max, int accumulate, int act_twice);
+uint16_t orc_f32_to_f16(float f);
+float    orc_f16_to_f32(uint16_t h);
+void     orc_gemmlowp_f16(const void *A, int a_signed, int64_t lda, const void *B, int b_signed, int64_t ldb,
+                          const float *bias, uint16_t *dst, int64_t ldd, int M, int N, int K, int32_t a_offset,
+                          int32_t b_offset, float scale, float act_min, float act_max, int accumulate, int act_twice);
 
 /* ---- convolution lowering ------------------------------------------------------------------ */
 /* NHWC src [batch][H][W][C] -> patch matrix [batch*OH*OW][KH*KW*C], K ordered (ky, kx, c) */

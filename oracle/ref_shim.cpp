@@ -9,6 +9,7 @@
  */
 #include "arm_compute/core/utils/quantization/AsymmHelpers.h"
 #include "tests/SimpleTensor.h"
+#include "tests/validation/reference/ArithmeticOperations.h"
 #include "tests/validation/reference/Convolution3d.h"
 #include "tests/validation/reference/DequantizationLayer.h"
 #include "tests/validation/reference/GEMMLowp.h"
@@ -156,6 +157,24 @@ extern "C"
             make<int32_t>(TensorShape(count), DataType::S32, in, QuantizationInfo(scale, 0));
         const SimpleTensor<float> d = reference::dequantization_layer<float, int32_t>(t);
         std::memcpy(out, d.data(), sizeof(float) * d.num_elements());
+    }
+
+    /* tests/validation/reference/DequantizationLayer.cpp:69-116 with a half destination, and - when prev is given -
+     * tests/validation/reference/ArithmeticOperations.cpp (ADD, SATURATE) on halfs: the F16 GEMMLowp reference of
+     * tests/validation/fixtures/GEMMLowpFixture.h:908-920. Halfs travel as their 16 bits. */
+    void ref_dequantize_s32_f16(const int32_t *in, int count, float scale, const uint16_t *prev, uint16_t *out)
+    {
+        const SimpleTensor<int32_t> t =
+            make<int32_t>(TensorShape(count), DataType::S32, in, QuantizationInfo(scale, 0));
+        SimpleTensor<half> d = reference::dequantization_layer<half, int32_t>(t);
+        if (prev != nullptr)
+        {
+            SimpleTensor<half> o = make<half>(TensorShape(count), DataType::F16, prev);
+            reference::arithmetic_operation<half>(reference::ArithmeticOperation::ADD, o, d, o, ConvertPolicy::SATURATE);
+            std::memcpy(out, o.data(), sizeof(half) * o.num_elements());
+            return;
+        }
+        std::memcpy(out, d.data(), sizeof(half) * d.num_elements());
     }
 
     /* tests/validation/reference/Im2Col.cpp:108-170 (NHWC branch; instantiated for uint8 storage only,

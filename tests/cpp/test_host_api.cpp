@@ -451,6 +451,37 @@ static void test_gemmlowp_accumulate_and_3d()
                          INFINITY, 1, 0);
         EXPECT(dense_copy<float>(dst) == want);
     }
+    for (int accumulate = 0; accumulate < 2; ++accumulate)
+    {
+        // F16 destination (tests/validation/NEON/GEMMLowp.cpp:598-621: the reference's small dataset, signed operands,
+        // QuantizationInfo(1/255, a_offset) x QuantizationInfo(5/255, b_offset), with and without accumulation)
+        Tensor a, b, dst;
+        init_tensor(a, TensorShape(K, M), DataType::QASYMM8_SIGNED, QuantizationInfo(1.f / 255, -3));
+        init_tensor(b, TensorShape(N, K), DataType::QASYMM8_SIGNED, QuantizationInfo(5.f / 255, 2));
+        init_tensor(dst, TensorShape(N, M), DataType::F16);
+        a.allocator()->allocate(), b.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(a, -128, 127, 14), fill_uniform<int8_t>(b, -128, 127, 15);
+        std::mt19937                    rng(16);
+        std::normal_distribution<float> nd(0.f, 2.f);
+        for (size_t y = 0; y < (size_t)M; ++y)
+            for (size_t x = 0; x < (size_t)N; ++x)
+                *reinterpret_cast<uint16_t *>(dst.ptr_to_element(Coordinates(x, y))) = orc_f32_to_f16(nd(rng));
+        auto     want = dense_copy<uint16_t>(dst);
+        GEMMInfo info(false, false, true);
+        info.set_accumulate(accumulate != 0);
+        EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(a.info(), b.info(), nullptr, dst.info(), info)));
+        NEGEMMLowpMatrixMultiplyCore gemm;
+        gemm.configure(&a, &b, nullptr, &dst, info);
+        gemm.run();
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        orc_gemmlowp_f16(A.data(), 1, K, B.data(), 1, N, nullptr, want.data(), N, M, N, K, -3, 2, (1.f / 255) * (5.f / 255),
+                         -INFINITY, INFINITY, accumulate, 0);
+        EXPECT(dense_copy<uint16_t>(dst) == want);
+        // unsigned operands are not part of the half leg
+        Tensor ua;
+        init_tensor(ua, TensorShape(K, M), DataType::QASYMM8, QuantizationInfo(1.f / 255, 3));
+        EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(ua.info(), b.info(), nullptr, dst.info(), info)));
+    }
     {
         // a = [K, W, H, batch] -> M = W*H rows per batch; dst = [N, W, H, batch]
         const int W = 5, H = 4, batch = 2;

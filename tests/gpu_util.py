@@ -36,7 +36,7 @@ def run_gemm(A, B, epilogue, dst_dtype, a_offset=0, b_offset=0, bias=None, mult=
                       0 if per_channel or shift is None else int(np.atleast_1d(shift)[0]), result_offset, lo, hi,
                       per_channel, stage)
     dcode = {np.dtype(np.uint8): capi.U8, np.dtype(np.int8): capi.S8, np.dtype(np.int32): capi.S32,
-             np.dtype(np.float32): capi.F32}[np.dtype(dst_dtype)]
+             np.dtype(np.float32): capi.F32, np.dtype(np.float16): capi.F16}[np.dtype(dst_dtype)]
     lda = lda or K
     ldd = ldd or N
     g = capi.Gemm(M, N, K, CODE[A.dtype], CODE[B.dtype], dcode, epilogue, a_offset, b_offset, rq, scale, act[0],

@@ -145,6 +145,35 @@ def test_random_shape_sweep_against_oracle():
         assert np.array_equal(got, want), "case %d" % case
 
 
+@pytest.mark.parametrize("device", [True, False])
+def test_f16_destination(device):
+    """GEMMLowp dequantised into halfs (tests/validation/NEON/GEMMLowp.cpp:598-621: signed operands, with and without
+    accumulation; the reference accepts 0.2 relative error there). Here: the bits of the oracle - the float result
+    rounded to nearest even, added to the previous halfs the way the reference's test oracle adds halfs - on every
+    kernel path, with padded destination rows, a float bias and an activation clamp after the accumulation."""
+    rng = np.random.default_rng(1600)
+    scale = (1.0 / 255) * (5.0 / 255)
+    for (M, N, K) in [(21, 13, 33), (8, 300, 200), (150, 70, 520), (40, 4100, 128)]:
+        A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+        prev = rng.normal(0, 3, size=(M, N)).astype(np.float16)
+        biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+        for path in paths_for(M):
+            announce("f16 destination", (M, N, K), ao, bo, "path", path, "device", device)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float16, ao, bo, scale=scale, path=path, device=device, ldd=N + 3)
+            np.testing.assert_array_equal(got.view(np.uint16), oracle.gemmlowp_f16(A, B, None, ao, bo, scale).view(np.uint16))
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float16, ao, bo, scale=scale, path=path, device=device, prev=prev,
+                              flags=capi.GEMM_ACCUMULATE)
+            np.testing.assert_array_equal(got.view(np.uint16),
+                                          oracle.gemmlowp_f16(A, B, None, ao, bo, scale, prev=prev).view(np.uint16))
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float16, ao, bo, scale=scale, bias_f32=biasf, act=(0.0, 6.0), path=path,
+                              device=device, prev=prev, flags=capi.GEMM_ACCUMULATE)
+            want = oracle.gemmlowp_f16(A, B, biasf, ao, bo, scale, 0.0, 6.0, prev=prev)
+            np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+            assert 0.05 < (want == 0).mean() < 0.95 or M * N < 400
+
+
 PIPELINED_CONFIGS = ["pp_256x128x128_s3", "pp_128x128x128_s3", "pp_128x64x128_s3", "pp_64x64x128_s3", "pp_64x64x128_s6",
                      "pp_128x64x256_s3", "pp_256x128x64_s4"]
 

@@ -234,3 +234,73 @@ def test_fused_against_live_reference_config1_shape():
         if ao < 0:
             inside = ((want > 0) & (want < 255)).mean()
             assert 0.2 < inside < 0.6  # a meaningful share of outputs is not clamped
+
+
+def test_half_conversion_against_numpy_and_by_construction():
+    """float -> half of the oracle: every half value survives the round trip; exact midpoints between neighbouring
+    halfs go to the even one; the overflow and underflow thresholds; 200k random floats against numpy's conversion
+    (IEEE round-to-nearest-even)."""
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    vals = oracle.f16_bits_to_f32(bits)
+    finite = np.isfinite(vals)
+    np.testing.assert_array_equal(vals[finite], bits.view(np.float16).astype(np.float32)[finite])
+    np.testing.assert_array_equal(oracle.f32_to_f16_bits(vals[finite]), bits[finite])
+    assert np.isnan(vals[~finite & ((bits & 0x3FF) != 0)]).all() and np.isinf(vals[(bits & 0x7FFF) == 0x7C00]).all()
+    # midpoints of neighbouring positive halfs (exact in float): ties to even
+    lo = np.arange(0, 0x7BFF, dtype=np.uint16)
+    mid = (oracle.f16_bits_to_f32(lo).astype(np.float64) + oracle.f16_bits_to_f32(lo + 1).astype(np.float64)) / 2
+    assert (mid.astype(np.float32).astype(np.float64) == mid).all()
+    want = np.where(lo % 2 == 0, lo, lo + 1).astype(np.uint16)
+    np.testing.assert_array_equal(oracle.f32_to_f16_bits(mid.astype(np.float32)), want)
+    np.testing.assert_array_equal(oracle.f32_to_f16_bits(-mid.astype(np.float32)), want | 0x8000)
+    # thresholds
+    for v, h in [(65504.0, 0x7BFF), (65519.996, 0x7BFF), (65520.0, 0x7C00), (1e9, 0x7C00), (2.0 ** -24, 0x0001),
+                 (2.0 ** -25, 0x0000), (np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 0x0001), (0.0, 0x0000),
+                 (2.0 ** -14, 0x0400), (np.inf, 0x7C00)]:
+        assert int(oracle.f32_to_f16_bits(np.float32(v)).item()) == h, v
+        assert int(oracle.f32_to_f16_bits(np.float32(-v)).item()) == (h | 0x8000), v
+    rng = np.random.default_rng(16)
+    x = np.concatenate([rng.normal(0, 1, 50000), rng.normal(0, 1e-6, 50000), rng.normal(0, 3e4, 50000),
+                        np.exp(rng.uniform(np.log(1e-9), np.log(1e6), 50000)) * rng.choice([-1, 1], 50000)]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(oracle.f32_to_f16_bits(x), x.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.skipif(not oracle.ref_available(), reason="oracle/_ref not built (needs the reference checkout)")
+def test_f16_destination_against_live_reference():
+    """The reference's F16 GEMMLowp values (GEMMLowpFixture.h:908-920: half(float(s32) * scale), plus the previous halfs,
+    added as halfs, when accumulating) through its own code. Without offsets the oracle must give the same bits, with
+    and without accumulation; with offsets the float underneath follows the NEON rounding order (<= 1e-5 relative),
+    which may cross a half rounding boundary now and then: at most one half ulp apart before the accumulation, and
+    equal almost everywhere."""
+    rng = np.random.default_rng(5)
+    A = rng.integers(-128, 128, size=(37, 120), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(120, 53), dtype=np.int8)
+    scale = (1.0 / 255) * (5.0 / 255)
+    prev = rng.normal(0, 2, size=(37, 53)).astype(np.float16)
+    t = oracle.ref_gemmlowp_core(A, B, 0, 0)
+    np.testing.assert_array_equal(oracle.gemmlowp_f16(A, B, None, 0, 0, scale).view(np.uint16),
+                                  oracle.ref_dequantize_s32_f16(t, scale).view(np.uint16))
+    np.testing.assert_array_equal(oracle.gemmlowp_f16(A, B, None, 0, 0, scale, prev=prev).view(np.uint16),
+                                  oracle.ref_dequantize_s32_f16(t, scale, prev=prev).view(np.uint16))
+
+    def ulps(a, b):  # distance in representable halfs
+        def key(h):
+            u = h.view(np.uint16).astype(np.int32)
+            return np.where(u & 0x8000, -(u & 0x7FFF), u)
+        return np.abs(key(a) - key(b))
+
+    t = oracle.ref_gemmlowp_core(A, B, 3, -7)
+    got = oracle.gemmlowp_f16(A, B, None, 3, -7, scale)
+    want = oracle.ref_dequantize_s32_f16(t, scale)
+    assert ulps(got, want).max() <= 1 and (got.view(np.uint16) == want.view(np.uint16)).mean() > 0.99
+    got = oracle.gemmlowp_f16(A, B, None, 3, -7, scale, prev=prev)
+    want = oracle.ref_dequantize_s32_f16(t, scale, prev=prev)
+    assert (got.view(np.uint16) == want.view(np.uint16)).mean() > 0.99
+    # the oracle's own definition, restated with numpy's conversions
+    f = oracle.gemmlowp_f32(A, B, None, 3, -7, scale)
+    np.testing.assert_array_equal(oracle.gemmlowp_f16(A, B, None, 3, -7, scale).view(np.uint16), f.astype(np.float16).view(np.uint16))
+    acc = (prev.astype(np.float32) + f.astype(np.float16).astype(np.float32)).astype(np.float16)
+    np.testing.assert_array_equal(got.view(np.uint16), acc.view(np.uint16))
+    clamped = oracle.gemmlowp_f16(A, B, None, 3, -7, scale, 0.0, 1.5, prev=prev)
+    np.testing.assert_array_equal(clamped.view(np.uint16), np.clip(acc.astype(np.float32), 0.0, 1.5).astype(np.float16).view(np.uint16))

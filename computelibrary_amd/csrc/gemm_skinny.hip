@@ -23,11 +23,12 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 // Row pitch of the staged copy of A (STAGE_A): 1 KiB of a row's K slice + 64 bytes, which spreads the 8 rows an
 // operand read touches over the LDS banks
 constexpr int SK_A_PITCH = 1024 + 64;
-
-template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A, int MR>
+template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A, int MR, bool STEP_A = false,
+          int STEP_KB = (MR == 4 ? 4 : 8)>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 {
     static_assert(MR >= 1 && MR <= SK_WAVES && (!STAGE_A || MR == 1), "row blocks");
+    static_assert(!STEP_A || (!STAGE_A && SK_UNROLL == 8), "per-step staging: steps of 8 k blocks");
     __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
     extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][SK_A_PITCH]
 
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     // copies its slice of A into LDS once, with all 64 lanes per load, and takes the operand blocks from there.
     // Loading them from global memory inside the stream costs one half-empty load instruction (rows 8..15 are padding)
     // per B load and 16 % of the kernel's time, although A never leaves the L2.
-    char *a_lds = a_stage + wave * 8 * SK_A_PITCH;
+    char *a_lds = a_stage + (STEP_A ? wave * MR * 16 * (STEP_KB * 64 + 16) : wave * 8 * SK_A_PITCH);
     v4i   ta[STAGE_A ? 8 : 1];
     if (STAGE_A)
     {
@@ -130,7 +131,63 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
             *(v4i *)(a_lds + r * SK_A_PITCH + lane * 16) = ta[r];
         }
     }
-    if constexpr (MR == 1)
+    if constexpr (STEP_A)
+    {
+        // More than 8 rows: the bytes of A that a step needs go through LDS, STEP_KB k blocks at a time - loads of 2
+        // (or 4) rows x 512 (256) contiguous bytes, whole cache lines with every lane busy, instead of gathers of 16
+        // rows x 64 bytes, which cost the L2 twice the requests. No branches (a branch per load would put a full wait
+        // behind every load): rows past M re-read row M-1 and are multiplied into accumulator rows that are never stored. LDS operations of one wave execute in order, so
+        // the next pass's writes cannot overtake this pass's reads.
+        constexpr int SKB   = STEP_KB;              // k blocks per staging pass
+        constexpr int LPR   = SKB * 4;               // lanes per row (16 bytes each)
+        constexpr int RPL   = 64 / LPR;              // rows per load instruction
+        constexpr int PITCH = SKB * 64 + 16;         // 16 rows of an operand read fall into 16 different bank groups
+        const int     sub = lane / LPR, col = (lane % LPR) * 16;
+        bool          more = whole_step(kb);
+        if (more)
+            load_b(kb);
+        while (more)
+        {
+#pragma unroll
+            for (int h = 0; h < SK_UNROLL / SKB; ++h)
+            {
+#pragma unroll
+                for (int c = 0; c < MR; ++c)
+                {
+                    v4i ts[16 / RPL];
+#pragma unroll
+                    for (int q = 0; q < 16 / RPL; ++q)
+                        ts[q] = *(const v4i *)(g.A + (int64_t)min(c * 16 + q * RPL + sub, g.M - 1) * g.lda +
+                                               (int64_t)(kb + h * SKB) * 64 + col);
+#pragma unroll
+                    for (int q = 0; q < 16 / RPL; ++q)
+                    {
+                        if (FLIP_A)
+                            ts[q] ^= (int)0x80808080;
+                        *(v4i *)(a_lds + (c * 16 + q * RPL + sub) * PITCH + col) = ts[q];
+                    }
+                }
+#pragma unroll
+                for (int u = h * SKB; u < (h + 1) * SKB; ++u)
+                {
+                    v4i fa[MR];
+#pragma unroll
+                    for (int rb = 0; rb < MR; ++rb)
+                        fa[rb] = *(const v4i *)(a_lds + (rb * 16 + arow) * PITCH + (u - h * SKB) * 64 + akc);
+#pragma unroll
+                    for (int rb = 0; rb < MR; ++rb)
+#pragma unroll
+                        for (int n = 0; n < NG; ++n)
+                            acc[rb][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb], fb[u][n], acc[rb][n], 0, 0, 0);
+                }
+            }
+            kb += SK_UNROLL;
+            more = whole_step(kb);
+            if (more)
+                load_b(kb);
+        }
+    }
+    else if constexpr (MR == 1)
     {
         bool more = whole_step(kb);
         if (more)
@@ -307,13 +364,26 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     }
 }
 
-template <int NG, int WAVES, int UNROLL, bool STAGE_A, int MR = 1>
+template <int NG, int WAVES, int UNROLL, bool STAGE_A, int MR = 1, bool STEP_A = false>
 static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
 {
     const int    groups = (a.N + 15) / 16;
     const dim3   grid((groups + NG - 1) / NG), block(WAVES * 64);
-    const size_t lds = STAGE_A ? (size_t)WAVES * 8 * SK_A_PITCH : 0;
-#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR><<<grid, block, lds, s>>>(a)
+    const size_t lds = STAGE_A ? (size_t)WAVES * 8 * SK_A_PITCH : (STEP_A ? (size_t)WAVES * MR * 16 * ((MR == 4 ? 4 : 8) * 64 + 16) : 0);
+    if (lds > 48 * 1024)
+    {
+#define MI355_SKA(E, F)                                                                                                  \
+    (void)hipFuncSetAttribute((const void *)gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>,            \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+        if (epi == EPI_S32)
+            flip_a ? MI355_SKA(EPI_S32, true) : MI355_SKA(EPI_S32, false);
+        else if (epi == EPI_FIXEDPOINT)
+            flip_a ? MI355_SKA(EPI_FIXEDPOINT, true) : MI355_SKA(EPI_FIXEDPOINT, false);
+        else if (epi == EPI_F32)
+            flip_a ? MI355_SKA(EPI_F32, true) : MI355_SKA(EPI_F32, false);
+#undef MI355_SKA
+    }
+#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A><<<grid, block, lds, s>>>(a)
     if (epi == EPI_S32)
         flip_a ? MI355_SK(EPI_S32, true) : MI355_SK(EPI_S32, false);
     else if (epi == EPI_FIXEDPOINT)
@@ -339,6 +409,27 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     const int  per   = ((int)(args.Kp / 64) + waves - 1) / waves;
     const bool stage = args.M <= 8 && per <= 16 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
                        ((uintptr_t)args.A & 15) == 0 && getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    // more than 8 rows: per-step staging (dword-aligned rows are enough: the staging loads are plain 16-byte loads)
+    const bool step = args.M > 8 && args.lda % 4 == 0 && ((uintptr_t)args.A & 3) == 0 &&
+                      getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    // (17..24 rows: the gathers of the unstaged variants below re-read row M-1 for the missing rows of the second
+    // block, which costs less than staging 32 rows)
+    if (args.M > 24 && step)
+    {
+        // LDS: 8.25 KiB per wave and block of 16 rows; a workgroup covers 2 column groups when there are many
+        static const char *force_ng = getenv("MI355_SKINNY_NG");
+        const int          ng       = force_ng ? (atoi(force_ng) >= 2 ? 2 : 1) : (groups >= 512 ? 2 : 1);
+        const int          blocks   = (groups + ng - 1) / ng;
+        if (args.M > 32)
+            return ng == 2 ? skinny_launch_v<2, 4, 8, false, 4, true>(epi, flip_a, args, s)
+                           : skinny_launch_v<1, 4, 8, false, 4, true>(epi, flip_a, args, s);
+        const int w = force ? atoi(force) : (blocks >= 320 ? 4 : 8);
+        if (ng == 2)
+            return w == 4 ? skinny_launch_v<2, 4, 8, false, 2, true>(epi, flip_a, args, s)
+                          : skinny_launch_v<2, 8, 8, false, 2, true>(epi, flip_a, args, s);
+        return w == 4 ? skinny_launch_v<1, 4, 8, false, 2, true>(epi, flip_a, args, s)
+                      : skinny_launch_v<1, 8, 8, false, 2, true>(epi, flip_a, args, s);
+    }
     if (args.M > 16)
     {
         // More than one block of 16 rows: A (L2 resident) is re-read once per block of the grid, which costs as much as
@@ -359,6 +450,9 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
         return ng == 4 ? MI355_SKV(4, 4) : (ng == 2 ? MI355_SKV(2, 4) : MI355_SKV(1, 4));
 #undef MI355_SKV
     }
+    if (step) // 9..16 rows
+        return waves == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, s)
+                          : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, s);
     if (stage)
         return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, s);
     return waves == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);

@@ -205,12 +205,38 @@ def test_every_pipelined_configuration(cfg, monkeypatch):
         np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
 
 
-@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 63, 64])
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 12, 16])
+def test_skinny_kernel_with_staged_a(M):
+    """Up to 8 rows the streaming kernel copies each wave's K slice of A into LDS once, 9 to 16 rows it stages the 512
+    bytes per row of every step; both with 4 waves (many column groups) and 8 waves (few), signed and unsigned A,
+    K with and without whole steps, row strides that are only dword aligned."""
+    rng = np.random.default_rng(300 + M)
+    for (N, K, lda) in [(300, 512, 512), (300, 4096, 4096), (8200, 1024, 1024), (8200, 1088, 1092), (520, 640, 656),
+                        (100, 200, 200)]:
+        a_dt = np.uint8 if (N + K) % 3 == 0 else np.int8
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+        announce("skinny staged", (M, N, K), "lda", lda, a_dt.__name__)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_SKINNY, device=True, lda=lda)
+        assert name.startswith("skinny"), name
+        np.testing.assert_array_equal(got, oracle.gemmlowp_s32(A, B, ao, bo))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, 0, bias, mult, shift, off, lo, hi, path=capi.PATH_SKINNY,
+                          device=True, lda=lda)
+        np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
+
+
+@pytest.mark.parametrize("M", [17, 24, 25, 31, 32, 33, 48, 63, 64])
 def test_skinny_kernel_with_several_row_blocks(M):
-    """17 to 64 rows run as 2 or 4 blocks of 16 rows in the streaming kernel; N picks 1, 2 or 4 column groups per
-    workgroup and 4 or 8 waves; K covers whole steps only, a tail of whole 64-byte blocks, and a ragged tail."""
+    """17 to 64 rows run as 2 or 4 blocks of 16 rows in the streaming kernel (from 25 rows on with A staged through LDS
+    step by step); N picks 1, 2 or 4 column groups per workgroup and 4 or 8 waves; K covers whole steps only, a tail of
+    whole 64-byte blocks, and a ragged tail."""
     rng = np.random.default_rng(900 + M)
-    for (N, K) in [(100, 200), (4100, 1024), (8200, 333), (16400, 448), (21000, 192)]:
+    for (N, K) in [(100, 200), (4100, 1024), (8200, 333), (16400, 448), (21000, 192), (300, 4160), (11000, 2112)]:
         a_dt = np.int8 if (N // 100) % 2 else np.uint8
         A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
         B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)

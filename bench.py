@@ -200,6 +200,32 @@ def main():
         for h in handles:
             h.close()
 
+        # the same weights with larger decode batches (not BASELINE configurations; B rotated the same way)
+        out["secondary"]["decode_batches"] = {}
+        for Mb in (16, 32, 64):
+            Ab = torch.from_numpy(np.random.default_rng(30 + Mb).integers(-128, 128, size=(Mb, K3), dtype=np.int8)).cuda()
+            Db = torch.zeros((Mb, N3), dtype=torch.int8, device="cuda")
+            hb = []
+            for r in range(9):
+                h = capi.Gemm(Mb, N3, K3, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
+                h.prepare(torch.from_numpy(np.roll(B3, r, axis=1) if r else B3).cuda(), b3, m3, s3, stream)
+                hb.append(h)
+            torch.cuda.synchronize()
+            st = {"i": 0}
+
+            def rotated_b():
+                hb[st["i"] % len(hb)].run(Ab, Db, None, stream)
+                st["i"] += 1
+
+            _, evt_b = time_launches(torch, rotated_b, steps3, args.warmup)
+            bytes_b = N3 * K3 + Mb * K3 + Mb * N3 + 3 * 4 * N3
+            out["secondary"]["decode_batches"]["m%d" % Mb] = {
+                "kernel": hb[0].kernel_name, "kernel_us": round(evt_b / steps3 * 1e6, 3),
+                "achieved_GBs": round(bytes_b / (evt_b / steps3) / 1e9, 1),
+                "TOPS": round(2.0 * Mb * N3 * K3 / (evt_b / steps3) / 1e12, 1)}
+            for h in hb:
+                h.close()
+
         # config 4: NHWC 3x3 convolution as an implicit GEMM (M = 32*56*56, N = 64, K = 576), near the roofline ridge
         rng = np.random.default_rng(4)
         src = torch.from_numpy(rng.integers(-128, 128, size=(32, 56, 56, 64), dtype=np.int8)).cuda()

@@ -15,9 +15,10 @@ GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
 NHWC, NCHW = 0, 1
 
 EXPORTS = [
-    "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_run",
+    "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_set_strides",
+    "mi355_gemmlowp_run",
     "mi355_gemmlowp_destroy", "mi355_gemmlowp_kernel_name", "mi355_output_stage_run", "mi355_conv_create",
-    "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
+    "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_set_strides", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
     "mi355_im2col_nhwc_run", "mi355_last_error", "mi355_device_info",
 ]
 
@@ -77,6 +78,7 @@ def lib():
         l.mi355_gemmlowp_create.argtypes = [C.POINTER(GemmDesc), C.POINTER(vp)]
         l.mi355_gemmlowp_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
         l.mi355_gemmlowp_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(Requant), C.c_float, vp]
+        l.mi355_gemmlowp_set_strides.argtypes = [vp] + [C.c_int64] * 6
         l.mi355_gemmlowp_run.argtypes = [vp, vp, f32p, vp, vp]
         l.mi355_gemmlowp_destroy.argtypes = [vp]
         l.mi355_gemmlowp_destroy.restype = None
@@ -86,6 +88,7 @@ def lib():
         l.mi355_conv_create.argtypes = [C.POINTER(ConvDesc), C.POINTER(vp)]
         l.mi355_conv_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
         l.mi355_conv_run.argtypes = [vp, vp, vp, vp]
+        l.mi355_conv_set_strides.argtypes = [vp, C.c_int64, C.c_int64, C.c_int64]
         l.mi355_conv_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Requant), i32p, i32p, vp]
         l.mi355_conv_out_dims.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         l.mi355_conv_out_dims.restype = None
@@ -161,6 +164,15 @@ class Gemm:
         _check(lib().mi355_gemmlowp_update_quant(self._h, a_offset, b_offset, C.byref(rq) if rq else None, scale,
                                                  stream))
 
+    def set_strides(self, lda, ldb, ldd, a_batch_stride=None, b_batch_stride=None, d_batch_stride=None):
+        d = self.desc
+        a_bs = d.M * lda if a_batch_stride is None else a_batch_stride
+        d_bs = d.M * ldd if d_batch_stride is None else d_batch_stride
+        b_bs = ((d.N if d.b_transposed else d.K) * ldb if d.b_batch_stride else 0) if b_batch_stride is None \
+            else b_batch_stride
+        _check(lib().mi355_gemmlowp_set_strides(self._h, lda, ldb, ldd, a_bs, b_bs, d_bs))
+        d.lda, d.ldb, d.ldd, d.a_batch_stride, d.b_batch_stride, d.d_batch_stride = lda, ldb, ldd, a_bs, b_bs, d_bs
+
     def run(self, A, D, bias_f32=None, stream=None):
         _check(lib().mi355_gemmlowp_run(self._h, ptr(A), ptr(bias_f32), ptr(D), stream))
 
@@ -212,6 +224,9 @@ class Conv:
     def update_quant(self, src_offset, weights_offset, pad_value, rq, mult=None, shift=None, stream=None):
         _check(lib().mi355_conv_update_quant(self._h, src_offset, weights_offset, pad_value, C.byref(rq), ptr(mult),
                                              ptr(shift), stream))
+
+    def set_strides(self, src_pixel_stride, weights_pixel_stride, dst_pixel_stride):
+        _check(lib().mi355_conv_set_strides(self._h, src_pixel_stride, weights_pixel_stride, dst_pixel_stride))
 
     def run(self, src, dst, stream=None):
         _check(lib().mi355_conv_run(self._h, ptr(src), ptr(dst), stream))

@@ -56,6 +56,23 @@ bool is_device_ptr(const void *p)
     return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
+// What kind of memory an argument slot of a handle was last given. Device allocations live in an address range the
+// driver reserves for them, so a pointer value does not change sides while the process lives: asking once per value
+// and slot is enough, and a steady-state run() asks nothing.
+struct PtrKind
+{
+    const void *p   = nullptr;
+    bool        dev = false;
+    bool        is_device(const void *q)
+    {
+        if (q == nullptr)
+            return false;
+        if (q != p)
+            dev = is_device_ptr(q), p = q;
+        return dev;
+    }
+};
+
 struct DevBuf
 {
     void  *p   = nullptr;
@@ -89,14 +106,14 @@ struct DevBuf
 };
 
 // brings `bytes` at `src` to the device if it is host memory; returns the device pointer to use
-int to_device(const void *src, size_t bytes, DevBuf &stage, hipStream_t s, const void **out)
+int to_device(const void *src, size_t bytes, DevBuf &stage, hipStream_t s, const void **out, PtrKind *kind = nullptr)
 {
     if (src == nullptr)
     {
         *out = nullptr;
         return 0;
     }
-    if (is_device_ptr(src))
+    if (kind ? kind->is_device(src) : is_device_ptr(src))
     {
         *out = src;
         return 0;
@@ -145,8 +162,7 @@ struct GemmCore
     bool    has_bias = false, has_pc = false, prepared = false;
     std::string kname;
     DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp;
-    bool    qp_ok = false; // all multipliers >= 0: the branch-free epilogue applies
-    bool    qp_std = false; // ... and every column has a normalised multiplier (>= 2^30) and a right shift of 2..31
+    bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
 
@@ -205,7 +221,7 @@ struct GemmCore
             {
                 int    best = -1, best_lds = 0;
                 double best_cost = 0;
-                for (int i = 0; i < DMA_AUTO_CONFIGS; ++i)
+                for (int i = 0; i < dma_num_configs(); ++i)
                 {
                     const MfmaConfig c = dma_config(i);
                     if ((N <= 64 && c.BN > 64) || Kp % c.BK != 0)
@@ -285,28 +301,27 @@ struct GemmCore
         return 0;
     }
 
-    // digest multipliers / shifts for the pipelined kernel's epilogue; synchronises the stream to learn whether it applies
+    // Digest multipliers / shifts for the pipelined kernel's epilogue. Whether the branch-free forms apply (no negative
+    // multiplier; every column normalised) is left in a flag word behind the vectors, which the kernel reads itself:
+    // nothing here waits for the device.
     int refresh_qparams(hipStream_t s)
     {
-        qp_ok = qp_std = false;
+        qp_on = false;
         if (epi != EPI_FIXEDPOINT || rq.stage != MI355_STAGE_FIXEDPOINT)
             return 0;
         TRY(qp.ensure(sizeof(int32_t) * ((size_t)QP_COUNT * Np + 4)));
         int32_t *flag = qp.as<int32_t>() + (size_t)QP_COUNT * Np;
         HIP_TRY(qparams_launch(has_pc ? mult.as<int32_t>() : nullptr, has_pc ? shift.as<int32_t>() : nullptr,
                                rq.multiplier, rq.shift, N, Np, qp.as<int32_t>(), flag, s));
-        int32_t neg = 1;
-        HIP_TRY(hipMemcpyAsync(&neg, flag, sizeof(neg), hipMemcpyDeviceToHost, s));
-        HIP_TRY(hipStreamSynchronize(s));
-        qp_ok  = (neg & 1) == 0;
-        qp_std = neg == 0;
+        qp_on = true;
         return 0;
     }
 
     void fill_epi(EpiParams &p, const float *bias_f32) const
     {
-        p.qp                  = qp_ok ? qp.as<int32_t>() : nullptr;
-        p.qp_std              = (qp_ok && qp_std && rq.result_offset > -(1 << 28) && rq.result_offset < (1 << 28)) ? 1 : 0;
+        p.qp                  = qp_on ? qp.as<int32_t>() : nullptr;
+        p.qp_flag             = qp_on ? qp.as<int32_t>() + (size_t)QP_COUNT * Np : nullptr;
+        p.qp_std              = (qp_on && rq.result_offset > -(1 << 28) && rq.result_offset < (1 << 28)) ? 1 : 0;
         p.qp_stride           = Np;
         p.colvec              = colvec.as<int32_t>();
         p.rowvec              = nullptr;
@@ -432,9 +447,16 @@ int check_requant(const mi355_requant &rq, int dst_dtype)
         return fail("unknown output stage %d", rq.stage);
     if (rq.stage == MI355_STAGE_SCALE && !rq.per_channel && (rq.shift < 0 || rq.shift > 31))
         return fail("QUANTIZE_DOWN needs a shift in [0, 31] (got %d)", rq.shift);
+    // Bounds inside the destination type's range clamp; bounds that cover it only saturate. Bounds with one end inside
+    // and one outside are refused: the reference's three implementations disagree there (the stand-alone kernel narrows
+    // the bound to 8 bits, src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:502-503; the assembly path
+    // clamps in int32 and keeps the low byte, src/core/NEON/kernels/arm_gemm/quantized.cpp:36-46,254-261)
     const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
-    if (rq.max_bound < tlo || rq.min_bound > thi)
-        return fail("clamp bounds [%d,%d] do not intersect the destination type's range", rq.min_bound, rq.max_bound);
+    const bool    covers = rq.min_bound <= tlo && rq.max_bound >= thi;
+    const bool    inside = rq.min_bound >= tlo && rq.max_bound <= thi;
+    if (!covers && !inside)
+        return fail("clamp bounds [%d,%d] are partly outside the destination type's range [%d,%d]", rq.min_bound,
+                    rq.max_bound, tlo, thi);
     return 0;
 }
 } // namespace
@@ -445,6 +467,7 @@ struct mi355_gemm_handle
     GemmCore        core;
     DevBuf          stageA, stageB, stageD, stageBiasF, stageBias, stageMult, stageShift;
     DevBuf          wsF32; // MI355_F16 destination: the dense F32 matrix the kernels write
+    PtrKind         kindA, kindD, kindBiasF; // host or device memory, per argument of run()
 };
 
 struct mi355_conv_handle
@@ -457,6 +480,7 @@ struct mi355_conv_handle
     DevBuf          nhwcSrc, nhwcW, nhwcDst; // MI355_NCHW: the tensors in the kernels' layout
     DevBuf          biasF;                   // F32 destination: the float bias
     bool            has_bias_f32 = false;
+    PtrKind         kindSrc, kindDst; // host or device memory, per argument of run()
 };
 
 extern "C"
@@ -612,6 +636,26 @@ int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t 
     return 0;
 }
 
+int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                               int64_t b_batch_stride, int64_t d_batch_stride)
+{
+    if (!h)
+        return fail("null argument");
+    mi355_gemm_desc &d = h->d;
+    if (lda < d.K || ldb < (d.b_transposed ? d.K : d.N) || ldd < d.N)
+        return fail("row stride smaller than the row");
+    if (d.batch > 1 && (a_batch_stride < (int64_t)(d.M - 1) * lda + d.K || d_batch_stride < (int64_t)(d.M - 1) * ldd + d.N))
+        return fail("batch stride smaller than one matrix");
+    if (d.batch > 1 && (b_batch_stride == 0) != h->core.b_shared)
+        return fail("set_strides cannot switch between one shared B and one B per batch entry");
+    if (d.batch > 1 && b_batch_stride != 0 &&
+        b_batch_stride < (d.b_transposed ? (int64_t)(d.N - 1) * ldb + d.K : (int64_t)(d.K - 1) * ldb + d.N))
+        return fail("B batch stride smaller than one matrix");
+    d.lda = lda, d.ldb = ldb, d.ldd = ldd;
+    d.a_batch_stride = a_batch_stride, d.b_batch_stride = b_batch_stride, d.d_batch_stride = d_batch_stride;
+    return 0;
+}
+
 int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream)
 {
     if (!h || !A || !D)
@@ -626,9 +670,9 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     const size_t a_bytes = (size_t)(d.batch - 1) * d.a_batch_stride + (size_t)(d.M - 1) * d.lda + d.K;
     const size_t d_elems = (size_t)(d.batch - 1) * d.d_batch_stride + (size_t)(d.M - 1) * d.ldd + d.N;
     const void  *Ad, *bfd;
-    TRY(to_device(A, a_bytes, h->stageA, s, &Ad));
-    TRY(to_device(bias_f32, sizeof(float) * d.N, h->stageBiasF, s, &bfd));
-    const bool d_host = !is_device_ptr(D);
+    TRY(to_device(A, a_bytes, h->stageA, s, &Ad, &h->kindA));
+    TRY(to_device(bias_f32, sizeof(float) * d.N, h->stageBiasF, s, &bfd, &h->kindBiasF));
+    const bool d_host = !h->kindD.is_device(D);
     void      *Dd     = D;
     if (d_host)
     {
@@ -944,6 +988,18 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
     return 0;
 }
 
+int mi355_conv_set_strides(mi355_conv_handle *h, int64_t src_pixel_stride, int64_t weights_pixel_stride,
+                           int64_t dst_pixel_stride)
+{
+    if (!h)
+        return fail("null argument");
+    mi355_conv_desc d = h->d;
+    d.src_pixel_stride = src_pixel_stride, d.weights_pixel_stride = weights_pixel_stride, d.dst_pixel_stride = dst_pixel_stride;
+    TRY(conv_check(d));
+    h->d = d;
+    return 0;
+}
+
 int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream)
 {
     if (!h || !src || !dst)
@@ -960,14 +1016,15 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     const bool    d_pad     = d.dst_pixel_stride != 0 && d.dst_pixel_stride != (int64_t)d.OFM * (int64_t)desz;
     const size_t  dst_ext   = d_pad ? (size_t)((int64_t)(c.M - 1) * d.dst_pixel_stride + c.N) : dst_bytes;
     const void   *srcd;
-    TRY(to_device(src, s_pad ? (size_t)((pixels - 1) * d.src_pixel_stride + d.C) : src_bytes, h->stageSrc, s, &srcd));
+    TRY(to_device(src, s_pad ? (size_t)((pixels - 1) * d.src_pixel_stride + d.C) : src_bytes, h->stageSrc, s, &srcd,
+                  &h->kindSrc));
     if (s_pad)
     {
         TRY(h->nhwcSrc.ensure(src_bytes));
         HIP_TRY(restride_launch(srcd, h->nhwcSrc.p, pixels, d.C, d.src_pixel_stride, d.C, s));
         srcd = h->nhwcSrc.p;
     }
-    const bool d_host = !is_device_ptr(dst);
+    const bool d_host = !h->kindDst.is_device(dst);
     void      *Dd     = dst;
     if (d_host)
     {
@@ -1030,7 +1087,7 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         HIP_TRY(hipMemcpyAsync(dst, Dd, dst_ext, hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
     }
-    else if (!is_device_ptr(src))
+    else if (!h->kindSrc.is_device(src))
         HIP_TRY(hipStreamSynchronize(s));
     return 0;
 }

@@ -40,7 +40,10 @@ struct EpiParams
     // multiplier is negative and the general formula has to be used
     const int32_t *qp;
     int64_t        qp_stride;
-    int32_t        qp_std; // every column: multiplier >= 2^30, shift in [2, 31]; |result_offset| < 2^28 (see std_requant)
+    int32_t        qp_std; // |result_offset| < 2^28: std_requant may be used where the flag word allows it
+    // One word written together with qp: 0 when every column has a multiplier >= 2^30 and a shift in [2, 31]
+    // (std_requant applies), bit 0 set when some multiplier is negative (then only the general formula applies)
+    const int32_t *qp_flag;
     int32_t        accumulate; // EPI_S32 / EPI_F32: add the destination's previous contents (GEMMInfo::accumulate)
     int32_t        act_twice;  // EPI_F32: the activation clamp is also applied before the offset term is added
 };

@@ -35,6 +35,8 @@
 // 128-byte tile rows, 16 bytes per lane; where the destination is not 16-byte aligned they are stored directly.
 #include "mfma_common.hpp"
 
+#include <atomic>
+
 namespace mi355
 {
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr)
@@ -252,6 +254,11 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         tile_coords_batched(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, bz, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = (g.K + BK - 1) / BK;
+    // which requantisation formula applies was decided on the device when the per-column constants were digested
+    int qflag = 1;
+    if (EPI == EPI_FIXEDPOINT && g.epi.qp_flag != nullptr)
+        qflag = __builtin_amdgcn_readfirstlane(*g.epi.qp_flag);
+    const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
 
     // Barrier protocol (b = number of barriers a wave has executed): consumer group 0 reads stage kt between barriers
     // 2kt and 2kt+1 and multiplies it between 2kt+1 and 2kt+2; group 1 does the same one barrier later. Producers make
@@ -289,7 +296,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
             block_barrier(); // barrier 2kt+2
         }
         block_barrier(); // barrier 2nk+1
-        if (EPI == EPI_FIXEDPOINT && g.epi.qp != nullptr)
+        if (fast)
         {
             __syncthreads(); // the consumers' staging of the epilogue constants
             if (g.epi.vec_store16)
@@ -308,7 +315,6 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
     constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
     constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
     int32_t       par_reg[PPT > 0 ? PPT : 1];
-    const bool    fast = EPI == EPI_FIXEDPOINT && g.epi.qp != nullptr;
     if (fast)
     {
 #pragma unroll
@@ -435,7 +441,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         if (EPI == EPI_FIXEDPOINT)
         {
             char *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
-            if (g.epi.vec_store16 && g.epi.qp_std)
+            if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0)
                 epilogue_store_staged<true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
                                                                 [] { __syncthreads(); });
             else if (g.epi.vec_store16)
@@ -485,7 +491,6 @@ static const DmaEntry g_dma[] = {
     MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
     MI355_DCFG("pp_64x64x128_s6", 64, 64, 128, 1, 2, 6),
     MI355_DCFG("pp_128x64x256_s3", 128, 64, 256, 2, 2, 3),
-    MI355_DCFG("pp_256x128x64_s4", 256, 128, 64, 2, 2, 4),
 };
 
 int dma_num_configs()
@@ -518,9 +523,19 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
         return (int)hipErrorInvalidValue;
     if (c.lds_bytes > 48 * 1024)
     {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, c.lds_bytes);
-        if (e != hipSuccess)
-            return (int)e;
+        // once per kernel and device
+        static std::atomic<uint32_t> raised[sizeof(g_dma) / sizeof(g_dma[0])][3][2][2];
+        std::atomic<uint32_t>       &done = raised[cfg_idx][epi][flip_a ? 1 : 0][conv ? 1 : 0];
+        int                          dev  = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
+            return (int)hipErrorInvalidDevice;
+        if ((done.load(std::memory_order_acquire) & (1u << dev)) == 0)
+        {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, c.lds_bytes);
+            if (e != hipSuccess)
+                return (int)e;
+            done.fetch_or(1u << dev, std::memory_order_release);
+        }
     }
     GemmArgs a       = args;
     // reciprocals for the tile map: floor(2^32 / d) + 1 gives x / d exactly while x * d < 2^32; the 4-wide groups are

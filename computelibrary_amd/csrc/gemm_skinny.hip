@@ -13,6 +13,7 @@
 // number of waves per block is chosen from the number of column groups.
 #include "internal.hpp"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace mi355
@@ -20,9 +21,10 @@ namespace mi355
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 
-// Row pitch of the staged copy of A (STAGE_A): 1 KiB of a row's K slice + 64 bytes, which spreads the 8 rows an
-// operand read touches over the LDS banks
-constexpr int SK_A_PITCH = 1024 + 64;
+// STAGE_A: a wave's K slice of A is at most 4 KiB / WAVES per row (K <= 4096); the row pitch of its staged copy adds
+// 64 bytes, which spreads the 8 rows an operand read touches over the LDS banks
+constexpr int sk_a_slice(int waves) { return 4096 / waves; }
+constexpr int sk_a_pitch(int waves) { return sk_a_slice(waves) + 64; }
 template <int EPI, bool FLIP_A, int NG, int SK_WAVES, int SK_UNROLL, bool STAGE_A, int MR, bool STEP_A = false,
           int STEP_KB = (MR == 4 ? 4 : 8)>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
@@ -30,7 +32,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     static_assert(MR >= 1 && MR <= SK_WAVES && (!STAGE_A || MR == 1), "row blocks");
     static_assert(!STEP_A || (!STAGE_A && SK_UNROLL == 8), "per-step staging: steps of 8 k blocks");
     __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
-    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][SK_A_PITCH]
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][sk_a_pitch(SK_WAVES)]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -90,27 +92,30 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     const v4i zero4 = {0, 0, 0, 0};
     int       kb    = kb0;
 
-    // STAGE_A (M <= 8, every wave's K slice at most 1 KiB per row, K a multiple of 64, 16-byte aligned rows): the wave
+    // STAGE_A (M <= 8, every wave's K slice at most A_SLICE bytes per row, K a multiple of 64, 16-byte aligned rows): the wave
     // copies its slice of A into LDS once, with all 64 lanes per load, and takes the operand blocks from there.
     // Loading them from global memory inside the stream costs one half-empty load instruction (rows 8..15 are padding)
     // per B load and 16 % of the kernel's time, although A never leaves the L2.
-    char *a_lds = a_stage + (STEP_A ? wave * MR * 16 * (STEP_KB * 64 + 16) : wave * 8 * SK_A_PITCH);
-    v4i   ta[STAGE_A ? 8 : 1];
+    constexpr int A_SLICE = sk_a_slice(SK_WAVES), A_PITCH = sk_a_pitch(SK_WAVES);
+    constexpr int NA      = 8 * A_SLICE / 1024; // load instructions (1 KiB each) that cover 8 rows of a slice
+    constexpr int LPR     = A_SLICE / 16;       // lanes per row
+    char *a_lds = a_stage + (STEP_A ? wave * MR * 16 * (STEP_KB * 64 + 16) : wave * 8 * A_PITCH);
+    v4i   ta[STAGE_A ? NA : 1];
+    const int a_sr = lane / LPR, a_sc = (lane % LPR) * 16; // this lane's row (of 1024 / A_SLICE per load) and column
     if (STAGE_A)
     {
         // branch-free (a branch per row would put a full wait behind every load): rows past M re-read row M-1 into
-        // staging rows nobody reads, lanes past the slice re-read its first 16 bytes into the unused end of the pitch
-        const int slice = max(kb1 - kb0, 0) * 64; // bytes per row, <= 1024
-        const int col   = lane * 16 < slice ? lane * 16 : 0;
+        // staging rows nobody reads, lanes past the slice re-read its first 16 bytes into columns nobody reads
+        const int slice = max(kb1 - kb0, 0) * 64; // bytes per row, <= A_SLICE
+        const int col   = a_sc < slice ? a_sc : 0;
         const int8_t *src = g.A + (int64_t)min(kb0, KB - 1) * 64 + col;
 #pragma unroll
-        for (int r = 0; r < 8; ++r)
-            ta[r] = *(const v4i *)(src + (int64_t)min(r, g.M - 1) * g.lda);
+        for (int i = 0; i < NA; ++i)
+            ta[i] = *(const v4i *)(src + (int64_t)min(i * (1024 / A_SLICE) + a_sr, g.M - 1) * g.lda);
     }
-    const char *a_frag = a_lds + arow * SK_A_PITCH + akc; // this lane's piece of the operand block of k block kb0
+    const char *a_frag = a_lds + arow * A_PITCH + akc; // this lane's piece of the operand block of k block kb0
     // whole steps inside the wave's range and inside K: straight-line loads, all in flight together; the loads of the
-    // next step directly follow the matrix instructions of this one. (Issuing the first step's loads before the wave
-    // waits for its slice of A measured 1 % slower: the 8 + 8 registers of both are then live together.)
+    // next step directly follow the matrix instructions of this one.
     v4i  fb[SK_UNROLL][NG];
     auto whole_step = [&](int k) { return k + SK_UNROLL <= kb1 && (k + SK_UNROLL) * 64 <= g.K; };
     auto load_b     = [&](int k)
@@ -121,14 +126,21 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
             for (int n = 0; n < NG; ++n)
                 fb[u][n] = __builtin_nontemporal_load((const v4i *)(b_ptr[n] + (int64_t)(k + u) * 1024));
     };
+    // STAGE_A: the first step of the B stream is issued before the wave waits for its slice of A. Loads return in order,
+    // so the wait for A (the older loads) does not wait for B, and one memory latency leaves the critical path
+    // (M = 8, N = 11008, K = 4096: 9.7 -> 9.4 us).
+    bool more = false;
     if (STAGE_A)
     {
+        more = whole_step(kb);
+        if (more)
+            load_b(kb);
 #pragma unroll
-        for (int r = 0; r < 8; ++r)
+        for (int i = 0; i < NA; ++i)
         {
             if (FLIP_A)
-                ta[r] ^= (int)0x80808080;
-            *(v4i *)(a_lds + r * SK_A_PITCH + lane * 16) = ta[r];
+                ta[i] ^= (int)0x80808080;
+            *(v4i *)(a_lds + (i * (1024 / A_SLICE) + a_sr) * A_PITCH + a_sc) = ta[i];
         }
     }
     if constexpr (STEP_A)
@@ -143,7 +155,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
         constexpr int RPL   = 64 / LPR;              // rows per load instruction
         constexpr int PITCH = SKB * 64 + 16;         // 16 rows of an operand read fall into 16 different bank groups
         const int     sub = lane / LPR, col = (lane % LPR) * 16;
-        bool          more = whole_step(kb);
+        more = whole_step(kb);
         if (more)
             load_b(kb);
         while (more)
@@ -189,35 +201,47 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     }
     else if constexpr (MR == 1)
     {
-        bool more = whole_step(kb);
-        if (more)
-            load_b(kb);
+        if (!STAGE_A)
+        {
+            more = whole_step(kb);
+            if (more)
+                load_b(kb);
+        }
         while (more)
         {
-            v4i fa[SK_UNROLL];
+            // staged operands are read in two halves (the scheduler would otherwise hoist all reads and hold 8
+            // operand blocks next to the 8 blocks of B: 86 registers, one too few waves per SIMD for the 8-wave variant)
+            constexpr int HALVES = STAGE_A ? 2 : 1, HU = SK_UNROLL / HALVES;
 #pragma unroll
-            for (int u = 0; u < SK_UNROLL; ++u)
-                fa[u] = zero4;
-            if (a_live[0])
+            for (int h = 0; h < HALVES; ++h)
             {
+                v4i fa[HU];
 #pragma unroll
-                for (int u = 0; u < SK_UNROLL; ++u)
+                for (int u = 0; u < HU; ++u)
+                    fa[u] = zero4;
+                if (a_live[0])
                 {
-                    if (STAGE_A)
-                        fa[u] = *(const v4i *)(a_frag + (kb + u - kb0) * 64);
-                    else
+#pragma unroll
+                    for (int u = 0; u < HU; ++u)
                     {
-                        fa[u] = *(const v4i *)(a_ptr[0] + (int64_t)(kb + u) * 64);
-                        if (FLIP_A)
-                            fa[u] ^= (int)0x80808080;
+                        if (STAGE_A)
+                            fa[u] = *(const v4i *)(a_frag + (kb + h * HU + u - kb0) * 64);
+                        else
+                        {
+                            fa[u] = *(const v4i *)(a_ptr[0] + (int64_t)(kb + u) * 64);
+                            if (FLIP_A)
+                                fa[u] ^= (int)0x80808080;
+                        }
                     }
                 }
+#pragma unroll
+                for (int u = 0; u < HU; ++u)
+#pragma unroll
+                    for (int n = 0; n < NG; ++n)
+                        acc[0][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[h * HU + u][n], acc[0][n], 0, 0, 0);
+                if (HALVES > 1)
+                    __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int u = 0; u < SK_UNROLL; ++u)
-#pragma unroll
-                for (int n = 0; n < NG; ++n)
-                    acc[0][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[u][n], acc[0][n], 0, 0, 0);
             kb += SK_UNROLL;
             more = whole_step(kb);
             if (more)
@@ -259,7 +283,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
                         acc[rb][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u][rb], b[u][n], acc[rb][n], 0, 0, 0);
                 }
         };
-        bool more = whole_step(kb);
+        more = whole_step(kb);
         if (more)
             load_ab(fb, fa, kb);
         while (more)
@@ -364,66 +388,96 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     }
 }
 
+// A kernel that needs more than 48 KiB of dynamic LDS has to be told so once per device
+static int raise_lds_limit(const void *fn, size_t lds, std::atomic<uint32_t> &done)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
+        return (int)hipErrorInvalidDevice;
+    if (done.load(std::memory_order_acquire) & (1u << dev))
+        return 0;
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+        done.fetch_or(1u << dev, std::memory_order_release);
+    return (int)e;
+}
+
 template <int NG, int WAVES, int UNROLL, bool STAGE_A, int MR = 1, bool STEP_A = false>
 static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
 {
     const int    groups = (a.N + 15) / 16;
     const dim3   grid((groups + NG - 1) / NG), block(WAVES * 64);
-    const size_t lds = STAGE_A ? (size_t)WAVES * 8 * SK_A_PITCH : (STEP_A ? (size_t)WAVES * MR * 16 * ((MR == 4 ? 4 : 8) * 64 + 16) : 0);
+    const size_t lds = STAGE_A ? (size_t)WAVES * 8 * sk_a_pitch(WAVES) : (STEP_A ? (size_t)WAVES * MR * 16 * ((MR == 4 ? 4 : 8) * 64 + 16) : 0);
+    if (epi != EPI_S32 && epi != EPI_FIXEDPOINT && epi != EPI_F32)
+        return (int)hipErrorInvalidValue;
+    static const void *const fns[3][2] = {
+        {(const void *)gemm_skinny_kernel<EPI_S32, false, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>,
+         (const void *)gemm_skinny_kernel<EPI_S32, true, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>},
+        {(const void *)gemm_skinny_kernel<EPI_FIXEDPOINT, false, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>,
+         (const void *)gemm_skinny_kernel<EPI_FIXEDPOINT, true, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>},
+        {(const void *)gemm_skinny_kernel<EPI_F32, false, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>,
+         (const void *)gemm_skinny_kernel<EPI_F32, true, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>}};
+    static std::atomic<uint32_t> lds_raised[3][2];
+    const void *fn = fns[epi][flip_a ? 1 : 0];
     if (lds > 48 * 1024)
     {
-#define MI355_SKA(E, F)                                                                                                  \
-    (void)hipFuncSetAttribute((const void *)gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A>,            \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-        if (epi == EPI_S32)
-            flip_a ? MI355_SKA(EPI_S32, true) : MI355_SKA(EPI_S32, false);
-        else if (epi == EPI_FIXEDPOINT)
-            flip_a ? MI355_SKA(EPI_FIXEDPOINT, true) : MI355_SKA(EPI_FIXEDPOINT, false);
-        else if (epi == EPI_F32)
-            flip_a ? MI355_SKA(EPI_F32, true) : MI355_SKA(EPI_F32, false);
-#undef MI355_SKA
+        const int e = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
+        if (e)
+            return e;
     }
-#define MI355_SK(E, F) gemm_skinny_kernel<E, F, NG, WAVES, UNROLL, STAGE_A, MR, STEP_A><<<grid, block, lds, s>>>(a)
-    if (epi == EPI_S32)
-        flip_a ? MI355_SK(EPI_S32, true) : MI355_SK(EPI_S32, false);
-    else if (epi == EPI_FIXEDPOINT)
-        flip_a ? MI355_SK(EPI_FIXEDPOINT, true) : MI355_SK(EPI_FIXEDPOINT, false);
-    else if (epi == EPI_F32)
-        flip_a ? MI355_SK(EPI_F32, true) : MI355_SK(EPI_F32, false);
-    else
-        return (int)hipErrorInvalidValue;
-#undef MI355_SK
-    return (int)hipGetLastError();
+    GemmArgs copy    = a;
+    void    *kargs[] = {&copy};
+    return (int)hipLaunchKernel(fn, grid, block, kargs, lds, s);
 }
+
+// Environment overrides for experiments, read once: MI355_SKINNY_WAVES (4 or 8; anything else is ignored),
+// MI355_SKINNY_NG (column groups per workgroup), MI355_SKINNY_NO_STAGE (A operands straight from global memory)
+struct SkinnyEnv
+{
+    int  waves = 0, ng = 0;
+    bool no_stage = false;
+    SkinnyEnv()
+    {
+        const char *w = getenv("MI355_SKINNY_WAVES"), *n = getenv("MI355_SKINNY_NG");
+        if (w && (atoi(w) == 4 || atoi(w) == 8))
+            waves = atoi(w);
+        if (n && atoi(n) >= 1 && atoi(n) <= 4)
+            ng = atoi(n);
+        no_stage = getenv("MI355_SKINNY_NO_STAGE") != nullptr;
+    }
+};
 
 int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
 {
     if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
         return (int)hipErrorInvalidValue;
-    // about 2000-4000 waves fill the 256 compute units with enough loads in flight: split K over 4 waves per block
-    // when there are many column groups, over 8 otherwise
-    static const char *force  = getenv("MI355_SKINNY_WAVES");
-    const int          groups = (args.N + 15) / 16;
-    const int          waves  = force ? atoi(force) : (groups >= 512 ? 4 : 8);
-    // A goes through LDS when a wave's K slice fits 1 KiB per row and nothing about it needs guarding
-    const int  per   = ((int)(args.Kp / 64) + waves - 1) / waves;
-    const bool stage = args.M <= 8 && per <= 16 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
-                       ((uintptr_t)args.A & 15) == 0 && getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    static const SkinnyEnv env;
+    const int groups = (args.N + 15) / 16;
+    const int KB     = (int)(args.Kp / 64);
+    // Up to 8 rows every wave copies its K slice of A (at most 1 KiB per row) into LDS once and takes its operands
+    // from there; that needs nothing to guard
+    const bool stage_ok = args.M <= 8 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
+                          ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
+    // The kernel lives on loads in flight: 8 waves per workgroup while each of them still has at least one whole
+    // step of 8 k blocks and all workgroups are resident together (24 waves of this size per compute unit), 4 otherwise
+    int waves = (groups >= 512 && !(stage_ok && KB >= 64 && (int64_t)groups * 8 <= 24 * 256)) ? 4 : 8;
+    if (env.waves)
+        waves = env.waves;
+    const int  per   = (KB + waves - 1) / waves;
+    const bool stage = stage_ok && per * 64 <= sk_a_slice(waves);
     // more than 8 rows: per-step staging (dword-aligned rows are enough: the staging loads are plain 16-byte loads)
-    const bool step = args.M > 8 && args.lda % 4 == 0 && ((uintptr_t)args.A & 3) == 0 &&
-                      getenv("MI355_SKINNY_NO_STAGE") == nullptr;
+    const bool step = args.M > 8 && args.lda % 4 == 0 && ((uintptr_t)args.A & 3) == 0 && !env.no_stage;
     // (17..24 rows: the gathers of the unstaged variants below re-read row M-1 for the missing rows of the second
     // block, which costs less than staging 32 rows)
     if (args.M > 24 && step)
     {
         // LDS: 8.25 KiB per wave and block of 16 rows; a workgroup covers 2 column groups when there are many
-        static const char *force_ng = getenv("MI355_SKINNY_NG");
-        const int          ng       = force_ng ? (atoi(force_ng) >= 2 ? 2 : 1) : (groups >= 512 ? 2 : 1);
-        const int          blocks   = (groups + ng - 1) / ng;
+        const int ng     = env.ng ? (env.ng >= 2 ? 2 : 1) : (groups >= 512 ? 2 : 1);
+        const int blocks = (groups + ng - 1) / ng;
         if (args.M > 32)
             return ng == 2 ? skinny_launch_v<2, 4, 8, false, 4, true>(epi, flip_a, args, s)
                            : skinny_launch_v<1, 4, 8, false, 4, true>(epi, flip_a, args, s);
-        const int w = force ? atoi(force) : (blocks >= 320 ? 4 : 8);
+        const int w = env.waves ? env.waves : (blocks >= 320 ? 4 : 8);
         if (ng == 2)
             return w == 4 ? skinny_launch_v<2, 4, 8, false, 2, true>(epi, flip_a, args, s)
                           : skinny_launch_v<2, 8, 8, false, 2, true>(epi, flip_a, args, s);
@@ -434,14 +488,13 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     {
         // More than one block of 16 rows: A (L2 resident) is re-read once per block of the grid, which costs as much as
         // the B stream unless a block covers several column groups - as many as still leave a few hundred blocks.
-        static const char *force_ng = getenv("MI355_SKINNY_NG");
-        const int          mr       = args.M > 32 ? 4 : 2;
-        int                ng       = groups >= 1024 ? 4 : (groups >= 512 ? 2 : 1);
-        if (force_ng)
-            ng = atoi(force_ng);
+        const int mr = args.M > 32 ? 4 : 2;
+        int       ng = groups >= 1024 ? 4 : (groups >= 512 ? 2 : 1);
+        if (env.ng)
+            ng = env.ng;
         ng = ng >= 4 && mr == 4 ? 4 : (ng >= 2 ? 2 : 1);
         const int blocks = (groups + ng - 1) / ng;
-        const int w      = force ? atoi(force) : (blocks >= 320 ? 4 : 8);
+        const int w      = env.waves ? env.waves : (blocks >= 320 ? 4 : 8);
 #define MI355_SKV(NG_, MR_)                                                                          \
     (w == 4 ? skinny_launch_v<NG_, 4, 2, false, MR_>(epi, flip_a, args, s)                           \
             : skinny_launch_v<NG_, 8, 2, false, MR_>(epi, flip_a, args, s))
@@ -450,11 +503,13 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
         return ng == 4 ? MI355_SKV(4, 4) : (ng == 2 ? MI355_SKV(2, 4) : MI355_SKV(1, 4));
 #undef MI355_SKV
     }
+    // the waves of the unstaged / per-step variants follow the old rule
+    const int w1 = env.waves ? env.waves : (groups >= 512 ? 4 : 8);
     if (step) // 9..16 rows
-        return waves == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, s)
-                          : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, s);
+        return w1 == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, s)
+                       : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, s);
     if (stage)
         return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, s);
-    return waves == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);
+    return w1 == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);
 }
 } // namespace mi355

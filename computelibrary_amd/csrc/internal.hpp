@@ -94,7 +94,6 @@ int         mfma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const Gemm
 int         dma_num_configs();
 MfmaConfig  dma_config(int idx);
 int         dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
-constexpr int DMA_AUTO_CONFIGS = 6; // the first entries are the ones the heuristic picks from; the rest are experiments
 
 // gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 64;

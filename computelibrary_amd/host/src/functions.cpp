@@ -93,9 +93,70 @@ Status check_matrix_layout(const ITensorInfo *t, const char *name)
     return Status{};
 }
 
+// Clamp bounds of an 8-bit output stage must lie inside the destination type's range (a bounded activation) or cover it
+// (saturation only). With one end inside and one outside, the reference's own paths disagree: the stand-alone kernel
+// narrows the bound to 8 bits (src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:502-503), the assembly
+// path clamps in int32 and keeps the low byte (src/core/NEON/kernels/arm_gemm/quantized.cpp:36-46,254-261).
+Status check_8bit_bounds(const GEMMLowpOutputStageInfo &stage, DataType dt)
+{
+    if (dt != DataType::QASYMM8 && dt != DataType::QASYMM8_SIGNED)
+        return Status{};
+    if (stage.type == GEMMLowpOutputStageType::QUANTIZE_DOWN && stage.gemmlowp_min_bound == stage.gemmlowp_max_bound)
+        return Status{}; // "no bounded activation" for that stage
+    const int32_t lo = dt == DataType::QASYMM8 ? 0 : -128, hi = dt == DataType::QASYMM8 ? 255 : 127;
+    const bool    covers = stage.gemmlowp_min_bound <= lo && stage.gemmlowp_max_bound >= hi;
+    const bool    inside = stage.gemmlowp_min_bound >= lo && stage.gemmlowp_max_bound <= hi;
+    ARM_COMPUTE_RETURN_ERROR_ON_MSG(!covers && !inside, "Output stage bounds partly outside the output type's range");
+    return Status{};
+}
+
 const std::set<ActivationLayerInfo::ActivationFunction> fusable_acts = {
     ActivationLayerInfo::ActivationFunction::RELU, ActivationLayerInfo::ActivationFunction::BOUNDED_RELU,
     ActivationLayerInfo::ActivationFunction::LU_BOUNDED_RELU};
+
+// Row and batch strides of the three matrices as the tensor infos give them now; an info that is not at hand (nullptr)
+// leaves its fields as they are
+void read_gemm_strides(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorInfo *oi, const GEMMInfo &gemm_info,
+                       mi355_gemm_desc &d)
+{
+    const bool a3d = gemm_info.reinterpret_input_as_3d();
+    if (ai != nullptr)
+    {
+        d.lda            = ai->strides_in_bytes()[1];
+        d.a_batch_stride = ai->strides_in_bytes()[a3d ? 3 : 2];
+    }
+    if (bi != nullptr)
+    {
+        d.ldb            = bi->strides_in_bytes()[1];
+        d.b_batch_stride = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
+    }
+    if (oi != nullptr)
+    {
+        d.ldd = oi->strides_in_bytes()[1] / oi->element_size();
+        if (gemm_info.depth_output_gemm3d() != 0)
+            d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
+        else
+            d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
+    }
+}
+
+// Padding may be added to a tensor between configure() and the first run (the reference's fixtures do exactly that:
+// tests/validation/fixtures/GEMMLowpFixture.h:300-304, CpuGEMMLowpFixture.h:117) and the reference reads strides when
+// it runs. Re-reads them from the infos at hand and tells the handle when they differ from what it holds. Once B is
+// packed its strides no longer matter.
+void sync_gemm_strides(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorInfo *oi, const GEMMInfo &info,
+                       mi355_gemm_desc &d, mi355_gemm_handle *handle, bool b_is_packed, const char *where)
+{
+    mi355_gemm_desc now = d;
+    read_gemm_strides(ai, b_is_packed ? nullptr : bi, oi, info, now);
+    if (now.lda == d.lda && now.ldb == d.ldb && now.ldd == d.ldd && now.a_batch_stride == d.a_batch_stride &&
+        now.b_batch_stride == d.b_batch_stride && now.d_batch_stride == d.d_batch_stride)
+        return;
+    check_abi(mi355_gemmlowp_set_strides(handle, now.lda, now.ldb, now.ldd, now.a_batch_stride, now.b_batch_stride,
+                                         now.d_batch_stride),
+              where);
+    d = now;
+}
 
 // the C-ABI descriptor of a GEMMLowp on these tensor infos (shapes are x-fastest: a = [K, M, batch], b = [N, K(, batch)],
 // output = [N, M, batch]); per-channel multipliers / shifts are cut to exactly N entries
@@ -113,15 +174,7 @@ void fill_gemm_desc(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorI
     d.a_dtype          = to_mi355(ai->data_type());
     d.b_dtype          = to_mi355(bi->data_type());
     d.dst_dtype        = to_mi355(oi->data_type());
-    d.lda              = ai->strides_in_bytes()[1];
-    d.ldb              = bi->strides_in_bytes()[1];
-    d.ldd              = oi->strides_in_bytes()[1] / oi->element_size();
-    d.a_batch_stride   = ai->strides_in_bytes()[a3d ? 3 : 2];
-    d.b_batch_stride   = bi->num_dimensions() > 2 ? bi->strides_in_bytes()[2] : 0;
-    if (gemm_info.depth_output_gemm3d() != 0)
-        d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
-    else
-        d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
+    read_gemm_strides(ai, bi, oi, gemm_info, d);
     d.a_offset = ai->quantization_info().uniform().offset;
     d.b_offset = is_data_type_quantized_per_channel(bi->data_type()) ? 0 : bi->quantization_info().uniform().offset;
     d.act_min  = -std::numeric_limits<float>::infinity();
@@ -311,6 +364,7 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
             ARM_COMPUTE_RETURN_ERROR_ON_MSG(!is_one_of(output->data_type(), {DataType::QASYMM8, DataType::QASYMM8_SIGNED}),
                                             "The integer output stages write QASYMM8 or QASYMM8_SIGNED");
             ARM_COMPUTE_RETURN_ERROR_ON(stage.gemmlowp_min_bound > stage.gemmlowp_max_bound);
+            ARM_COMPUTE_RETURN_ON_ERROR(check_8bit_bounds(stage, output->data_type()));
             if (c != nullptr)
             {
                 ARM_COMPUTE_RETURN_ERROR_ON(c->data_type() != DataType::S32);
@@ -354,41 +408,17 @@ void NEGEMMLowpMatrixMultiplyCore::configure(const ITensor *a, const ITensor *b,
     check_abi(mi355_gemmlowp_create(&d, &s.handle), "NEGEMMLowpMatrixMultiplyCore::configure");
 }
 
-namespace
-{
-// Padding may be added to a tensor between configure() and the first run (the reference's fixtures do exactly that:
-// tests/validation/fixtures/GEMMLowpFixture.h:300-304) and the reference reads strides when it runs. The strides are
-// part of the descriptor here: when they have changed, the handle is made again (nothing is packed yet in that flow).
-bool gemm_strides_changed(const ITensorInfo *ai, const ITensorInfo *bi, const ITensorInfo *oi, const GEMMInfo &info,
-                          mi355_gemm_desc &d)
-{
-    mi355_gemm_desc       now;
-    std::vector<int32_t> m, sh;
-    fill_gemm_desc(ai, bi, oi, info, now, m, sh);
-    const bool changed = now.lda != d.lda || now.ldb != d.ldb || now.ldd != d.ldd || now.a_batch_stride != d.a_batch_stride ||
-                         now.b_batch_stride != d.b_batch_stride || now.d_batch_stride != d.d_batch_stride;
-    if (changed)
-        d.lda = now.lda, d.ldb = now.ldb, d.ldd = now.ldd, d.a_batch_stride = now.a_batch_stride,
-        d.b_batch_stride = now.b_batch_stride, d.d_batch_stride = now.d_batch_stride;
-    return changed;
-}
-} // namespace
-
 void NEGEMMLowpMatrixMultiplyCore::prepare()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMLowpMatrixMultiplyCore::prepare() before configure()");
-    if (gemm_strides_changed(s.a->info(), s.b->info(), s.output->info(), s.info, s.desc))
-    {
-        ARM_COMPUTE_ERROR_THROW_ON(validate(s.a->info(), s.b->info(), s.c != nullptr ? s.c->info() : nullptr,
-                                            s.output->info(), s.info));
-        mi355_gemmlowp_destroy(s.handle);
-        s.handle = nullptr;
-        check_abi(mi355_gemmlowp_create(&s.desc, &s.handle), "NEGEMMLowpMatrixMultiplyCore::prepare");
-        s.is_prepared = false;
-    }
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(s.a->info(), "a"));
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(s.output->info(), "output"));
+    sync_gemm_strides(s.a->info(), s.b->info(), s.output->info(), s.info, s.desc, s.handle, s.is_prepared,
+                      "NEGEMMLowpMatrixMultiplyCore::prepare");
     if (s.is_prepared)
         return;
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(s.b->info(), "b"));
     ARM_COMPUTE_ERROR_ON_MSG(s.b->buffer() == nullptr, "matrix B has no memory");
     const int32_t *bias = nullptr;
     if (s.desc.epilogue == MI355_EPI_FIXEDPOINT && s.c != nullptr)
@@ -523,6 +553,7 @@ Status NEGEMMLowpOutputStage::validate(const ITensorInfo *input, const ITensorIn
     }
     ARM_COMPUTE_RETURN_ERROR_ON(input->data_type() != DataType::S32 || input->num_channels() != 1);
     ARM_COMPUTE_RETURN_ERROR_ON(info.gemmlowp_min_bound > info.gemmlowp_max_bound);
+    ARM_COMPUTE_RETURN_ON_ERROR(check_8bit_bounds(info, output->data_type()));
     ARM_COMPUTE_RETURN_ERROR_ON_MSG(info.is_quantized_per_channel, "The stand-alone output stage is per-tensor");
     if (bias != nullptr)
     {
@@ -890,16 +921,20 @@ void NEGEMMConvolutionLayer::configure(const ITensor *input, const ITensor *weig
 
 namespace
 {
-// see gemm_strides_changed: the same for the convolution's pixel strides
-bool conv_strides_changed(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, mi355_conv_desc &d)
+// see sync_gemm_strides: the same for the convolution's pixel strides (an info that is not at hand, or weights that
+// are already packed, leave their stride as it is)
+void sync_conv_strides(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, mi355_conv_desc &d,
+                       mi355_conv_handle *handle, const char *where)
 {
     if (d.layout != MI355_NHWC)
-        return false;
-    const int64_t sp = static_cast<int64_t>(ii->strides_in_bytes()[1]), wp = static_cast<int64_t>(wi->strides_in_bytes()[1]);
-    const int64_t dp = static_cast<int64_t>(oi->strides_in_bytes()[1]);
-    const bool    changed = sp != d.src_pixel_stride || wp != d.weights_pixel_stride || dp != d.dst_pixel_stride;
+        return;
+    const int64_t sp = ii ? static_cast<int64_t>(ii->strides_in_bytes()[1]) : d.src_pixel_stride;
+    const int64_t wp = wi ? static_cast<int64_t>(wi->strides_in_bytes()[1]) : d.weights_pixel_stride;
+    const int64_t dp = oi ? static_cast<int64_t>(oi->strides_in_bytes()[1]) : d.dst_pixel_stride;
+    if (sp == d.src_pixel_stride && wp == d.weights_pixel_stride && dp == d.dst_pixel_stride)
+        return;
+    check_abi(mi355_conv_set_strides(handle, sp, wp, dp), where);
     d.src_pixel_stride = sp, d.weights_pixel_stride = wp, d.dst_pixel_stride = dp;
-    return changed;
 }
 } // namespace
 
@@ -907,13 +942,8 @@ void NEGEMMConvolutionLayer::prepare()
 {
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEGEMMConvolutionLayer::prepare() before configure()");
-    if (conv_strides_changed(s.src->info(), s.weights->info(), s.dst->info(), s.desc))
-    {
-        mi355_conv_destroy(s.handle);
-        s.handle = nullptr;
-        check_abi(mi355_conv_create(&s.desc, &s.handle), "NEGEMMConvolutionLayer::prepare");
-        s.is_prepared = false;
-    }
+    sync_conv_strides(s.src->info(), s.is_prepared ? nullptr : s.weights->info(), s.dst->info(), s.desc, s.handle,
+                      "NEGEMMConvolutionLayer::prepare");
     if (s.is_prepared)
         return;
     ARM_COMPUTE_ERROR_ON_MSG(s.weights->buffer() == nullptr, "weights have no memory");
@@ -1192,7 +1222,7 @@ void NEFullyConnectedLayer::prepare()
     Impl &s = *_impl;
     ARM_COMPUTE_ERROR_ON_MSG(s.handle == nullptr, "NEFullyConnectedLayer::prepare() before configure()");
     {
-        // padding added after configure() (see gemm_strides_changed)
+        // padding added after configure() (see sync_gemm_strides)
         FcGeometry g;
         ARM_COMPUTE_ERROR_THROW_ON(fc_geometry(s.src->info(), s.weights->info(), s.dst->info(), s.fc_info, g));
         if (fc_strides(s.src->info(), s.weights->info(), s.dst->info(), g, s.desc))
@@ -1295,6 +1325,8 @@ struct CpuGEMMLowp::Impl
 {
     mi355_gemm_desc      desc{};
     mi355_gemm_handle   *handle{nullptr};
+    GEMMInfo             info{};
+    bool                 b_per_channel{false};
     ActivationLayerInfo  act_info{};
     bool                 is_prepared{false};
     bool                 b_constant{true};
@@ -1334,6 +1366,8 @@ void CpuGEMMLowp::configure(const ITensorInfo *a, const ITensorInfo *b, const IT
         s.handle = nullptr;
     }
     s.act_info    = gemm_info.activation_info();
+    s.info        = gemm_info;
+    s.b_per_channel = is_data_type_quantized_per_channel(b->data_type());
     s.is_prepared = false;
     s.b_constant  = gemm_info.reshape_b_only_on_first_run(); // CpuGEMMLowp.cpp:60-66 of the reference
     s.has_bias    = c != nullptr;
@@ -1361,8 +1395,12 @@ void CpuGEMMLowp::update_quantization_parameters(const QuantizationInfo &a, cons
     out.is_quantized_per_channel = false;
     out.output_data_type         = data_type;
     ARM_COMPUTE_ERROR_THROW_ON(quantization::calculate_quantized_multipliers(a, b, c, out));
-    s.desc.a_offset = negated_offsets ? -a.uniform().offset : a.uniform().offset;
-    s.desc.b_offset = negated_offsets ? -b.uniform().offset : b.uniform().offset;
+    // negated_offsets == true: the offsets in a / b are already the values ADDED to every element (what the tensors of
+    // NEGEMMLowpMatrixMultiplyCore carry); false: they are true zero points, which are subtracted
+    // (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:213-215: arm_gemm's subtracted zero point is
+    // -offset * (negated ? 1 : -1))
+    s.desc.a_offset = negated_offsets ? a.uniform().offset : -a.uniform().offset;
+    s.desc.b_offset = negated_offsets ? b.uniform().offset : -b.uniform().offset;
     s.desc.requant  = make_requant(out);
     check_abi(mi355_gemmlowp_update_quant(s.handle, s.desc.a_offset, s.desc.b_offset, &s.desc.requant, s.desc.scale, nullptr),
               "CpuGEMMLowp::update_quantization_parameters");
@@ -1377,6 +1415,9 @@ void CpuGEMMLowp::prepare(ITensorPack &tensors)
         return;
     const ITensor *b = tensors.get_const_tensor(ACL_SRC_1);
     ARM_COMPUTE_ERROR_ON_MSG(b == nullptr || b->buffer() == nullptr, "matrix B (ACL_SRC_1) is missing or has no memory");
+    // the strides are those of the tensor in the pack, which may have been padded after configure()
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(b->info(), "b"));
+    sync_gemm_strides(nullptr, b->info(), nullptr, s.info, s.desc, s.handle, false, "CpuGEMMLowp::prepare");
     const int32_t *bias = nullptr;
     if (s.desc.epilogue == MI355_EPI_FIXEDPOINT && s.has_bias)
     {
@@ -1402,7 +1443,27 @@ void CpuGEMMLowp::run(ITensorPack &tensors)
     ITensor       *dst = tensors.get_tensor(ACL_DST);
     ARM_COMPUTE_ERROR_ON_MSG(a == nullptr || dst == nullptr || a->buffer() == nullptr || dst->buffer() == nullptr,
                              "ACL_SRC_0 / ACL_DST missing or without memory");
+    // dynamic quantization: offsets (and the dequantisation scale) are those the tensors of this pack carry now
+    // (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:668-674,776-784 of the reference)
+    const ITensor *bq = tensors.get_const_tensor(ACL_SRC_1);
+    if (a->info()->quantization_info().is_dynamic() || (bq != nullptr && bq->info()->quantization_info().is_dynamic()))
+    {
+        const int32_t ao = a->info()->quantization_info().uniform().offset;
+        const int32_t bo = (s.b_per_channel || bq == nullptr) ? s.desc.b_offset : bq->info()->quantization_info().uniform().offset;
+        const float   sc = (s.desc.epilogue == MI355_EPI_F32 && bq != nullptr)
+                               ? a->info()->quantization_info().uniform().scale * bq->info()->quantization_info().uniform().scale
+                               : s.desc.scale;
+        if (ao != s.desc.a_offset || bo != s.desc.b_offset || sc != s.desc.scale)
+        {
+            s.desc.a_offset = ao, s.desc.b_offset = bo, s.desc.scale = sc;
+            check_abi(mi355_gemmlowp_update_quant(s.handle, ao, bo, nullptr, sc, nullptr), "CpuGEMMLowp::run");
+        }
+    }
     prepare(tensors);
+    // the strides of the tensors actually handed over (padding may have been added after configure())
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(a->info(), "a"));
+    ARM_COMPUTE_ERROR_THROW_ON(check_matrix_layout(dst->info(), "output"));
+    sync_gemm_strides(a->info(), nullptr, dst->info(), s.info, s.desc, s.handle, true, "CpuGEMMLowp::run");
     const float *bias_f32 = nullptr;
     if (s.desc.epilogue == MI355_EPI_F32 && s.has_bias)
     {
@@ -1486,6 +1547,8 @@ void CpuGemmConv2d::prepare(ITensorPack &tensors)
         return;
     const ITensor *w = tensors.get_const_tensor(ACL_SRC_1);
     ARM_COMPUTE_ERROR_ON_MSG(w == nullptr || w->buffer() == nullptr, "weights (ACL_SRC_1) are missing or have no memory");
+    // the strides are those of the tensor in the pack, which may have been padded after configure()
+    sync_conv_strides(nullptr, w->info(), nullptr, s.desc, s.handle, "CpuGemmConv2d::prepare");
     const int32_t *bias = nullptr;
     if (s.has_bias)
     {
@@ -1523,6 +1586,7 @@ void CpuGemmConv2d::run(ITensorPack &tensors)
     ARM_COMPUTE_ERROR_ON_MSG(src == nullptr || dst == nullptr || src->buffer() == nullptr || dst->buffer() == nullptr,
                              "ACL_SRC_0 / ACL_DST missing or without memory");
     prepare(tensors);
+    sync_conv_strides(src->info(), nullptr, dst->info(), s.desc, s.handle, "CpuGemmConv2d::run");
     check_abi(mi355_conv_run(s.handle, first_element(src), first_element(dst), nullptr), "CpuGemmConv2d::run");
 }
 } // namespace op

@@ -157,6 +157,14 @@ int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *b
 int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t b_offset,
                                 const mi355_requant *requant, float scale, void *stream);
 
+/* New row and batch strides (same units as in mi355_gemm_desc) for the calls that follow: ldb / b_batch_stride are read
+ * by the next mi355_gemmlowp_prepare, the others by the next mi355_gemmlowp_run; nothing already packed is touched.
+ * The reference reads every stride from the tensors when it runs, not when it is configured
+ * (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:658-672,696-697), and its fixtures add padding in between
+ * (tests/validation/fixtures/CpuGEMMLowpFixture.h:117). A shared B cannot become a batched one or the reverse. */
+int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                               int64_t b_batch_stride, int64_t d_batch_stride);
+
 /* Replaces CpuGemmLowpMatrixMultiplyCore::run (:647-811). bias_f32 (N floats, MI355_EPI_F32 only) may be NULL. */
 int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
 
@@ -233,6 +241,11 @@ int  mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const void *b
  * touching the packed weights. mult / shift (OFM int32 each) are read only when requant->per_channel. */
 int  mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t weights_offset, int32_t pad_value,
                              const mi355_requant *requant, const int32_t *mult, const int32_t *shift, void *stream);
+/* New pixel strides (see mi355_conv_desc) for the calls that follow: weights_pixel_stride is read by the next
+ * mi355_conv_prepare, the other two by the next mi355_conv_run. The reference reads strides when it runs and its
+ * fixtures pad the tensors after configure (tests/validation/fixtures/CpuGemmConv2dFixture.h:315-319). NHWC only. */
+int  mi355_conv_set_strides(mi355_conv_handle *h, int64_t src_pixel_stride, int64_t weights_pixel_stride,
+                            int64_t dst_pixel_stride);
 int  mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream);
 void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW);
 void mi355_conv_destroy(mi355_conv_handle *h);

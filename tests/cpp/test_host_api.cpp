@@ -167,6 +167,15 @@ static void test_validate_tables()
     EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o32, fused)));
     st.gemmlowp_min_bound = 5, st.gemmlowp_max_bound = 4;
     EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, GEMMInfo(false, false, true, 0, false, false, st))));
+    // bounds with one end inside the output type's range and one outside are refused (the reference's kernels disagree
+    // on them); bounds that cover the range only saturate and are accepted
+    st.gemmlowp_min_bound = -5, st.gemmlowp_max_bound = 200;
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, GEMMInfo(false, false, true, 0, false, false, st))));
+    st.gemmlowp_min_bound = 10, st.gemmlowp_max_bound = 300;
+    EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, GEMMInfo(false, false, true, 0, false, false, st))));
+    st.gemmlowp_min_bound = std::numeric_limits<int32_t>::lowest(), st.gemmlowp_max_bound = std::numeric_limits<int32_t>::max();
+    EXPECT(bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, &bias, &o8, GEMMInfo(false, false, true, 0, false, false, st))));
+    st.gemmlowp_min_bound = 5, st.gemmlowp_max_bound = 4;
     GEMMInfo acc;
     acc.set_accumulate(true);
     EXPECT(!bool(NEGEMMLowpMatrixMultiplyCore::validate(&a, &b, nullptr, &o8, acc)));
@@ -193,6 +202,10 @@ static void test_validate_tables()
     os.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
     os.gemmlowp_min_bound = 9, os.gemmlowp_max_bound = 1;
     EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
+    os.gemmlowp_min_bound = -1, os.gemmlowp_max_bound = 254; // partly outside [0, 255]
+    EXPECT(!bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
+    os.gemmlowp_min_bound = -1000, os.gemmlowp_max_bound = 1000; // covers it: saturation only
+    EXPECT(bool(NEGEMMLowpOutputStage::validate(&o32, &bias, &o8, os)));
 
     SECTION("NEGEMMConvolutionLayer::validate");
     TensorInfo src(TensorShape(64U, 8U, 8U, 2U), 1, DataType::QASYMM8_SIGNED, QuantizationInfo(0.02f, -1));
@@ -1097,15 +1110,104 @@ static void test_stateless_operator()
     orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 7, -3, &st.gemmlowp_multiplier,
                             &st.gemmlowp_shift, 1, 11, -128, 127);
     EXPECT(dense_copy<int8_t>(dst2) == want);
-    // new quantization, offsets negated as a convolution / fully connected caller would ask
+    // new quantization; negated_offsets = true: the offsets handed over are already the added ones, which is how
+    // NEGEMMLowpMatrixMultiplyCore and the reference's own fixture call this
+    // (tests/validation/fixtures/CpuGEMMLowpFixture.h:109; src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:213-215)
     const QuantizationInfo aq2(0.03f, -4), bq2(0.006f, 2), oq2(0.08f, -6);
     op.update_quantization_parameters(aq2, bq2, oq2, DataType::QASYMM8_SIGNED, true, true);
     op.run(pack2);
     GEMMLowpOutputStageInfo st2;
     EXPECT(bool(quantization::calculate_quantized_multipliers(aq2, bq2, oq2, st2)));
-    orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 4, -2, &st2.gemmlowp_multiplier,
+    orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, -4, 2, &st2.gemmlowp_multiplier,
                             &st2.gemmlowp_shift, 1, -6, -128, 127);
     EXPECT(dense_copy<int8_t>(dst2) == want);
+    // negated_offsets = false: true zero points (what a CpuMatMul-style caller holds); they are subtracted
+    const QuantizationInfo aq3(0.025f, 9), bq3(0.005f, -5), oq3(0.09f, 3);
+    op.update_quantization_parameters(aq3, bq3, oq3, DataType::QASYMM8_SIGNED, true, false);
+    op.run(pack2);
+    GEMMLowpOutputStageInfo st3;
+    EXPECT(bool(quantization::calculate_quantized_multipliers(aq3, bq3, oq3, st3)));
+    orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, -9, 5, &st3.gemmlowp_multiplier,
+                            &st3.gemmlowp_shift, 1, 3, -128, 127);
+    EXPECT(dense_copy<int8_t>(dst2) == want);
+}
+
+// The flow of the reference's fixtures for the stateless operators: configure on tensor infos, THEN pad the tensors
+// along x, allocate and run (tests/validation/fixtures/CpuGEMMLowpFixture.h:95-124, CpuGemmConv2dFixture.h:300-330).
+// The strides the operator walks must be those of the tensors in the pack; dynamic offsets are re-read from them too.
+static void test_stateless_operators_padded_after_configure()
+{
+    SECTION("experimental::op::CpuGEMMLowp / CpuGemmConv2d: x-padding added after configure, dynamic offsets");
+    {
+        const int M = 37, N = 50, K = 96;
+        const QuantizationInfo aq(0.02f, 5, true), bq(0.004f, -2, true), oq(0.06f, 9);
+        TensorInfo ai(TensorShape(K, M), 1, DataType::QASYMM8_SIGNED, aq), bi(TensorShape(N, K), 1, DataType::QASYMM8_SIGNED, bq);
+        TensorInfo ci(TensorShape(N), 1, DataType::S32), oi(TensorShape(N, M), 1, DataType::QASYMM8_SIGNED, oq);
+        GEMMLowpOutputStageInfo st;
+        st.type = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT, st.output_data_type = DataType::QASYMM8_SIGNED;
+        st.gemmlowp_offset = 9, st.gemmlowp_min_bound = -128, st.gemmlowp_max_bound = 127;
+        EXPECT(bool(quantization::calculate_quantized_multipliers(aq, bq, oq, st)));
+        experimental::op::CpuGEMMLowp op;
+        op.configure(&ai, &bi, &ci, &oi, GEMMInfo(false, false, true, 0, false, false, st));
+        Tensor a, b, c, dst;
+        a.allocator()->init(ai), b.allocator()->init(bi), c.allocator()->init(ci), dst.allocator()->init(oi);
+        a.info()->extend_padding(PaddingSize(0, 7, 0, 4)), b.info()->extend_padding(PaddingSize(0, 13, 0, 1));
+        dst.info()->extend_padding(PaddingSize(0, 2, 0, 16));
+        a.allocator()->allocate(), b.allocator()->allocate(), c.allocator()->allocate(), dst.allocator()->allocate();
+        EXPECT(a.info()->strides_in_bytes()[1] != (size_t)K && dst.info()->strides_in_bytes()[1] != (size_t)N);
+        fill_uniform<int8_t>(a, -128, 127, 201), fill_uniform<int8_t>(b, -128, 127, 202), fill_uniform<int32_t>(c, -2000, 2000, 203);
+        std::memset(dst.buffer(), 0x55, dst.info()->total_size());
+        ITensorPack pack{{ACL_SRC_0, &a}, {ACL_SRC_1, &b}, {ACL_SRC_2, &c}, {ACL_DST, &dst}};
+        op.run(pack);
+        const auto A = dense_copy<int8_t>(a), B = dense_copy<int8_t>(b);
+        const auto Cb = dense_copy<int32_t>(c);
+        std::vector<int8_t> want(M * N);
+        orc_gemmlowp_fixedpoint(A.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, 5, -2, &st.gemmlowp_multiplier,
+                                &st.gemmlowp_shift, 1, 9, -128, 127);
+        EXPECT(dense_copy<int8_t>(dst) == want);
+        // the destination's padding bytes are not touched
+        bool pad_ok = true;
+        const size_t ld = dst.info()->strides_in_bytes()[1], off0 = dst.info()->offset_first_element_in_bytes();
+        for (size_t i = 0; i < dst.info()->total_size(); ++i)
+        {
+            const bool inside = i >= off0 && (i - off0) % ld < (size_t)N && (i - off0) / ld < (size_t)M;
+            pad_ok = pad_ok && (inside || dst.buffer()[i] == 0x55);
+        }
+        EXPECT(pad_ok);
+        // dynamic quantization info: new offsets on the pack's tensors are picked up by the next run
+        a.info()->set_quantization_info(QuantizationInfo(0.02f, -11, true));
+        b.info()->set_quantization_info(QuantizationInfo(0.004f, 6, true));
+        op.run(pack);
+        orc_gemmlowp_fixedpoint(A.data(), 1, K, B.data(), 1, N, Cb.data(), want.data(), N, 1, M, N, K, -11, 6, &st.gemmlowp_multiplier,
+                                &st.gemmlowp_shift, 1, 9, -128, 127);
+        EXPECT(dense_copy<int8_t>(dst) == want);
+    }
+    {
+        const int batch = 2, H = 9, W = 8, C = 16, OFM = 24, KH = 3, KW = 3, in_zp = -4, out_zp = 6;
+        const QuantizationInfo iq(0.03f, in_zp), wq(0.01f, 0), oq(0.9f, out_zp);
+        TensorInfo si(TensorShape(C, W, H, batch), 1, DataType::QASYMM8_SIGNED, iq), wi(TensorShape(C, KW, KH, OFM), 1, DataType::QASYMM8_SIGNED, wq);
+        TensorInfo bi(TensorShape(OFM), 1, DataType::S32), di(TensorShape(), 1, DataType::QASYMM8_SIGNED, oq);
+        si.set_data_layout(DataLayout::NHWC), wi.set_data_layout(DataLayout::NHWC), di.set_data_layout(DataLayout::NHWC);
+        const PadStrideInfo psi(1, 1, 1, 1);
+        experimental::op::CpuGemmConv2d op;
+        op.configure(&si, &wi, &bi, &di, psi);
+        Tensor src, w, bias, dst;
+        src.allocator()->init(si), w.allocator()->init(wi), bias.allocator()->init(bi), dst.allocator()->init(di);
+        src.info()->extend_padding(PaddingSize(0, 5, 0, 3)), w.info()->extend_padding(PaddingSize(0, 16, 0, 2));
+        dst.info()->extend_padding(PaddingSize(0, 8, 0, 1));
+        src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
+        fill_uniform<int8_t>(src, -128, 127, 211), fill_uniform<int8_t>(w, -127, 127, 212), fill_uniform<int32_t>(bias, -500, 500, 213);
+        ITensorPack pack{{ACL_SRC_0, &src}, {ACL_SRC_1, &w}, {ACL_SRC_2, &bias}, {ACL_DST, &dst}};
+        op.run(pack);
+        const auto S = dense_copy<int8_t>(src), Wd = dense_copy<int8_t>(w);
+        const auto Bv = dense_copy<int32_t>(bias);
+        GEMMLowpOutputStageInfo st;
+        EXPECT(bool(quantization::calculate_quantized_multipliers(iq, wq, oq, st)));
+        std::vector<int8_t> want(batch * H * W * OFM);
+        orc_conv_nhwc_direct(S.data(), 1, Wd.data(), 1, Bv.data(), want.data(), 1, batch, H, W, C, OFM, KH, KW, 1, 1, 1, 1, 1, 1, 1, 1,
+                             in_zp, 0, &st.gemmlowp_multiplier, &st.gemmlowp_shift, 1, out_zp, -128, 127);
+        EXPECT(dense_copy<int8_t>(dst) == want);
+    }
 }
 
 // the channel-planar layout through NEGEMMConvolutionLayer and the stateless operator on an ITensorPack: both against
@@ -1309,6 +1411,7 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), true);
             test_gemm_conv2d();
             test_stateless_operator();
+            test_stateless_operators_padded_after_configure();
             test_convolution_nchw_and_stateless();
             test_convolution_f32_destination();
             test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);

@@ -63,3 +63,41 @@ def test_create_rejects_bad_descriptors_without_a_gpu():
     g = capi.Gemm(4, 4, 4, capi.U8, capi.U8, capi.U8, capi.EPI_FIXEDPOINT, rq=rq)
     assert g.kernel_name.startswith("skinny")
     g.close()
+
+
+def test_clamp_bounds_partly_outside_the_output_type_are_rejected():
+    """Bounds inside the 8-bit range clamp, bounds that cover it saturate; one end in and one end out is refused, for the
+    fused GEMM, the convolution and a later update alike (the reference's own kernels disagree on such bounds)."""
+    import pytest
+    for dt, bad, good in ((capi.U8, [(-5, 200), (10, 300), (-1, 254)], [(0, 255), (3, 250), (-(1 << 31), (1 << 31) - 1), (-9, 999)]),
+                          (capi.S8, [(-129, 0), (0, 128), (-200, 100)], [(-128, 127), (-100, 5), (-128, 200), (-500, 127)])):
+        for lo, hi in bad:
+            with pytest.raises(capi.Mi355Error, match="partly outside"):
+                capi.Gemm(4, 4, 4, dt, dt, dt, capi.EPI_FIXEDPOINT, rq=capi.requant(1 << 30, 1, 0, lo, hi))
+            with pytest.raises(capi.Mi355Error, match="partly outside"):
+                capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 3, 3, src_dtype=dt, weights_dtype=dt, dst_dtype=dt,
+                                         rq=capi.requant(1 << 30, 1, 0, lo, hi)))
+        for lo, hi in good:
+            g = capi.Gemm(4, 4, 4, dt, dt, dt, capi.EPI_FIXEDPOINT, rq=capi.requant(1 << 30, 1, 0, lo, hi))
+            with pytest.raises(capi.Mi355Error, match="partly outside"):
+                g.update_quant(0, 0, capi.requant(1 << 30, 1, 0, bad[0][0], bad[0][1]))
+            g.close()
+
+
+def test_set_strides_checks_what_create_checks():
+    import pytest
+    g = capi.Gemm(8, 12, 16, capi.S8, capi.S8, capi.S32, capi.EPI_S32, batch=2)
+    g.set_strides(20, 12, 16)
+    assert (g.desc.lda, g.desc.ldd, g.desc.a_batch_stride, g.desc.d_batch_stride) == (20, 16, 160, 128)
+    with pytest.raises(capi.Mi355Error, match="row stride"):
+        g.set_strides(15, 12, 16)
+    with pytest.raises(capi.Mi355Error, match="batch stride"):
+        g.set_strides(20, 12, 16, a_batch_stride=100)
+    with pytest.raises(capi.Mi355Error, match="shared"):
+        g.set_strides(20, 12, 16, b_batch_stride=16 * 12)
+    g.close()
+    c = capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 3, 3))
+    c.set_strides(24, 16, 8)
+    with pytest.raises(capi.Mi355Error, match="pixel stride"):
+        c.set_strides(8, 16, 8)
+    c.close()

@@ -175,7 +175,7 @@ def test_f16_destination(device):
 
 
 PIPELINED_CONFIGS = ["pp_256x128x128_s3", "pp_128x128x128_s3", "pp_128x64x128_s3", "pp_64x64x128_s3", "pp_64x64x128_s6",
-                     "pp_128x64x256_s3", "pp_256x128x64_s4"]
+                     "pp_128x64x256_s3"]
 
 
 @pytest.mark.parametrize("cfg", range(len(PIPELINED_CONFIGS)))

@@ -16,7 +16,7 @@ NHWC, NCHW = 0, 1
 
 EXPORTS = [
     "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_set_strides",
-    "mi355_gemmlowp_run",
+    "mi355_gemmlowp_run", "mi355_gemmlowp_run_noalloc", "mi355_gemmlowp_noalloc_workspace_bytes",
     "mi355_gemmlowp_destroy", "mi355_gemmlowp_kernel_name", "mi355_output_stage_run", "mi355_conv_create",
     "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_set_strides", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
     "mi355_im2col_nhwc_run", "mi355_last_error", "mi355_device_info",
@@ -80,6 +80,9 @@ def lib():
         l.mi355_gemmlowp_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(Requant), C.c_float, vp]
         l.mi355_gemmlowp_set_strides.argtypes = [vp] + [C.c_int64] * 6
         l.mi355_gemmlowp_run.argtypes = [vp, vp, f32p, vp, vp]
+        l.mi355_gemmlowp_run_noalloc.argtypes = [vp, vp, f32p, vp, vp]
+        l.mi355_gemmlowp_noalloc_workspace_bytes.argtypes = []
+        l.mi355_gemmlowp_noalloc_workspace_bytes.restype = C.c_size_t
         l.mi355_gemmlowp_destroy.argtypes = [vp]
         l.mi355_gemmlowp_destroy.restype = None
         l.mi355_gemmlowp_kernel_name.argtypes = [vp]
@@ -175,6 +178,9 @@ class Gemm:
 
     def run(self, A, D, bias_f32=None, stream=None):
         _check(lib().mi355_gemmlowp_run(self._h, ptr(A), ptr(bias_f32), ptr(D), stream))
+
+    def run_noalloc(self, A, D, bias_f32=None, stream=None):
+        _check(lib().mi355_gemmlowp_run_noalloc(self._h, ptr(A), ptr(bias_f32), ptr(D), stream))
 
     def close(self):
         if self._h:

@@ -13,6 +13,11 @@
 
 using namespace mi355;
 
+// Workspace of mi355_gemmlowp_run_noalloc: row sums of A, then (rows that are not dword aligned) the padded copy of A.
+// One array per GPU for the life of the process; every call on a GPU shares it.
+#define MI355_NOALLOC_SCRATCH_BYTES (8u << 20)
+static __device__ __align__(256) unsigned char scratch[MI355_NOALLOC_SCRATCH_BYTES];
+
 namespace
 {
 thread_local std::string g_err;
@@ -165,6 +170,8 @@ struct GemmCore
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
+    void   *ext_ws = nullptr; // set around a run that must not allocate: see run_dense
+    size_t  ext_ws_bytes = 0;
 
     int32_t a_off_eff() const { return (int32_t)((uint32_t)a_offset + (flip_a ? 128u : 0u)); }
     int32_t b_off_eff() const { return (int32_t)((uint32_t)b_offset + (flip_b ? 128u : 0u)); }
@@ -359,26 +366,44 @@ struct GemmCore
         const bool direct =
             path == MI355_PATH_SIMPLE || ((((uintptr_t)A | (uintptr_t)lda | (uintptr_t)a_bs) & 3) == 0);
         const bool need_rowvec = b_off_eff() != 0;
-        if (need_rowvec)
-            TRY(rowvec.ensure(sizeof(int32_t) * (size_t)M * batch));
+        // the two workspaces of a run: owned by the handle and grown on demand, or carved out of a buffer the caller of
+        // this function brings (ext_ws != nullptr: nothing is allocated, sizes beyond ext_ws_bytes are an error)
+        const size_t rv_bytes = need_rowvec ? ((sizeof(int32_t) * (size_t)M * batch + 255) & ~(size_t)255) : 0;
+        const size_t ap_bytes = direct ? 0 : (size_t)batch * M * Kp;
+        int32_t     *rv       = nullptr;
+        int8_t      *ap       = nullptr;
+        if (ext_ws != nullptr)
+        {
+            if (rv_bytes + ap_bytes > ext_ws_bytes)
+                return fail("this run needs %zu bytes of workspace (row sums %zu + padded copy of A %zu); the fixed "
+                            "workspace holds %zu",
+                            rv_bytes + ap_bytes, rv_bytes, ap_bytes, ext_ws_bytes);
+            rv = (int32_t *)ext_ws, ap = (int8_t *)ext_ws + rv_bytes;
+        }
+        else
+        {
+            if (need_rowvec)
+                TRY(rowvec.ensure(rv_bytes));
+            if (!direct)
+                TRY(Ap.ensure(ap_bytes));
+            rv = rowvec.as<int32_t>(), ap = Ap.as<int8_t>();
+        }
         if (!direct)
         {
             // rows not dword aligned: padded, sign-normalised copy (and the row sums in the same pass)
-            TRY(Ap.ensure((size_t)batch * M * Kp));
             for (int b = 0; b < batch; ++b)
-                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, Ap.as<int8_t>() + (size_t)b * M * Kp,
-                                         Kp, need_rowvec ? rowvec.as<int32_t>() + (size_t)b * M : nullptr, b_off_eff(),
-                                         s));
-            A = Ap.as<int8_t>(), lda = Kp, a_bs = (int64_t)M * Kp, k_valid = Kp, flip_in_loader = false;
+                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, ap + (size_t)b * M * Kp, Kp,
+                                         need_rowvec ? rv + (size_t)b * M : nullptr, b_off_eff(), s));
+            A = ap, lda = Kp, a_bs = (int64_t)M * Kp, k_valid = Kp, flip_in_loader = false;
         }
         else if (need_rowvec)
         {
             for (int b = 0; b < batch; ++b)
-                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, nullptr, Kp,
-                                         rowvec.as<int32_t>() + (size_t)b * M, b_off_eff(), s));
+                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, nullptr, Kp, rv + (size_t)b * M,
+                                         b_off_eff(), s));
         }
         if (need_rowvec)
-            g.epi.rowvec = rowvec.as<int32_t>();
+            g.epi.rowvec = rv;
         g.A = A, g.lda = lda, g.a_batch_stride = a_bs;
         g.Bp = Bp.as<int8_t>(), g.Kp = Kp, g.bp_batch_stride = b_shared ? 0 : (int64_t)Np * Kp;
         g.D = D, g.ldd = ldd, g.d_batch_stride = d_bs;
@@ -707,6 +732,54 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     else if (Ad != A || bfd != bias_f32)
         HIP_TRY(hipStreamSynchronize(s)); // staged inputs must be consumed before the caller may reuse them
     return 0;
+}
+
+// The address of this GPU's copy of the workspace array, asked once per device (with that device current)
+static int noalloc_scratch(void **out)
+{
+    static void *ptrs[64];
+    int          dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64)
+        return fail("device index %d out of range", dev);
+    void *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr)
+    {
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr)
+            return fail("hipGetSymbolAddress returned no address for the workspace");
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+    }
+    *out = p;
+    return 0;
+}
+
+size_t mi355_gemmlowp_noalloc_workspace_bytes(void)
+{
+    return MI355_NOALLOC_SCRATCH_BYTES;
+}
+
+int mi355_gemmlowp_run_noalloc(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream)
+{
+    if (!h || !A || !D)
+        return fail("null argument");
+    hipStream_t            s = (hipStream_t)stream;
+    GemmCore              &c = h->core;
+    const mi355_gemm_desc &d = h->d;
+    if (!c.prepared)
+        return fail("run before prepare");
+    if (bias_f32 && c.epi != EPI_F32)
+        return fail("float bias is only valid with the F32 epilogue");
+    if (d.dst_dtype == MI355_F16)
+        return fail("mi355_gemmlowp_run_noalloc does not write F16 destinations (they need a float matrix as workspace)");
+    if (!h->kindA.is_device(A) || !h->kindD.is_device(D) || (bias_f32 && !h->kindBiasF.is_device(bias_f32)))
+        return fail("mi355_gemmlowp_run_noalloc takes device memory only");
+    void *ws = nullptr;
+    TRY(noalloc_scratch(&ws));
+    c.ext_ws = ws, c.ext_ws_bytes = MI355_NOALLOC_SCRATCH_BYTES;
+    const int rc = c.run_dense((const int8_t *)A, d.lda, d.a_batch_stride, D, d.ldd, d.d_batch_stride, bias_f32, s);
+    c.ext_ws = nullptr, c.ext_ws_bytes = 0;
+    return rc;
 }
 
 void mi355_gemmlowp_destroy(mi355_gemm_handle *h)

@@ -168,6 +168,19 @@ int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, i
 /* Replaces CpuGemmLowpMatrixMultiplyCore::run (:647-811). bias_f32 (N floats, MI355_EPI_F32 only) may be NULL. */
 int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
 
+/* mi355_gemmlowp_run for callers that cannot allocate device memory while they run (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arguments and
+ * result as mi355_gemmlowp_run, with these differences: A, D and bias_f32 must be device memory; the run's workspace -
+ * the row sums of A (4 bytes per row and batch entry, rounded up to 256; needed when b_offset != 0 or B is unsigned)
+ * followed by the padded copy of A (batch * M * round_up(K, 128) bytes; needed when a row of A does not start on a
+ * 4-byte boundary) - lives in one fixed array of mi355_gemmlowp_noalloc_workspace_bytes() (8 MiB) that each GPU holds
+ * for the life of the process; a run that needs more is refused with an error, as is an F16 destination. The call
+ * allocates and frees nothing and only enqueues kernels on `stream`. Every call on a GPU uses that GPU's one array
+ * (nothing in it has to start at zero: the kernels overwrite what they read), so calls that overlap in time on one GPU
+ * - different streams, different handles - race; serialise them. The handle must be prepared. */
+int    mi355_gemmlowp_run_noalloc(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
+size_t mi355_gemmlowp_noalloc_workspace_bytes(void);
+
 void mi355_gemmlowp_destroy(mi355_gemm_handle *h);
 
 /* Name of the kernel variant the handle dispatches to, e.g. "mfma_256x128x64" (static string). */

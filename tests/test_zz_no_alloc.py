@@ -1,0 +1,88 @@
+"""mi355_gemmlowp_run_noalloc (the entry point that allocates nothing: its workspace is a fixed array on the device)
+against mi355_gemmlowp_run on the same handle and inputs, to the same bar: identical bytes. Two calls in a row, the
+second with a smaller input, so that what the first call left in the shared workspace is still there."""
+import numpy as np
+import pytest
+
+import oracle
+from computelibrary_amd import capi
+from gpu_util import announce, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(M, N, K, lda, a_dt, b_dt, b_off, seed):
+    """one handle, one input: (A on the device, handle, result of the allocating entry point, oracle result)"""
+    import torch
+    rng = np.random.default_rng(seed)
+    A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+    B = rng.integers(np.iinfo(b_dt).min, np.iinfo(b_dt).max + 1, size=(K, N)).astype(b_dt)
+    bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+    mult, shift = oracle.calculate_quantized_multipliers(1.0, [3e-4 * 128.0 / np.sqrt(K)], 1.0)
+    lo, hi = (-128, 127) if a_dt == np.int8 else (0, 255)
+    code = capi.S8 if a_dt == np.int8 else capi.U8
+    g = capi.Gemm(M, N, K, code, capi.S8 if b_dt == np.int8 else capi.U8, code, capi.EPI_FIXEDPOINT, -7, b_off,
+                  capi.requant(int(mult[0]), int(shift[0]), 5, lo, hi), lda=lda)
+    Ah = np.zeros((M, lda), dtype=a_dt)
+    Ah[:, :K] = A
+    Ad = to_dev(Ah)
+    keep = [to_dev(B), to_dev(bias)]
+    g.prepare(keep[0], keep[1])
+    D_ref = torch.zeros((M, N), dtype=torch.int8 if a_dt == np.int8 else torch.uint8, device="cuda")
+    g.run(Ad, D_ref)
+    torch.cuda.synchronize()
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -7, b_off, mult, shift, 5, lo, hi, a_dt)
+    return Ad, g, D_ref.cpu().numpy(), want, keep
+
+
+@pytest.mark.parametrize("lda_extra", [0, 3])  # rows 16-byte aligned (row sums only) / unaligned (row sums + copy of A)
+def test_noalloc_matches_the_allocating_entry_point_twice_in_a_row(lda_extra):
+    import torch
+    assert capi.lib().mi355_gemmlowp_noalloc_workspace_bytes() == 8 << 20
+    shapes = [(300, 200, 528), (70, 96, 272)]  # the second call is smaller than the first
+    for rep, (M, N, K) in enumerate(shapes):
+        announce("no-alloc", (M, N, K), "lda +", lda_extra, "call", rep)
+        Ad, g, ref, want, keep = _case(M, N, K, K + lda_extra, np.uint8, np.uint8, 9, 500 + rep)
+        np.testing.assert_array_equal(ref, want)
+        D = torch.full((M, N), 77, dtype=torch.uint8, device="cuda")
+        g.run_noalloc(Ad, D)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(D.cpu().numpy(), ref)
+        # and once more on the same handle: the workspace still holds this call's own values
+        D.fill_(0)
+        g.run_noalloc(Ad, D)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(D.cpu().numpy(), ref)
+        g.close()
+
+
+def test_noalloc_skinny_and_signed_paths():
+    import torch
+    for (M, N, K, a_dt, b_dt, b_off) in [(8, 256, 512, np.int8, np.int8, 11), (33, 130, 192, np.int8, np.int8, -4),
+                                          (16, 64, 128, np.int8, np.int8, 0)]:
+        announce("no-alloc", (M, N, K), a_dt.__name__, "b_off", b_off)
+        Ad, g, ref, want, keep = _case(M, N, K, K, a_dt, b_dt, b_off, 600 + M)
+        np.testing.assert_array_equal(ref, want)
+        D = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+        g.run_noalloc(Ad, D)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(D.cpu().numpy(), ref)
+        g.close()
+
+
+def test_noalloc_rejects_what_does_not_fit_and_host_memory():
+    import torch
+    # unaligned rows: the padded copy of A would need 5000 * 2048 bytes > 8 MiB
+    M, N, K = 5000, 32, 2045
+    g = capi.Gemm(M, N, K, capi.S8, capi.S8, capi.S32, capi.EPI_S32, 0, 3, lda=K)
+    Bd = torch.zeros((K, N), dtype=torch.int8, device="cuda")
+    g.prepare(Bd)
+    Ad = torch.zeros((M, K), dtype=torch.int8, device="cuda")
+    Dd = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    with pytest.raises(capi.Mi355Error, match="workspace"):
+        g.run_noalloc(Ad, Dd)
+    with pytest.raises(capi.Mi355Error, match="device memory"):
+        g.run_noalloc(np.zeros((M, K), np.int8), Dd)
+    g.run(Ad, Dd)  # the allocating entry point still takes it
+    torch.cuda.synchronize()
+    g.close()

@@ -208,6 +208,28 @@ def f32_dequant():
     np.savez_compressed(os.path.join(HERE, "gemmlowp_f32.npz"), **out)
 
 
+def f16_dequant():
+    """The reference's test oracle for the F16 output (tests/validation/fixtures/GEMMLowpFixture.h:908-920): the S32
+    result dequantised to half with scale a.scale*b.scale, and, when accumulating, added to the previous halfs as halfs.
+    Signed operands (tests/validation/NEON/GEMMLowp.cpp:598-621), with and without offsets and previous contents."""
+    rng = np.random.default_rng(116)
+    out = {}
+    scale = np.float32(np.float32(1.0 / 255) * np.float32(5.0 / 255))
+    cases = [(M, N, K, 0, 0) for (M, N, K, _, _) in SMALL_GEMMLOWP] + [(37, 53, 120, 0, 0), (5, 9, 1000, 0, 0),
+                                                                      (37, 53, 120, 3, -7), (27, 23, 31, 5, 13)]
+    for n, (M, N, K, ao, bo) in enumerate(cases):
+        A, B = rnd8(rng, (M, K), 1), rnd8(rng, (K, N), 1)
+        prev = rng.normal(0, 2, size=(M, N)).astype(np.float16)
+        t = oracle.ref_gemmlowp_core(A, B, ao, bo)
+        out["a%d" % n], out["b%d" % n], out["prev%d" % n] = A, B, prev
+        out["off%d" % n] = np.array([ao, bo], dtype=np.int32)
+        out["dst%d" % n] = oracle.ref_dequantize_s32_f16(t, float(scale)).view(np.uint16)
+        out["acc%d" % n] = oracle.ref_dequantize_s32_f16(t, float(scale), prev=prev).view(np.uint16)
+    out["count"] = np.array(len(cases))
+    out["scale"] = np.array(scale, dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "gemmlowp_f16.npz"), **out)
+
+
 IM2COL = [  # (batch, H, W, C, KH, KW, (sx, sy), (pl, pt, pr, pb), zero_point)
     (1, 5, 5, 3, 3, 3, (1, 1), (1, 1, 1, 1), 10), (2, 7, 6, 1, 3, 3, (2, 2), (0, 0, 0, 0), 0),
     (1, 6, 6, 64, 1, 1, (1, 1), (0, 0, 0, 0), -1), (1, 9, 8, 3, 5, 5, (1, 1), (2, 2, 2, 2), -1),
@@ -264,8 +286,9 @@ def conv():
 
 if __name__ == "__main__":
     assert oracle.ref_available(), "build oracle/_ref first (make -C oracle ref)"
-    for fn in (gemmlowp_s32, gemmlowp_batched, fused_fixedpoint, output_stage, output_stage_scale, requant_sweep,
-               quant_multiplier,
-               f32_dequant, im2col, conv):
+    every = (gemmlowp_s32, gemmlowp_batched, fused_fixedpoint, output_stage, output_stage_scale, requant_sweep,
+             quant_multiplier, f32_dequant, f16_dequant, im2col, conv)
+    # python tests/golden/make_fixtures.py [name ...]: only the named fixtures (all of them without arguments)
+    for fn in [f for f in every if not sys.argv[1:] or f.__name__ in sys.argv[1:]]:
         fn()
         print("wrote", fn.__name__)

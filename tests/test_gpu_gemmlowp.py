@@ -174,6 +174,25 @@ def test_f16_destination(device):
             assert 0.05 < (want == 0).mean() < 0.95 or M * N < 400
 
 
+def test_f16_fixture(golden):
+    """Halfs produced by the reference's own code (tests/golden/gemmlowp_f16.npz): with zero offsets the device result
+    has the same bits, with and without accumulation into previous halfs."""
+    g = golden("gemmlowp_f16.npz")
+    scale = float(g["scale"])
+    for n in range(int(g["count"])):
+        A, B, prev = g["a%d" % n], g["b%d" % n], g["prev%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        if ao or bo:
+            continue
+        for path in paths_for(A.shape[0]):
+            announce("f16 fixture", n, A.shape, B.shape, "path", path)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float16, 0, 0, scale=scale, path=path, device=True)
+            np.testing.assert_array_equal(got.view(np.uint16), g["dst%d" % n])
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float16, 0, 0, scale=scale, path=path, device=True, prev=prev,
+                              flags=capi.GEMM_ACCUMULATE)
+            np.testing.assert_array_equal(got.view(np.uint16), g["acc%d" % n])
+
+
 PIPELINED_CONFIGS = ["pp_256x128x128_s3", "pp_128x128x128_s3", "pp_128x64x128_s3", "pp_64x64x128_s3", "pp_64x64x128_s6",
                      "pp_128x64x256_s3"]
 

@@ -219,6 +219,37 @@ def test_f32_accumulate_and_double_clamp_against_numpy_float32():
     np.testing.assert_array_equal(oracle.gemmlowp_f32(A, B, bias, 0, 0, float(s)), acc.astype(np.float32) * s + bias)
 
 
+def _half_ulps(a_bits, b_bits):
+    def key(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+def test_f16_destination_fixture(golden):
+    """orc_gemmlowp_f16 against halfs the reference's own code produced (dequantization_layer<half, int32_t> and the half
+    arithmetic_operation behind tests/validation/fixtures/GEMMLowpFixture.h:908-920), committed as a fixture so the pin
+    holds without the reference checkout. Zero offsets: identical bits, with and without accumulation. Non-zero
+    offsets: the float underneath follows the NEON order of operations (two roundings), which crosses a half rounding
+    boundary now and then: never more than one half apart before the accumulation, equal almost everywhere."""
+    g = golden("gemmlowp_f16.npz")
+    scale = float(g["scale"])
+    seen_offsets = 0
+    for n in range(int(g["count"])):
+        A, B, prev = g["a%d" % n], g["b%d" % n], g["prev%d" % n]
+        ao, bo = (int(x) for x in g["off%d" % n])
+        got = oracle.gemmlowp_f16(A, B, None, ao, bo, scale).view(np.uint16)
+        acc = oracle.gemmlowp_f16(A, B, None, ao, bo, scale, prev=prev).view(np.uint16)
+        if ao == 0 and bo == 0:
+            np.testing.assert_array_equal(got, g["dst%d" % n])
+            np.testing.assert_array_equal(acc, g["acc%d" % n])
+        else:
+            seen_offsets += 1
+            assert _half_ulps(got, g["dst%d" % n]).max() <= 1
+            assert (got == g["dst%d" % n]).mean() > 0.99 and (acc == g["acc%d" % n]).mean() > 0.99
+    assert seen_offsets >= 2
+
+
 @pytest.mark.skipif(not oracle.ref_available(), reason="oracle/_ref not built (needs the reference checkout)")
 def test_fused_against_live_reference_config1_shape():
     """BASELINE config 1 at full size (256^3, QASYMM8, both zero-point conventions) through the reference's code."""

@@ -67,6 +67,143 @@ def time_launches(torch, fn, steps, warmup):
     return wall, ev0.elapsed_time(ev1) * 1e-3
 
 
+def time_graph(torch, fns, launches):
+    """The kernels' own duration with no host work inside the timed region: fns (called round-robin with the capture
+    stream) are captured into one HIP graph of about 200 launches, which is replayed until `launches` launches have
+    run, after one untimed replay. Returns seconds per launch."""
+    per_graph = max(len(fns), min(launches, 200) // len(fns) * len(fns))
+    replays = (launches + per_graph - 1) // per_graph
+    side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        cs = torch.cuda.current_stream().cuda_stream
+        for i in range(per_graph):
+            fns[i % len(fns)](cs)
+    graph.replay()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(replays):
+        graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    return ev0.elapsed_time(ev1) * 1e-3 / (per_graph * replays)
+
+
+def ceilings_lib():
+    """ctypes handle of the measurement-only kernels (computelibrary_amd/csrc/ceilings.hip), or None if not built"""
+    import ctypes as C
+    path = os.path.join(ROOT, "computelibrary_amd", "lib", "libmi355ceilings.so")
+    if not os.path.exists(path):
+        return None
+    l = C.CDLL(path)
+    vp, i64 = C.c_void_p, C.c_int64
+    l.mi355_ceiling_read.argtypes = [vp, i64, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp]
+    l.mi355_ceiling_mfma.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
+    l.mi355_ceiling_mfma_lds.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp]
+    l.mi355_ceiling_dma.argtypes = [vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]
+    l.mi355_ceiling_clock.argtypes = [i64, i64, vp, vp]
+    return l
+
+
+def shader_clock_during(torch, cl, work, span_us=2000.0, delay_us=300.0):
+    """MHz of the shader clock while work() (which enqueues a few ms of launches on the current stream) runs: a
+    one-wave kernel on a second stream counts shader-clock ticks over span_us of the 100 MHz real-time counter."""
+    ticks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    rc = cl.mi355_ceiling_clock(int(delay_us * 100), int(span_us * 100), ticks.data_ptr(), side.cuda_stream)
+    assert rc == 0, rc
+    work()
+    torch.cuda.synchronize()
+    t = ticks.cpu().numpy()
+    return float(t[0]) / max(float(t[1]), 1.0) * 100.0
+
+
+def run_ceilings(torch, args):
+    """What the machine reaches on the parts the kernels are made of (see ceilings.hip); one JSON line."""
+    cl = ceilings_lib()
+    assert cl is not None, "libmi355ceilings.so is missing: run `python -m computelibrary_amd.build`"
+    out = {"ceilings": True, "launches": args.steps}
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    KIB = 11008 * 4096 // 1024  # the config-3 B matrix: 44032 KiB
+    ROT = 9
+    bufs = [torch.randint(-128, 128, (KIB * 1024,), dtype=torch.int8, device="cuda", generator=gen) for _ in range(ROT)]
+    sink = torch.zeros(256 * 768, dtype=torch.int32, device="cuda")
+    ticks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    steps = max(args.steps, 10 * ROT) // ROT * ROT
+
+    def read_fn(buf, pattern, grid, waves, unroll):
+        def f(cs):
+            rc = cl.mi355_ceiling_read(buf.data_ptr(), KIB, pattern, grid, waves, unroll, sink.data_ptr(), cs)
+            assert rc == 0, rc
+        return f
+
+    out["read_45MB"] = []
+    for (pattern, grid, waves, unroll) in [(0, 688, 8, 8), (0, 1376, 4, 8), (0, 2752, 4, 4), (1, 256, 8, 8), (1, 512, 8, 8),
+                                           (1, 512, 8, 4), (1, 1024, 8, 4), (1, 2048, 4, 4), (1, 688, 8, 8)]:
+        hbm = time_graph(torch, [read_fn(b, pattern, grid, waves, unroll) for b in bufs], steps)
+        cache = time_graph(torch, [read_fn(bufs[0], pattern, grid, waves, unroll)], steps)
+        out["read_45MB"].append({
+            "pattern": "chunk per workgroup" if pattern == 0 else "grid-wide window", "grid": grid, "waves": waves,
+            "unroll": unroll, "hbm_us": round(hbm * 1e6, 3), "hbm_GBs": round(KIB * 1024 / hbm / 1e9, 1),
+            "cache_resident_us": round(cache * 1e6, 3), "cache_resident_GBs": round(KIB * 1024 / cache / 1e9, 1)})
+
+    # matrix instructions of config 2 (2048 x 4096 x 4096): 1024 16x16x64 instructions per wave on 256 x 8 waves
+    ops = 2.0 * 2048 * 4096 * 4096
+    rnd = bufs[0][:16 << 20]
+    zero = torch.zeros(16 << 20, dtype=torch.int8, device="cuda")
+    out["mfma_cfg2_instruction_count"] = []
+
+    def timed(name, fn, data):
+        s = time_graph(torch, [fn], args.steps)
+        torch.cuda.synchronize()
+        t = ticks.cpu().numpy()
+        out["mfma_cfg2_instruction_count"].append({
+            "what": name, "operands": data, "us": round(s * 1e6, 3), "TOPS": round(ops / s / 1e12, 1),
+            "frac_of_5.0_POPs": round(ops / s / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "loop_clocks": int(t[0]), "shader_MHz_in_loop": round(float(t[0]) / max(float(t[1]), 1.0) * 100.0, 1)})
+
+    for data, src in (("random", rnd), ("zero", zero)):
+        for shape in (16, 32):
+            timed("registers only, v_mfma_i32_%dx%dx%d_i8" % (shape, shape, 64 if shape == 16 else 32),
+                  lambda cs, shape=shape, src=src: cl.mi355_ceiling_mfma(src.data_ptr(), shape, 256, 1024, sink.data_ptr(),
+                                                                         ticks.data_ptr(), cs), data)
+        timed("operands read from LDS (64x64 wave tiles), 16x16x64",
+              lambda cs, src=src: cl.mi355_ceiling_mfma_lds(src.data_ptr(), 256, 32, sink.data_ptr(), ticks.data_ptr(), cs),
+              data)
+    A = bufs[1][:2048 * 4096]
+    B = bufs[2][:4096 * 4096]
+    out["dma_stream_cfg2"] = []
+    for waves in (4, 12):
+        s = time_graph(torch, [lambda cs, waves=waves: cl.mi355_ceiling_dma(A.data_ptr(), B.data_ptr(), 4096, 32, waves,
+                                                                            sink.data_ptr(), ticks.data_ptr(), cs)],
+                       args.steps)
+        torch.cuda.synchronize()
+        t = ticks.cpu().numpy()
+        out["dma_stream_cfg2"].append({"issuing_waves": waves, "us": round(s * 1e6, 3), "bytes_to_lds": 256 * 32 * 49152,
+                                       "TBs": round(256 * 32 * 49152 / s / 1e12, 2), "loop_clocks": int(t[0]),
+                                       "bytes_per_clock_per_cu": round(32 * 49152 / max(float(t[0]), 1.0), 1)})
+    # the vendor library's int8 GEMM on the config-2 shape (int32 output, no epilogue)
+    try:
+        Am = A.view(2048, 4096)
+        Bm = B.view(4096, 4096)
+        for _ in range(50):
+            torch._int_mm(Am, Bm)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(args.steps):
+            torch._int_mm(Am, Bm)
+        ev1.record()
+        torch.cuda.synchronize()
+        s = ev0.elapsed_time(ev1) * 1e-3 / args.steps
+        out["vendor_int8_gemm_cfg2"] = {"what": "torch._int_mm 2048x4096x4096 -> s32", "us": round(s * 1e6, 3),
+                                        "TOPS": round(ops / s / 1e12, 1)}
+    except Exception as e:  # not every build has it
+        out["vendor_int8_gemm_cfg2"] = {"error": str(e)[:200]}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,6 +217,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only run the measurement-only kernels (read stream, matrix instructions, LDS, direct-to-LDS "
+                         "stream, vendor int8 GEMM) and print their figures as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -103,6 +243,10 @@ def main():
                           "launches": max(args.steps, 1)}))
         return
 
+    if args.ceilings:
+        run_ceilings(torch, args)
+        return
+
     M, N, K = 2048, 4096, 4096
     A, B, bias, mult, shift = synth_config2(M, N, K)
     rq = capi.requant(0, 0, -5, -128, 127, per_channel=True)
@@ -118,25 +262,17 @@ def main():
     wall, evt = time_launches(torch, lambda: g.run(Ad, Dd, None, stream), args.steps, args.warmup)
     ops = 2.0 * M * N * K
     tops = ops * args.steps / wall / 1e12
-    # The kernel's own duration, with no host work inside the timed region: the launches captured once into a HIP
-    # graph (GL per replay) and replayed until K launches have run, after one untimed replay.
-    GL = min(args.steps, 200)
-    replays = (args.steps + GL - 1) // GL
-    side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        cs = torch.cuda.current_stream().cuda_stream
-        for _ in range(GL):
-            g.run(Ad, Dd, None, cs)
-    graph.replay()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev0.record()
-    for _ in range(replays):
-        graph.replay()
-    ev1.record()
-    torch.cuda.synchronize()
-    kern_s = ev0.elapsed_time(ev1) * 1e-3 / (GL * replays)
+    # The kernel's own duration, with no host work inside the timed region: graph replays of the same launch
+    kern_s = time_graph(torch, [lambda cs: g.run(Ad, Dd, None, cs)], args.steps)
     achieved = ops / kern_s / 1e12
+    # shader clock while this kernel runs back to back (a one-wave probe on a second stream counts clock ticks over
+    # 2 ms of real time), and the matrix peak at that clock: CUs x 4 SIMDs x 1024 multiply-accumulates x 2
+    clock_mhz, cl = None, ceilings_lib()
+    if cl is not None:
+        def burst():
+            for _ in range(300):
+                g.run(Ad, Dd, None, stream)
+        clock_mhz = shader_clock_during(torch, cl, burst)
 
     out = {
         "metric": "int8 GEMMLowp TOPS & %MFMA peak at 2048x4096x4096; HBM GB/s at M=8",
@@ -149,6 +285,11 @@ def main():
                      "frac": round(achieved / INT8_DENSE_PEAK_TOPS, 4), "traffic": CFG2_MEASURED_TRAFFIC_BYTES,
                      "kernel_us": round(kern_s * 1e6, 3), "eager_us": round(evt / args.steps * 1e6, 3)},
     }
+    if clock_mhz:
+        cus = capi.device_info()[1]
+        peak_at_clock = clock_mhz * 1e6 * cus * 4 * 1024 * 2 / 1e12
+        out["roofline"].update({"shader_clock_MHz": round(clock_mhz, 1), "peak_at_measured_clock": round(peak_at_clock, 1),
+                                "frac_of_peak_at_measured_clock": round(achieved / peak_at_clock, 4)})
 
     if not args.no_cpu:
         import oracle
@@ -169,98 +310,135 @@ def main():
         fg.close()
 
     if not args.no_secondary:
+        check = not args.no_cpu  # every timed output is compared with the CPU restatement of the same arithmetic
+        if check:
+            import oracle
         M3, N3, K3 = 8, 11008, 4096
         A3, B3, bias3, mult3, shift3 = synth_config2(M3, N3, K3, seed=3)
         A3d = torch.from_numpy(A3).cuda()
         D3d = torch.zeros((M3, N3), dtype=torch.int8, device="cuda")
         b3, m3, s3 = torch.from_numpy(bias3).cuda(), torch.from_numpy(mult3).cuda(), torch.from_numpy(shift3).cuda()
-        handles = []
-        for r in range(9):  # 9 x 45 MB of packed B > 256 MB Infinity Cache
-            h = capi.Gemm(M3, N3, K3, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
-            h.prepare(torch.from_numpy(np.roll(B3, r, axis=1) if r else B3).cuda(), b3, m3, s3, stream)
-            handles.append(h)
-        torch.cuda.synchronize()
-        bytes3 = N3 * K3 + M3 * K3 + M3 * N3 + 3 * 4 * N3
-        state = {"i": 0}
+        ROT = 9  # 9 x 45 MB of packed B > 256 MB Infinity Cache
+        fg3 = [oracle.FastGemm(np.roll(B3, r, axis=1) if r else B3) for r in (0, ROT - 1)] if check else None
 
-        def rotated():
-            handles[state["i"] % len(handles)].run(A3d, D3d, None, stream)
-            state["i"] += 1
+        def decode_leg(Mb, Ab_host):
+            """M = Mb rows against the config-3 weights, B rotated over ROT packed copies so it is read from HBM;
+            eager launches and graph replays; the last launch's output compared with the CPU port."""
+            Ab = torch.from_numpy(Ab_host).cuda()
+            Db = torch.zeros((Mb, N3), dtype=torch.int8, device="cuda")
+            hs = []
+            for r in range(ROT):
+                h = capi.Gemm(Mb, N3, K3, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
+                h.prepare(torch.from_numpy(np.roll(B3, r, axis=1) if r else B3).cuda(), b3, m3, s3, stream)
+                hs.append(h)
+            torch.cuda.synchronize()
+            st = {"i": 0}
 
-        steps3 = max(args.steps, 90)
-        _, evt_rot = time_launches(torch, rotated, steps3, args.warmup)
-        _, evt_one = time_launches(torch, lambda: handles[0].run(A3d, D3d, None, stream), steps3, args.warmup)
+            def rotated():
+                hs[st["i"] % ROT].run(Ab, Db, None, stream)
+                st["i"] += 1
+
+            steps3 = max(args.steps, 10 * ROT) // ROT * ROT
+            _, evt_rot = time_launches(torch, rotated, steps3, args.warmup // ROT * ROT)
+            graph_s = time_graph(torch, [(lambda cs, h=h: h.run(Ab, Db, None, cs)) for h in hs], steps3)
+            # the last launch of either loop used the last handle: bias/multipliers are not rolled, only B's columns
+            ok = None
+            if check:
+                torch.cuda.synchronize()
+                ok = bool(np.array_equal(Db.cpu().numpy(),
+                                         fg3[1].run(Ab_host, bias3, -3, 0, mult3, shift3, -5, -128, 127, np.int8)))
+            _, evt_one = time_launches(torch, lambda: hs[0].run(Ab, Db, None, stream), steps3, args.warmup)
+            if check:
+                torch.cuda.synchronize()
+                ok = ok and bool(np.array_equal(Db.cpu().numpy(),
+                                                fg3[0].run(Ab_host, bias3, -3, 0, mult3, shift3, -5, -128, 127, np.int8)))
+            name = hs[0].kernel_name
+            for h in hs:
+                h.close()
+            bytes_b = N3 * K3 + Mb * K3 + Mb * N3 + 3 * 4 * N3
+            return name, bytes_b, evt_rot / steps3, graph_s, evt_one / steps3, ok
+
+        name3, bytes3, eager3, graph3, one3, ok3 = decode_leg(M3, A3)
         out["secondary"] = {"skinny_m8": {
-            "workload": "M=8 N=11008 K=4096 s8 x per-channel s8 -> s8", "kernel": handles[0].kernel_name,
-            "bound": "hbm", "bytes": bytes3, "kernel_us": round(evt_rot / steps3 * 1e6, 3),
-            "achieved_GBs": round(bytes3 / (evt_rot / steps3) / 1e9, 1), "peak_GBs": HBM_PEAK_GBS,
-            "frac": round(bytes3 / (evt_rot / steps3) / 1e9 / HBM_PEAK_GBS, 4),
-            "cache_resident_GBs": round(bytes3 / (evt_one / steps3) / 1e9, 1),
-            "note": "B rotated over 9 packed copies (405 MB) so reads come from HBM"}}
-        for h in handles:
-            h.close()
+            "workload": "M=8 N=11008 K=4096 s8 x per-channel s8 -> s8", "kernel": name3,
+            "bound": "hbm", "bytes": bytes3, "kernel_us": round(graph3 * 1e6, 3), "eager_us": round(eager3 * 1e6, 3),
+            "achieved_GBs": round(bytes3 / graph3 / 1e9, 1), "peak_GBs": HBM_PEAK_GBS,
+            "frac": round(bytes3 / graph3 / 1e9 / HBM_PEAK_GBS, 4),
+            "eager_GBs": round(bytes3 / eager3 / 1e9, 1), "cache_resident_GBs": round(bytes3 / one3 / 1e9, 1),
+            "bit_exact_vs_cpu": ok3,
+            "note": "B rotated over 9 packed copies (405 MB) so reads come from HBM; kernel_us from graph replays "
+                    "of the 9 rotating launches, eager_us from back-to-back host launches"}}
 
         # the same weights with larger decode batches (not BASELINE configurations; B rotated the same way)
         out["secondary"]["decode_batches"] = {}
         for Mb in (16, 32, 64):
-            Ab = torch.from_numpy(np.random.default_rng(30 + Mb).integers(-128, 128, size=(Mb, K3), dtype=np.int8)).cuda()
-            Db = torch.zeros((Mb, N3), dtype=torch.int8, device="cuda")
-            hb = []
-            for r in range(9):
-                h = capi.Gemm(Mb, N3, K3, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
-                h.prepare(torch.from_numpy(np.roll(B3, r, axis=1) if r else B3).cuda(), b3, m3, s3, stream)
-                hb.append(h)
-            torch.cuda.synchronize()
-            st = {"i": 0}
-
-            def rotated_b():
-                hb[st["i"] % len(hb)].run(Ab, Db, None, stream)
-                st["i"] += 1
-
-            _, evt_b = time_launches(torch, rotated_b, steps3, args.warmup)
-            bytes_b = N3 * K3 + Mb * K3 + Mb * N3 + 3 * 4 * N3
+            Abh = np.random.default_rng(30 + Mb).integers(-128, 128, size=(Mb, K3), dtype=np.int8)
+            nm, by, eg, gr, _, okb = decode_leg(Mb, Abh)
             out["secondary"]["decode_batches"]["m%d" % Mb] = {
-                "kernel": hb[0].kernel_name, "kernel_us": round(evt_b / steps3 * 1e6, 3),
-                "achieved_GBs": round(bytes_b / (evt_b / steps3) / 1e9, 1),
-                "TOPS": round(2.0 * Mb * N3 * K3 / (evt_b / steps3) / 1e12, 1)}
-            for h in hb:
-                h.close()
+                "kernel": nm, "kernel_us": round(gr * 1e6, 3), "eager_us": round(eg * 1e6, 3),
+                "achieved_GBs": round(by / gr / 1e9, 1), "TOPS": round(2.0 * Mb * N3 * K3 / gr / 1e12, 1),
+                "bit_exact_vs_cpu": okb}
+        if check:
+            for f in fg3:
+                f.close()
 
         # config 4: NHWC 3x3 convolution as an implicit GEMM (M = 32*56*56, N = 64, K = 576), near the roofline ridge
         rng = np.random.default_rng(4)
-        src = torch.from_numpy(rng.integers(-128, 128, size=(32, 56, 56, 64), dtype=np.int8)).cuda()
-        wts = torch.from_numpy(np.clip(np.rint(rng.normal(0.0, 24.0, size=(64, 3, 3, 64))), -127, 127).astype(np.int8)).cuda()
+        src_h = rng.integers(-128, 128, size=(32, 56, 56, 64), dtype=np.int8)
+        wts_h = np.clip(np.rint(rng.normal(0.0, 24.0, size=(64, 3, 3, 64))), -127, 127).astype(np.int8)
+        src, wts = torch.from_numpy(src_h).cuda(), torch.from_numpy(wts_h).cuda()
         m4, s4 = quantized_multipliers(rng.uniform(1e-4, 1e-3, size=64).astype(np.float32))
-        b4 = torch.from_numpy(np.rint(rng.normal(0.0, 500.0, size=64)).astype(np.int32)).cuda()
+        b4_h = np.rint(rng.normal(0.0, 500.0, size=64)).astype(np.int32)
+        b4 = torch.from_numpy(b4_h).cuda()
         cv = capi.Conv(capi.conv_desc(32, 56, 56, 64, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.S8,
                                       1, 0, -1, rq, 0))
         dst4 = torch.zeros((32, 56, 56, 64), dtype=torch.int8, device="cuda")
         cv.prepare(wts, b4, torch.from_numpy(m4).cuda(), torch.from_numpy(s4).cuda(), stream)
         _, evt4 = time_launches(torch, lambda: cv.run(src, dst4, stream), args.steps, args.warmup)
+        k4 = time_graph(torch, [lambda cs: cv.run(src, dst4, cs)], args.steps)
+        ok4 = None
+        if check:
+            torch.cuda.synchronize()
+            fg = oracle.FastGemm(oracle.weights_reshape(wts_h))
+            want4 = fg.run(oracle.im2col_nhwc(src_h, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), -1), b4_h, 1, 0, m4, s4, -5,
+                           -128, 127, np.int8)
+            fg.close()
+            ok4 = bool(np.array_equal(dst4.cpu().numpy().reshape(-1, 64), want4))
         ops4, bytes4 = 2.0 * 32 * 56 * 56 * 64 * 576, 2 * 32 * 56 * 56 * 64 + 64 * 576 + 3 * 4 * 64
         out["secondary"]["conv_cfg4"] = {
             "workload": "NHWC s8 [32,56,56,64] * 3x3x64x64 per-channel, s1 p1 -> s8", "kernel": cv.kernel_name,
-            "kernel_us": round(evt4 / args.steps * 1e6, 3), "TOPS": round(ops4 / (evt4 / args.steps) / 1e12, 1),
-            "frac_mfma": round(ops4 / (evt4 / args.steps) / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
-            "GBs": round(bytes4 / (evt4 / args.steps) / 1e9, 1),
-            "frac_hbm": round(bytes4 / (evt4 / args.steps) / 1e9 / HBM_PEAK_GBS, 4)}
+            "kernel_us": round(k4 * 1e6, 3), "eager_us": round(evt4 / args.steps * 1e6, 3),
+            "TOPS": round(ops4 / k4 / 1e12, 1), "frac_mfma": round(ops4 / k4 / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "GBs": round(bytes4 / k4 / 1e9, 1), "frac_hbm": round(bytes4 / k4 / 1e9 / HBM_PEAK_GBS, 4),
+            "bit_exact_vs_cpu": ok4}
         cv.close()
 
         # config 5: 16 x (1024 x 1000) * (1000 x 1024) s8 -> f32 dequantised, store-bound
-        A5 = torch.from_numpy(rng.integers(-128, 128, size=(16, 1024, 1000), dtype=np.int8)).cuda()
-        B5 = torch.from_numpy(rng.integers(-128, 128, size=(16, 1000, 1024), dtype=np.int8)).cuda()
+        A5_h = rng.integers(-128, 128, size=(16, 1024, 1000), dtype=np.int8)
+        B5_h = rng.integers(-128, 128, size=(16, 1000, 1024), dtype=np.int8)
+        A5, B5 = torch.from_numpy(A5_h).cuda(), torch.from_numpy(B5_h).cuda()
         D5 = torch.zeros((16, 1024, 1024), dtype=torch.float32, device="cuda")
-        g5 = capi.Gemm(1024, 1024, 1000, capi.S8, capi.S8, capi.F32, capi.EPI_F32, 0, 0, None,
-                       float(np.float32(0.02) * np.float32(0.005)), batch=16, b_batched=True)
+        scale5 = np.float32(0.02) * np.float32(0.005)
+        g5 = capi.Gemm(1024, 1024, 1000, capi.S8, capi.S8, capi.F32, capi.EPI_F32, 0, 0, None, float(scale5), batch=16,
+                       b_batched=True)
         g5.prepare(B5, None, None, None, stream)
         _, evt5 = time_launches(torch, lambda: g5.run(A5, D5, None, stream), args.steps, args.warmup)
+        k5 = time_graph(torch, [lambda cs: g5.run(A5, D5, None, cs)], args.steps)
+        ok5 = None
+        if check:
+            # |acc| < 2^24: the double-precision product is the exact integer, its float conversion is exact and the
+            # multiplication by the scale is the only rounding (the scalar oracle agrees; tests/ holds that check)
+            torch.cuda.synchronize()
+            got5 = D5.cpu().numpy()
+            ok5 = all(np.array_equal((A5_h[z].astype(np.float64) @ B5_h[z].astype(np.float64)).astype(np.float32) * scale5,
+                                     got5[z]) for z in range(16))
         ops5, bytes5 = 2.0 * 16 * 1024 * 1024 * 1000, 16 * (2 * 1024 * 1000 + 4 * 1024 * 1024)
         out["secondary"]["batched_f32_cfg5"] = {
             "workload": "16 x (1024x1000)*(1000x1024) s8 -> f32 dequantised", "kernel": g5.kernel_name,
-            "kernel_us": round(evt5 / args.steps * 1e6, 3), "TOPS": round(ops5 / (evt5 / args.steps) / 1e12, 1),
-            "frac_mfma": round(ops5 / (evt5 / args.steps) / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
-            "GBs": round(bytes5 / (evt5 / args.steps) / 1e9, 1),
-            "frac_hbm": round(bytes5 / (evt5 / args.steps) / 1e9 / HBM_PEAK_GBS, 4)}
+            "kernel_us": round(k5 * 1e6, 3), "eager_us": round(evt5 / args.steps * 1e6, 3),
+            "TOPS": round(ops5 / k5 / 1e12, 1), "frac_mfma": round(ops5 / k5 / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "GBs": round(bytes5 / k5 / 1e9, 1), "frac_hbm": round(bytes5 / k5 / 1e9 / HBM_PEAK_GBS, 4),
+            "bit_exact_vs_cpu": bool(ok5) if ok5 is not None else None}
         g5.close()
 
     g.close()

@@ -165,8 +165,9 @@ struct GemmCore
     int     Kp = 0, Np = 0;
     bool    b_shared = true; // one B for all batches
     bool    has_bias = false, has_pc = false, prepared = false;
+    bool    pt_vectors = false; // streaming path, per-tensor requantisation: mult / shift hold the scalars, replicated
     std::string kname;
-    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp;
+    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros;
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -180,7 +181,7 @@ struct GemmCore
     void release()
     {
         Bp.release(), Bs.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
-        shift.release(), bias.release(), Ap.release(), fill.release(), qp.release();
+        shift.release(), bias.release(), Ap.release(), fill.release(), qp.release(), zeros.release();
     }
 
     int choose_kernel()
@@ -292,6 +293,12 @@ struct GemmCore
         }
         TRY(fill.ensure(16));
         HIP_TRY(fill_i32_launch(fill.as<int32_t>(), (int32_t)(0x01010101u * fill_byte), 4, s));
+        if (path == MI355_PATH_SKINNY)
+        {
+            // the streaming kernel fetches its per-row vector without asking whether there is one
+            TRY(zeros.ensure(sizeof(int32_t) * SKINNY_MAX_M));
+            HIP_TRY(fill_i32_launch(zeros.as<int32_t>(), 0, SKINNY_MAX_M, s));
+        }
         TRY(refresh_colvec(s));
         TRY(refresh_qparams(s));
         prepared = true;
@@ -314,6 +321,16 @@ struct GemmCore
     int refresh_qparams(hipStream_t s)
     {
         qp_on = false;
+        if (path == MI355_PATH_SKINNY && epi == EPI_FIXEDPOINT && !has_pc)
+        {
+            // the streaming kernel always reads per-column vectors (a fetch behind a condition would cost it the exact
+            // count of its loads in flight): per-tensor constants are replicated
+            TRY(mult.ensure(sizeof(int32_t) * (size_t)Np));
+            TRY(shift.ensure(sizeof(int32_t) * (size_t)Np));
+            HIP_TRY(fill_i32_launch(mult.as<int32_t>(), rq.multiplier, Np, s));
+            HIP_TRY(fill_i32_launch(shift.as<int32_t>(), rq.shift, Np, s));
+            pt_vectors = true;
+        }
         if (epi != EPI_FIXEDPOINT || rq.stage != MI355_STAGE_FIXEDPOINT)
             return 0;
         TRY(qp.ensure(sizeof(int32_t) * ((size_t)QP_COUNT * Np + 4)));
@@ -332,8 +349,8 @@ struct GemmCore
         p.qp_stride           = Np;
         p.colvec              = colvec.as<int32_t>();
         p.rowvec              = nullptr;
-        p.mult                = has_pc ? mult.as<int32_t>() : nullptr;
-        p.shift               = has_pc ? shift.as<int32_t>() : nullptr;
+        p.mult                = (has_pc || pt_vectors) ? mult.as<int32_t>() : nullptr;
+        p.shift               = (has_pc || pt_vectors) ? shift.as<int32_t>() : nullptr;
         p.bias_f32            = bias_f32;
         p.colvec_batch_stride = b_shared ? 0 : Np;
         p.rowvec_batch_stride = M;
@@ -404,6 +421,8 @@ struct GemmCore
         }
         if (need_rowvec)
             g.epi.rowvec = rv;
+        else if (path == MI355_PATH_SKINNY)
+            g.epi.rowvec = zeros.as<int32_t>();
         g.A = A, g.lda = lda, g.a_batch_stride = a_bs;
         g.Bp = Bp.as<int8_t>(), g.Kp = Kp, g.bp_batch_stride = b_shared ? 0 : (int64_t)Np * Kp;
         g.D = D, g.ldd = ldd, g.d_batch_stride = d_bs;

@@ -1,0 +1,294 @@
+// Measurement-only kernels: what the machine reaches on the parts a GEMM kernel is made of, at the shapes the library's
+// kernels use them. Built into its own shared library (libmi355ceilings.so) that bench.py --ceilings loads; the product
+// library does not link this file and nothing here is on the hot path.
+//
+//   mi355_ceiling_read        one streaming pass over a buffer (the skinny GEMM's B stream, without any arithmetic)
+//   mi355_ceiling_mfma        int8 matrix instructions out of registers only (no LDS, no global traffic)
+//   mi355_ceiling_mfma_lds    the same instruction count with every operand read from LDS first (64 x 64 wave tiles)
+//   mi355_ceiling_dma         the pipelined GEMM's global -> LDS stream alone (direct-to-LDS loads, 3-slot ring)
+//   mi355_ceiling_clock       shader clock while other work runs: shader-clock ticks over a span of real time
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace
+{
+// PATTERN 0: workgroup b owns the contiguous chunk b of the buffer and its waves split that chunk into contiguous
+// slices (what a kernel with one workgroup per group of output columns does). PATTERN 1: the whole grid reads one
+// contiguous window per iteration (wave w of the grid takes block it * waves + w), the DRAM-friendliest order.
+template <int PATTERN, int UNROLL>
+__global__ __launch_bounds__(512) void read_kernel(const v4i *__restrict__ src, int64_t kib, int *sink)
+{
+    const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int64_t waves = (int64_t)gridDim.x * nw, gw = (int64_t)blockIdx.x * nw + wave;
+    v4i           acc = {0, 0, 0, 0};
+    if (PATTERN == 0)
+    {
+        const int64_t per = kib / waves; // 1 KiB blocks per wave (the host passes a multiple)
+        const v4i    *p   = src + gw * per * 64 + lane;
+        for (int64_t i = 0; i + UNROLL <= per; i += UNROLL)
+        {
+            v4i t[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+                t[u] = __builtin_nontemporal_load(p + (i + u) * 64);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+                acc += t[u];
+        }
+    }
+    else
+    {
+        for (int64_t blk = gw * UNROLL; blk + UNROLL <= kib; blk += waves * UNROLL)
+        {
+            v4i t[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+                t[u] = __builtin_nontemporal_load(src + (blk + u) * 64 + lane);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+                acc += t[u];
+        }
+    }
+    if (acc[0] + acc[1] + acc[2] + acc[3] == 0x12345678)
+        sink[0] = 1;
+}
+
+// SHAPE 16: v_mfma_i32_16x16x64_i8, SHAPE 32: v_mfma_i32_32x32x32_i8 (the same multiply-accumulates per instruction
+// pair). Every wave issues `mfma16` instructions' worth of work (counted in 16x16x64 units) on operands it read once.
+template <int SHAPE>
+__global__ __launch_bounds__(512) void mfma_kernel(const v4i *__restrict__ src, int mfma16, int *sink, int64_t *ticks)
+{
+    const int tid = blockIdx.x * blockDim.x + threadIdx.x;
+    v4i       a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+    {
+        a[i] = src[(tid * 16 + i) & 0xFFFFF];
+        b[i] = src[(tid * 16 + 8 + i) & 0xFFFFF];
+    }
+    const int64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    int           s  = 0;
+    if (SHAPE == 32)
+    {
+        v16i acc[4];
+        for (int i = 0; i < 4; ++i)
+            for (int r = 0; r < 16; ++r)
+                acc[i][r] = 0;
+        for (int it = 0; it < mfma16 / 32; ++it)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                acc[i & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 7], b[(i * 3) & 7], acc[i & 3], 0, 0, 0);
+        for (int i = 0; i < 4; ++i)
+            for (int r = 0; r < 16; ++r)
+                s += acc[i][r];
+    }
+    else
+    {
+        v4i acc[8];
+        for (int i = 0; i < 8; ++i)
+            acc[i] = (v4i){0, 0, 0, 0};
+        for (int it = 0; it < mfma16 / 32; ++it)
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                acc[i & 7] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i & 7], b[(i * 3) & 7], acc[i & 7], 0, 0, 0);
+        for (int i = 0; i < 8; ++i)
+            for (int r = 0; r < 4; ++r)
+                s += acc[i][r];
+    }
+    const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    sink[tid] = s;
+    if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
+        ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+}
+
+// 8 waves per workgroup; per K step of 128 every wave reads the operands of a 64 x 64 wave tile (16 x ds_read_b128)
+// from a 48 KiB stage of random bytes and issues 32 matrix instructions; one barrier per step.
+__global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ src, int steps, int *sink, int64_t *ticks)
+{
+    extern __shared__ __attribute__((aligned(1024))) char smem[]; // 3 x 48 KiB
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 3 * 49152 / 16; i += blockDim.x)
+        ((v4i *)smem)[i] = src[(blockIdx.x * 9216 + i) & 0xFFFFF];
+    __syncthreads();
+    v4i acc[16];
+    for (int i = 0; i < 16; ++i)
+        acc[i] = (v4i){0, 0, 0, 0};
+    const int64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    for (int kt = 0; kt < steps; ++kt)
+    {
+        // rows of 128 bytes; lane -> row lane % 16 of an operand block, 16-byte column (kk * 4 + lane / 16) ^ (row & 7):
+        // conflict free. A blocks: wave's 4 of the 16 A row blocks, B blocks: 4 of the 8 B row blocks
+        const char *s = smem + (kt % 3) * 49152;
+        v4i         fa[2][4], fb[2][4];
+        const int   row = lane & 15, lh = lane >> 4;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+            {
+                const int ra = ((wave >> 1) * 4 + f) * 16 + row, rb = 256 + ((wave & 1) * 4 + f) * 16 + row;
+                fa[kk][f]    = *(const v4i *)(s + ra * 128 + (((kk * 4 + lh) ^ (ra & 7)) << 4));
+                fb[kk][f]    = *(const v4i *)(s + rb * 128 + (((kk * 4 + lh) ^ (rb & 7)) << 4));
+            }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i * 4 + j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[kk][j], fa[kk][i], acc[i * 4 + j], 0, 0, 0);
+        __syncthreads();
+    }
+    const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    int           sum = 0;
+    for (int i = 0; i < 16; ++i)
+        sum += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+    if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
+        ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+}
+
+__device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+}
+
+// The 256 x 128 x 128 tile's stream: workgroup (tm, tn) of an 8 x 32 tile grid (XCD-major order as in the GEMM) moves 48
+// units of 1 KiB per K step (32 of its A panel, 16 of its B panel) into a 3-slot ring with `blockDim.x / 64` issuing
+// waves, two steps in flight, nothing reads the LDS.
+__global__ __launch_bounds__(768) void dma_kernel(const char *A, const char *B, int64_t ld, int steps, int tiles_n, int *sink,
+                                                  int64_t *ticks)
+{
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const int      lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
+    const int      l    = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int      tm = (l / (4 * tiles_n)) * 4 + (l % (4 * tiles_n)) % 4, tn = (l % (4 * tiles_n)) / 4;
+    const char    *a0 = A + (int64_t)tm * 256 * ld, *b0 = B + (int64_t)tn * 128 * ld;
+    const uint32_t vo = (uint32_t)((lane >> 3) * ld + (lane & 7) * 16);
+    const int64_t  t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    for (int kt = 0; kt < steps; ++kt)
+    {
+        const uint32_t base = lds0 + (uint32_t)(kt % 3) * 49152u;
+        for (int u = wave; u < 48; u += nw)
+            dma16s((u < 32 ? a0 + (int64_t)u * 8 * ld : b0 + (int64_t)(u - 32) * 8 * ld) + kt * 128, vo, base + (uint32_t)u * 1024u);
+        // at most two steps of this wave's loads in flight
+        if (48 / nw == 12)
+            asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+        else if (48 / nw == 6)
+            asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    __syncthreads();
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = ((int *)smem)[threadIdx.x];
+    if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
+        ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+}
+
+// One wave: waits `delay` ticks of the 100 MHz real-time counter, then reports the shader-clock ticks that pass during the
+// next `span` ticks of it. Launched on a second stream next to the work whose clock is to be known.
+__global__ void clock_kernel(int64_t delay, int64_t span, int64_t *ticks)
+{
+    const int64_t start = wall_clock64();
+    while (wall_clock64() - start < delay)
+        __builtin_amdgcn_s_sleep(32);
+    const int64_t r0 = wall_clock64(), t0 = __builtin_readcyclecounter();
+    int64_t       r1 = r0;
+    while (r1 - r0 < span)
+    {
+        __builtin_amdgcn_s_sleep(32);
+        r1 = wall_clock64();
+    }
+    const int64_t t1 = __builtin_readcyclecounter();
+    if (threadIdx.x == 0)
+        ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+}
+} // namespace
+
+extern "C"
+{
+// kib: size of the buffer in KiB, a multiple of grid * waves * unroll (pattern 1: of unroll); pattern 0 / 1 (see
+// read_kernel); unroll 4 or 8
+int mi355_ceiling_read(const void *buf, int64_t kib, int pattern, int grid, int waves, int unroll, int *sink, void *stream)
+{
+    if (!buf || !sink || grid < 1 || waves < 1 || waves > 8 || (unroll != 4 && unroll != 8) || kib < 1 ||
+        kib % (pattern == 0 ? (int64_t)grid * waves * unroll : (int64_t)unroll) != 0)
+        return (int)hipErrorInvalidValue;
+    const v4i  *p = (const v4i *)buf;
+    hipStream_t s = (hipStream_t)stream;
+    if (pattern == 0 && unroll == 8)
+        hipLaunchKernelGGL((read_kernel<0, 8>), dim3(grid), dim3(waves * 64), 0, s, p, kib, sink);
+    else if (pattern == 0)
+        hipLaunchKernelGGL((read_kernel<0, 4>), dim3(grid), dim3(waves * 64), 0, s, p, kib, sink);
+    else if (unroll == 8)
+        hipLaunchKernelGGL((read_kernel<1, 8>), dim3(grid), dim3(waves * 64), 0, s, p, kib, sink);
+    else
+        hipLaunchKernelGGL((read_kernel<1, 4>), dim3(grid), dim3(waves * 64), 0, s, p, kib, sink);
+    return (int)hipGetLastError();
+}
+
+// src: 16 MiB of operand bytes; grid workgroups of 8 waves, each wave issuing mfma16 (a multiple of 32) 16x16x64-sized
+// instructions; sink: grid * 512 ints; ticks: 2 x int64 (shader-clock ticks, 100 MHz ticks of one wave's loop) or null
+int mi355_ceiling_mfma(const void *src, int shape, int grid, int mfma16, int *sink, int64_t *ticks, void *stream)
+{
+    if (!src || !sink || grid < 1 || mfma16 < 32 || mfma16 % 32 != 0 || (shape != 16 && shape != 32))
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = (hipStream_t)stream;
+    if (shape == 16)
+        hipLaunchKernelGGL(mfma_kernel<16>, dim3(grid), dim3(512), 0, s, (const v4i *)src, mfma16, sink, ticks);
+    else
+        hipLaunchKernelGGL(mfma_kernel<32>, dim3(grid), dim3(512), 0, s, (const v4i *)src, mfma16, sink, ticks);
+    return (int)hipGetLastError();
+}
+
+int mi355_ceiling_mfma_lds(const void *src, int grid, int steps, int *sink, int64_t *ticks, void *stream)
+{
+    if (!src || !sink || grid < 1 || steps < 1)
+        return (int)hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised)
+    {
+        hipError_t e = hipFuncSetAttribute((const void *)mfma_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
+        if (e != hipSuccess)
+            return (int)e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(mfma_lds_kernel, dim3(grid), dim3(512), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps, sink,
+                       ticks);
+    return (int)hipGetLastError();
+}
+
+// A: at least 2048 rows, B: at least 4096 rows of ld bytes (ld >= steps * 128); grid = 256 (8 x 32 tiles); waves 4, 8 or 12
+int mi355_ceiling_dma(const void *A, const void *B, int64_t ld, int steps, int waves, int *sink, int64_t *ticks, void *stream)
+{
+    if (!A || !B || !sink || (waves != 4 && waves != 8 && waves != 12) || steps < 1 || ld < (int64_t)steps * 128 || ld % 16 != 0 ||
+        ld * 8 >= ((int64_t)1 << 32))
+        return (int)hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised)
+    {
+        hipError_t e = hipFuncSetAttribute((const void *)dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
+        if (e != hipSuccess)
+            return (int)e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(dma_kernel, dim3(256), dim3(waves * 64), 3 * 49152, (hipStream_t)stream, (const char *)A, (const char *)B, ld,
+                       steps, 32, sink, ticks);
+    return (int)hipGetLastError();
+}
+
+// delay, span in 100 MHz ticks (10 ns); afterwards ticks[0] / ticks[1] * 100 MHz is the shader clock over the span
+int mi355_ceiling_clock(int64_t delay, int64_t span, int64_t *ticks, void *stream)
+{
+    if (!ticks || delay < 0 || span < 1 || delay + span > 100000000)
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(clock_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, delay, span, ticks);
+    return (int)hipGetLastError();
+}
+}

@@ -13,7 +13,9 @@
 // number of waves per block is chosen from the number of column groups.
 #include "internal.hpp"
 
+#include <algorithm>
 #include <atomic>
+#include <type_traits>
 #include <cstdlib>
 
 namespace mi355
@@ -388,6 +390,215 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     }
 }
 
+
+// M <= 8, K <= 4096: the stage-once form. One workgroup of 16 waves per compute unit walks the column groups
+// blockIdx.x, blockIdx.x + gridDim.x, ... (at most ONCE_MAX_GROUPS of them); wave w owns the k blocks
+// [w * PER, (w + 1) * PER) of every group and copies its slice of A into LDS once for all groups. With one workgroup per
+// group, A (which never leaves the L2) crosses the compute unit's vector-memory path once per group and takes a third
+// of its requests; here it crosses once per compute unit. Two groups of B loads are in flight per wave. Partial sums
+// meet in double-buffered LDS (one barrier per group) and 8 x 16 threads finish one output each, so the only work
+// behind the last byte of B is one short chain; their per-column constants are fetched before the stream starts.
+constexpr int ONCE_WAVES      = 16;
+constexpr int ONCE_MAX_GROUPS = 4;
+// The arguments this kernel uses, packed into 136 bytes: it reads all of them in one batch of scalar loads before
+// anything else. With the general argument block (three times the size, the used fields scattered over it) the
+// compiler fetched some fields where they were first used, which put a second round trip to memory in front of the B
+// stream and a third one behind it, in the epilogue; the number of workgroups is passed for the same reason (gridDim is
+// a hidden argument behind the block).
+struct OnceArgs
+{
+    const int8_t  *A, *Bp;
+    void          *D;
+    const int32_t *colvec, *rowvec, *mult, *shift;
+    const float   *bias_f32;
+    int64_t        lda, ldd;
+    int32_t        M, N, KB, grid;
+    int32_t        result_offset, stage, lo, hi;
+    float          scale, act_min, act_max;
+    int32_t        has_offsets, accumulate, act_twice;
+};
+template <int EPI, bool FLIP_A, int PER, bool MULTI>
+__global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g)
+{
+    constexpr int SLICE = PER * 64, PITCH = SLICE + 64; // bytes of a row of A per wave; the pitch spreads 8 rows over the banks
+    constexpr int NA    = 8 * SLICE / 1024 > 0 ? 8 * SLICE / 1024 : 1; // 1 KiB loads that cover 8 rows of a slice
+    constexpr int LPR   = SLICE / 16;                                  // lanes per row
+    constexpr int RPL   = 64 / LPR > 8 ? 8 : 64 / LPR;                 // rows per load
+    __shared__ __attribute__((aligned(16))) int32_t red[2][ONCE_WAVES][32][4];
+    __shared__ int32_t                              par[4][64]; // [vector][group * 16 + column]; row vector: [3][row]
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][8][PITCH]
+
+    // Everything is pinned in registers here, so that it is all fetched before this point. A pointer that went through the
+    // asm as an integer is a generic pointer no more: it comes back as a pointer to global memory (generic loads would
+    // wait for LDS and memory alike).
+#define MI355_GLOBAL __attribute__((address_space(1)))
+    uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_d = (uintptr_t)g.D, u_cv = (uintptr_t)g.colvec, u_rv = (uintptr_t)g.rowvec,
+              u_mu = (uintptr_t)g.mult, u_sh = (uintptr_t)g.shift, u_bf = (uintptr_t)g.bias_f32;
+    asm volatile(""
+                 : "+s"(g.result_offset), "+s"(g.stage), "+s"(g.lo), "+s"(g.hi), "+s"(g.scale), "+s"(g.act_min), "+s"(g.act_max),
+                   "+s"(g.has_offsets), "+s"(g.accumulate), "+s"(g.act_twice), "+s"(g.lda), "+s"(g.ldd), "+s"(g.M), "+s"(g.N),
+                   "+s"(g.KB), "+s"(g.grid), "+s"(u_a), "+s"(u_b), "+s"(u_d), "+s"(u_cv), "+s"(u_rv), "+s"(u_mu), "+s"(u_sh),
+                   "+s"(u_bf));
+    const MI355_GLOBAL int8_t *const  gA = (const MI355_GLOBAL int8_t *)u_a, *const gB = (const MI355_GLOBAL int8_t *)u_b;
+    MI355_GLOBAL char *const          gD = (MI355_GLOBAL char *)u_d;
+    const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_rowvec = (const MI355_GLOBAL int32_t *)u_rv,
+                                     *const g_mult = (const MI355_GLOBAL int32_t *)u_mu, *const g_shift = (const MI355_GLOBAL int32_t *)u_sh,
+                                     *const g_bias = (const MI355_GLOBAL int32_t *)u_bf;
+    const bool has_bias = u_bf != 0;
+    EpiParams  p{};
+    p.result_offset = g.result_offset, p.stage = g.stage, p.lo = g.lo, p.hi = g.hi;
+    p.scale = g.scale, p.act_min = g.act_min, p.act_max = g.act_max;
+    p.has_offsets = g.has_offsets, p.accumulate = g.accumulate, p.act_twice = g.act_twice;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int KB   = g.KB;
+    const int NGT  = (g.N + 15) / 16;
+    const int G    = g.grid; // == gridDim.x
+    const int mine = (NGT - (int)blockIdx.x + G - 1) / G; // column groups of this workgroup, 1..ONCE_MAX_GROUPS
+    const int kb0  = wave * PER;
+    const bool busy = kb0 < KB; // K < 1024 * PER leaves the last waves without k blocks
+
+    // The epilogue's constants: 4 vectors (column term, multiplier or float bias, shift, row term) x 4 groups x 16 columns
+    // are one dword per lane of four waves. Wave w fetches vector w % 4, before anything else - every wave, without a
+    // condition (behind a branch the compiler would no longer know how many loads are in flight and would make the
+    // wait for A wait for B too); the host passes every vector (replicated scalars, a zero row vector) and only the
+    // float bias may be missing, in which case the column term stands in. Every wave leaves its dword in LDS (four
+    // waves write the same value to the same place) for the epilogue threads.
+    const int t = (int)threadIdx.x, erow = t >> 4, ecol = t & 15;
+    int32_t   par_v;
+    {
+        const int                   v   = wave & 3;
+        const int                   j   = min(((int)blockIdx.x + (lane >> 4) * G) * 16 + (lane & 15), g.N - 1);
+        const MI355_GLOBAL int32_t *vec = v == 0   ? g_colvec
+                                          : v == 1 ? (EPI == EPI_FIXEDPOINT ? g_mult : (EPI == EPI_F32 && has_bias ? g_bias : g_colvec))
+                                          : v == 2 ? (EPI == EPI_FIXEDPOINT ? g_shift : g_colvec)
+                                                   : g_rowvec;
+        par_v                           = vec[v == 3 ? min(lane & 7, g.M - 1) : j];
+    }
+
+    // this wave's slice of A: rows past M re-read row M-1 into staging rows whose results are never stored
+    char *a_lds = a_stage + wave * 8 * PITCH;
+    v4i   ta[NA];
+    const int a_sr = lane / LPR, a_sc = (lane % LPR) * 16;
+    {
+        // lanes past the end of K (last busy wave) re-read the slice's first 16 bytes into columns nobody reads; waves
+        // without k blocks re-read the last k block
+        const int col = a_sc < min(PER, KB - kb0) * 64 ? a_sc : 0;
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+            ta[i] = *(const MI355_GLOBAL v4i *)(gA + (int64_t)min(i * RPL + a_sr, g.M - 1) * g.lda + (int64_t)min(kb0, KB - 1) * 64 + col);
+    }
+    const MI355_GLOBAL int8_t *bp = gB + ((int64_t)min(kb0, KB - 1) * 64 + lane) * 16; // (waves without k blocks re-read the last one)
+    v4i           fb[2][PER];
+    auto load_b = [&](int slot, int gi)
+    {
+        const int grp = min((int)blockIdx.x + gi * G, NGT - 1);
+#pragma unroll
+        for (int u = 0; u < PER; ++u) // k blocks past KB (last busy wave, K not a multiple of 64 * PER) re-read the last one
+            fb[slot][u] = __builtin_nontemporal_load((const MI355_GLOBAL v4i *)(bp + ((int64_t)grp * KB + max(min(u, KB - 1 - kb0), 0)) * 1024));
+    };
+    // MULTI: every workgroup has at least two groups. Nothing between here and the wait for A may sit behind a branch:
+    // the compiler would no longer know how many loads are in flight and would make the wait for A wait for B as well
+    // (loads return in order) - hence also the unconditional fetches of the epilogue constants below.
+    load_b(0, 0);
+    if (MULTI)
+        load_b(1, 1);
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+    {
+        if (FLIP_A)
+            ta[i] ^= (int)0x80808080;
+        if (i * RPL + a_sr < 8 && a_sr < RPL)
+            *(v4i *)(a_lds + (i * RPL + a_sr) * PITCH + a_sc) = ta[i];
+    }
+    par[wave & 3][lane] = par_v; // read behind the first group's barrier
+    // operand blocks of A: lane -> row lane % 16 (rows 8..15 are zero), 16 bytes at k offset (lane / 16) * 16
+    const int arow = lane & 15, akc = (lane >> 4) * 16;
+    v4i       fa[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        fa[u] = (v4i){0, 0, 0, 0};
+        if (busy && arow < 8 && kb0 + u < KB)
+            fa[u] = *(const v4i *)(a_lds + arow * PITCH + u * 64 + akc);
+    }
+
+    // The groups of a workgroup, written out for each possible count: with the count a run-time value the fetch of
+    // group gi + 2 sits behind a condition, the compiler loses count of the loads in flight, and the matrix instructions
+    // of group gi + 1 wait for the loads of group gi + 2 as well.
+    auto groups = [&](auto count)
+    {
+        constexpr int MINE = decltype(count)::value;
+#pragma unroll
+        for (int gi = 0; gi < MINE; ++gi)
+        {
+            v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+            if (busy)
+            {
+                // The two chains are added and the sum is held back for 32 issue slots in the same basic block as the
+                // matrix instructions: their results may not be read by another instruction type for about a dozen
+                // slots, and the compiler only pads that distance inside a block - with the first reader behind a taken
+                // branch it came 3 slots after the instruction and read the last register of the result too early.
+#pragma unroll
+                for (int u = 0; u < PER; ++u)
+                    (u & 1 ? acc1 : acc0) = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[gi & 1][u], u & 1 ? acc1 : acc0, 0, 0, 0);
+                acc0 += acc1;
+                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0));
+            }
+            if (gi + 2 < MINE)
+                load_b(gi & 1, gi + 2);
+            // accumulator r of lane l is row 4 * (l / 16) + r, column l % 16: lanes 32..63 hold rows 8..15
+            if (lane < 32)
+                *(v4i *)&red[gi & 1][wave][lane][0] = acc0;
+            __syncthreads();
+            if (t < 128)
+            {
+                const int      j = ((int)blockIdx.x + gi * G) * 16 + ecol;
+                const int32_t *r = &red[gi & 1][0][(erow >> 2) * 16 + ecol][erow & 3];
+                int32_t        sum = 0;
+#pragma unroll
+                for (int w = 0; w < ONCE_WAVES; ++w)
+                    sum += r[w * 32 * 4];
+                const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & 7];
+                if (j < g.N && erow < g.M)
+                {
+                    const int64_t idx = (int64_t)erow * g.ldd + j;
+                    if (EPI == EPI_S32)
+                        ((MI355_GLOBAL int32_t *)gD)[idx] = (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv +
+                                                                      (p.accumulate ? (uint32_t)((MI355_GLOBAL int32_t *)gD)[idx] : 0u));
+                    else if (EPI == EPI_FIXEDPOINT)
+                    {
+                        const int32_t v = (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv);
+                        int32_t       q;
+                        if (p.stage == 0 && m >= 0 && sh > -32 && sh < 32)
+                            // the branch-free form of the same arithmetic (see fast_requant), its constants derived here
+                            q = fast_requant(v, (int32_t)((uint32_t)m << 1), (uint32_t)m >= 0x40000000u ? -1 : 0, sh < 0 ? -sh : 0,
+                                             sh > 1 ? sh - 1 : 0, sh > 0 ? 1 : 0, p.result_offset, p.lo, p.hi);
+                        else
+                            q = epi_fixedpoint(sum, c, rv, m, sh, p);
+                        ((MI355_GLOBAL int8_t *)gD)[idx] = (int8_t)q;
+                    }
+                    else
+                        ((MI355_GLOBAL float *)gD)[idx] = epi_f32(sum, (int32_t)((uint32_t)c + (uint32_t)rv), __int_as_float(m), has_bias,
+                                                                  p, p.accumulate ? ((MI355_GLOBAL float *)gD)[idx] : 0.f);
+                }
+            }
+        }
+    };
+    if (!MULTI || mine == 1)
+        groups(std::integral_constant<int, 1>{});
+    else if (mine == 2)
+        groups(std::integral_constant<int, 2>{});
+    else if (mine == 3)
+        groups(std::integral_constant<int, 3>{});
+    else
+        groups(std::integral_constant<int, 4>{});
+}
+static_assert(ONCE_MAX_GROUPS == 4, "the group loop is written out for 1 to 4 groups");
+
+#undef MI355_GLOBAL
+
 // A kernel that needs more than 48 KiB of dynamic LDS has to be told so once per device
 static int raise_lds_limit(const void *fn, size_t lds, std::atomic<uint32_t> &done)
 {
@@ -430,12 +641,59 @@ static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t 
     return (int)hipLaunchKernel(fn, grid, block, kargs, lds, s);
 }
 
+
+// compute units of the current device, asked once per device
+static int device_cus()
+{
+    static std::atomic<int> cus[32];
+    int                     dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
+        return 0;
+    int n = cus[dev].load(std::memory_order_acquire);
+    if (n == 0)
+    {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+            return 0;
+        cus[dev].store(n, std::memory_order_release);
+    }
+    return n;
+}
+
+template <int PER, bool MULTI>
+static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
+{
+    static const void *const fns[3][2] = {
+        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI>,
+         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI>},
+        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI>,
+         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI>},
+        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI>,
+         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI>}};
+    // the kernel fetches these without asking
+    if (a.epi.colvec == nullptr || a.epi.rowvec == nullptr || (epi == EPI_FIXEDPOINT && (a.epi.mult == nullptr || a.epi.shift == nullptr)))
+        return (int)hipErrorInvalidValue;
+    static std::atomic<uint32_t> lds_raised[3][2];
+    const size_t                 lds = (size_t)ONCE_WAVES * 8 * (PER * 64 + 64);
+    const void                  *fn  = fns[epi][flip_a ? 1 : 0];
+    // 16 KiB of static LDS on top: declare the dynamic part whatever its size
+    const int e = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
+    if (e)
+        return e;
+    const EpiParams &p = a.epi;
+    OnceArgs         o{a.A,    a.Bp,   a.D,    p.colvec, p.rowvec,  p.mult,    p.shift,       p.bias_f32,   a.lda,       a.ldd,        a.M,
+               a.N,    (int32_t)(a.Kp / 64), grid, p.result_offset, p.stage, p.lo, p.hi, p.scale, p.act_min, p.act_max,
+               p.has_offsets, p.accumulate, p.act_twice};
+    void *kargs[] = {&o};
+    return (int)hipLaunchKernel(fn, dim3(grid), dim3(ONCE_WAVES * 64), kargs, lds, s);
+}
+
 // Environment overrides for experiments, read once: MI355_SKINNY_WAVES (4 or 8; anything else is ignored),
-// MI355_SKINNY_NG (column groups per workgroup), MI355_SKINNY_NO_STAGE (A operands straight from global memory)
+// MI355_SKINNY_NG (column groups per workgroup), MI355_SKINNY_NO_STAGE (A operands straight from global memory),
+// MI355_SKINNY_NO_ONCE (one workgroup per column group also where the stage-once form applies)
 struct SkinnyEnv
 {
     int  waves = 0, ng = 0;
-    bool no_stage = false;
+    bool no_stage = false, no_once = false;
     SkinnyEnv()
     {
         const char *w = getenv("MI355_SKINNY_WAVES"), *n = getenv("MI355_SKINNY_NG");
@@ -444,6 +702,7 @@ struct SkinnyEnv
         if (n && atoi(n) >= 1 && atoi(n) <= 4)
             ng = atoi(n);
         no_stage = getenv("MI355_SKINNY_NO_STAGE") != nullptr;
+        no_once  = getenv("MI355_SKINNY_NO_ONCE") != nullptr;
     }
 };
 
@@ -458,6 +717,27 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     // from there; that needs nothing to guard
     const bool stage_ok = args.M <= 8 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
                           ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
+    // Up to 4096 of K the stage-once form: one workgroup per column group while there are no more groups than compute
+    // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
+    // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside
+    // the first on a compute unit: one workgroup of 8 waves per group below. Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
+    if (stage_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    {
+        const int cus = device_cus();
+        if (cus > 0 && (groups <= cus || groups >= 2 * cus))
+        {
+            const bool multi = groups >= 2 * cus;
+            const int  grid  = multi ? std::max(cus, (groups + ONCE_MAX_GROUPS - 1) / ONCE_MAX_GROUPS) : groups;
+            const int  per   = KB <= ONCE_WAVES ? 1 : (KB <= 2 * ONCE_WAVES ? 2 : 4);
+            if (multi)
+                return per == 1   ? skinny_once_launch_v<1, true>(epi, flip_a, args, grid, s)
+                       : per == 2 ? skinny_once_launch_v<2, true>(epi, flip_a, args, grid, s)
+                                  : skinny_once_launch_v<4, true>(epi, flip_a, args, grid, s);
+            return per == 1   ? skinny_once_launch_v<1, false>(epi, flip_a, args, grid, s)
+                   : per == 2 ? skinny_once_launch_v<2, false>(epi, flip_a, args, grid, s)
+                              : skinny_once_launch_v<4, false>(epi, flip_a, args, grid, s);
+        }
+    }
     // The kernel lives on loads in flight: 8 waves per workgroup while each of them still has at least one whole
     // step of 8 k blocks and all workgroups are resident together (24 waves of this size per compute unit), 4 otherwise
     int waves = (groups >= 512 && !(stage_ok && KB >= 64 && (int64_t)groups * 8 <= 24 * 256)) ? 4 : 8;

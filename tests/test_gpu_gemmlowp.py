@@ -249,6 +249,47 @@ def test_skinny_kernel_with_staged_a(M):
         np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
 
 
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_skinny_stage_once_kernel(M):
+    """Up to 8 rows and K <= 4096 (whole 64-byte blocks, 16-byte aligned rows) one workgroup of 16 waves per compute unit
+    walks several column groups with A staged once: K picks 1, 2 or 4 k blocks per wave, with the last busy wave short
+    (K = 2112, 3136) or waves without any k block (K = 64, 640); N covers a single ragged group, fewer groups than compute
+    units, 2 to 3 groups per workgroup and more than four times the compute units; every epilogue, signed and unsigned
+    A, a non-zero B offset (row vector) and accumulation."""
+    rng = np.random.default_rng(3300 + M)
+    for once in (True,):
+        for (N, K) in [(7, 64), (300, 640), (8200, 1024), (11008, 4096), (5000, 2112), (4100, 3136), (70000, 256),
+                       (16400, 2048)]:
+            a_dt = np.uint8 if (N + K) % 3 == 0 else np.int8
+            A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+            B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+            ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
+            lda = K + (0 if K % 128 else 16)
+            announce("skinny stage-once", once, (M, N, K), "lda", lda, a_dt.__name__)
+            want = oracle.gemmlowp_s32(A, B, ao, bo)
+            got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_AUTO, device=True, lda=lda, ldd=N + 3)
+            assert name.startswith("skinny"), name
+            np.testing.assert_array_equal(got, want)
+            prev = rng.integers(-10**6, 10**6, size=(M, N), dtype=np.int32)
+            got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, device=True, lda=lda, prev=prev, flags=capi.GEMM_ACCUMULATE)
+            np.testing.assert_array_equal(got, (want.astype(np.int64) + prev).astype(np.int32))
+            bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+            reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+            got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, 0, bias, mult, shift, off, lo, hi, device=True, lda=lda)
+            np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
+            got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, bo, bias, [int(mult[0])], [int(shift[0])], off, lo, hi,
+                              device=True, lda=lda)
+            np.testing.assert_array_equal(
+                got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, bo, [int(mult[0])], [int(shift[0])], off, lo, hi, a_dt))
+            if a_dt == np.int8:
+                biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+                got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, device=True, lda=lda)
+                np.testing.assert_array_equal(got.view(np.uint32),
+                                              oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
+
+
 @pytest.mark.parametrize("M", [17, 24, 25, 31, 32, 33, 48, 63, 64])
 def test_skinny_kernel_with_several_row_blocks(M):
     """17 to 64 rows run as 2 or 4 blocks of 16 rows in the streaming kernel (from 25 rows on with A staged through LDS

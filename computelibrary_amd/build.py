@@ -16,7 +16,7 @@ LIB = os.path.join(LIBDIR, "libmi355gemmlowp.so")
 # measurement-only kernels for `bench.py --ceilings`: a library of their own, never linked into the product library
 CEILINGS_LIB = os.path.join(LIBDIR, "libmi355ceilings.so")
 CEILINGS_SOURCES = ["ceilings.hip"]
-SOURCES = ["gemm_dma.hip", "gemm_mfma.hip", "gemm_skinny.hip", "kernels_aux.hip", "capi.hip"]
+SOURCES = ["gemm_dma.hip", "gemm_mfma.hip", "gemm_skinny.hip", "gemm_narrow.hip", "kernels_aux.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -165,9 +165,10 @@ struct GemmCore
     int     Kp = 0, Np = 0;
     bool    b_shared = true; // one B for all batches
     bool    has_bias = false, has_pc = false, prepared = false;
+    bool    has_narrow = false; // Bn holds the narrow kernel's image of B
     bool    pt_vectors = false; // streaming path, per-tensor requantisation: mult / shift hold the scalars, replicated
     std::string kname;
-    DevBuf  Bp, Bs, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros;
+    DevBuf  Bp, Bs, Bn, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros;
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -180,7 +181,7 @@ struct GemmCore
 
     void release()
     {
-        Bp.release(), Bs.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
+        Bp.release(), Bs.release(), Bn.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
         shift.release(), bias.release(), Ap.release(), fill.release(), qp.release(), zeros.release();
     }
 
@@ -290,6 +291,14 @@ struct GemmCore
         {
             TRY(Bs.ensure((size_t)Np * Kp));
             HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>(), Kp, Np, Bs.as<int8_t>(), s));
+        }
+        // few output columns and a short K: the image of the B panel the narrow kernel copies into LDS
+        has_narrow = path == MI355_PATH_MFMA && nb() == 1 && N <= 64 && narrow_panel_chunks(K) > 0;
+        if (has_narrow)
+        {
+            const int chunks = narrow_panel_chunks(K);
+            TRY(Bn.ensure((size_t)64 * (chunks + 1) * 16));
+            HIP_TRY(pack_b_narrow_launch(Bp.as<int8_t>(), Kp, Np, chunks, Bn.as<int8_t>(), s));
         }
         TRY(fill.ensure(16));
         HIP_TRY(fill_i32_launch(fill.as<int32_t>(), (int32_t)(0x01010101u * fill_byte), 4, s));
@@ -460,7 +469,17 @@ struct GemmCore
             const int64_t span = conv ? (int64_t)((g.M + g.conv.OH * g.conv.OW - 1) / (g.conv.OH * g.conv.OW)) *
                                             g.conv.H * g.conv.W * g.conv.C
                                       : (int64_t)g.lda * 256 + g.K;
-            if (dma_idx >= 0 && aligned && g.K >= 16 && span < ((int64_t)1 << 32))
+            // few output columns and a short K: every wave for itself, weights resident in LDS (gemm_narrow.hip)
+            static const bool no_narrow = getenv("MI355_NO_NARROW") != nullptr;
+            if (!no_narrow && has_narrow && batch == 1 && conv && !g.epi.accumulate && span < ((int64_t)1 << 31) &&
+                narrow_applies(g, conv))
+            {
+                kname           = kprefix + "narrow_32x64";
+                g.Bp            = Bn.as<int8_t>();
+                g.conv.pad_word = 0x01010101u * fill_byte; // as in the image: the kernel flips what it loads
+                HIP_TRY(narrow_launch(epi, flip_in_loader, conv, g, s));
+            }
+            else if (dma_idx >= 0 && aligned && g.K >= 16 && span < ((int64_t)1 << 32))
             {
                 const MfmaConfig c = dma_config(dma_idx);
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;

@@ -1,0 +1,379 @@
+// K5: implicit-GEMM convolution (and dense GEMM) with few output columns: N <= 64, K <= 1152.
+//
+// CpuGemmConv2d lowers a convolution with 64 output channels to a GEMM with M = batch * OH * OW rows and 64 columns
+// (src/cpu/operators/CpuGemmConv2d.cpp:923-1008); the work per output tile is then so small (K = KH * KW * C) that a
+// tile kernel built around a ring of K steps spends its time on start-up, barriers and epilogues. Here nothing is
+// shared between waves but the weights:
+//   * the whole B panel (64 columns x K, K contiguous, from the packed Bp) is copied into LDS once per workgroup, rows
+//     padded by 16 bytes so that the 16 rows of an operand read fall into 16 different bank groups;
+//   * every wave owns 32 output rows x all 64 columns and fetches its A operands straight from global memory into the
+//     matrix cores' operand layout - lane l holds 16 bytes of row l % 16 at k offset (l / 16) * 16, for NHWC with
+//     C % 16 == 0 that is 16 channels of one tap of one pixel, so a wave load covers whole pixels, and every A byte is
+//     used against all 64 columns out of registers;
+//   * loads go out in batches of 3 k blocks (6 loads of 1 KiB per wave), two batches in flight, and the number of
+//     batches is a template parameter, so the code is straight-line and the compiler knows exactly how many loads
+//     are outstanding at every wait;
+//   * no barrier after the one that publishes the B panel; 4 workgroups of 4 waves fit a compute unit.
+#include "mfma_common.hpp"
+
+#include <atomic>
+#include <type_traits>
+
+namespace mi355
+{
+// global -> LDS without registers: 64 lanes x 16 bytes land at M0 + lane * 16
+// (scalar base + one 32-bit offset per lane)
+__device__ __forceinline__ void narrow_dma16(const void *sbase, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+}
+
+// x / d with the reciprocal of ConvGeom::magic_* (0 stands for d == 1), without a branch on the reciprocal
+__device__ __forceinline__ int narrow_div(int x, uint32_t magic)
+{
+    const uint32_t one = (uint32_t)(magic != 0) - 1u; // all ones when d == 1
+    return (int)(__umulhi((uint32_t)x, magic) + ((uint32_t)x & one));
+}
+
+constexpr int NARROW_WAVES  = 4;
+constexpr int NARROW_ROWS   = 32;  // per wave
+constexpr int NARROW_BN     = 64;
+constexpr int NARROW_MAX_NB = 6;   // batches of 3 k blocks of 64: K <= 1152
+
+// UNI: C % 64 == 0 - a k block of 64 lies inside one tap, so the tap of a load is decoded with scalar arithmetic
+template <int EPI, bool FLIP_A, bool CONV, bool UNI, int NB>
+// (4 waves per SIMD, i.e. 4 workgroups per compute unit: at most 128 registers per lane)
+__global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_narrow_kernel(GemmArgs g)
+{
+    constexpr int RS = NARROW_ROWS / 16, QS = NARROW_BN / 16;
+    constexpr int KBLK  = NB * 3;         // k blocks the loop covers (the B panel is zero beyond K)
+    constexpr int PITCH = KBLK * 64 + 16; // bytes per B row in LDS
+    constexpr int NPAR  = 1 + QP_COUNT;
+    extern __shared__ __attribute__((aligned(16))) char smem[]; // B panel [64][PITCH], then par[NPAR][64]
+    int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
+
+    // Everything the main part uses is fetched here in one batch of scalar loads and pinned in registers (left alone, the
+    // compiler fetches kernel arguments where they are first used: a round trip to memory each time). Pointers go
+    // through the asm as integers and come back as pointers to global memory.
+#define MI355_GLOBAL __attribute__((address_space(1)))
+    ConvGeom  cg = g.conv;
+    uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp,
+              u_fl = (uintptr_t)g.epi.qp_flag;
+    int32_t   a_M = g.M, a_K = g.K, a_lda = (int32_t)g.lda, a_kp = (int32_t)g.Kp, a_qps = (int32_t)g.epi.qp_stride;
+    asm volatile(""
+                 : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x), "+s"(cg.stride_y),
+                   "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word), "+s"(cg.magic_C),
+                   "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(cg.magic_OH), "+s"(a_M), "+s"(a_K), "+s"(a_lda), "+s"(a_kp),
+                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl));
+    const MI355_GLOBAL int8_t *const  gA = (const MI355_GLOBAL int8_t *)u_a, *const gB = (const MI355_GLOBAL int8_t *)u_b;
+    const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lh = lane >> 4;
+    const int row0 = blockIdx.x * (NARROW_WAVES * NARROW_ROWS) + wave * NARROW_ROWS;
+
+    // the epilogue's per-column constants (column term + the digested requantisation vectors), where they exist: 6 x 64
+    // dwords, one or two per thread, fetched first and parked in LDS with the B panel
+    const bool have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
+    int32_t    tp[2]   = {0, 0};
+    if (have_qp)
+    {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+        {
+            const int idx = min(tid + i * NARROW_WAVES * 64, NPAR * NARROW_BN - 1);
+            const int v = idx / NARROW_BN, col = idx - v * NARROW_BN;
+            tp[i]       = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
+        }
+    }
+    int qflag = 1;
+    if (have_qp && u_fl != 0)
+        qflag = *(const MI355_GLOBAL int32_t *)u_fl;
+
+    // ---- B panel: straight into LDS (no registers), issued before the A loads, which are needed later. The host keeps
+    // the panel in global memory exactly as it lies in LDS (rows of CHUNKS pieces of 16 bytes plus one of padding,
+    // zero beyond Kp), so it moves as NDMA linear transfers of 1 KiB; wave w issues transfers w, w + 4, ... ----
+    constexpr int  CHUNKS = KBLK * 4;       // 16-byte pieces of a row that hold data
+    constexpr int  NDMA   = CHUNKS + 1;     // 64 rows x (CHUNKS + 1) pieces / 64 pieces per transfer
+    constexpr int  DPW    = (NDMA + NARROW_WAVES - 1) / NARROW_WAVES;
+    const uint32_t lds0   = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+    int            my_dma = 0; // transfers this wave issues (wave-uniform)
+#pragma unroll
+    for (int i = 0; i < DPW; ++i)
+    {
+        const int ins = wave + i * NARROW_WAVES;
+        if (ins < NDMA)
+        {
+            narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
+            ++my_dma;
+        }
+    }
+    (void)my_dma;
+
+    // ---- A: per-lane source of row rb*16 + lr ----
+    // conv: pix[rb] = byte offset of the (possibly out-of-image) top-left tap of the row's pixel, iy0/ix0 its coordinates;
+    // dense: byte offset of the row. Rows past M re-use row M-1 (never stored).
+    int32_t pix[RS], iy0[RS], ix0[RS];
+#pragma unroll
+    for (int rb = 0; rb < RS; ++rb)
+    {
+        const int gr = min(row0 + rb * 16 + lr, a_M - 1);
+        if (CONV)
+        {
+            const int t  = narrow_div(gr, cg.magic_OW);
+            const int ox = gr - t * cg.OW;
+            const int n  = narrow_div(t, cg.magic_OH);
+            const int oy = t - n * cg.OH;
+            iy0[rb]      = oy * cg.stride_y - cg.pad_top;
+            ix0[rb]      = ox * cg.stride_x - cg.pad_left;
+            pix[rb]      = n * (cg.H * cg.W * cg.C) + (iy0[rb] * cg.W + ix0[rb]) * cg.C;
+        }
+        else
+        {
+            iy0[rb] = ix0[rb] = 0;
+            pix[rb]           = gr * a_lda;
+        }
+    }
+    // A piece outside the image (or past K) is fetched from offset 0 instead - a load that depends on nothing - and
+    // replaced by the padding value when it is used (past K its value is irrelevant: B is zero there).
+    v4i      fa[2][3][RS];
+    uint32_t oob = 0; // bit (slot * 3 + kk) * RS + rb: that piece is padding
+    auto     load_a = [&](int slot, int batch)
+    {
+        oob &= ~(((1u << (3 * RS)) - 1u) << (slot * 3 * RS));
+#pragma unroll
+        for (int kk = 0; kk < 3; ++kk)
+        {
+            const int kb = batch * 3 + kk;
+            const int k  = kb * 64 + lh * 16; // this lane's 16 bytes of the k block
+            int       dy = 0, dx = 0, off = k;
+            if (CONV)
+            {
+                int tap, c0;
+                if (UNI)
+                {
+                    tap = narrow_div(kb * 64, cg.magic_C); // scalar
+                    c0  = kb * 64 - tap * cg.C + lh * 16;
+                }
+                else
+                {
+                    tap = narrow_div(k, cg.magic_C);
+                    c0  = k - tap * cg.C;
+                }
+                const int ky = narrow_div(tap, cg.magic_KW);
+                const int kx = tap - ky * cg.KW;
+                dy           = ky * cg.dil_y;
+                dx           = kx * cg.dil_x;
+                off          = (dy * cg.W + dx) * cg.C + c0;
+            }
+#pragma unroll
+            for (int rb = 0; rb < RS; ++rb)
+            {
+                // (bitwise, not short-circuit: no branches between the loads)
+                const bool ok = CONV ? ((k < a_K) & ((unsigned)(iy0[rb] + dy) < (unsigned)cg.H) & ((unsigned)(ix0[rb] + dx) < (unsigned)cg.W))
+                                     : (k < a_K);
+                oob |= (uint32_t)(!ok) << ((slot * 3 + kk) * RS + rb);
+                fa[slot][kk][rb] = *(const MI355_GLOBAL v4i *)(gA + (uint32_t)(ok ? pix[rb] + off : 0));
+            }
+        }
+    };
+    load_a(0, 0);
+    if (NB > 1)
+        load_a(1, 1);
+    __builtin_amdgcn_sched_barrier(0); // nothing that waits for a load may move up between the loads
+
+    // ---- the B panel has landed when at most the A loads issued after it are still in flight; epilogue constants ----
+    if (NB > 1)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * 3 * RS) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * RS) : "memory");
+    if (have_qp)
+    {
+        par[tid] = tp[0];
+        if (tid < NPAR * NARROW_BN - NARROW_WAVES * 64)
+            par[tid + NARROW_WAVES * 64] = tp[1];
+    }
+    qflag           = __builtin_amdgcn_readfirstlane(qflag);
+    const bool fast = have_qp && (qflag & 1) == 0;
+    __syncthreads();
+
+    v4i acc[RS][QS];
+#pragma unroll
+    for (int i = 0; i < RS; ++i)
+#pragma unroll
+        for (int j = 0; j < QS; ++j)
+            acc[i][j] = (v4i){0, 0, 0, 0};
+
+    // The waves of a SIMD would otherwise share the matrix pipe evenly, finish together and then all queue for the vector
+    // ALU with their epilogues: different priorities let one wave at a time through the matrix instructions, and its
+    // epilogue then runs beside the matrix instructions of the next.
+    // (workgroups go to the 8 XCDs round-robin: those that meet on a compute unit differ in the bits above the low three)
+    switch ((blockIdx.x >> 3) & 3)
+    {
+    case 0: __builtin_amdgcn_s_setprio(3); break;
+    case 1: __builtin_amdgcn_s_setprio(2); break;
+    case 2: __builtin_amdgcn_s_setprio(1); break;
+    default: break;
+    }
+    const char *b_rd = smem + lr * PITCH + lh * 16; // + q * 16 * PITCH + kb * 64
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+    {
+#pragma unroll
+        for (int kk = 0; kk < 3; ++kk)
+        {
+            v4i fb[QS];
+#pragma unroll
+            for (int q = 0; q < QS; ++q)
+                fb[q] = *(const v4i *)(b_rd + q * 16 * PITCH + (b * 3 + kk) * 64);
+#pragma unroll
+            for (int rb = 0; rb < RS; ++rb)
+            {
+                v4i a = fa[b & 1][kk][rb];
+                if (oob & (1u << (((b & 1) * 3 + kk) * RS + rb)))
+                    a = (v4i){(int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word};
+                if (FLIP_A)
+                    a ^= (int)0x80808080;
+#pragma unroll
+                for (int q = 0; q < QS; ++q)
+                    acc[rb][q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[q], a, acc[rb][q], 0, 0, 0);
+            }
+        }
+        if (b + 2 < NB)
+            load_a(b & 1, b + 2);
+    }
+
+    __builtin_amdgcn_s_setprio(0);
+    if (fast && g.epi.qp_std && (qflag & 3) == 0 && g.epi.vec_store)
+    {
+        // every column has a normalised multiplier and a right shift of 2..31: the short form of the requantisation.
+        // Lane l holds, for row rb * 16 + l % 16, the 4 consecutive columns q * 16 + 4 * (l / 16) + {0..3}: one dword.
+        const int32_t  off2p1 = 2 * g.epi.result_offset + 1, lo = g.epi.lo, hi = g.epi.hi;
+        const int32_t *rowvec = g.epi.rowvec;
+        char          *D      = (char *)g.D;
+        int32_t        rv[RS];
+#pragma unroll
+        for (int rb = 0; rb < RS; ++rb)
+            rv[rb] = (rowvec && row0 + rb * 16 + lr < a_M) ? rowvec[row0 + rb * 16 + lr] : 0;
+#pragma unroll
+        for (int q = 0; q < QS; ++q)
+        {
+            const int c  = q * 16 + 4 * lh;
+            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * NARROW_BN + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * NARROW_BN + c);
+            const v4i cv = *(const v4i *)(par + c);
+#pragma unroll
+            for (int rb = 0; rb < RS; ++rb)
+            {
+                const int i = row0 + rb * 16 + lr;
+                int32_t   o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                {
+                    // std_requant with the clamp as one median instruction (lo <= hi)
+                    const int32_t v = (int32_t)((uint32_t)acc[rb][q][t] + (uint32_t)cv[t] + (uint32_t)rv[rb]);
+                    const int32_t h = __mulhi(v, s2[t]) + v;
+                    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(o[t]) : "v"(((h >> r1[t]) + off2p1) >> 1), "s"(lo), "v"(hi));
+                }
+                const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
+                const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
+                if (i < a_M && c + 3 < g.N)
+                    *(uint32_t *)(D + (int64_t)i * g.ldd + c) = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+                else if (i < a_M)
+                    for (int t = 0; t < 4; ++t)
+                        if (c + t < g.N)
+                            D[(int64_t)i * g.ldd + c + t] = (char)o[t];
+            }
+        }
+    }
+    else if (fast)
+        epilogue_store_fast<RS, QS, NARROW_BN>(acc, g, par, row0, 0, 0, lane, 0);
+    else
+        epilogue_store_t<EPI, RS, QS>(acc, g, row0, 0, lane, 0);
+#undef MI355_GLOBAL
+}
+
+template <int EPI, bool FLIP_A, bool CONV, bool UNI>
+static const void *narrow_fn(int nb)
+{
+    switch (nb)
+    {
+    case 1: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 1>;
+    case 2: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 2>;
+    case 3: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 3>;
+    case 4: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 4>;
+    case 5: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 5>;
+    case 6: return (const void *)gemm_narrow_kernel<EPI, FLIP_A, CONV, UNI, 6>;
+    }
+    return nullptr;
+}
+
+template <int EPI>
+static const void *narrow_fn_e(bool flip_a, bool conv, bool uni, int nb)
+{
+    if (conv)
+    {
+        if (uni)
+            return flip_a ? narrow_fn<EPI, true, true, true>(nb) : narrow_fn<EPI, false, true, true>(nb);
+        return flip_a ? narrow_fn<EPI, true, true, false>(nb) : narrow_fn<EPI, false, true, false>(nb);
+    }
+    return flip_a ? narrow_fn<EPI, true, false, false>(nb) : narrow_fn<EPI, false, false, false>(nb);
+}
+
+int narrow_panel_chunks(int K)
+{
+    if (K < 16 || K > NARROW_MAX_NB * 192)
+        return 0;
+    return (K + 191) / 192 * 12;
+}
+
+bool narrow_applies(const GemmArgs &a, bool conv)
+{
+    if (a.N < 1 || a.N > NARROW_BN || a.K < 16 || a.K > NARROW_MAX_NB * 192 || a.K > a.Kp || a.Kp % 64 != 0 || a.M < 1)
+        return false;
+    if (conv)
+    {
+        // whole 16-byte columns of one tap; the image batch within 31 bits of offset
+        const ConvGeom &c = a.conv;
+        const int64_t   images = ((int64_t)a.M + (int64_t)c.OH * c.OW - 1) / ((int64_t)c.OH * c.OW);
+        return c.C % 16 == 0 && ((uintptr_t)a.A & 15) == 0 && a.K % 16 == 0 && images * c.H * c.W * c.C < ((int64_t)1 << 31);
+    }
+    // dense: 16-byte aligned rows of whole 16-byte columns, offsets within 31 bits
+    return ((uintptr_t)a.A & 15) == 0 && a.lda % 16 == 0 && a.K % 16 == 0 && (int64_t)a.M * a.lda < ((int64_t)1 << 31);
+}
+
+int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s)
+{
+    if (!narrow_applies(args, conv) || args.fill16 == nullptr || epi < 0 || epi > 2)
+        return (int)hipErrorInvalidValue;
+    const int   nb  = (args.K + 191) / 192;
+    const bool  uni = conv && args.conv.C % 64 == 0;
+    const void *fn  = epi == EPI_S32 ? narrow_fn_e<EPI_S32>(flip_a, conv, uni, nb)
+                      : epi == EPI_FIXEDPOINT ? narrow_fn_e<EPI_FIXEDPOINT>(flip_a, conv, uni, nb)
+                                              : narrow_fn_e<EPI_F32>(flip_a, conv, uni, nb);
+    if (fn == nullptr)
+        return (int)hipErrorInvalidValue;
+    const size_t lds = (size_t)NARROW_BN * (nb * 192 + 16) + (size_t)(1 + QP_COUNT) * NARROW_BN * sizeof(int32_t);
+    if (lds > 48 * 1024)
+    {
+        // once per kernel and device
+        static std::atomic<uint32_t> raised[3][2][2][2][NARROW_MAX_NB];
+        std::atomic<uint32_t>       &done = raised[epi][flip_a ? 1 : 0][conv ? 1 : 0][uni ? 1 : 0][nb - 1];
+        int                          dev  = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
+            return (int)hipErrorInvalidDevice;
+        if ((done.load(std::memory_order_acquire) & (1u << dev)) == 0)
+        {
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess)
+                return (int)e;
+            done.fetch_or(1u << dev, std::memory_order_release);
+        }
+    }
+    GemmArgs a       = args;
+    void    *kargs[] = {&a};
+    const int rows   = NARROW_WAVES * NARROW_ROWS;
+    return (int)hipLaunchKernel(fn, dim3((args.M + rows - 1) / rows), dim3(NARROW_WAVES * 64), kargs, lds, s);
+}
+} // namespace mi355

@@ -95,6 +95,13 @@ int         dma_num_configs();
 MfmaConfig  dma_config(int idx);
 int         dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &args, int batch, hipStream_t s);
 
+// gemm_narrow.hip — N <= 64, K <= 1152, 16-byte aligned operands: A straight from global memory into the matrix cores'
+// operand layout, B resident in LDS; dense or implicit convolution (C % 16 == 0). needs args.fill16
+// (args.Bp: the image written by pack_b_narrow_launch with narrow_panel_chunks(K) pieces per row)
+int  narrow_panel_chunks(int K); // 0: K outside the kernel's range
+bool narrow_applies(const GemmArgs &args, bool conv);
+int  narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s);
+
 // gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 64;
 int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
@@ -108,6 +115,8 @@ int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bo
                    hipStream_t s);
 // Bp [Np][Kp] -> operand order for the skinny kernel: [Np/16][Kp/64][64 lanes][16 bytes]
 int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream_t s);
+// rows 0..63 of Bp -> [64][chunks + 1] pieces of 16 bytes (the last one padding), zero beyond Kp
+int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int8_t *Bn, hipStream_t s);
 // colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j])
 int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int32_t b_off, int K, int N,
                   int32_t *colvec, hipStream_t s);

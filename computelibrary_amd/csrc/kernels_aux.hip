@@ -170,6 +170,29 @@ int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream
     return launch_status();
 }
 
+// The first 64 rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus one piece of
+// padding, zero beyond Kp - the workgroups copy this image into LDS with plain linear transfers
+__global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__restrict__ Bp, int Kp, int chunks,
+                                                            int8_t *__restrict__ Bn)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= 64 * (chunks + 1))
+        return;
+    const int r = idx / (chunks + 1), c = idx - r * (chunks + 1);
+    v4i       v = {0, 0, 0, 0};
+    if (c < chunks && c * 16 < Kp)
+        v = *(const v4i *)(Bp + (int64_t)r * Kp + c * 16);
+    *(v4i *)(Bn + (int64_t)idx * 16) = v;
+}
+
+int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int8_t *Bn, hipStream_t s)
+{
+    if (Kp % 16 || Np < 64 || chunks < 1)
+        return (int)hipErrorInvalidValue;
+    pack_b_narrow_kernel<<<dim3((64 * (chunks + 1) + 255) / 256), dim3(256), 0, s>>>(Bp, Kp, chunks, Bn);
+    return launch_status();
+}
+
 // colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j]); the per-column part of the offset contribution, folded with the
 // bias like arm_gemm's col_bias (src/core/NEON/kernels/arm_gemm/quantized.cpp:963-968)
 __global__ void colvec_kernel(const int32_t *__restrict__ colsum, const int32_t *__restrict__ bias, uint32_t a_off,

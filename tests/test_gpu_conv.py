@@ -114,6 +114,57 @@ def test_conv_seeded_strides_dilation_uint8():
             np.testing.assert_array_equal(got, want)
 
 
+def test_conv_few_output_channels_kernel():
+    """Up to 64 output channels and K = KH * KW * C <= 1152 with C a multiple of 16 run on the kernel that keeps the
+    weights in LDS and reads the patches straight into the matrix cores' operand layout: 1 to 6 batches of 3 k blocks
+    (K from 16 to 1152, with a last batch that is partly or mostly empty), C = 16 / 32 / 48 (a k block spans several
+    taps) and 64 / 128 (one tap per k block), unsigned sources (flipped in the loader, non-zero padding value), strides,
+    dilation, asymmetric padding, ragged channel counts, and row counts that do not fill the last workgroup. Above
+    those limits the tiled kernels take over."""
+    rng = np.random.default_rng(77)
+    cases = [
+        # (src shape, weights shape, stride, pad, dilation, dtype)
+        ((1, 5, 5, 16), (1, 1, 1, 16), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),        # K = 16
+        ((2, 9, 8, 16), (7, 3, 3, 16), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8),       # K = 144, taps inside a k block
+        ((1, 11, 13, 32), (63, 3, 3, 32), (2, 2), (1, 0, 2, 1), (1, 1), np.int8),     # K = 288
+        ((2, 8, 8, 48), (64, 3, 3, 48), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8),      # K = 432, dilation 2
+        ((3, 14, 14, 64), (64, 3, 3, 64), (1, 1), (1, 1, 1, 1), (1, 1), np.int8),     # K = 576 (config 4's geometry)
+        ((1, 7, 9, 128), (33, 3, 3, 128), (1, 2), (1, 1, 1, 1), (1, 1), np.uint8),    # K = 1152
+        ((1, 6, 6, 64), (40, 4, 4, 64), (1, 1), (1, 1, 1, 1), (1, 1), np.int8),       # K = 1024
+        ((2, 20, 20, 64), (64, 1, 1, 64), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),     # K = 64, 800 rows
+        ((1, 9, 9, 80), (16, 3, 3, 80), (1, 1), (1, 1, 1, 1), (1, 1), np.int8),       # K = 720, C = 80
+    ]
+    for (shape, wshape, stride, pad, dil, dt) in cases:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(-127, 128, size=wshape).astype(np.int8)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        for per_channel in (True, False):
+            reals = rng.uniform(0.5, 2.0, wshape[0] if per_channel else 1) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            if per_channel and wshape[0] > 2:
+                mult[1], shift[1] = 1 << 29, -1   # a multiplier below 2^30 and a left shift: not the short form
+            want = oracle.conv_nhwc_direct(src, w, bias, zp, 0, mult, shift, ozp, lo, hi, stride, pad, dil)
+            announce("conv few channels", shape, wshape, stride, pad, dil, dt.__name__, "per_channel", per_channel)
+            got, name = run_conv(src, w, bias, zp, 0, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert name.startswith("implicit_narrow"), name
+            np.testing.assert_array_equal(got, want)
+            assert 0.1 < ((want > lo) & (want < hi)).mean()
+    # 65 output channels, K = 1168: the tiled kernel
+    for (shape, wshape) in [((1, 8, 8, 64), (65, 3, 3, 64)), ((1, 6, 6, 16), (8, 9, 9, 16))]:
+        src = rng.integers(-128, 128, size=shape).astype(np.int8)
+        w = rng.integers(-127, 128, size=wshape).astype(np.int8)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multipliers(0.02, rng.uniform(0.01, 0.1, wshape[0]), 1.1)
+        announce("conv beyond few channels", shape, wshape)
+        got, name = run_conv(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4))
+        assert name.startswith("implicit_pp"), name
+        np.testing.assert_array_equal(
+            got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
+
+
 def test_conv_nchw_fixture(golden):
     """The reference oracle's outputs (tests/golden/conv_nhwc.npz) with every tensor handed over channel-planar"""
     g = golden("conv_nhwc.npz")

@@ -64,13 +64,21 @@ enum : int
     QP_COUNT
 };
 
+// min(max(x, lo), hi) for lo <= hi as one instruction (the compiler keeps min and max apart: it cannot know lo <= hi)
+__device__ __forceinline__ int32_t clamp_med3(int32_t x, int32_t lo, int32_t hi)
+{
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(lo), "v"(hi));
+    return r;
+}
+
 __device__ __forceinline__ int32_t fast_requant(int32_t v, int32_t s2, int32_t cmask, int32_t ls, int32_t rsm1,
                                                 int32_t rmask, int32_t result_offset, int32_t lo, int32_t hi)
 {
     const int32_t pre = (int32_t)((uint32_t)v << ls);
     const int32_t h   = __mulhi(pre, s2) + (pre & cmask);
     const int32_t r   = ((h >> rsm1) + rmask) >> rmask;
-    return min(max((int32_t)((uint32_t)r + (uint32_t)result_offset), lo), hi);
+    return clamp_med3((int32_t)((uint32_t)r + (uint32_t)result_offset), lo, hi);
 }
 
 // The common case of fast_requant (cmask = -1, ls = 0, rmask = 1, rsm1 >= 1): the rounding increment and the result
@@ -79,7 +87,7 @@ __device__ __forceinline__ int32_t fast_requant(int32_t v, int32_t s2, int32_t c
 __device__ __forceinline__ int32_t std_requant(int32_t v, int32_t s2, int32_t rsm1, int32_t off2p1, int32_t lo, int32_t hi)
 {
     const int32_t h = __mulhi(v, s2) + v;
-    return min(max(((h >> rsm1) + off2p1) >> 1, lo), hi);
+    return clamp_med3(((h >> rsm1) + off2p1) >> 1, lo, hi);
 }
 
 // (a * b * 2) >> 32 with the single saturating case, without 64-bit VALU arithmetic

@@ -213,8 +213,28 @@ struct PanelProducer
 
 // GWM x GWN consumer waves per group, 2 groups stacked along M, plus NP = GWM*GWN producer waves
 template <int BM, int BN, int BK, int GWM, int GWN, int NS, int EPI, bool FLIP_A, bool CONV>
-__global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
+__global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
 {
+    // What a workgroup needs before its first loads go out is read here, in one batch of scalar loads, and pinned in
+    // registers. Left alone, the compiler fetches kernel arguments where they are first used: five dependent round trips
+    // to memory lay between the start of the kernel and its first load. Only scalars and the three pointers of the
+    // epilogue constants go through the asm: a pointer that did is generic afterwards, and a generic load waits for LDS
+    // and memory alike, so those three come back as pointers to global memory; the operand pointers sit next to pinned
+    // scalars in the argument block and arrive with the same loads.
+    GemmArgs g = g_in;
+    asm volatile(""
+                 : "+s"(g.tiles_m), "+s"(g.tiles_n), "+s"(g.magic_tiles), "+s"(g.magic_group), "+s"(g.tile_magic_ok), "+s"(g.lda),
+                   "+s"(g.a_batch_stride), "+s"(g.Kp), "+s"(g.bp_batch_stride), "+s"(g.M), "+s"(g.N), "+s"(g.K),
+                   "+s"(g.epi.qp_stride), "+s"(g.epi.colvec_batch_stride), "+s"(g.nblocks));
+    typedef const __attribute__((address_space(1))) int32_t *global_i32;
+    uintptr_t u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp, u_fl = (uintptr_t)g.epi.qp_flag;
+    asm volatile("" : "+s"(u_cv), "+s"(u_qp), "+s"(u_fl));
+    if (CONV)
+        asm volatile(""
+                     : "+s"(g.conv.H), "+s"(g.conv.W), "+s"(g.conv.C), "+s"(g.conv.KW), "+s"(g.conv.OW), "+s"(g.conv.OH),
+                       "+s"(g.conv.stride_x), "+s"(g.conv.stride_y), "+s"(g.conv.pad_left), "+s"(g.conv.pad_top), "+s"(g.conv.dil_x),
+                       "+s"(g.conv.dil_y), "+s"(g.conv.magic_C), "+s"(g.conv.magic_KW), "+s"(g.conv.magic_OW), "+s"(g.conv.magic_OH));
+
     constexpr int GW    = GWM * GWN; // waves per consumer group
     constexpr int NW    = 2 * GW;    // consumer waves
     constexpr int NP    = GW;        // producer waves (one per SIMD when GW == 4)
@@ -249,15 +269,15 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
 
     int tm, tn, bz;
     if (g.tile_magic_ok)
-        tile_coords_batched_fast(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, g.magic_tiles, g.magic_group, bz, tm, tn);
+        tile_coords_batched_fast(blockIdx.x, g.nblocks, g.tiles_m, g.tiles_n, g.magic_tiles, g.magic_group, bz, tm, tn);
     else
-        tile_coords_batched(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, bz, tm, tn);
+        tile_coords_batched(blockIdx.x, g.nblocks, g.tiles_m, g.tiles_n, bz, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = (g.K + BK - 1) / BK;
     // which requantisation formula applies was decided on the device when the per-column constants were digested
     int qflag = 1;
-    if (EPI == EPI_FIXEDPOINT && g.epi.qp_flag != nullptr)
-        qflag = __builtin_amdgcn_readfirstlane(*g.epi.qp_flag);
+    if (EPI == EPI_FIXEDPOINT && u_fl != 0)
+        qflag = __builtin_amdgcn_readfirstlane(*(global_i32)u_fl);
     const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
 
     // Barrier protocol (b = number of barriers a wave has executed): consumer group 0 reads stage kt between barriers
@@ -325,8 +345,8 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
             if (idx < NPAR * BN)
             {
                 const int par = idx / BN, col = idx % BN;
-                par_reg[t]    = par == 0 ? g.epi.colvec[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
-                                         : g.epi.qp[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
+                par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
+                                         : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
             }
         }
     }
@@ -441,12 +461,16 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g)
         if (EPI == EPI_FIXEDPOINT)
         {
             char *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
-            if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0)
-                epilogue_store_staged<true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
-                                                                [] { __syncthreads(); });
+            const bool rowv = g.epi.rowvec != nullptr;
+            if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0 && !rowv)
+                epilogue_store_staged<true, false, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                       [] { __syncthreads(); });
+            else if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0)
+                epilogue_store_staged<true, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                      [] { __syncthreads(); });
             else if (g.epi.vec_store16)
-                epilogue_store_staged<false, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
-                                                                 [] { __syncthreads(); });
+                epilogue_store_staged<false, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                       [] { __syncthreads(); });
             else
                 epilogue_store_fast<RS, QS, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
         }
@@ -548,6 +572,7 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
                                 : 0;
     a.magic_tiles = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_tiles) + 1u : 0u;
     a.magic_group = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_group) + 1u : 0u;
+    a.nblocks     = (int32_t)nblocks;
     void    *kargs[] = {&a};
     dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block(c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);

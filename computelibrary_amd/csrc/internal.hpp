@@ -50,6 +50,7 @@ struct GemmArgs
     // launch; tile_magic_ok == 0: divide
     uint32_t magic_tiles, magic_group;
     int32_t  tile_magic_ok;
+    int32_t  nblocks; // workgroups of the launch (gridDim.x is a hidden argument behind this block: one more fetch)
 };
 
 struct MfmaConfig

@@ -321,8 +321,8 @@ __device__ __forceinline__ void epilogue_store_fast(const v4i (&acc)[RS][QS], co
 // 64 different banks) and then written with 16 bytes per lane, BN/16 lanes per output row, so a wave instruction writes
 // whole rows of the tile instead of 16-byte pieces of 16 different rows. All NW consumer waves of the block call this
 // together; `barrier` is executed once between the two phases by every wave of the block. Requires p.vec_store16.
-// stage must not overlap par.
-template <bool STD, int RS, int QS, int BM, int BN, int NW, typename Barrier>
+// stage must not overlap par. ROWV: a per-row term exists (b_offset != 0) and is added.
+template <bool STD, bool ROWV, int RS, int QS, int BM, int BN, int NW, typename Barrier>
 __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], const GemmArgs &g, const int32_t *par,
                                                       char *stage, int m0, int n0, int row_in_tile, int col_in_tile,
                                                       int wave, int lane, int bz, Barrier barrier)
@@ -337,7 +337,7 @@ __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], 
     for (int rs = 0; rs < RS; ++rs)
     {
         const int i = m0 + row_in_tile + rs * 16 + lr;
-        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+        rv[rs]      = (ROWV && rowvec && i < g.M) ? rowvec[i] : 0;
     }
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs)
@@ -360,7 +360,8 @@ __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], 
 #pragma unroll
             for (int t = 0; t < 4; ++t)
             {
-                const int32_t v = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv[rs]);
+                const int32_t v = ROWV ? (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv[rs])
+                                       : (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t]);
                 o[t] = STD ? std_requant(v, s2[t], r1[t], off2p1, p.lo, p.hi)
                            : fast_requant(v, s2[t], cm[t], ls[t], r1[t], rm[t], p.result_offset, p.lo, p.hi);
             }

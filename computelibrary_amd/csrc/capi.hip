@@ -1000,9 +1000,10 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         delete h;
         return 1;
     }
-    // the on-the-fly loader moves 16-byte pieces of one tap: needs C % 16 == 0; it has no row sums: needs b_off == 0
-    // (the F32 epilogue only exists on the dense kernels: that destination always takes the explicit lowering)
-    h->implicit      = !f32 && d.path == 0 && (d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(d, h->geom);
+    // The patch matrix is only materialised on request (path 1) or where the loaders' reciprocal divisions would not be
+    // exact. Channel counts that are not a multiple of 16 take the register-staged kernel, whose loader then looks up
+    // every byte; a weights offset adds a pass over the source for the patches' row sums.
+    h->implicit      = d.path == 0 && conv_fast_div_ok(d, h->geom);
     h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
     if (h->implicit)
         c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
@@ -1076,7 +1077,7 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
         return fail("update cannot switch between per-tensor and per-channel requantisation");
     h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
     c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
-    h->implicit      = h->d.path == 0 && (h->d.C % 16 == 0) && c.b_off_eff() == 0 && conv_fast_div_ok(h->d, h->geom);
+    h->implicit      = h->d.path == 0 && conv_fast_div_ok(h->d, h->geom);
     h->geom.pad_word = ((uint32_t)pad_value & 0xFFu) * 0x01010101u;
     c.fill_byte      = (uint8_t)(pad_value & 0xFF);
     c.kprefix        = h->implicit ? "implicit_" : "im2col+";
@@ -1161,10 +1162,18 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         srcd = h->nhwcSrc.p;
         Dd   = h->nhwcDst.p;
     }
-    if (h->implicit && (((uintptr_t)srcd) & 15) == 0)
+    if (h->implicit)
     {
         GemmArgs g{};
-        c.fill_epi(g.epi, nullptr);
+        c.fill_epi(g.epi, h->has_bias_f32 ? h->biasF.as<float>() : nullptr);
+        if (c.b_off_eff() != 0)
+        {
+            ConvGeom gr = h->geom;
+            gr.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
+            TRY(c.rowvec.ensure(sizeof(int32_t) * (size_t)c.M));
+            HIP_TRY(conv_rowsum_launch(srcd, gr, c.M, c.flip_a, c.b_off_eff(), c.rowvec.as<int32_t>(), s));
+            g.epi.rowvec = c.rowvec.as<int32_t>();
+        }
         g.A = (const int8_t *)srcd, g.lda = 0, g.a_batch_stride = 0;
         g.Bp = c.Bp.as<int8_t>(), g.Kp = c.Kp, g.bp_batch_stride = 0;
         g.D = Dd, g.ldd = c.N, g.d_batch_stride = 0;

@@ -503,8 +503,8 @@ struct DmaEntry
              {MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, false), nullptr}},                                           \
                 {{MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, true)}, \
                  {MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, true)}}, \
-                {{MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, false), nullptr},                                       \
-                 {MI355_DFN(BM, BN, BK, WM, WN, NS, 2, true, false), nullptr}},                                       \
+                {{MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, true)}, \
+                 {MI355_DFN(BM, BN, BK, WM, WN, NS, 2, true, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, true, true)}}, \
         }                                                                                                            \
     }
 

@@ -85,6 +85,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_mfma_kernel(GemmArgs g)
     }
 
     v4i ra[A_CHUNKS], rb[B_CHUNKS];
+    const bool gather = CONV && ((g.conv.C & 15) != 0 || ((uintptr_t)g.A & 15) != 0);
 
     auto load_tiles = [&](int k0)
     {
@@ -95,7 +96,32 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_mfma_kernel(GemmArgs g)
             v4i       v = {0, 0, 0, 0};
             if (k < g.K)
             {
-                if (CONV)
+                if (CONV && gather)
+                {
+                    // channel counts that are not a multiple of 16: a 16-byte piece crosses taps, every byte is looked up
+                    uint32_t w[4] = {0, 0, 0, 0};
+                    for (int b = 0; b < 16; ++b)
+                    {
+                        const int kb = k + b;
+                        uint32_t  byte = 0;
+                        if (kb < g.K)
+                        {
+                            const int tap = kb / g.conv.C;
+                            const int c0  = kb - tap * g.conv.C;
+                            const int ky  = tap / g.conv.KW;
+                            const int kx  = tap - ky * g.conv.KW;
+                            const int iy  = a_iy0[i] + ky * g.conv.dil_y;
+                            const int ix  = a_ix0[i] + kx * g.conv.dil_x;
+                            if (iy >= 0 && iy < g.conv.H && ix >= 0 && ix < g.conv.W)
+                                byte = (uint8_t)A[a_off[i] + ((int64_t)iy * g.conv.W + ix) * g.conv.C + c0] ^ (FLIP_A ? 0x80u : 0u);
+                            else
+                                byte = g.conv.pad_word & 0xFFu;
+                        }
+                        w[b >> 2] |= byte << (8 * (b & 3));
+                    }
+                    v = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                }
+                else if (CONV)
                 {
                     const int tap = k / g.conv.C;
                     const int c0  = k - tap * g.conv.C;
@@ -219,8 +245,8 @@ struct CfgEntry
              {MI355_FN(BM, BN, BK, WM, WN, 0, true, false), nullptr}},                                               \
                 {{MI355_FN(BM, BN, BK, WM, WN, 1, false, false), MI355_FN(BM, BN, BK, WM, WN, 1, false, true)},      \
                  {MI355_FN(BM, BN, BK, WM, WN, 1, true, false), MI355_FN(BM, BN, BK, WM, WN, 1, true, true)}},       \
-                {{MI355_FN(BM, BN, BK, WM, WN, 2, false, false), nullptr},                                           \
-                 {MI355_FN(BM, BN, BK, WM, WN, 2, true, false), nullptr}},                                           \
+                {{MI355_FN(BM, BN, BK, WM, WN, 2, false, false), MI355_FN(BM, BN, BK, WM, WN, 2, false, true)},      \
+                 {MI355_FN(BM, BN, BK, WM, WN, 2, true, false), MI355_FN(BM, BN, BK, WM, WN, 2, true, true)}},       \
         }                                                                                                           \
     }
 

@@ -127,6 +127,8 @@ int qparams_launch(const int32_t *mult, const int32_t *shift, int32_t mult_s, in
 // A pre-pass: optional padded + flipped copy Ap[M][Kp] and/or rowvec[i] = b_off * sum_k(flip(A[i][k]))
 int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
                      int32_t b_off, hipStream_t s);
+// rowvec[m] = b_off * (sum of the sign-normalised patch of output pixel m); g.pad_word = the raw padding byte, replicated
+int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int32_t b_off, int32_t *rowvec, hipStream_t s);
 int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                         int N, const EpiParams &epi, hipStream_t s);
 int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,

@@ -170,6 +170,51 @@ int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream
     return launch_status();
 }
 
+// Row sums of the patch matrix without the patch matrix: rowvec[m] = b_off * sum over the taps and channels of output
+// pixel m of the (sign-normalised) source byte, the padding value where a tap lies outside the image - what
+// CpuGemmLowpMatrixAReductionKernel computes from the im2col buffer
+// (src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:133-204). One thread per output pixel.
+__global__ __launch_bounds__(256) void conv_rowsum_kernel(const uint8_t *__restrict__ src, ConvGeom g, int M, uint8_t flip,
+                                                          uint32_t b_off, int32_t *__restrict__ rowvec)
+{
+    const int m = blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= M)
+        return;
+    const int     ox = m % g.OW, t = m / g.OW, oy = t % g.OH, n = t / g.OH;
+    const int     pad = (int8_t)((g.pad_word & 0xFFu) ^ flip);
+    const int64_t img = (int64_t)n * g.H * g.W * g.C;
+    int32_t       sum = 0;
+    for (int ky = 0; ky < g.KH; ++ky)
+        for (int kx = 0; kx < g.KW; ++kx)
+        {
+            const int iy = oy * g.stride_y - g.pad_top + ky * g.dil_y, ix = ox * g.stride_x - g.pad_left + kx * g.dil_x;
+            if (iy < 0 || iy >= g.H || ix < 0 || ix >= g.W)
+            {
+                sum += pad * g.C;
+                continue;
+            }
+            const uint8_t *p = src + img + ((int64_t)iy * g.W + ix) * g.C;
+            int            c = 0;
+            if ((((uintptr_t)p) & 3) == 0)
+                for (; c + 4 <= g.C; c += 4)
+                {
+                    const uint32_t w = *(const uint32_t *)(p + c) ^ (flip * 0x01010101u);
+                    sum += (int8_t)(w & 0xFF) + (int8_t)((w >> 8) & 0xFF) + (int8_t)((w >> 16) & 0xFF) + (int8_t)(w >> 24);
+                }
+            for (; c < g.C; ++c)
+                sum += (int8_t)(p[c] ^ flip);
+        }
+    rowvec[m] = (int32_t)(b_off * (uint32_t)sum);
+}
+
+// g.pad_word: the raw padding byte replicated
+int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int32_t b_off, int32_t *rowvec, hipStream_t s)
+{
+    conv_rowsum_kernel<<<dim3((M + 255) / 256), dim3(256), 0, s>>>((const uint8_t *)src, g, M, flip ? 0x80 : 0, (uint32_t)b_off,
+                                                                  rowvec);
+    return launch_status();
+}
+
 // The first 64 rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus one piece of
 // padding, zero beyond Kp - the workgroups copy this image into LDS with plain linear transfers
 __global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__restrict__ Bp, int Kp, int chunks,

@@ -165,6 +165,34 @@ def test_conv_few_output_channels_kernel():
             got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
 
 
+def test_conv_weights_offset_and_odd_channels_on_the_fly():
+    """QASYMM8 weights with a non-zero offset need the row sums of the patch matrix (a pass over the source, padding
+    included), channel counts that are not a multiple of 16 the byte-wise loader: neither materialises the patches.
+    Few and many output channels (both kernels), unsigned and signed sources."""
+    rng = np.random.default_rng(88)
+    for (shape, wshape, stride, pad, dil, dt, w_zp) in [
+            ((2, 9, 8, 16), (24, 3, 3, 16), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8, 131),
+            ((1, 12, 11, 64), (80, 3, 3, 64), (2, 1), (1, 0, 1, 2), (1, 1), np.uint8, 120),
+            ((2, 7, 7, 3), (8, 3, 3, 3), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8, 128),
+            ((1, 10, 9, 20), (70, 2, 3, 20), (1, 2), (0, 1, 1, 0), (2, 1), np.int8, 0),
+            ((3, 6, 6, 5), (9, 1, 1, 5), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, 7)]:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w_dt = np.uint8 if w_zp else np.int8
+        w = rng.integers(np.iinfo(w_dt).min + (0 if w_zp else 1), np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        mult, shift = oracle.calculate_quantized_multiplier(float(40.0 / (K ** 0.5 * 74.0 * 74.0)))
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil)
+        assert 0.1 < ((want > lo) & (want < hi)).mean()
+        for device in (True, False):
+            announce("conv offsets / odd channels", shape, wshape, stride, pad, dil, dt.__name__, "w_zp", w_zp, "device", device)
+            got, name = run_conv(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil, device=device)
+            assert name.startswith("implicit_"), name
+            np.testing.assert_array_equal(got, want)
+
+
 def test_conv_nchw_fixture(golden):
     """The reference oracle's outputs (tests/golden/conv_nhwc.npz) with every tensor handed over channel-planar"""
     g = golden("conv_nhwc.npz")
@@ -260,8 +288,11 @@ def test_conv_random_geometry_sweep():
         device = bool(rng.integers(2))
         announce("conv sweep", done, src.shape, w.shape, stride, pad, dil, dt.__name__, "pc", per_channel, "layout", layout,
                  "path", path, "dev", device)
-        got, _ = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dil, path=path, device=device,
-                          layout=layout)
+        got, name = run_conv(src, w, bias, in_zp, w_zp, mult, shift, out_zp, lo, hi, stride, pad, dil, path=path, device=device,
+                             layout=layout)
+        # the patch matrix only exists on request: channel counts off the 16-byte granularity and weights with an offset
+        # (row sums of the patches) run on the on-the-fly loaders too
+        assert name.startswith("implicit_" if path == 0 else "im2col+"), name
         np.testing.assert_array_equal(got, want, err_msg="case %d" % done)
         done += 1
 
@@ -269,7 +300,9 @@ def test_conv_random_geometry_sweep():
 @pytest.mark.parametrize("device", [True, False])
 def test_conv_with_f32_destination(device):
     """QASYMM8_SIGNED input and weights, F32 destination (src/cpu/operators/CpuGemmConv2d.cpp:297-305 of the reference):
-    the im2col matrix through the dequantising GEMM; checked against the oracle's im2col + F32 GEMM, identical bits"""
+    the same on-the-fly lowering as the 8-bit destination with the dequantising epilogue (few output channels: the
+    LDS-resident-weights kernel; 5 input channels: the byte-wise loader; a weights offset: row sums of the patches);
+    checked against the oracle's im2col + F32 GEMM, identical bits"""
     import torch
     rng = np.random.default_rng(91)
     for (B_, H, W, C, OFM, KH, KW, stride, pad, in_zp, w_zp, act, twice) in [
@@ -298,5 +331,6 @@ def test_conv_with_f32_destination(device):
         else:
             cv.prepare(w, bias)
             cv.run(src, out)
+        assert cv.kernel_name.startswith("implicit_"), cv.kernel_name
         cv.close()
         assert np.array_equal(out.reshape(-1, OFM).view(np.uint32), want.view(np.uint32))

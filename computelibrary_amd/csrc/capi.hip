@@ -192,9 +192,11 @@ struct GemmCore
         if (path == MI355_PATH_AUTO)
             // measured: up to 32 rows the streaming kernel always wins; up to 64 rows only while N is small enough
             // that the pipelined kernel would leave most compute units without a tile
-            path = (batch == 1 && (M <= 32 || (M <= SKINNY_MAX_M && N < 8192))) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
-        if (path == MI355_PATH_SKINNY && (M > SKINNY_MAX_M || batch != 1))
-            return fail("skinny path needs M <= %d and batch == 1", SKINNY_MAX_M);
+            // (a batch of small products runs the streaming kernel once per entry: the tiled kernels would spend a 64-row
+            // tile, mostly padding, on each)
+            path = (M <= 32 || (batch == 1 && M <= SKINNY_MAX_M && N < 8192)) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
+        if (path == MI355_PATH_SKINNY && M > SKINNY_MAX_M)
+            return fail("skinny path needs M <= %d", SKINNY_MAX_M);
         if (path == MI355_PATH_SIMPLE)
             kname = "simple";
         else if (path == MI355_PATH_SKINNY)
@@ -289,8 +291,9 @@ struct GemmCore
         }
         if (path == MI355_PATH_SKINNY)
         {
-            TRY(Bs.ensure((size_t)Np * Kp));
-            HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>(), Kp, Np, Bs.as<int8_t>(), s));
+            TRY(Bs.ensure((size_t)nb() * Np * Kp));
+            for (int b = 0; b < nb(); ++b)
+                HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>() + (size_t)b * Np * Kp, Kp, Np, Bs.as<int8_t>() + (size_t)b * Np * Kp, s));
         }
         // few output columns and a short K: the image of the B panel the narrow kernel copies into LDS
         has_narrow = path == MI355_PATH_MFMA && nb() == 1 && N <= 64 && narrow_panel_chunks(K) > 0;
@@ -454,8 +457,18 @@ struct GemmCore
             HIP_TRY(simple_gemm_launch(epi, flip_in_loader, g, batch, s));
         else if (path == MI355_PATH_SKINNY)
         {
-            g.Bp = Bs.as<int8_t>();
-            HIP_TRY(skinny_launch(epi, flip_in_loader, g, s));
+            // one launch per batch entry, each with its own operands and per-column / per-row vectors
+            for (int b = 0; b < batch; ++b)
+            {
+                GemmArgs gb = g;
+                gb.A        = g.A + (int64_t)b * g.a_batch_stride;
+                gb.Bp       = Bs.as<int8_t>() + (b_shared ? 0 : (int64_t)b * Np * Kp);
+                gb.D        = (char *)g.D + (int64_t)b * g.d_batch_stride * (epi == EPI_FIXEDPOINT ? 1 : 4);
+                gb.epi.colvec += (int64_t)b * g.epi.colvec_batch_stride;
+                if (g.epi.rowvec != zeros.as<int32_t>() && g.epi.rowvec != nullptr)
+                    gb.epi.rowvec += (int64_t)b * g.epi.rowvec_batch_stride;
+                HIP_TRY(skinny_launch(epi, flip_in_loader, gb, s));
+            }
         }
         else
         {
@@ -667,8 +680,6 @@ int mi355_gemmlowp_prepare(mi355_gemm_handle *h, const void *B, const int32_t *b
         else
             HIP_TRY(pack_b_launch(src, d.ldb, d.K, d.N, c.Kp, c.Np, c.flip_b, d.b_k_interleave, dst, cs, s));
     }
-    if (c.path == MI355_PATH_SKINNY && nb != 1)
-        return fail("skinny path does not batch");
     TRY(c.finish_prepare((const int32_t *)biasd, (const int32_t *)multd, (const int32_t *)shiftd, s));
     // staging buffers are reused by later calls: make sure the copies out of them have finished
     HIP_TRY(hipStreamSynchronize(s));

@@ -15,7 +15,7 @@ PATHS = [capi.PATH_SIMPLE, capi.PATH_MFMA, capi.PATH_SKINNY]
 
 
 def paths_for(M, batch=1):
-    return [p for p in PATHS if p != capi.PATH_SKINNY or (M <= 64 and batch == 1)]
+    return [p for p in PATHS if p != capi.PATH_SKINNY or M <= 64]
 
 
 def test_device_is_gfx950():
@@ -41,7 +41,7 @@ def test_s32_batched_fixture(golden):
     for n in range(int(g["count"])):
         A, B = g["a%d" % n], g["b%d" % n]
         ao, bo = (int(x) for x in g["off%d" % n])
-        for path in (capi.PATH_SIMPLE, capi.PATH_MFMA):
+        for path in paths_for(A.shape[1], A.shape[0]):
             announce("batched fixture", n, A.shape, B.shape, "path", path)
             got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=path, device=True)
             np.testing.assert_array_equal(got, g["dst%d" % n])
@@ -172,6 +172,33 @@ def test_f16_destination(device):
             want = oracle.gemmlowp_f16(A, B, biasf, ao, bo, scale, 0.0, 6.0, prev=prev)
             np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
             assert 0.05 < (want == 0).mean() < 0.95 or M * N < 400
+
+
+def test_batched_small_products_take_the_streaming_kernel():
+    """Batches of small products (tests/datasets/GEMMLowpFusedOffsetOutputDataset.h:142-162: up to 32 entries of a few
+    rows) run the streaming kernel once per entry instead of a mostly empty tile per entry: per-entry and shared B, a
+    B offset (row sums per entry), padded rows and batch strides, every epilogue."""
+    rng = np.random.default_rng(4242)
+    for (batch, M, N, K, b_batched) in [(3, 4, 5, 2, True), (3, 7, 29, 15, True), (32, 17, 5, 56, True), (32, 13, 19, 256, True),
+                                        (5, 8, 300, 1024, False), (4, 32, 130, 200, True)]:
+        A = rng.integers(-128, 128, size=(batch, M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, size=(batch, K, N) if b_batched else (K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multiplier(float(40.0 / (max(K, 4) ** 0.5 * 74.0 * 74.0)))
+        announce("batched small", (batch, M, N, K), "b_batched", b_batched)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, device=True, lda=K + 4 - K % 4, ldd=N + 1)
+        assert name.startswith("skinny"), name
+        for z in range(batch):
+            np.testing.assert_array_equal(got[z], oracle.gemmlowp_s32(A[z], B[z] if b_batched else B, ao, bo))
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, bo, bias, [mult], [shift], -3, -128, 127, device=True)
+        for z in range(batch):
+            np.testing.assert_array_equal(
+                got[z], oracle.gemmlowp_fixedpoint(A[z], B[z] if b_batched else B, bias, ao, bo, [mult], [shift], -3, -128, 127, np.int8))
+        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, device=False)
+        for z in range(batch):
+            np.testing.assert_array_equal(got[z].view(np.uint32),
+                                          oracle.gemmlowp_f32(A[z], B[z] if b_batched else B, None, ao, bo, 3e-4).view(np.uint32))
 
 
 def test_f16_fixture(golden):

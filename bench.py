@@ -102,6 +102,7 @@ def ceilings_lib():
     l.mi355_ceiling_mfma_lds.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp]
     l.mi355_ceiling_dma.argtypes = [vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]
     l.mi355_ceiling_clock.argtypes = [i64, i64, vp, vp]
+    l.mi355_ceiling_lds_read.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp]
     return l
 
 
@@ -171,6 +172,16 @@ def run_ceilings(torch, args):
         timed("operands read from LDS (64x64 wave tiles), 16x16x64",
               lambda cs, src=src: cl.mi355_ceiling_mfma_lds(src.data_ptr(), 256, 32, sink.data_ptr(), ticks.data_ptr(), cs),
               data)
+    # LDS operand reads alone: 16 KiB per wave and step, 32 steps (config 2 reads 128 KiB per compute unit and step)
+    out["lds_operand_reads"] = []
+    sink2 = torch.zeros(256 * 1024, dtype=torch.int32, device="cuda")
+    for waves in (4, 8, 16):
+        s = time_graph(torch, [lambda cs, waves=waves: cl.mi355_ceiling_lds_read(256, waves, 32, sink2.data_ptr(),
+                                                                                 ticks.data_ptr(), cs)], args.steps)
+        torch.cuda.synchronize()
+        t = ticks.cpu().numpy()
+        out["lds_operand_reads"].append({"waves_per_cu": waves, "us": round(s * 1e6, 3), "loop_clocks": int(t[0]),
+                                         "bytes_per_clock_per_cu": round(32 * waves * 16384 / max(float(t[0]), 1.0), 1)})
     A = bufs[1][:2048 * 4096]
     B = bufs[2][:4096 * 4096]
     out["dma_stream_cfg2"] = []

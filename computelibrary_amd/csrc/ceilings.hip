@@ -5,6 +5,7 @@
 //   mi355_ceiling_read        one streaming pass over a buffer (the skinny GEMM's B stream, without any arithmetic)
 //   mi355_ceiling_mfma        int8 matrix instructions out of registers only (no LDS, no global traffic)
 //   mi355_ceiling_mfma_lds    the same instruction count with every operand read from LDS first (64 x 64 wave tiles)
+//   mi355_ceiling_lds_read    the operand reads of the pipelined GEMM alone (LDS bandwidth per compute unit)
 //   mi355_ceiling_dma         the pipelined GEMM's global -> LDS stream alone (direct-to-LDS loads, 3-slot ring)
 //   mi355_ceiling_clock       shader clock while other work runs: shader-clock ticks over a span of real time
 #include <hip/hip_runtime.h>
@@ -151,6 +152,45 @@ __global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ s
         ticks[0] = t1 - t0, ticks[1] = r1 - r0;
 }
 
+// LDS operand reads alone: `waves` waves per workgroup, each reading the 16 operand blocks of a 64 x 64 wave tile
+// (ds_read_b128, 1 KiB per wave instruction, the conflict-free swizzled addresses of the GEMM) per step, nothing else.
+__global__ __launch_bounds__(1024) void lds_read_kernel(int steps, int *sink, int64_t *ticks)
+{
+    extern __shared__ __attribute__((aligned(1024))) char smem[]; // 48 KiB
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 49152 / 16; i += blockDim.x)
+        ((v4i *)smem)[i] = (v4i){i, lane, wave, 1};
+    __syncthreads();
+    const int      row = lane & 15, lh = lane >> 4;
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+    uint32_t       addr[2][8];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int f = 0; f < 8; ++f)
+        {
+            const int r = (f < 4 ? ((wave >> 1) & 3) * 64 + f * 16 : 256 + (wave & 1) * 64 + (f - 4) * 16) + row;
+            addr[kk][f] = lds0 + (uint32_t)(r * 128 + (((kk * 4 + lh) ^ (r & 7)) << 4));
+        }
+    v4i           acc = {0, 0, 0, 0};
+    const int64_t t0  = __builtin_readcyclecounter(), r0 = wall_clock64();
+    for (int kt = 0; kt < steps; ++kt)
+    {
+        v4i f[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            asm volatile("ds_read_b128 %0, %1" : "=v"(f[i]) : "v"(addr[i >> 3][i & 7]));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc ^= f[i];
+    }
+    const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+    if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
+        ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+}
+
 __device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_addr)
 {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
@@ -280,6 +320,15 @@ int mi355_ceiling_dma(const void *A, const void *B, int64_t ld, int steps, int w
     }
     hipLaunchKernelGGL(dma_kernel, dim3(256), dim3(waves * 64), 3 * 49152, (hipStream_t)stream, (const char *)A, (const char *)B, ld,
                        steps, 32, sink, ticks);
+    return (int)hipGetLastError();
+}
+
+// grid workgroups of `waves` (4, 8, 12 or 16) waves, each wave reading 16 KiB per step; sink: grid * waves * 64 ints
+int mi355_ceiling_lds_read(int grid, int waves, int steps, int *sink, int64_t *ticks, void *stream)
+{
+    if (!sink || grid < 1 || steps < 1 || (waves != 4 && waves != 8 && waves != 12 && waves != 16))
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(lds_read_kernel, dim3(grid), dim3(waves * 64), 49152, (hipStream_t)stream, steps, sink, ticks);
     return (int)hipGetLastError();
 }
 

@@ -15,10 +15,10 @@ GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
 NHWC, NCHW = 0, 1
 
 EXPORTS = [
-    "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_set_strides",
+    "mi355_gemmlowp_create", "mi355_gemmlowp_prepare", "mi355_gemmlowp_update_quant", "mi355_gemmlowp_set_strides", "mi355_gemmlowp_set_strides_3d",
     "mi355_gemmlowp_run", "mi355_gemmlowp_run_noalloc", "mi355_gemmlowp_noalloc_workspace_bytes",
     "mi355_gemmlowp_destroy", "mi355_gemmlowp_kernel_name", "mi355_output_stage_run", "mi355_conv_create",
-    "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_set_strides", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
+    "mi355_conv_prepare", "mi355_conv_update_quant", "mi355_conv_set_strides", "mi355_conv_set_strides_nd", "mi355_conv_run", "mi355_conv_out_dims", "mi355_conv_destroy", "mi355_conv_kernel_name",
     "mi355_im2col_nhwc_run", "mi355_last_error", "mi355_device_info",
 ]
 
@@ -37,7 +37,8 @@ class GemmDesc(C.Structure):
                 ("a_offset", C.c_int32), ("b_offset", C.c_int32), ("requant", Requant),
                 ("scale", C.c_float), ("act_min", C.c_float), ("act_max", C.c_float),
                 ("path", C.c_int32), ("b_transposed", C.c_int32), ("b_k_interleave", C.c_int32),
-                ("flags", C.c_int32)]
+                ("flags", C.c_int32), ("a_plane_rows", C.c_int32), ("d_plane_rows", C.c_int32),
+                ("a_plane_stride", C.c_int64), ("d_plane_stride", C.c_int64)]
 
 
 class OutputStageDesc(C.Structure):
@@ -55,7 +56,10 @@ class ConvDesc(C.Structure):
                                                                   ("weights_pixel_stride", C.c_int64),
                                                                   ("dst_pixel_stride", C.c_int64),
                                                                   ("scale", C.c_float), ("act_min", C.c_float),
-                                                                  ("act_max", C.c_float), ("flags", C.c_int32)]
+                                                                  ("act_max", C.c_float), ("flags", C.c_int32)] + [
+                                                                      (n, C.c_int64) for n in
+                                                                      ("src_stride2", "src_stride3", "weights_stride2",
+                                                                       "weights_stride3", "dst_stride2", "dst_stride3")]
 
 
 _lib = None
@@ -79,6 +83,7 @@ def lib():
         l.mi355_gemmlowp_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
         l.mi355_gemmlowp_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(Requant), C.c_float, vp]
         l.mi355_gemmlowp_set_strides.argtypes = [vp] + [C.c_int64] * 6
+        l.mi355_gemmlowp_set_strides_3d.argtypes = [vp] + [C.c_int64] * 8
         l.mi355_gemmlowp_run.argtypes = [vp, vp, f32p, vp, vp]
         l.mi355_gemmlowp_run_noalloc.argtypes = [vp, vp, f32p, vp, vp]
         l.mi355_gemmlowp_noalloc_workspace_bytes.argtypes = []
@@ -92,6 +97,7 @@ def lib():
         l.mi355_conv_prepare.argtypes = [vp, vp, i32p, i32p, i32p, vp]
         l.mi355_conv_run.argtypes = [vp, vp, vp, vp]
         l.mi355_conv_set_strides.argtypes = [vp, C.c_int64, C.c_int64, C.c_int64]
+        l.mi355_conv_set_strides_nd.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.mi355_conv_update_quant.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Requant), i32p, i32p, vp]
         l.mi355_conv_out_dims.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         l.mi355_conv_out_dims.restype = None
@@ -147,12 +153,17 @@ class Gemm:
 
     def __init__(self, M, N, K, a_dtype, b_dtype, dst_dtype, epilogue, a_offset=0, b_offset=0, rq=None, scale=1.0,
                  act_min=-np.inf, act_max=np.inf, batch=1, b_batched=False, lda=None, ldb=None, ldd=None,
-                 path=PATH_AUTO, b_transposed=False, b_k_interleave=0, flags=0):
+                 path=PATH_AUTO, b_transposed=False, b_k_interleave=0, flags=0, a_planes=None, d_planes=None,
+                 a_batch_stride=None, d_batch_stride=None):
+        """a_planes / d_planes: (rows per plane, plane stride) of matrices whose rows come as planes with gaps between
+        them (A: bytes, D: elements); the batch strides then have to be given too."""
         lda, ldb, ldd = lda or K, ldb or (K if b_transposed else N), ldd or N
         b_rows = N if b_transposed else K
-        self.desc = GemmDesc(M, N, K, batch, a_dtype, b_dtype, dst_dtype, epilogue, lda, ldb, ldd, M * lda,
-                             b_rows * ldb if b_batched else 0, M * ldd, a_offset, b_offset, rq or requant(), scale,
-                             act_min, act_max, path, 1 if b_transposed else 0, b_k_interleave, flags)
+        ap, dp = a_planes or (0, 0), d_planes or (0, 0)
+        self.desc = GemmDesc(M, N, K, batch, a_dtype, b_dtype, dst_dtype, epilogue, lda, ldb, ldd,
+                             a_batch_stride or M * lda, b_rows * ldb if b_batched else 0, d_batch_stride or M * ldd,
+                             a_offset, b_offset, rq or requant(), scale, act_min, act_max, path,
+                             1 if b_transposed else 0, b_k_interleave, flags, ap[0], dp[0], ap[1], dp[1])
         self._h = C.c_void_p()
         _check(lib().mi355_gemmlowp_create(C.byref(self.desc), C.byref(self._h)))
 
@@ -162,6 +173,10 @@ class Gemm:
 
     def prepare(self, B, bias=None, mult=None, shift=None, stream=None):
         _check(lib().mi355_gemmlowp_prepare(self._h, ptr(B), ptr(bias), ptr(mult), ptr(shift), stream))
+
+    def set_strides_3d(self, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride, a_plane_stride, d_plane_stride):
+        _check(lib().mi355_gemmlowp_set_strides_3d(self._h, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride,
+                                                   a_plane_stride, d_plane_stride))
 
     def update_quant(self, a_offset, b_offset, rq, scale=1.0, stream=None):
         _check(lib().mi355_gemmlowp_update_quant(self._h, a_offset, b_offset, C.byref(rq) if rq else None, scale,
@@ -202,11 +217,13 @@ def output_stage(src, bias, dst, rq, stream=None, ld_src=None, ld_dst=None):
 
 def conv_desc(batch, H, W, Cc, OFM, KH, KW, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), src_dtype=S8,
               weights_dtype=S8, dst_dtype=S8, src_offset=0, weights_offset=0, pad_value=0, rq=None, path=0, layout=0, pixel_strides=(0, 0, 0), scale=1.0,
-              act=(-np.inf, np.inf), flags=0):
+              act=(-np.inf, np.inf), flags=0, outer_strides=((0, 0), (0, 0), (0, 0))):
+    """pixel_strides: strides_in_bytes()[1] of src, weights and dst; outer_strides: their ([2], [3]); 0 = no gap."""
     return ConvDesc(batch, H, W, Cc, OFM, KH, KW, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0],
                     dilation[1], src_dtype, weights_dtype, dst_dtype, src_offset, weights_offset, pad_value,
                     rq or requant(), path, layout, pixel_strides[0], pixel_strides[1], pixel_strides[2], scale,
-                    act[0], act[1], flags)
+                    act[0], act[1], flags, outer_strides[0][0], outer_strides[0][1], outer_strides[1][0],
+                    outer_strides[1][1], outer_strides[2][0], outer_strides[2][1])
 
 
 class Conv:
@@ -233,6 +250,11 @@ class Conv:
 
     def set_strides(self, src_pixel_stride, weights_pixel_stride, dst_pixel_stride):
         _check(lib().mi355_conv_set_strides(self._h, src_pixel_stride, weights_pixel_stride, dst_pixel_stride))
+
+    def set_strides_nd(self, src, weights, dst):
+        """Each argument: (strides_in_bytes()[1], [2], [3]) of that tensor, 0 = no gap."""
+        a3 = C.c_int64 * 3
+        _check(lib().mi355_conv_set_strides_nd(self._h, a3(*src), a3(*weights), a3(*dst)))
 
     def run(self, src, dst, stream=None):
         _check(lib().mi355_conv_run(self._h, ptr(src), ptr(dst), stream))

@@ -543,8 +543,35 @@ struct mi355_gemm_handle
     GemmCore        core;
     DevBuf          stageA, stageB, stageD, stageBiasF, stageBias, stageMult, stageShift;
     DevBuf          wsF32; // MI355_F16 destination: the dense F32 matrix the kernels write
+    DevBuf          denseA, denseD; // matrices handed over as planes with gaps between them, without the gaps
     PtrKind         kindA, kindD, kindBiasF; // host or device memory, per argument of run()
+    bool a_planes() const { return d.a_plane_rows > 0 && d.a_plane_stride != (int64_t)d.a_plane_rows * d.lda; }
+    bool d_planes() const { return d.d_plane_rows > 0 && d.d_plane_stride != (int64_t)d.d_plane_rows * d.ldd; }
 };
+
+static int check_planes(const mi355_gemm_desc &d)
+{
+    if (d.a_plane_rows < 0 || d.d_plane_rows < 0 || (d.a_plane_rows > 0 && d.M % d.a_plane_rows != 0) ||
+        (d.d_plane_rows > 0 && d.M % d.d_plane_rows != 0))
+        return fail("plane_rows must divide M");
+    if (d.a_plane_rows > 0 && d.a_plane_stride < (int64_t)(d.a_plane_rows - 1) * d.lda + d.K)
+        return fail("A plane stride smaller than one plane");
+    if (d.d_plane_rows > 0 && d.d_plane_stride < (int64_t)(d.d_plane_rows - 1) * d.ldd + d.N)
+        return fail("D plane stride smaller than one plane");
+    return 0;
+}
+
+// bytes (A) / elements (D) from the first element of a batch entry's matrix to one past its last
+static int64_t a_span(const mi355_gemm_desc &d)
+{
+    return d.a_plane_rows > 0 ? (int64_t)(d.M / d.a_plane_rows - 1) * d.a_plane_stride + (int64_t)(d.a_plane_rows - 1) * d.lda + d.K
+                              : (int64_t)(d.M - 1) * d.lda + d.K;
+}
+static int64_t d_span(const mi355_gemm_desc &d)
+{
+    return d.d_plane_rows > 0 ? (int64_t)(d.M / d.d_plane_rows - 1) * d.d_plane_stride + (int64_t)(d.d_plane_rows - 1) * d.ldd + d.N
+                              : (int64_t)(d.M - 1) * d.ldd + d.N;
+}
 
 struct mi355_conv_handle
 {
@@ -554,6 +581,7 @@ struct mi355_conv_handle
     bool            implicit = false;
     DevBuf          stageSrc, stageW, stageDst, stageBias, stageMult, stageShift, cols;
     DevBuf          nhwcSrc, nhwcW, nhwcDst; // MI355_NCHW: the tensors in the kernels' layout
+    DevBuf          denseSrc, denseW, denseDst; // tensors that came with gaps, without them
     DevBuf          biasF;                   // F32 destination: the float bias
     bool            has_bias_f32 = false;
     PtrKind         kindSrc, kindDst; // host or device memory, per argument of run()
@@ -625,7 +653,8 @@ int mi355_gemmlowp_create(const mi355_gemm_desc *desc, mi355_gemm_handle **out)
         return fail("unknown flag bits 0x%x", d.flags);
     if ((d.flags & MI355_GEMM_ACCUMULATE) && d.epilogue == MI355_EPI_FIXEDPOINT)
         return fail("accumulation is only possible into an S32 or F32 destination");
-    if (d.batch > 1 && (d.a_batch_stride < (int64_t)(d.M - 1) * d.lda + d.K || d.d_batch_stride < (int64_t)(d.M - 1) * d.ldd + d.N))
+    TRY(check_planes(d));
+    if (d.batch > 1 && (d.a_batch_stride < a_span(d) || d.d_batch_stride < d_span(d)))
         return fail("batch stride smaller than one matrix");
     if (d.batch > 1 && d.b_batch_stride != 0 &&
         d.b_batch_stride < (d.b_transposed ? (int64_t)(d.N - 1) * d.ldb + d.K : (int64_t)(d.K - 1) * d.ldb + d.N))
@@ -710,24 +739,45 @@ int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t 
     return 0;
 }
 
-int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
-                               int64_t b_batch_stride, int64_t d_batch_stride)
+static int set_gemm_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                            int64_t b_batch_stride, int64_t d_batch_stride, int64_t a_plane_stride, int64_t d_plane_stride)
 {
-    if (!h)
-        return fail("null argument");
-    mi355_gemm_desc &d = h->d;
+    const mi355_gemm_desc &d = h->d;
     if (lda < d.K || ldb < (d.b_transposed ? d.K : d.N) || ldd < d.N)
         return fail("row stride smaller than the row");
-    if (d.batch > 1 && (a_batch_stride < (int64_t)(d.M - 1) * lda + d.K || d_batch_stride < (int64_t)(d.M - 1) * ldd + d.N))
+    mi355_gemm_desc n = d;
+    n.lda = lda, n.ldb = ldb, n.ldd = ldd;
+    n.a_plane_stride = a_plane_stride, n.d_plane_stride = d_plane_stride;
+    n.a_batch_stride = a_batch_stride, n.b_batch_stride = b_batch_stride, n.d_batch_stride = d_batch_stride;
+    TRY(check_planes(n));
+    if (d.batch > 1 && (a_batch_stride < a_span(n) || d_batch_stride < d_span(n)))
         return fail("batch stride smaller than one matrix");
     if (d.batch > 1 && (b_batch_stride == 0) != h->core.b_shared)
         return fail("set_strides cannot switch between one shared B and one B per batch entry");
     if (d.batch > 1 && b_batch_stride != 0 &&
         b_batch_stride < (d.b_transposed ? (int64_t)(d.N - 1) * ldb + d.K : (int64_t)(d.K - 1) * ldb + d.N))
         return fail("B batch stride smaller than one matrix");
-    d.lda = lda, d.ldb = ldb, d.ldd = ldd;
-    d.a_batch_stride = a_batch_stride, d.b_batch_stride = b_batch_stride, d.d_batch_stride = d_batch_stride;
+    h->d = n;
     return 0;
+}
+
+int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                               int64_t b_batch_stride, int64_t d_batch_stride)
+{
+    if (!h)
+        return fail("null argument");
+    // planes keep following one another without a gap under the new row strides
+    return set_gemm_strides(h, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride,
+                            (int64_t)h->d.a_plane_rows * lda, (int64_t)h->d.d_plane_rows * ldd);
+}
+
+int mi355_gemmlowp_set_strides_3d(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                                  int64_t b_batch_stride, int64_t d_batch_stride, int64_t a_plane_stride,
+                                  int64_t d_plane_stride)
+{
+    if (!h)
+        return fail("null argument");
+    return set_gemm_strides(h, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride, a_plane_stride, d_plane_stride);
 }
 
 int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream)
@@ -741,8 +791,8 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
         return fail("float bias is only valid with the F32 epilogue");
     const bool   f16     = d.dst_dtype == MI355_F16;
     const size_t esz     = d.dst_dtype == MI355_S32 || d.dst_dtype == MI355_F32 ? 4 : (f16 ? 2 : 1);
-    const size_t a_bytes = (size_t)(d.batch - 1) * d.a_batch_stride + (size_t)(d.M - 1) * d.lda + d.K;
-    const size_t d_elems = (size_t)(d.batch - 1) * d.d_batch_stride + (size_t)(d.M - 1) * d.ldd + d.N;
+    const size_t a_bytes = (size_t)(d.batch - 1) * d.a_batch_stride + (size_t)a_span(d);
+    const size_t d_elems = (size_t)(d.batch - 1) * d.d_batch_stride + (size_t)d_span(d);
     const void  *Ad, *bfd;
     TRY(to_device(A, a_bytes, h->stageA, s, &Ad, &h->kindA));
     TRY(to_device(bias_f32, sizeof(float) * d.N, h->stageBiasF, s, &bfd, &h->kindBiasF));
@@ -752,8 +802,30 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     {
         TRY(h->stageD.ensure(d_elems * esz));
         Dd = h->stageD.p;
-        if (c.accumulate || d.ldd != d.N || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
+        if (c.accumulate || d.ldd != d.N || h->d_planes() || (d.batch > 1 && d.d_batch_stride != (int64_t)d.M * d.ldd))
             HIP_TRY(hipMemcpyAsync(Dd, D, d_elems * esz, hipMemcpyHostToDevice, s)); // previous values / padding
+    }
+    const bool staged_in = Ad != A || bfd != bias_f32;
+    // planes with gaps between them: the kernels see dense copies
+    int64_t lda = d.lda, a_bs = d.a_batch_stride, ldd = d.ldd, d_bs = d.d_batch_stride;
+    void   *Dplanes = nullptr;
+    if (h->a_planes())
+    {
+        const int64_t row = round_up(d.K, 16);
+        TRY(h->denseA.ensure((size_t)d.batch * d.M * row));
+        HIP_TRY(restride_nd_launch(Ad, h->denseA.p, d.K, d.a_plane_rows, d.M / d.a_plane_rows, d.batch,
+                                   RestrideSteps{{d.lda, d.a_plane_stride, d.a_batch_stride}},
+                                   RestrideSteps{{row, row * d.a_plane_rows, row * d.M}}, s));
+        Ad = h->denseA.p, lda = row, a_bs = row * d.M;
+    }
+    const RestrideSteps d_given{{d.ldd * (int64_t)esz, d.d_plane_stride * (int64_t)esz, d.d_batch_stride * (int64_t)esz}};
+    const RestrideSteps d_dense{{d.N * (int64_t)esz, d.N * (int64_t)esz * d.d_plane_rows, d.N * (int64_t)esz * d.M}};
+    if (h->d_planes())
+    {
+        TRY(h->denseD.ensure((size_t)d.batch * d.M * d.N * esz));
+        Dplanes = Dd, Dd = h->denseD.p, ldd = d.N, d_bs = (int64_t)d.M * d.N;
+        if (c.accumulate) // the previous values
+            HIP_TRY(restride_nd_launch(Dplanes, Dd, (int)(d.N * esz), d.d_plane_rows, d.M / d.d_plane_rows, d.batch, d_given, d_dense, s));
     }
     if (f16)
     {
@@ -765,20 +837,25 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
         const float lo = c.act_min, hi = c.act_max;
         if (acc)
             c.accumulate = false, c.act_twice = false, c.act_min = -INFINITY, c.act_max = INFINITY;
-        const int rc = c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, ws, d.N, (int64_t)d.M * d.N, (const float *)bfd, s);
+        const int rc = c.run_dense((const int8_t *)Ad, lda, a_bs, ws, d.N, (int64_t)d.M * d.N, (const float *)bfd, s);
         c.accumulate = acc, c.act_twice = twice, c.act_min = lo, c.act_max = hi;
         if (rc)
             return rc;
-        HIP_TRY(f32_to_f16_launch(ws, Dd, d.batch, d.M, d.N, d.ldd, d.d_batch_stride, acc, lo, hi, s));
+        HIP_TRY(f32_to_f16_launch(ws, Dd, d.batch, d.M, d.N, ldd, d_bs, acc, lo, hi, s));
     }
     else
-        TRY(c.run_dense((const int8_t *)Ad, d.lda, d.a_batch_stride, Dd, d.ldd, d.d_batch_stride, (const float *)bfd, s));
+        TRY(c.run_dense((const int8_t *)Ad, lda, a_bs, Dd, ldd, d_bs, (const float *)bfd, s));
+    if (Dplanes)
+    {
+        HIP_TRY(restride_nd_launch(Dd, Dplanes, (int)(d.N * esz), d.d_plane_rows, d.M / d.d_plane_rows, d.batch, d_dense, d_given, s));
+        Dd = Dplanes;
+    }
     if (d_host)
     {
         HIP_TRY(hipMemcpyAsync(D, Dd, d_elems * esz, hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
     }
-    else if (Ad != A || bfd != bias_f32)
+    else if (staged_in)
         HIP_TRY(hipStreamSynchronize(s)); // staged inputs must be consumed before the caller may reuse them
     return 0;
 }
@@ -821,6 +898,8 @@ int mi355_gemmlowp_run_noalloc(mi355_gemm_handle *h, const void *A, const float 
         return fail("float bias is only valid with the F32 epilogue");
     if (d.dst_dtype == MI355_F16)
         return fail("mi355_gemmlowp_run_noalloc does not write F16 destinations (they need a float matrix as workspace)");
+    if (h->a_planes() || h->d_planes())
+        return fail("mi355_gemmlowp_run_noalloc does not take planes with gaps between them (they need dense copies)");
     if (!h->kindA.is_device(A) || !h->kindD.is_device(D) || (bias_f32 && !h->kindBiasF.is_device(bias_f32)))
         return fail("mi355_gemmlowp_run_noalloc takes device memory only");
     void *ws = nullptr;
@@ -837,7 +916,7 @@ void mi355_gemmlowp_destroy(mi355_gemm_handle *h)
         return;
     h->core.release();
     h->stageA.release(), h->stageB.release(), h->stageD.release(), h->stageBiasF.release(), h->stageBias.release();
-    h->stageMult.release(), h->stageShift.release(), h->wsF32.release();
+    h->stageMult.release(), h->stageShift.release(), h->wsF32.release(), h->denseA.release(), h->denseD.release();
     delete h;
 }
 
@@ -944,6 +1023,57 @@ void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW)
         *OW = g.OW;
 }
 
+// One tensor of a convolution as runs of contiguous bytes: seg bytes per run, n1 x n2 x n3 runs along dimensions 1..3 of
+// the tensor, 'given' the caller's byte strides of those dimensions (0 resolved to "no gap"), 'dense' the gap-free ones
+struct ConvTensorSteps
+{
+    int           seg = 0;
+    int64_t       n1 = 0, n2 = 0, n3 = 0;
+    RestrideSteps given{}, dense{};
+    bool          padded = false;
+    size_t        extent = 0, bytes = 0; // bytes spanned from the first element with and without the gaps
+};
+
+static int conv_tensor_steps(const char *name, int64_t seg, int64_t n1, int64_t n2, int64_t n3, int64_t s1, int64_t s2,
+                             int64_t s3, ConvTensorSteps &t)
+{
+    const int64_t g1 = s1 ? s1 : seg, g2 = s2 ? s2 : g1 * n1, g3 = s3 ? s3 : g2 * n2;
+    if (g1 < seg || g2 < g1 * n1 || g3 < g2 * n2)
+        return fail("%s: a stride is smaller than what it steps over", name);
+    t.seg = (int)seg, t.n1 = n1, t.n2 = n2, t.n3 = n3;
+    t.given  = RestrideSteps{{g1, g2, g3}};
+    t.dense  = RestrideSteps{{seg, seg * n1, seg * n1 * n2}};
+    t.padded = g1 != t.dense.st[0] || g2 != t.dense.st[1] || g3 != t.dense.st[2];
+    t.extent = (size_t)((n1 - 1) * g1 + (n2 - 1) * g2 + (n3 - 1) * g3 + seg);
+    t.bytes  = (size_t)(seg * n1 * n2 * n3);
+    return 0;
+}
+
+static int conv_src_steps(const mi355_conv_desc &d, ConvTensorSteps &t)
+{
+    return d.layout == MI355_NHWC
+               ? conv_tensor_steps("src", d.C, d.W, d.H, d.batch, d.src_pixel_stride, d.src_stride2, d.src_stride3, t)
+               : conv_tensor_steps("src", d.W, d.H, d.C, d.batch, d.src_pixel_stride, d.src_stride2, d.src_stride3, t);
+}
+
+static int conv_weights_steps(const mi355_conv_desc &d, ConvTensorSteps &t)
+{
+    return d.layout == MI355_NHWC ? conv_tensor_steps("weights", d.C, d.KW, d.KH, d.OFM, d.weights_pixel_stride,
+                                                      d.weights_stride2, d.weights_stride3, t)
+                                  : conv_tensor_steps("weights", d.KW, d.KH, d.C, d.OFM, d.weights_pixel_stride,
+                                                      d.weights_stride2, d.weights_stride3, t);
+}
+
+static int conv_dst_steps(const mi355_conv_desc &d, ConvTensorSteps &t)
+{
+    ConvGeom g;
+    conv_geom(d, g);
+    const int64_t esz = d.dst_dtype == MI355_F32 ? 4 : 1;
+    return d.layout == MI355_NHWC
+               ? conv_tensor_steps("dst", d.OFM * esz, g.OW, g.OH, d.batch, d.dst_pixel_stride, d.dst_stride2, d.dst_stride3, t)
+               : conv_tensor_steps("dst", g.OW * esz, g.OH, d.OFM, d.batch, d.dst_pixel_stride, d.dst_stride2, d.dst_stride3, t);
+}
+
 static int conv_check(const mi355_conv_desc &d)
 {
     if (d.batch < 1 || d.H < 1 || d.W < 1 || d.C < 1 || d.OFM < 1 || d.KH < 1 || d.KW < 1)
@@ -956,20 +1086,19 @@ static int conv_check(const mi355_conv_desc &d)
         return fail("convolution source and weights must be 8-bit, the destination 8-bit or F32");
     if (d.dst_dtype == MI355_F32)
     {
-        if (d.layout != MI355_NHWC || (d.dst_pixel_stride != 0 && d.dst_pixel_stride != (int64_t)d.OFM * 4))
-            return fail("the F32 destination of a convolution must be dense NHWC");
         if ((d.flags & ~MI355_GEMM_ACT_TWICE) != 0)
             return fail("unknown flag bits 0x%x", d.flags);
     }
     if (d.layout != MI355_NHWC && d.layout != MI355_NCHW)
         return fail("unknown layout %d", d.layout);
-    if ((d.src_pixel_stride != 0 && d.src_pixel_stride < d.C) || (d.weights_pixel_stride != 0 && d.weights_pixel_stride < d.C) ||
-        (d.dst_pixel_stride != 0 && d.dst_pixel_stride < (int64_t)d.OFM * (d.dst_dtype == MI355_F32 ? 4 : 1)))
-        return fail("pixel stride smaller than the pixel");
-    if (d.layout != MI355_NHWC && ((d.src_pixel_stride != 0 && d.src_pixel_stride != d.C) ||
-                                   (d.weights_pixel_stride != 0 && d.weights_pixel_stride != d.C) ||
-                                   (d.dst_pixel_stride != 0 && d.dst_pixel_stride != d.OFM)))
-        return fail("pixel strides are an NHWC notion");
+    ConvGeom g;
+    conv_geom(d, g);
+    if (g.OH < 1 || g.OW < 1)
+        return fail("the kernel does not fit into the padded image");
+    ConvTensorSteps t;
+    TRY(conv_src_steps(d, t));
+    TRY(conv_weights_steps(d, t));
+    TRY(conv_dst_steps(d, t));
     return 0;
 }
 
@@ -1044,15 +1173,14 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const void *bi
         }
         bias = nullptr;
     }
-    const int64_t wps   = h->d.weights_pixel_stride;
-    const int64_t wtaps = (int64_t)c.N * h->d.KH * h->d.KW;
-    const bool    w_pad = wps != 0 && wps != h->d.C;
-    TRY(to_device(weights, w_pad ? (size_t)((wtaps - 1) * wps + h->d.C) : (size_t)c.N * c.K, h->stageW, s, &wd));
-    if (w_pad)
+    ConvTensorSteps wt;
+    TRY(conv_weights_steps(h->d, wt));
+    TRY(to_device(weights, wt.extent, h->stageW, s, &wd));
+    if (wt.padded)
     {
-        TRY(h->nhwcW.ensure((size_t)c.N * c.K));
-        HIP_TRY(restride_launch(wd, h->nhwcW.p, wtaps, h->d.C, wps, h->d.C, s));
-        wd = h->nhwcW.p;
+        TRY(h->denseW.ensure(wt.bytes));
+        HIP_TRY(restride_nd_launch(wd, h->denseW.p, wt.seg, wt.n1, wt.n2, wt.n3, wt.given, wt.dense, s));
+        wd = h->denseW.p;
     }
     if (h->d.layout == MI355_NCHW)
     {
@@ -1116,8 +1244,18 @@ int mi355_conv_set_strides(mi355_conv_handle *h, int64_t src_pixel_stride, int64
 {
     if (!h)
         return fail("null argument");
+    const int64_t a[3] = {src_pixel_stride, 0, 0}, b[3] = {weights_pixel_stride, 0, 0}, c[3] = {dst_pixel_stride, 0, 0};
+    return mi355_conv_set_strides_nd(h, a, b, c);
+}
+
+int mi355_conv_set_strides_nd(mi355_conv_handle *h, const int64_t src[3], const int64_t weights[3], const int64_t dst[3])
+{
+    if (!h || !src || !weights || !dst)
+        return fail("null argument");
     mi355_conv_desc d = h->d;
-    d.src_pixel_stride = src_pixel_stride, d.weights_pixel_stride = weights_pixel_stride, d.dst_pixel_stride = dst_pixel_stride;
+    d.src_pixel_stride = src[0], d.src_stride2 = src[1], d.src_stride3 = src[2];
+    d.weights_pixel_stride = weights[0], d.weights_stride2 = weights[1], d.weights_stride3 = weights[2];
+    d.dst_pixel_stride = dst[0], d.dst_stride2 = dst[1], d.dst_stride3 = dst[2];
     TRY(conv_check(d));
     h->d = d;
     return 0;
@@ -1132,20 +1270,18 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     const mi355_conv_desc &d = h->d;
     if (!c.prepared)
         return fail("run before prepare");
-    const size_t  desz      = c.epi == EPI_F32 ? 4 : 1;
-    const size_t  src_bytes = (size_t)d.batch * d.H * d.W * d.C, dst_bytes = (size_t)c.M * c.N * desz;
-    const int64_t pixels    = (int64_t)d.batch * d.H * d.W;
-    const bool    s_pad     = d.src_pixel_stride != 0 && d.src_pixel_stride != d.C;
-    const bool    d_pad     = d.dst_pixel_stride != 0 && d.dst_pixel_stride != (int64_t)d.OFM * (int64_t)desz;
-    const size_t  dst_ext   = d_pad ? (size_t)((int64_t)(c.M - 1) * d.dst_pixel_stride + c.N) : dst_bytes;
-    const void   *srcd;
-    TRY(to_device(src, s_pad ? (size_t)((pixels - 1) * d.src_pixel_stride + d.C) : src_bytes, h->stageSrc, s, &srcd,
-                  &h->kindSrc));
+    ConvTensorSteps st, dt;
+    TRY(conv_src_steps(d, st));
+    TRY(conv_dst_steps(d, dt));
+    const size_t src_bytes = st.bytes, dst_bytes = dt.bytes, dst_ext = dt.extent;
+    const bool   s_pad = st.padded, d_pad = dt.padded;
+    const void  *srcd;
+    TRY(to_device(src, st.extent, h->stageSrc, s, &srcd, &h->kindSrc));
     if (s_pad)
     {
-        TRY(h->nhwcSrc.ensure(src_bytes));
-        HIP_TRY(restride_launch(srcd, h->nhwcSrc.p, pixels, d.C, d.src_pixel_stride, d.C, s));
-        srcd = h->nhwcSrc.p;
+        TRY(h->denseSrc.ensure(src_bytes));
+        HIP_TRY(restride_nd_launch(srcd, h->denseSrc.p, st.seg, st.n1, st.n2, st.n3, st.given, st.dense, s));
+        srcd = h->denseSrc.p;
     }
     const bool d_host = !h->kindDst.is_device(dst);
     void      *Dd     = dst;
@@ -1159,8 +1295,8 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     void *Dpadded = Dd;
     if (d_pad)
     {
-        TRY(h->nhwcDst.ensure(dst_bytes));
-        Dd = h->nhwcDst.p;
+        TRY(h->denseDst.ensure(dst_bytes));
+        Dd = h->denseDst.p;
     }
     const bool nchw   = d.layout == MI355_NCHW;
     void      *Dfinal = Dd;
@@ -1205,12 +1341,12 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
     }
     if (nchw)
     {
-        HIP_TRY(transpose_bytes_launch(Dd, Dfinal, d.batch, h->geom.OH * h->geom.OW, c.N, s));
+        HIP_TRY((c.epi == EPI_F32 ? transpose_words_launch : transpose_bytes_launch)(Dd, Dfinal, d.batch, h->geom.OH * h->geom.OW, c.N, s));
         Dd = Dfinal;
     }
     if (d_pad)
     {
-        HIP_TRY(restride_launch(Dd, Dpadded, c.M, c.N, c.N, d.dst_pixel_stride, s));
+        HIP_TRY(restride_nd_launch(Dd, Dpadded, dt.seg, dt.n1, dt.n2, dt.n3, dt.dense, dt.given, s));
         Dd = Dpadded;
     }
     if (d_host)
@@ -1231,6 +1367,7 @@ void mi355_conv_destroy(mi355_conv_handle *h)
     h->stageSrc.release(), h->stageW.release(), h->stageDst.release(), h->stageBias.release();
     h->stageMult.release(), h->stageShift.release(), h->cols.release();
     h->nhwcSrc.release(), h->nhwcW.release(), h->nhwcDst.release(), h->biasF.release();
+    h->denseSrc.release(), h->denseW.release(), h->denseDst.release();
     delete h;
 }
 

@@ -135,11 +135,19 @@ int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *b
                             int N, const EpiParams &epi, hipStream_t s);
 // [batch][R][C] bytes -> [batch][C][R]
 int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
+int transpose_words_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
 // dst[s * dst_stride + c] = src[s * src_stride + c] for s < segments, c < seg (bytes)
 // dense F32 [batch][M][N] -> F16 destination (row stride ldh, batch stride, in elements), optionally added to its
 // previous contents in half arithmetic and clamped
 int f32_to_f16_launch(const float *dense_f32, void *half_matrix, int batch, int M, int N, int64_t ldh,
                       int64_t h_batch_stride, bool accumulate, float act_min, float act_max, hipStream_t s);
+// byte steps of dimensions 1, 2 and 3 of a tensor whose dimension 0 is a run of contiguous bytes
+struct RestrideSteps
+{
+    int64_t st[3];
+};
+int restride_nd_launch(const void *src, void *dst, int seg, int64_t n1, int64_t n2, int64_t n3, const RestrideSteps &ss,
+                       const RestrideSteps &ds, hipStream_t s);
 int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64_t src_stride, int64_t dst_stride,
                     hipStream_t s);
 int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g, int64_t ld_dst, hipStream_t s);

@@ -546,13 +546,14 @@ int im2col_nhwc_launch(const void *src, void *dst, int batch, const ConvGeom &g,
     return launch_status();
 }
 
-// ---- byte-matrix transpose: [batch][R][C] -> [batch][C][R] ---------------------------------------------------------
-// The NCHW <-> NHWC conversions around the NHWC convolution kernel (one image is a C x HW byte matrix) and of NCHW
-// weights ([OFM][C][KH*KW] -> [OFM][KH*KW][C]). 64 x 64 tiles through LDS so that reads and writes both run along rows.
-__global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                              int R, int C)
+// ---- matrix transpose of bytes or 32-bit words: [batch][R][C] -> [batch][C][R] --------------------------------------
+// The NCHW <-> NHWC conversions around the NHWC convolution kernel (one image is a C x HW matrix of bytes, or of floats
+// for the dequantised destination) and of NCHW weights ([OFM][C][KH*KW] -> [OFM][KH*KW][C]). 64 x 64 tiles through LDS
+// so that reads and writes both run along rows.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ src, T *__restrict__ dst, int R, int C)
 {
-    __shared__ uint8_t tile[64][65];
+    __shared__ T tile[64][65];
     const int64_t      base = (int64_t)blockIdx.z * R * C;
     const int          r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
     const int          tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -574,34 +575,55 @@ int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, 
     if (batch > 65535 || (R + 63) / 64 > 65535)
         return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)batch), block(256);
-    transpose_bytes_kernel<<<grid, block, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, R, C);
+    transpose_kernel<uint8_t><<<grid, block, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, R, C);
     return launch_status();
 }
 
-// ---- segment gather / scatter: dst[s * dst_stride + c] = src[s * src_stride + c], c < seg ------------------------------
-// Tensors that carry padding along the channel dimension (pixels seg bytes long, src_stride apart) to dense and back.
+int transpose_words_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s)
+{
+    if (batch <= 0 || R <= 0 || C <= 0)
+        return 0;
+    if (batch > 65535 || (R + 63) / 64 > 65535)
+        return (int)hipErrorInvalidValue;
+    const dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)batch), block(256);
+    transpose_kernel<uint32_t><<<grid, block, 0, s>>>((const uint32_t *)src, (uint32_t *)dst, R, C);
+    return launch_status();
+}
+
+// ---- segment gather / scatter between two stride sets ------------------------------------------------------------------
+// Segment (i1, i2, i3) of seg bytes lives at i1*st[0] + i2*st[1] + i3*st[2] on either side: tensors that carry padding
+// (along the channel dimension, between rows, between planes or images; ITensorInfo::strides_in_bytes()) to dense and back.
 __global__ __launch_bounds__(256) void restride_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                       int64_t segments, int seg, int64_t src_stride, int64_t dst_stride)
+                                                       int64_t total, int seg, int64_t n1, int64_t n2, RestrideSteps ss,
+                                                       RestrideSteps ds)
 {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= segments * seg)
+    if (idx >= total)
         return;
     const int64_t sgm = idx / seg;
     const int     c   = (int)(idx - sgm * seg);
-    dst[sgm * dst_stride + c] = src[sgm * src_stride + c];
+    const int64_t q1  = sgm / n1, i1 = sgm - q1 * n1;
+    const int64_t i3 = q1 / n2, i2 = q1 - i3 * n2;
+    dst[i1 * ds.st[0] + i2 * ds.st[1] + i3 * ds.st[2] + c] = src[i1 * ss.st[0] + i2 * ss.st[1] + i3 * ss.st[2] + c];
+}
+
+int restride_nd_launch(const void *src, void *dst, int seg, int64_t n1, int64_t n2, int64_t n3, const RestrideSteps &ss,
+                       const RestrideSteps &ds, hipStream_t s)
+{
+    if (seg <= 0 || n1 <= 0 || n2 <= 0 || n3 <= 0)
+        return 0;
+    const int64_t total = n1 * n2 * n3 * seg;
+    if ((total + 255) / 256 > 0x7FFFFFFF)
+        return (int)hipErrorInvalidValue;
+    restride_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)src, (uint8_t *)dst, total,
+                                                                                 seg, n1, n2, ss, ds);
+    return launch_status();
 }
 
 int restride_launch(const void *src, void *dst, int64_t segments, int seg, int64_t src_stride, int64_t dst_stride,
                     hipStream_t s)
 {
-    if (segments <= 0 || seg <= 0)
-        return 0;
-    const int64_t total = segments * seg;
-    if ((total + 255) / 256 > 0x7FFFFFFF)
-        return (int)hipErrorInvalidValue;
-    restride_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)src, (uint8_t *)dst,
-                                                                                 segments, seg, src_stride, dst_stride);
-    return launch_status();
+    return restride_nd_launch(src, dst, seg, segments, 1, 1, RestrideSteps{{src_stride, 0, 0}}, RestrideSteps{{dst_stride, 0, 0}}, s);
 }
 
 // ---- F16 destinations: [batch][M][N] halfs with row / batch strides <- the dense F32 matrix the GEMM kernels write --------

@@ -124,6 +124,10 @@ void read_gemm_strides(const ITensorInfo *ai, const ITensorInfo *bi, const ITens
     {
         d.lda            = ai->strides_in_bytes()[1];
         d.a_batch_stride = ai->strides_in_bytes()[a3d ? 3 : 2];
+        // [K, W, H, batch] read as W*H rows: planes of W rows, strides_in_bytes()[2] apart (more than W rows when the
+        // tensor is padded along y)
+        d.a_plane_rows   = a3d ? static_cast<int32_t>(ai->dimension(1)) : 0;
+        d.a_plane_stride = a3d ? static_cast<int64_t>(ai->strides_in_bytes()[2]) : 0;
     }
     if (bi != nullptr)
     {
@@ -134,9 +138,17 @@ void read_gemm_strides(const ITensorInfo *ai, const ITensorInfo *bi, const ITens
     {
         d.ldd = oi->strides_in_bytes()[1] / oi->element_size();
         if (gemm_info.depth_output_gemm3d() != 0)
-            d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size(); // [N, W, H, batch] planes are contiguous
+        {
+            // [N, W, H, batch]: planes of W rows
+            d.d_batch_stride = oi->strides_in_bytes()[3] / oi->element_size();
+            d.d_plane_rows   = static_cast<int32_t>(oi->dimension(1));
+            d.d_plane_stride = static_cast<int64_t>(oi->strides_in_bytes()[2] / oi->element_size());
+        }
         else
+        {
             d.d_batch_stride = oi->strides_in_bytes()[2] / oi->element_size();
+            d.d_plane_rows = 0, d.d_plane_stride = 0;
+        }
     }
 }
 
@@ -150,10 +162,11 @@ void sync_gemm_strides(const ITensorInfo *ai, const ITensorInfo *bi, const ITens
     mi355_gemm_desc now = d;
     read_gemm_strides(ai, b_is_packed ? nullptr : bi, oi, info, now);
     if (now.lda == d.lda && now.ldb == d.ldb && now.ldd == d.ldd && now.a_batch_stride == d.a_batch_stride &&
-        now.b_batch_stride == d.b_batch_stride && now.d_batch_stride == d.d_batch_stride)
+        now.b_batch_stride == d.b_batch_stride && now.d_batch_stride == d.d_batch_stride &&
+        now.a_plane_stride == d.a_plane_stride && now.d_plane_stride == d.d_plane_stride)
         return;
-    check_abi(mi355_gemmlowp_set_strides(handle, now.lda, now.ldb, now.ldd, now.a_batch_stride, now.b_batch_stride,
-                                         now.d_batch_stride),
+    check_abi(mi355_gemmlowp_set_strides_3d(handle, now.lda, now.ldb, now.ldd, now.a_batch_stride, now.b_batch_stride,
+                                            now.d_batch_stride, now.a_plane_stride, now.d_plane_stride),
               where);
     d = now;
 }
@@ -298,10 +311,6 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
         ARM_COMPUTE_RETURN_ERROR_ON_MSG(stage.type != GEMMLowpOutputStageType::NONE,
                                         "Accumulation is not supported for output QASYMM8/QASYMM8_SIGNED");
     }
-    // [K, W, H, batch] read as W*H rows per batch: the rows of consecutive planes must be evenly spaced
-    ARM_COMPUTE_RETURN_ERROR_ON_MSG(gemm_info.reinterpret_input_as_3d() &&
-                                        a->strides_in_bytes()[2] != a->dimension(1) * a->strides_in_bytes()[1],
-                                    "reinterpret_input_as_3d needs planes without padding between them");
 
     // shapes
     ARM_COMPUTE_RETURN_ERROR_ON(b->dimension(0) != output->dimension(0));
@@ -317,9 +326,6 @@ Status NEGEMMLowpMatrixMultiplyCore::validate(const ITensorInfo *a, const ITenso
         }
         else
             ARM_COMPUTE_RETURN_ERROR_ON(a->dimension(1) != output->dimension(1) * output->dimension(2));
-        ARM_COMPUTE_RETURN_ERROR_ON_MSG(output->strides_in_bytes()[2] !=
-                                            output->dimension(1) * output->strides_in_bytes()[1],
-                                        "GEMM3D output planes must be contiguous (no y padding)");
     }
     else
     {
@@ -719,8 +725,6 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
     {
         ARM_COMPUTE_RETURN_ERROR_ON_MSG(weights->data_type() != DataType::QASYMM8_SIGNED,
                                         "The F32 destination needs QASYMM8_SIGNED weights");
-        ARM_COMPUTE_RETURN_ERROR_ON_MSG(input->data_layout() != DataLayout::NHWC || output->has_padding(),
-                                        "The F32 destination is built for dense NHWC tensors");
     }
     if (biases != nullptr)
     {
@@ -745,19 +749,15 @@ Status NEGEMMConvolutionLayer::validate(const ITensorInfo *input, const ITensorI
         ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(dm.w) != conv_w || output->dimension(dm.h) != conv_h);
         ARM_COMPUTE_RETURN_ERROR_ON(output->dimension(3) != input->dimension(3));
     }
-    // padding along the channel dimension of NHWC tensors (what the reference's fixtures add: add_padding_x,
-    // tests/validation/Helpers.cpp:335-357) is taken as a pixel stride; anything else has to be dense
+    // Padding in any dimension of either layout (what the reference's fixtures add is add_padding_x,
+    // tests/validation/Helpers.cpp:335-357; its kernels read ITensorInfo::strides_in_bytes()) travels as the byte
+    // strides of dimensions 1 to 3; the elements of dimension 0 must be contiguous
     for (const ITensorInfo *t : {input, weights, output})
     {
         if (t->total_size() == 0)
             continue;
-        if (input->data_layout() == DataLayout::NHWC)
-            ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->strides_in_bytes()[2] != t->dimension(1) * t->strides_in_bytes()[1] ||
-                                                (t->num_dimensions() > 3 &&
-                                                 t->strides_in_bytes()[3] != t->dimension(2) * t->strides_in_bytes()[2]),
-                                            "Only padding along the channel dimension is supported by this convolution");
-        else
-            ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->has_padding(), "Padded NCHW tensors are not supported by this convolution");
+        ARM_COMPUTE_RETURN_ERROR_ON_MSG(t->strides_in_bytes()[0] != t->element_size(),
+                                        "The elements of dimension 0 must be contiguous");
     }
     if (!dequant)
     {
@@ -801,6 +801,25 @@ void conv_auto_init_output(const ITensorInfo *ii, const ITensorInfo *wi, ITensor
     oi->set_data_type(ii->data_type());
     oi->set_data_layout(ii->data_layout());
     oi->set_quantization_info(keep.empty() ? ii->quantization_info() : keep);
+}
+
+// strides_in_bytes()[1..3] of the three tensors of a convolution (zeros, i.e. "dense", for an info that is not at hand)
+struct ConvStrides
+{
+    int64_t src[3] = {0, 0, 0}, weights[3] = {0, 0, 0}, dst[3] = {0, 0, 0};
+};
+ConvStrides conv_strides_of(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi)
+{
+    ConvStrides cs;
+    const auto  take = [](const ITensorInfo *t, int64_t *out)
+    {
+        if (t == nullptr || t->total_size() == 0)
+            return;
+        for (int i = 0; i < 3; ++i)
+            out[i] = static_cast<int64_t>(t->strides_in_bytes()[i + 1]);
+    };
+    take(ii, cs.src), take(wi, cs.weights), take(oi, cs.dst);
+    return cs;
 }
 
 // the C-ABI descriptor of a (validated) convolution on these tensor infos
@@ -860,12 +879,10 @@ void fill_conv_desc(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorI
     }
     else
         d.requant = make_requant(stage);
-    if (d.layout == MI355_NHWC)
-    {
-        d.src_pixel_stride     = static_cast<int64_t>(ii->strides_in_bytes()[1]);
-        d.weights_pixel_stride = static_cast<int64_t>(wi->strides_in_bytes()[1]);
-        d.dst_pixel_stride     = static_cast<int64_t>(oi->strides_in_bytes()[1]);
-    }
+    const ConvStrides cs = conv_strides_of(ii, wi, oi);
+    d.src_pixel_stride = cs.src[0], d.src_stride2 = cs.src[1], d.src_stride3 = cs.src[2];
+    d.weights_pixel_stride = cs.weights[0], d.weights_stride2 = cs.weights[1], d.weights_stride3 = cs.weights[2];
+    d.dst_pixel_stride = cs.dst[0], d.dst_stride2 = cs.dst[1], d.dst_stride3 = cs.dst[2];
     if (stage.is_quantized_per_channel)
     {
         multipliers.assign(stage.gemmlowp_multipliers.begin(), stage.gemmlowp_multipliers.begin() + d.OFM);
@@ -926,15 +943,23 @@ namespace
 void sync_conv_strides(const ITensorInfo *ii, const ITensorInfo *wi, const ITensorInfo *oi, mi355_conv_desc &d,
                        mi355_conv_handle *handle, const char *where)
 {
-    if (d.layout != MI355_NHWC)
+    ConvStrides now = conv_strides_of(ii, wi, oi);
+    const int64_t have[3][3] = {{d.src_pixel_stride, d.src_stride2, d.src_stride3},
+                                {d.weights_pixel_stride, d.weights_stride2, d.weights_stride3},
+                                {d.dst_pixel_stride, d.dst_stride2, d.dst_stride3}};
+    if (!ii)
+        std::copy(have[0], have[0] + 3, now.src);
+    if (!wi)
+        std::copy(have[1], have[1] + 3, now.weights);
+    if (!oi)
+        std::copy(have[2], have[2] + 3, now.dst);
+    if (std::equal(now.src, now.src + 3, have[0]) && std::equal(now.weights, now.weights + 3, have[1]) &&
+        std::equal(now.dst, now.dst + 3, have[2]))
         return;
-    const int64_t sp = ii ? static_cast<int64_t>(ii->strides_in_bytes()[1]) : d.src_pixel_stride;
-    const int64_t wp = wi ? static_cast<int64_t>(wi->strides_in_bytes()[1]) : d.weights_pixel_stride;
-    const int64_t dp = oi ? static_cast<int64_t>(oi->strides_in_bytes()[1]) : d.dst_pixel_stride;
-    if (sp == d.src_pixel_stride && wp == d.weights_pixel_stride && dp == d.dst_pixel_stride)
-        return;
-    check_abi(mi355_conv_set_strides(handle, sp, wp, dp), where);
-    d.src_pixel_stride = sp, d.weights_pixel_stride = wp, d.dst_pixel_stride = dp;
+    check_abi(mi355_conv_set_strides_nd(handle, now.src, now.weights, now.dst), where);
+    d.src_pixel_stride = now.src[0], d.src_stride2 = now.src[1], d.src_stride3 = now.src[2];
+    d.weights_pixel_stride = now.weights[0], d.weights_stride2 = now.weights[1], d.weights_stride3 = now.weights[2];
+    d.dst_pixel_stride = now.dst[0], d.dst_stride2 = now.dst[1], d.dst_stride3 = now.dst[2];
 }
 } // namespace
 

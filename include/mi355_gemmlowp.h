@@ -135,6 +135,15 @@ typedef struct mi355_gemm_desc
                                        (src/cpu/kernels/CpuConvertFullyConnectedWeightsKernel.cpp:60-66,118-121; f is its
                                        _factor2). 0 or 1: none. Must divide K. */
     int32_t       flags;            /* MI355_GEMM_* bits (enum mi355_gemm_flags) */
+    /* Matrices whose M rows are the rows of several planes with a gap between the planes: GEMMInfo::
+     * reinterpret_input_as_3d (A is [K, W, H, batch] read as W*H rows) and depth_output_gemm3d (D is [N, W, H, batch])
+     * on tensors padded along y (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:520-534; strides per
+     * arm_compute/core/ITensorInfo.h:81-334). Row r of a matrix is row r % plane_rows of plane r / plane_rows; planes
+     * are a_plane_stride bytes (d_plane_stride destination elements) apart. plane_rows = 0: no planes (rows lda / ldd
+     * apart throughout). plane_rows must divide M. Such a matrix is gathered into (scattered from) a dense device
+     * buffer by one extra pass. */
+    int32_t       a_plane_rows, d_plane_rows;
+    int64_t       a_plane_stride, d_plane_stride;
 } mi355_gemm_desc;
 
 typedef struct mi355_gemm_handle mi355_gemm_handle;
@@ -164,6 +173,11 @@ int mi355_gemmlowp_update_quant(mi355_gemm_handle *h, int32_t a_offset, int32_t 
  * (tests/validation/fixtures/CpuGEMMLowpFixture.h:117). A shared B cannot become a batched one or the reverse. */
 int mi355_gemmlowp_set_strides(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
                                int64_t b_batch_stride, int64_t d_batch_stride);
+/* The same with the plane strides of mi355_gemm_desc (a_plane_stride in bytes, d_plane_stride in destination
+ * elements; ignored for a matrix created without planes). mi355_gemmlowp_set_strides leaves planes without a gap. */
+int mi355_gemmlowp_set_strides_3d(mi355_gemm_handle *h, int64_t lda, int64_t ldb, int64_t ldd, int64_t a_batch_stride,
+                                  int64_t b_batch_stride, int64_t d_batch_stride, int64_t a_plane_stride,
+                                  int64_t d_plane_stride);
 
 /* Replaces CpuGemmLowpMatrixMultiplyCore::run (:647-811). bias_f32 (N floats, MI355_EPI_F32 only) may be NULL. */
 int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
@@ -230,18 +244,25 @@ typedef struct mi355_conv_desc
     mi355_requant requant;
     int32_t       path; /* 0 auto (implicit GEMM where the shape allows), 1 force explicit im2col + GEMM */
     int32_t       layout; /* mi355_conv_layout of src, weights and dst */
-    /* NHWC only: bytes from one pixel (one tap of the weights) to the next when the tensors carry padding along the
-     * channel dimension, as the reference's own fixtures give them (add_padding_x, tests/validation/Helpers.cpp:335-357;
-     * ITensorInfo::strides_in_bytes()[1]). Rows, planes and batches must follow without further gaps. 0 = dense (C, C,
-     * OFM). The pointers passed to prepare / run address the first element. Padded tensors are gathered into dense
-     * device buffers first (one extra pass) and the result is scattered into dst, leaving its padding untouched. */
+    /* Bytes from one pixel (one tap of the weights) to the next when the tensors carry padding along the channel
+     * dimension, as the reference's own fixtures give them (add_padding_x, tests/validation/Helpers.cpp:335-357;
+     * ITensorInfo::strides_in_bytes()[1]). 0 = dense (C, C, OFM x element size). For MI355_NCHW tensors the same field
+     * is the stride of dimension 1 there: bytes from one row of W (KW, OW) elements to the next. The strides of
+     * dimensions 2 and 3 are the *_stride2 / *_stride3 fields at the end of this struct. The pointers passed to
+     * prepare / run address the first element. Padded tensors are gathered into dense device buffers first (one
+     * extra pass) and the result is scattered into dst, leaving its padding untouched. */
     int64_t       src_pixel_stride, weights_pixel_stride, dst_pixel_stride;
     /* dst_dtype MI355_F32 only - the dequantising convolution (CpuGemmConv2d with a QASYMM8_SIGNED input and an F32
      * destination, src/cpu/operators/CpuGemmConv2d.cpp:297-305,391-393): no requantisation, dst = float(acc) * scale
      * (+ float bias) + float(offset terms) * scale, clamped to [act_min, act_max] as MI355_EPI_F32 does; flags takes
-     * MI355_GEMM_ACT_TWICE. Dense NHWC only; the bias passed to mi355_conv_prepare is then OFM floats. */
+     * MI355_GEMM_ACT_TWICE. The bias passed to mi355_conv_prepare is then OFM floats. */
     float         scale, act_min, act_max;
     int32_t       flags;
+    /* ITensorInfo::strides_in_bytes()[2] and [3] of the three tensors (arm_compute/core/ITensorInfo.h:81-334): NHWC -
+     * from one row of pixels to the next and from one image (one output channel's filter) to the next; NCHW - from one
+     * channel plane to the next and from one image (filter) to the next. 0 = follows without a gap from the stride of
+     * the dimension below (tensors padded along y, between planes or between images have larger values). */
+    int64_t       src_stride2, src_stride3, weights_stride2, weights_stride3, dst_stride2, dst_stride3;
 } mi355_conv_desc;
 
 typedef struct mi355_conv_handle mi355_conv_handle;
@@ -256,9 +277,12 @@ int  mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t w
                              const mi355_requant *requant, const int32_t *mult, const int32_t *shift, void *stream);
 /* New pixel strides (see mi355_conv_desc) for the calls that follow: weights_pixel_stride is read by the next
  * mi355_conv_prepare, the other two by the next mi355_conv_run. The reference reads strides when it runs and its
- * fixtures pad the tensors after configure (tests/validation/fixtures/CpuGemmConv2dFixture.h:315-319). NHWC only. */
+ * fixtures pad the tensors after configure (tests/validation/fixtures/CpuGemmConv2dFixture.h:315-319). */
 int  mi355_conv_set_strides(mi355_conv_handle *h, int64_t src_pixel_stride, int64_t weights_pixel_stride,
                             int64_t dst_pixel_stride);
+/* The same for all three strides of each tensor: { strides_in_bytes()[1], [2], [3] } of src, weights and dst, 0 = dense.
+ * mi355_conv_set_strides(h, a, b, c) is this call with { a, 0, 0 }, { b, 0, 0 }, { c, 0, 0 }. Both layouts. */
+int  mi355_conv_set_strides_nd(mi355_conv_handle *h, const int64_t src[3], const int64_t weights[3], const int64_t dst[3]);
 int  mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *stream);
 void mi355_conv_out_dims(const mi355_conv_desc *desc, int32_t *OH, int32_t *OW);
 void mi355_conv_destroy(mi355_conv_handle *h);

@@ -513,6 +513,45 @@ static void test_gemmlowp_accumulate_and_3d()
         std::vector<int32_t> want(batch * W * H * N);
         orc_gemmlowp_s32(A.data(), 1, K, B.data(), 1, N, want.data(), N, batch * W * H, N, K, 2, -1);
         EXPECT(dense_copy<int32_t>(dst) == want);
+        // the same with both 3D tensors padded along x and y after configure (gaps between the planes of W rows:
+        // strides_in_bytes()[2] > W * strides_in_bytes()[1]), a fused output stage, and the padding of dst left alone
+        {
+            Tensor a2, dst2;
+            init_tensor(a2, TensorShape(K, W, H, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.1f, 2));
+            init_tensor(dst2, TensorShape(N, W, H, batch), DataType::QASYMM8_SIGNED, QuantizationInfo(0.7f, 3));
+            GEMMLowpOutputStageInfo st;
+            EXPECT(bool(quantization::calculate_quantized_multipliers(QuantizationInfo(0.1f, 2), QuantizationInfo(0.2f, -1),
+                                                                      QuantizationInfo(0.7f, 3), st)));
+            st.type                = GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT;
+            st.gemmlowp_offset     = 3;
+            st.gemmlowp_min_bound  = -128;
+            st.gemmlowp_max_bound  = 127;
+            st.output_data_type    = DataType::QASYMM8_SIGNED;
+            st.gemmlowp_multiplier = st.gemmlowp_multipliers[0];
+            st.gemmlowp_shift      = st.gemmlowp_shifts[0];
+            GEMMInfo info2(false, false, true, H, true);
+            info2.set_gemmlowp_output_stage(st);
+            NEGEMMLowpMatrixMultiplyCore gemm2;
+            gemm2.configure(&a2, &b, nullptr, &dst2, info2);
+            a2.info()->extend_padding(PaddingSize(2, 5, 1, 3)); // top, right, bottom, left
+            dst2.info()->extend_padding(PaddingSize(1, 4, 2, 0));
+            a2.allocator()->allocate(), dst2.allocator()->allocate();
+            EXPECT(a2.info()->strides_in_bytes()[2] > W * a2.info()->strides_in_bytes()[1]);
+            fill_uniform<int8_t>(a2, -128, 127, 9);
+            std::memset(dst2.buffer(), 0x5A, dst2.info()->total_size());
+            gemm2.run();
+            const auto A2 = dense_copy<int8_t>(a2);
+            std::vector<int8_t> want2(batch * W * H * N);
+            orc_gemmlowp_fixedpoint(A2.data(), 1, K, B.data(), 1, N, nullptr, want2.data(), N, 1, batch * W * H, N, K, 2, -1,
+                                    &st.gemmlowp_multiplier, &st.gemmlowp_shift, 1, 3, -128, 127);
+            EXPECT(dense_copy<int8_t>(dst2) == want2);
+            size_t untouched = 0, padding = dst2.info()->total_size() - (size_t)batch * W * H * N;
+            for (size_t i = 0; i < dst2.info()->total_size(); ++i)
+                untouched += dst2.buffer()[i] == 0x5A;
+            EXPECT(untouched >= padding);
+            std::printf("       kernel: %s (planes %zu bytes apart for %d rows of %zu)\n", gemm2.kernel_name(),
+                        (size_t)a2.info()->strides_in_bytes()[2], W, (size_t)a2.info()->strides_in_bytes()[1]);
+        }
         // a 3D input without a 3D output is not built
         Tensor flat;
         init_tensor(flat, TensorShape(N, W * H, batch), DataType::S32);
@@ -841,9 +880,12 @@ static void test_quantize_down_scale()
 
 // padded: src / weights / dst carry padding along x (the channels), as the reference's fixture adds it with
 // add_padding_x (tests/validation/fixtures/ConvolutionLayerFixture.h:464-469)
-static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act, bool padded = false)
+// padded == 2: padding along y as well (rows above and below every plane; ITensorInfo::strides_in_bytes()[2] and the
+// offset of the first element change, arm_compute/core/ITensorInfo.h:81-334)
+static void test_convolution(DataType dt, bool per_channel, int C, const ActivationLayerInfo &act, int padded = 0)
 {
-    SECTION(padded ? "NEGEMMConvolutionLayer NHWC, tensors padded along x"
+    SECTION(padded == 2 ? "NEGEMMConvolutionLayer NHWC, tensors padded along x and y"
+            : padded   ? "NEGEMMConvolutionLayer NHWC, tensors padded along x"
                    : per_channel ? "NEGEMMConvolutionLayer NHWC per-channel weights" : "NEGEMMConvolutionLayer NHWC per-tensor weights");
     const bool is_signed = dt == DataType::QASYMM8_SIGNED;
     const int  batch = 2, H = 9, W = 8, OFM = 24, KH = 3, KW = 3;
@@ -867,10 +909,11 @@ static void test_convolution(DataType dt, bool per_channel, int C, const Activat
     if (padded)
     {
         // after configure and before allocation, like the fixture: PaddingSize(top, right, bottom, left)
-        src.info()->extend_padding(PaddingSize(0, 7, 0, 3));
-        w.info()->extend_padding(PaddingSize(0, 16, 0, 1));
+        const unsigned y = padded == 2 ? 1 : 0;
+        src.info()->extend_padding(PaddingSize(2 * y, 7, y, 3));
+        w.info()->extend_padding(PaddingSize(y, 16, 3 * y, 1));
         bias.info()->extend_padding(PaddingSize(0, 2, 0, 5));
-        dst.info()->extend_padding(PaddingSize(0, 4, 0, 9));
+        dst.info()->extend_padding(PaddingSize(y, 4, 2 * y, 9));
     }
     src.allocator()->allocate(), w.allocator()->allocate(), bias.allocator()->allocate(), dst.allocator()->allocate();
     if (is_signed)
@@ -1407,8 +1450,10 @@ int main(int argc, char **argv)
             test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
             test_convolution(DataType::QASYMM8, true, 32,
                              ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
-            test_convolution(DataType::QASYMM8_SIGNED, true, 32, ActivationLayerInfo(), true);
-            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), true);
+            test_convolution(DataType::QASYMM8_SIGNED, true, 32, ActivationLayerInfo(), 1);
+            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), 1);
+            test_convolution(DataType::QASYMM8_SIGNED, true, 16, ActivationLayerInfo(), 2);
+            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(), 2);
             test_gemm_conv2d();
             test_stateless_operator();
             test_stateless_operators_padded_after_configure();

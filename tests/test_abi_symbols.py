@@ -98,6 +98,6 @@ def test_set_strides_checks_what_create_checks():
     g.close()
     c = capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 3, 3))
     c.set_strides(24, 16, 8)
-    with pytest.raises(capi.Mi355Error, match="pixel stride"):
+    with pytest.raises(capi.Mi355Error, match="stride is smaller"):
         c.set_strides(8, 16, 8)
     c.close()

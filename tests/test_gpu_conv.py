@@ -249,8 +249,108 @@ def test_conv_tensors_padded_along_channels(device):
         cv.close()
         np.testing.assert_array_equal(got[..., :OFM], want)
         assert (got[..., OFM:] == 55).all(), "padding bytes of the destination were overwritten"
-    with pytest.raises(capi.Mi355Error, match="pixel stride"):
+    with pytest.raises(capi.Mi355Error, match="stride is smaller"):
         capi.Conv(capi.conv_desc(1, 4, 4, 16, 8, 1, 1, pixel_strides=(8, 0, 0)))
+
+
+def _padded_view(rng, dense, pads, fill):
+    """A buffer of `fill` bytes holding `dense` (4 dimensions, the last one contiguous) with pads[i] extra elements
+    after dimension i of each of the last three dimensions' rows / planes / images; returns (buffer, view on the
+    valid elements, byte strides of dimensions 1, 2 and 3 in the reference's order: innermost first)."""
+    n3, n2, n1, n0 = dense.shape
+    big = np.full((n3, n2 + pads[2], n1 + pads[1], n0 + pads[0]), fill, dtype=dense.dtype)
+    view = big[:, :n2, :n1, :n0]
+    view[...] = dense
+    e = dense.dtype.itemsize
+    s1 = (n0 + pads[0]) * e
+    s2 = s1 * (n1 + pads[1])
+    s3 = s2 * (n2 + pads[2])
+    return big, view, (s1, s2, s3)
+
+
+@pytest.mark.parametrize("layout", ["nhwc", "nchw"])
+@pytest.mark.parametrize("device", [True, False])
+def test_conv_tensors_padded_in_every_dimension(layout, device):
+    """Padding after every dimension of src, weights and dst (ITensorInfo::strides_in_bytes()[1..3] all larger than
+    dense, arm_compute/core/ITensorInfo.h:81-334), both layouts: same integers, padding of dst untouched. Strides
+    given at create for the first case and through mi355_conv_set_strides_nd after create for the second."""
+    import torch
+    rng = np.random.default_rng(67)
+    nchw = layout == "nchw"
+    for case, (B_, H, W, C, OFM, KH, KW, pads_s, pads_w, pads_d) in enumerate(
+            [(2, 9, 8, 16, 24, 3, 3, (5, 2, 1), (9, 1, 2), (3, 1, 2)),
+             (3, 7, 6, 5, 10, 2, 3, (0, 3, 0), (0, 0, 4), (0, 2, 1))]):
+        src = rng.integers(-128, 128, size=(B_, H, W, C), dtype=np.int8)
+        w = rng.integers(-127, 128, size=(OFM, KH, KW, C), dtype=np.int8)
+        bias = rng.integers(-500, 500, size=OFM, dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multipliers(0.02, rng.uniform(0.01, 1, OFM), 1.1)
+        pad = (1, 1, 1, 1) if KH == 3 else (0, 1, 1, 0)
+        want = oracle.conv_nhwc_direct(src, w, bias, 4, 0, mult, shift, -5, -128, 127, (1, 1), pad, (1, 1))
+        to_layout = (lambda a: np.ascontiguousarray(a.transpose(0, 3, 1, 2))) if nchw else (lambda a: a)
+        src_b, _, ss = _padded_view(rng, to_layout(src), pads_s, 99)
+        w_b, _, ws = _padded_view(rng, to_layout(w), pads_w, 77)
+        dst_b, dst_v, ds = _padded_view(rng, np.zeros_like(to_layout(want)), pads_d, 55)
+        dst_v[...] = 11
+        rq = capi.requant(0, 0, -5, -128, 127, True)
+        lay = capi.NCHW if nchw else capi.NHWC
+        if case == 0:
+            d = capi.conv_desc(B_, H, W, C, OFM, KH, KW, (1, 1), pad, (1, 1), capi.S8, capi.S8, capi.S8, -4, 0, 4, rq, 0,
+                               lay, (ss[0], ws[0], ds[0]), outer_strides=(ss[1:], ws[1:], ds[1:]))
+            cv = capi.Conv(d)
+        else:
+            cv = capi.Conv(capi.conv_desc(B_, H, W, C, OFM, KH, KW, (1, 1), pad, (1, 1), capi.S8, capi.S8, capi.S8, -4,
+                                          0, 4, rq, 0, lay))
+            cv.set_strides_nd(ss, ws, ds)
+        announce("conv padded in every dimension", layout, (B_, H, W, C, OFM, KH, KW), ss, ws, ds, "device", device)
+        m, sh = np.ascontiguousarray(mult, dtype=np.int32), np.ascontiguousarray(shift, dtype=np.int32)
+        if device:
+            sd, wd, od = to_dev(src_b), to_dev(w_b), to_dev(dst_b)
+            keep = [to_dev(bias), to_dev(m), to_dev(sh)]
+            cv.prepare(wd, *keep)
+            cv.run(sd, od)
+            torch.cuda.synchronize()
+            got = od.cpu().numpy()
+        else:
+            cv.prepare(w_b, bias, m, sh)
+            got = dst_b.copy()
+            cv.run(src_b, got)
+        cv.close()
+        n3, n2, n1, n0 = to_layout(want).shape
+        np.testing.assert_array_equal(got[:, :n2, :n1, :n0], to_layout(want))
+        mask = np.ones(got.shape, dtype=bool)
+        mask[:, :n2, :n1, :n0] = False
+        assert (got[mask] == 55).all(), "padding bytes of the destination were overwritten"
+
+
+def test_conv_f32_destination_padded():
+    """The dequantising convolution into an NHWC float tensor with padding after pixels and rows"""
+    import torch
+    rng = np.random.default_rng(68)
+    B_, H, W, C, OFM = 2, 6, 7, 16, 12
+    src = rng.integers(-128, 128, size=(B_, H, W, C), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(OFM, 3, 3, C), dtype=np.int8)
+    dense = capi.Conv(capi.conv_desc(B_, H, W, C, OFM, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.F32, -3,
+                                     0, 3, None, 0, capi.NHWC, scale=0.0123))
+    dense.prepare(to_dev(w))
+    want_d = torch.zeros((B_, H, W, OFM), dtype=torch.float32, device="cuda")
+    dense.run(to_dev(src), want_d)
+    torch.cuda.synchronize()
+    want = want_d.cpu().numpy()
+    dense.close()
+    dst_b, _, ds = _padded_view(rng, np.zeros_like(want), (3, 2, 0), 7.5)
+    announce("conv F32 padded destination", ds)
+    cv = capi.Conv(capi.conv_desc(B_, H, W, C, OFM, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.F32, -3, 0,
+                                  3, None, 0, capi.NHWC, (0, 0, ds[0]), scale=0.0123, outer_strides=((0, 0), (0, 0), ds[1:])))
+    od = to_dev(dst_b)
+    cv.prepare(to_dev(w))
+    cv.run(to_dev(src), od)
+    torch.cuda.synchronize()
+    got = od.cpu().numpy()
+    cv.close()
+    np.testing.assert_array_equal(got[:, :H, :W, :OFM].view(np.uint32), want.view(np.uint32))
+    mask = np.ones(got.shape, dtype=bool)
+    mask[:, :H, :W, :OFM] = False
+    assert (got[mask] == 7.5).all(), "padding of the destination was overwritten"
 
 
 def test_conv_random_geometry_sweep():

@@ -7,7 +7,7 @@ import pytest
 
 import oracle
 from computelibrary_amd import capi
-from gpu_util import announce, run_gemm
+from gpu_util import announce, run_gemm, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -528,6 +528,69 @@ def test_f32_activation_clamps_before_and_after_the_offset_term(M):
     assert np.array_equal(got.view(np.uint32), twice.view(np.uint32))
     got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, 40, 25, scale=1e-3, act=(0.0, 6.0))
     assert np.array_equal(got.view(np.uint32), once.view(np.uint32))
+
+
+@pytest.mark.parametrize("device", [False, True])
+@pytest.mark.parametrize("W,H,N,K,batch,epi", [(5, 4, 33, 40, 2, "s32"), (7, 9, 136, 64, 1, "s8"), (3, 2, 24, 19, 3, "f32acc"),
+                                               (40, 8, 72, 100, 1, "s8")])
+def test_rows_in_planes_with_gaps_between_them(W, H, N, K, batch, epi, device):
+    """GEMMInfo::reinterpret_input_as_3d / depth_output_gemm3d on tensors padded along y: A is [batch][H][W rows + gap][K],
+    D likewise (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:520-534 reads the tensors' strides): the same result
+    as on dense matrices, the gaps of D untouched, strides given at create or afterwards through set_strides_3d."""
+    import torch
+    rng = np.random.default_rng(zlib.crc32(("planes %d %d %d %d" % (W, H, N, K)).encode()))
+    M = W * H
+    lda, ldd, gap_a, gap_d = K + 5, N + 3, 2, 3  # gaps in rows
+    A = rng.integers(-128, 128, size=(batch, H, W, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    a_buf = np.full((batch, H, W + gap_a, lda), 99, dtype=np.int8)
+    a_buf[:, :, :W, :K] = A
+    dt = {"s32": np.int32, "s8": np.int8, "f32acc": np.float32}[epi]
+    fill = {"s32": 0x5A5A5A5A, "s8": 0x5A, "f32acc": 7.5}[epi]
+    d_buf = np.full((batch, H, W + gap_d, ldd), fill, dtype=dt)
+    prev = rng.normal(0, 3, size=(batch, H, W, N)).astype(np.float32)
+    if epi == "f32acc":
+        d_buf[:, :, :W, :N] = prev
+    A2 = A.reshape(batch * M, K)
+    if epi == "s32":
+        want = oracle.gemmlowp_s32(A2, B, 4, -2)
+        kw = dict(epilogue=capi.EPI_S32, dst_dtype=capi.S32)
+    elif epi == "s8":
+        mult, shift = oracle.calculate_quantized_multipliers(0.02, [0.03], 0.9)
+        want = oracle.gemmlowp_fixedpoint(A2, B, None, 4, -2, mult, shift, -3, -128, 127, np.int8)
+        kw = dict(epilogue=capi.EPI_FIXEDPOINT, dst_dtype=capi.S8, rq=capi.requant(int(mult[0]), int(shift[0]), -3, -128, 127))
+    else:
+        want = oracle.gemmlowp_f32(A2, B, None, 4, -2, 1e-3, prev=prev.reshape(batch * M, N))
+        kw = dict(epilogue=capi.EPI_F32, dst_dtype=capi.F32, scale=1e-3, flags=capi.GEMM_ACCUMULATE)
+    a_ps, d_ps = (W + gap_a) * lda, (W + gap_d) * ldd
+    late = (W + H) % 2 == 1
+    announce("rows in planes", W, H, N, K, batch, epi, "device", device, "strides set late", late)
+    if late:
+        g = capi.Gemm(M, N, K, capi.S8, capi.S8, a_offset=4, b_offset=-2, batch=batch, a_planes=(W, W * K), d_planes=(W, W * N),
+                      **kw)
+        g.set_strides_3d(lda, N, ldd, H * a_ps, 0, H * d_ps, a_ps, d_ps)
+    else:
+        g = capi.Gemm(M, N, K, capi.S8, capi.S8, a_offset=4, b_offset=-2, batch=batch, lda=lda, ldd=ldd, a_planes=(W, a_ps),
+                      d_planes=(W, d_ps), a_batch_stride=H * a_ps, d_batch_stride=H * d_ps, **kw)
+    if device:
+        bd, ad, dd = to_dev(B), to_dev(a_buf), to_dev(d_buf)
+        g.prepare(bd)
+        g.run(ad, dd)
+        torch.cuda.synchronize()
+        got = dd.cpu().numpy()
+    else:
+        g.prepare(B)
+        got = d_buf.copy()
+        g.run(a_buf, got)
+    g.close()
+    valid = got[:, :, :W, :N].reshape(batch * M, N)
+    if epi == "f32acc":
+        assert np.array_equal(valid.view(np.uint32), want.view(np.uint32))
+    else:
+        np.testing.assert_array_equal(valid, want)
+    mask = np.ones(got.shape, dtype=bool)
+    mask[:, :, :W, :N] = False
+    assert (got[mask] == d_buf[mask]).all(), "gaps of the destination were overwritten"
 
 
 def test_accumulate_is_rejected_with_an_output_stage():

@@ -13,6 +13,9 @@
 //   * loads go out in batches of 3 k blocks (6 loads of 1 KiB per wave), two batches in flight, and the number of
 //     batches is a template parameter, so the code is straight-line and the compiler knows exactly how many loads
 //     are outstanding at every wait;
+//   * the A loads are buffer loads with the hardware's range check (a tap above the first or below the last image row
+//     lies outside the tensor and reads as zero without a test), so a load costs one addition; which pieces are padding
+//     is worked out after the loads have been issued, while they are in flight;
 //   * no barrier after the one that publishes the B panel; 4 workgroups of 4 waves fit a compute unit.
 #include "mfma_common.hpp"
 
@@ -59,13 +62,17 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     ConvGeom  cg = g.conv;
     uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp,
               u_fl = (uintptr_t)g.epi.qp_flag;
+    uint32_t  a_bytes = (uint32_t)(g.a_end - g.A); // bytes of A: what the range check of the A loads compares with
     int32_t   a_M = g.M, a_K = g.K, a_lda = (int32_t)g.lda, a_kp = (int32_t)g.Kp, a_qps = (int32_t)g.epi.qp_stride;
     asm volatile(""
                  : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x), "+s"(cg.stride_y),
                    "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word), "+s"(cg.magic_C),
                    "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(cg.magic_OH), "+s"(a_M), "+s"(a_K), "+s"(a_lda), "+s"(a_kp),
-                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl));
-    const MI355_GLOBAL int8_t *const  gA = (const MI355_GLOBAL int8_t *)u_a, *const gB = (const MI355_GLOBAL int8_t *)u_b;
+                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl), "+s"(a_bytes));
+    const MI355_GLOBAL int8_t *const gB = (const MI355_GLOBAL int8_t *)u_b;
+    // raw buffer over A (stride 0, 32-bit elements untyped): loads at or past a_bytes - also "negative" offsets, which
+    // are huge as unsigned - return zero
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)u_a, 0, (int)a_bytes, 0x00020000);
     const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
 
     const int tid  = threadIdx.x;
@@ -136,53 +143,72 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
             pix[rb]           = gr * a_lda;
         }
     }
-    // A piece outside the image (or past K) is fetched from offset 0 instead - a load that depends on nothing - and
-    // replaced by the padding value when it is used (past K its value is irrelevant: B is zero there).
+    // A piece outside the image is replaced by the padding value when it is used; its load goes out all the same (inside
+    // the tensor it reads a neighbouring pixel, outside it reads zero). Past K the value is irrelevant: B is zero there.
     v4i      fa[2][3][RS];
     uint32_t oob = 0; // bit (slot * 3 + kk) * RS + rb: that piece is padding
-    auto     load_a = [&](int slot, int batch)
+    // tap of k block kb (UNI: scalar) or of this lane's 16 bytes of it
+    auto tap_of = [&](int kb, int &dy, int &dx, int &off)
     {
+        const int k = kb * 64 + lh * 16;
+        dy = 0, dx = 0, off = k;
+        if (CONV)
+        {
+            int tap, c0;
+            if (UNI)
+            {
+                tap = narrow_div(kb * 64, cg.magic_C); // scalar
+                c0  = kb * 64 - tap * cg.C + lh * 16;
+            }
+            else
+            {
+                tap = narrow_div(k, cg.magic_C);
+                c0  = k - tap * cg.C;
+            }
+            const int ky = narrow_div(tap, cg.magic_KW);
+            const int kx = tap - ky * cg.KW;
+            dy           = ky * cg.dil_y;
+            dx           = kx * cg.dil_x;
+            off          = (dy * cg.W + dx) * cg.C + c0;
+        }
+    };
+    auto load_a = [&](int slot, int batch)
+    {
+#pragma unroll
+        for (int kk = 0; kk < 3; ++kk)
+        {
+            int dy, dx, off;
+            tap_of(batch * 3 + kk, dy, dx, off);
+#pragma unroll
+            for (int rb = 0; rb < RS; ++rb)
+                fa[slot][kk][rb] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(a_rsrc, pix[rb] + off, 0, 0);
+        }
+    };
+    auto mask_a = [&](int slot, int batch)
+    {
+        if (!CONV)
+            return;
         oob &= ~(((1u << (3 * RS)) - 1u) << (slot * 3 * RS));
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk)
         {
-            const int kb = batch * 3 + kk;
-            const int k  = kb * 64 + lh * 16; // this lane's 16 bytes of the k block
-            int       dy = 0, dx = 0, off = k;
-            if (CONV)
-            {
-                int tap, c0;
-                if (UNI)
-                {
-                    tap = narrow_div(kb * 64, cg.magic_C); // scalar
-                    c0  = kb * 64 - tap * cg.C + lh * 16;
-                }
-                else
-                {
-                    tap = narrow_div(k, cg.magic_C);
-                    c0  = k - tap * cg.C;
-                }
-                const int ky = narrow_div(tap, cg.magic_KW);
-                const int kx = tap - ky * cg.KW;
-                dy           = ky * cg.dil_y;
-                dx           = kx * cg.dil_x;
-                off          = (dy * cg.W + dx) * cg.C + c0;
-            }
+            int dy, dx, off;
+            tap_of(batch * 3 + kk, dy, dx, off);
 #pragma unroll
             for (int rb = 0; rb < RS; ++rb)
             {
-                // (bitwise, not short-circuit: no branches between the loads)
-                const bool ok = CONV ? ((k < a_K) & ((unsigned)(iy0[rb] + dy) < (unsigned)cg.H) & ((unsigned)(ix0[rb] + dx) < (unsigned)cg.W))
-                                     : (k < a_K);
+                const bool ok = ((unsigned)(iy0[rb] + dy) < (unsigned)cg.H) & ((unsigned)(ix0[rb] + dx) < (unsigned)cg.W);
                 oob |= (uint32_t)(!ok) << ((slot * 3 + kk) * RS + rb);
-                fa[slot][kk][rb] = *(const MI355_GLOBAL v4i *)(gA + (uint32_t)(ok ? pix[rb] + off : 0));
             }
         }
     };
     load_a(0, 0);
     if (NB > 1)
         load_a(1, 1);
-    __builtin_amdgcn_sched_barrier(0); // nothing that waits for a load may move up between the loads
+    __builtin_amdgcn_sched_barrier(0); // nothing else moves up between the loads: they go out first
+    mask_a(0, 0);
+    if (NB > 1)
+        mask_a(1, 1);
 
     // ---- the B panel has landed when at most the A loads issued after it are still in flight; epilogue constants ----
     if (NB > 1)
@@ -242,21 +268,30 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
             }
         }
         if (b + 2 < NB)
+        {
             load_a(b & 1, b + 2);
+            mask_a(b & 1, b + 2);
+        }
     }
 
     __builtin_amdgcn_s_setprio(0);
-    if (fast && g.epi.qp_std && (qflag & 3) == 0 && g.epi.vec_store)
+    if (fast && g.epi.qp_std && (qflag & 3) == 0 && g.epi.vec_store && (g.N & 3) == 0)
     {
         // every column has a normalised multiplier and a right shift of 2..31: the short form of the requantisation.
-        // Lane l holds, for row rb * 16 + l % 16, the 4 consecutive columns q * 16 + 4 * (l / 16) + {0..3}: one dword.
+        // Lane l holds, for row rb * 16 + l % 16, the 4 consecutive columns q * 16 + 4 * (l / 16) + {0..3}: one dword
+        // (N is a multiple of 4 here, so a lane's four columns exist together or not at all).
         const int32_t  off2p1 = 2 * g.epi.result_offset + 1, lo = g.epi.lo, hi = g.epi.hi;
         const int32_t *rowvec = g.epi.rowvec;
-        char          *D      = (char *)g.D;
+        const int      a_N    = g.N;
         int32_t        rv[RS];
+        char          *drow[RS]; // this lane's row of D at column 4 * (l / 16)
 #pragma unroll
         for (int rb = 0; rb < RS; ++rb)
-            rv[rb] = (rowvec && row0 + rb * 16 + lr < a_M) ? rowvec[row0 + rb * 16 + lr] : 0;
+        {
+            const int i = row0 + rb * 16 + lr;
+            rv[rb]      = (rowvec && i < a_M) ? rowvec[i] : 0;
+            drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + 4 * lh;
+        }
 #pragma unroll
         for (int q = 0; q < QS; ++q)
         {
@@ -266,8 +301,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 #pragma unroll
             for (int rb = 0; rb < RS; ++rb)
             {
-                const int i = row0 + rb * 16 + lr;
-                int32_t   o[4];
+                int32_t o[4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                 {
@@ -278,12 +312,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
                 }
                 const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
                 const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
-                if (i < a_M && c + 3 < g.N)
-                    *(uint32_t *)(D + (int64_t)i * g.ldd + c) = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
-                else if (i < a_M)
-                    for (int t = 0; t < 4; ++t)
-                        if (c + t < g.N)
-                            D[(int64_t)i * g.ldd + c + t] = (char)o[t];
+                if (row0 + rb * 16 + lr < a_M && c < a_N)
+                    *(uint32_t *)(drow[rb] + q * 16) = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
             }
         }
     }
@@ -371,9 +401,18 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
             done.fetch_or(1u << dev, std::memory_order_release);
         }
     }
-    GemmArgs a       = args;
-    void    *kargs[] = {&a};
-    const int rows   = NARROW_WAVES * NARROW_ROWS;
+    GemmArgs a = args;
+    // what the A loads' range check compares with
+    if (conv)
+    {
+        const ConvGeom &c      = args.conv;
+        const int64_t   images = ((int64_t)args.M + (int64_t)c.OH * c.OW - 1) / ((int64_t)c.OH * c.OW);
+        a.a_end                = args.A + images * c.H * c.W * c.C;
+    }
+    else
+        a.a_end = args.A + (int64_t)(args.M - 1) * args.lda + args.K;
+    void     *kargs[] = {&a};
+    const int rows    = NARROW_WAVES * NARROW_ROWS;
     return (int)hipLaunchKernel(fn, dim3((args.M + rows - 1) / rows), dim3(NARROW_WAVES * 64), kargs, lds, s);
 }
 } // namespace mi355

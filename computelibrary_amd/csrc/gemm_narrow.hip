@@ -38,6 +38,19 @@ __device__ __forceinline__ int narrow_div(int x, uint32_t magic)
     return (int)(__umulhi((uint32_t)x, magic) + ((uint32_t)x & one));
 }
 
+// bitwise OR of x over the 64 lanes of the wave, as a scalar
+__device__ __forceinline__ uint32_t wave_or(uint32_t x)
+{
+    // row_shr within rows of 16 lanes (bound_ctrl: lanes without a source read 0), then the four row results
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, true); // row_shr:1
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, true); // row_shr:2
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, true); // row_shr:4
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, true); // row_shr:8
+    // lane 15 of every row now holds the row's OR
+    return (uint32_t)__builtin_amdgcn_readlane((int)x, 15) | (uint32_t)__builtin_amdgcn_readlane((int)x, 31) |
+           (uint32_t)__builtin_amdgcn_readlane((int)x, 47) | (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+}
+
 constexpr int NARROW_WAVES  = 4;
 constexpr int NARROW_ROWS   = 32;  // per wave
 constexpr int NARROW_BN     = 64;
@@ -64,11 +77,12 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
               u_fl = (uintptr_t)g.epi.qp_flag;
     uint32_t  a_bytes = (uint32_t)(g.a_end - g.A); // bytes of A: what the range check of the A loads compares with
     int32_t   a_M = g.M, a_K = g.K, a_lda = (int32_t)g.lda, a_kp = (int32_t)g.Kp, a_qps = (int32_t)g.epi.qp_stride;
+    int32_t   tail_start = g.tiles_m, tail_waves = g.tiles_n; // see narrow_launch
     asm volatile(""
                  : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x), "+s"(cg.stride_y),
                    "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word), "+s"(cg.magic_C),
                    "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(cg.magic_OH), "+s"(a_M), "+s"(a_K), "+s"(a_lda), "+s"(a_kp),
-                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl), "+s"(a_bytes));
+                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl), "+s"(a_bytes), "+s"(tail_start), "+s"(tail_waves));
     const MI355_GLOBAL int8_t *const gB = (const MI355_GLOBAL int8_t *)u_b;
     // raw buffer over A (stride 0, 32-bit elements untyped): loads at or past a_bytes - also "negative" offsets, which
     // are huge as unsigned - return zero
@@ -79,7 +93,12 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 15, lh = lane >> 4;
-    const int row0 = blockIdx.x * (NARROW_WAVES * NARROW_ROWS) + wave * NARROW_ROWS;
+    // Workgroups from tail_start on cover only tail_waves * 32 rows each (their other waves help with the B panel and
+    // leave): the last, partial round of workgroups is spread over more compute units in smaller pieces.
+    const int  tail   = (int)blockIdx.x - tail_start;
+    const int  row0   = tail < 0 ? (int)blockIdx.x * (NARROW_WAVES * NARROW_ROWS) + wave * NARROW_ROWS
+                                 : tail_start * (NARROW_WAVES * NARROW_ROWS) + (tail * tail_waves + wave) * NARROW_ROWS;
+    const bool active = (tail < 0 || wave < tail_waves) && row0 < a_M;
 
     // the epilogue's per-column constants (column term + the digested requantisation vectors), where they exist: 6 x 64
     // dwords, one or two per thread, fetched first and parked in LDS with the B panel
@@ -119,6 +138,20 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     }
     (void)my_dma;
 
+    if (!active)
+    {
+        // this wave's share of the B panel and of the constants, then out
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (have_qp)
+        {
+            par[tid] = tp[0];
+            if (tid < NPAR * NARROW_BN - NARROW_WAVES * 64)
+                par[tid + NARROW_WAVES * 64] = tp[1];
+        }
+        __syncthreads();
+        return;
+    }
+
     // ---- A: per-lane source of row rb*16 + lr ----
     // conv: pix[rb] = byte offset of the (possibly out-of-image) top-left tap of the row's pixel, iy0/ix0 its coordinates;
     // dense: byte offset of the row. Rows past M re-use row M-1 (never stored).
@@ -146,7 +179,9 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     // A piece outside the image is replaced by the padding value when it is used; its load goes out all the same (inside
     // the tensor it reads a neighbouring pixel, outside it reads zero). Past K the value is irrelevant: B is zero there.
     v4i      fa[2][3][RS];
-    uint32_t oob = 0; // bit (slot * 3 + kk) * RS + rb: that piece is padding
+    uint32_t oob = 0;      // bit (slot * 3 + kk) * RS + rb: that piece is padding
+    uint32_t oob_wave = 0; // the same bits, set where any lane of the wave has them set (scalar: most pieces of most
+                           // waves have nothing to replace, and a scalar test skips them without vector work)
     // tap of k block kb (UNI: scalar) or of this lane's 16 bytes of it
     auto tap_of = [&](int kb, int &dy, int &dx, int &off)
     {
@@ -201,6 +236,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
                 oob |= (uint32_t)(!ok) << ((slot * 3 + kk) * RS + rb);
             }
         }
+        oob_wave = wave_or(oob);
     };
     load_a(0, 0);
     if (NB > 1)
@@ -258,8 +294,14 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
             for (int rb = 0; rb < RS; ++rb)
             {
                 v4i a = fa[b & 1][kk][rb];
-                if (oob & (1u << (((b & 1) * 3 + kk) * RS + rb)))
-                    a = (v4i){(int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word};
+                if (CONV && (oob_wave & (1u << (((b & 1) * 3 + kk) * RS + rb))))
+                {
+                    // (the asm keeps this a branch - as selects it would cost every wave four instructions per piece -
+                    // and puts two idle cycles between the vector writes and the matrix instruction that reads them)
+                    if (oob & (1u << (((b & 1) * 3 + kk) * RS + rb)))
+                        a = (v4i){(int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word, (int)cg.pad_word};
+                    asm volatile("s_nop 1" : "+v"(a));
+                }
                 if (FLIP_A)
                     a ^= (int)0x80808080;
 #pragma unroll
@@ -411,8 +453,24 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
     }
     else
         a.a_end = args.A + (int64_t)(args.M - 1) * args.lda + args.K;
-    void     *kargs[] = {&a};
-    const int rows    = NARROW_WAVES * NARROW_ROWS;
-    return (int)hipLaunchKernel(fn, dim3((args.M + rows - 1) / rows), dim3(NARROW_WAVES * 64), kargs, lds, s);
+    // Workgroups of 4 waves x 32 rows, 4 to a compute unit. When the last round of workgroups would put a fourth
+    // workgroup on only a few compute units (they finish last: the kernel's time is theirs), its rows go out in
+    // workgroups with fewer working waves, to more compute units.
+    const int rows = NARROW_WAVES * NARROW_ROWS;
+    const int full = (args.M + rows - 1) / rows, cus = device_cus();
+    int       grid = full;
+    a.tiles_m = full, a.tiles_n = NARROW_WAVES;
+    static const int tw_env = getenv("MI355_NARROW_TAIL_WAVES") ? atoi(getenv("MI355_NARROW_TAIL_WAVES")) : 0;
+    const int tw = tw_env >= 1 && tw_env <= 4 ? tw_env : 2;
+    if (cus > 0 && full > cus && full % cus != 0 && full % cus <= cus / 4 && tw < NARROW_WAVES)
+    {
+        const int     start     = full - full % cus;
+        const int64_t tail_rows = (int64_t)args.M - (int64_t)start * rows;
+        a.tiles_m               = start;
+        a.tiles_n               = tw;
+        grid                    = start + (int)((tail_rows + tw * NARROW_ROWS - 1) / (tw * NARROW_ROWS));
+    }
+    void *kargs[] = {&a};
+    return (int)hipLaunchKernel(fn, dim3(grid), dim3(NARROW_WAVES * 64), kargs, lds, s);
 }
 } // namespace mi355

@@ -643,7 +643,7 @@ static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t 
 
 
 // compute units of the current device, asked once per device
-static int device_cus()
+int device_cus()
 {
     static std::atomic<int> cus[32];
     int                     dev = 0;

@@ -141,6 +141,8 @@ int transpose_words_launch(const void *src, void *dst, int batch, int R, int C, 
 // previous contents in half arithmetic and clamped
 int f32_to_f16_launch(const float *dense_f32, void *half_matrix, int batch, int M, int N, int64_t ldh,
                       int64_t h_batch_stride, bool accumulate, float act_min, float act_max, hipStream_t s);
+// compute units of the current device (0 when it cannot be asked)
+int device_cus();
 // byte steps of dimensions 1, 2 and 3 of a tensor whose dimension 0 is a run of contiguous bytes
 struct RestrideSteps
 {

@@ -133,6 +133,10 @@ def test_conv_few_output_channels_kernel():
         ((1, 6, 6, 64), (40, 4, 4, 64), (1, 1), (1, 1, 1, 1), (1, 1), np.int8),       # K = 1024
         ((2, 20, 20, 64), (64, 1, 1, 64), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),     # K = 64, 800 rows
         ((1, 9, 9, 80), (16, 3, 3, 80), (1, 1), (1, 1, 1, 1), (1, 1), np.int8),       # K = 720, C = 80
+        # more than one round of workgroups on every compute unit plus a few: the last rows go out in half-size
+        # workgroups, the very last of them ragged (33708 = 256 * 128 + 14 * 64 + 32 + 12 rows; 33800 rows, 7 columns)
+        ((3, 106, 106, 16), (64, 1, 1, 16), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),
+        ((2, 130, 130, 16), (7, 3, 3, 16), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8),
     ]
     for (shape, wshape, stride, pad, dil, dt) in cases:
         src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)

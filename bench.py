@@ -215,6 +215,59 @@ def run_ceilings(torch, args):
     print(json.dumps(out))
 
 
+def run_phase_clocks(torch, capi, args):
+    """Config 2 on the instrumented build (a library of its own: the product library carries no instrumentation): shader
+    clocks between the ends of the kernel's parts, read from the first lane of consumer wave 0 and producer wave 0 of
+    the first, the middle and the last workgroup of the last launch."""
+    import ctypes
+    from computelibrary_amd import build as _build
+    if not os.path.exists(_build.PHASES_LIB):
+        print("%s is missing: run `python -m computelibrary_amd.build`" % _build.PHASES_LIB, file=sys.stderr)
+        sys.exit(2)
+    capi.LIB_PATH = _build.PHASES_LIB  # before the first call into the library
+    stream = torch.cuda.current_stream().cuda_stream
+    M, N, K = 2048, 4096, 4096
+    A, B, bias, mult, shift = synth_config2(M, N, K)
+    rq = capi.requant(0, 0, -5, -128, 127, per_channel=True)
+    g = capi.Gemm(M, N, K, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    keep = [torch.from_numpy(x).cuda() for x in (bias, mult, shift)]
+    Dd = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    g.prepare(Bd, *keep, stream)
+    wall, evt = time_launches(torch, lambda: g.run(Ad, Dd, None, stream), args.steps, args.warmup)
+    kern_s = time_graph(torch, [lambda cs: g.run(Ad, Dd, None, cs)], args.steps)
+    clock_mhz, cl = None, ceilings_lib()
+    if cl is not None:
+        def burst():
+            for _ in range(300):
+                g.run(Ad, Dd, None, stream)
+        clock_mhz = shader_clock_during(torch, cl, burst)
+    for _ in range(50):
+        g.run(Ad, Dd, None, stream)
+    torch.cuda.synchronize()
+    buf = (ctypes.c_longlong * 48)()
+    rc = capi.lib().mi355_phase_clocks_read(buf)
+    if rc != 0:
+        print("mi355_phase_clocks_read failed: %d" % rc, file=sys.stderr)
+        sys.exit(1)
+    rows = []
+    for r in range(6):
+        v = [int(buf[r * 8 + i]) for i in range(5)]
+        who = ("first", "middle", "last")[r // 2] + " workgroup, " + ("consumer wave 0" if r % 2 == 0 else "producer wave 0")
+        if r % 2 == 0:
+            parts = {"set_up": v[1] - v[0], "wait_for_stage_0": v[2] - v[1], "k_loop": v[3] - v[2], "epilogue": v[4] - v[3]}
+        else:
+            parts = {"set_up": v[1] - v[0], "issue_first_stages": v[2] - v[1], "wait_for_stage_0": v[3] - v[2],
+                     "k_loop": v[4] - v[3]}
+        parts["total"] = v[4] - v[0]
+        rows.append({"wave": who, "clocks": parts})
+    print(json.dumps({"phase_clocks": True, "workload": "config 2: M=2048 N=4096 K=4096 s8 -> s8", "kernel": g.kernel_name,
+                      "kernel_us_instrumented_build": round(kern_s * 1e6, 3), "eager_us": round(evt / args.steps * 1e6, 3),
+                      "shader_clock_MHz": round(clock_mhz, 1) if clock_mhz else None, "k_steps": K // 128,
+                      "waves": rows}))
+    g.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,6 +284,9 @@ def main():
     ap.add_argument("--ceilings", action="store_true",
                     help="only run the measurement-only kernels (read stream, matrix instructions, LDS, direct-to-LDS "
                          "stream, vendor int8 GEMM) and print their figures as one JSON line")
+    ap.add_argument("--phase-clocks", action="store_true",
+                    help="only run config 2 on the build of the library whose pipelined kernel leaves clock readings at "
+                         "the ends of its parts, and print start-up / K loop / epilogue clocks as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -256,6 +312,10 @@ def main():
 
     if args.ceilings:
         run_ceilings(torch, args)
+        return
+
+    if args.phase_clocks:
+        run_phase_clocks(torch, capi, args)
         return
 
     M, N, K = 2048, 4096, 4096

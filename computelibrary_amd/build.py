@@ -16,15 +16,18 @@ LIB = os.path.join(LIBDIR, "libmi355gemmlowp.so")
 # measurement-only kernels for `bench.py --ceilings`: a library of their own, never linked into the product library
 CEILINGS_LIB = os.path.join(LIBDIR, "libmi355ceilings.so")
 CEILINGS_SOURCES = ["ceilings.hip"]
+# the product library once more with the pipelined kernel compiled to leave clock readings at the ends of its parts
+# (`bench.py --phase-clocks`); also a library of its own
+PHASES_LIB = os.path.join(LIBDIR, "libmi355phases.so")
 SOURCES = ["gemm_dma.hip", "gemm_mfma.hip", "gemm_skinny.hip", "gemm_narrow.hip", "kernels_aux.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def _compile(src):
-    obj = os.path.join(OBJDIR, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src, extra=(), suffix=""):
+    obj = os.path.join(OBJDIR, src.replace(".hip", suffix + ".o"))
+    cmd = [HIPCC] + FLAGS + list(extra) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -38,8 +41,11 @@ def build(verbose=True):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=4) as ex:
+        phases = ex.submit(_compile, "gemm_dma.hip", ("-DMI355_PHASE_CLOCKS",), "_phases")
         objs = list(ex.map(_compile, SOURCES + CEILINGS_SOURCES))
-    for lib, members in ((LIB, objs[:len(SOURCES)]), (CEILINGS_LIB, objs[len(SOURCES):])):
+        phases_obj = phases.result()
+    phases_members = [phases_obj if os.path.basename(o) == "gemm_dma.o" else o for o in objs[:len(SOURCES)]]
+    for lib, members in ((LIB, objs[:len(SOURCES)]), (CEILINGS_LIB, objs[len(SOURCES):]), (PHASES_LIB, phases_members)):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + members
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if r.returncode != 0:

@@ -211,6 +211,24 @@ struct PanelProducer
     }
 };
 
+// Measurement build only (-DMI355_PHASE_CLOCKS, a library of its own that the product never loads): the first lane of a
+// consumer wave and of a producer wave of three workgroups (first, middle, last) leaves the shader clock counter at the
+// ends of the kernel's parts, so that start-up, K loop and epilogue can be told apart without a profiler.
+#ifdef MI355_PHASE_CLOCKS
+__device__ long long phase_clocks[6][8];
+#define MI355_PHASE(i)                                                           \
+    do                                                                           \
+    {                                                                            \
+        if (phase_row >= 0 && lane == 0)                                         \
+            phase_clocks[phase_row][i] = (long long)__builtin_readcyclecounter(); \
+    } while (0)
+#else
+#define MI355_PHASE(i) \
+    do                 \
+    {                  \
+    } while (0)
+#endif
+
 // GWM x GWN consumer waves per group, 2 groups stacked along M, plus NP = GWM*GWN producer waves
 template <int BM, int BN, int BK, int GWM, int GWN, int NS, int EPI, bool FLIP_A, bool CONV>
 __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
@@ -253,6 +271,13 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     constexpr bool CDMA = !CONV && (BU % NW == 0) && (AU % NP == 0) && (AU / NP) % 2 == 0;
     constexpr int  CBU  = CDMA ? BU / NW : 0;   // B units per consumer wave per stage
     constexpr int  PLP  = CDMA ? AU / NP : LPP; // loads per producer wave per stage inside the loop
+    // Start-up of dense tiles: a wave gets one direct-to-LDS load accepted about every 190 clocks at the start of a kernel,
+    // so the first NS-1 stages took the 4 producers 2 x 12 loads = 4.6 k clocks while the consumers sat in barrier 0.
+    // All NW + NP waves issue them instead, unit u to wave u % (NW + NP), stage 0 first (4 loads per wave and stage).
+    constexpr int  NALL  = NW + NP;
+    constexpr int  LPW   = (AU + BU) / NALL; // loads per wave per start-up stage
+    constexpr bool SPREAD = CDMA && (AU + BU) % NALL == 0 && (NS - 1) * LPW < 64 &&
+                            (CPR <= 4 || (CPR == 8 && NALL % 2 == 0) || (CPR == 16 && NALL % 4 == 0));
     // Small wave tiles: a slot of matrix instructions is much shorter than a slot of operand reads, so running the two
     // consumer groups one slot apart only serialises their reads; both groups then read and multiply in the same slots.
     constexpr bool INPHASE = RS * QS * KK <= 16;
@@ -267,6 +292,11 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
+#ifdef MI355_PHASE_CLOCKS
+    const int phase_blk = blockIdx.x == 0 ? 0 : ((int)blockIdx.x == g.nblocks / 2 ? 1 : ((int)blockIdx.x == g.nblocks - 1 ? 2 : -1));
+    const int phase_row = phase_blk < 0 ? -1 : (wave == 0 ? phase_blk * 2 : (wave == NW ? phase_blk * 2 + 1 : -1));
+    MI355_PHASE(0); // arguments fetched, first instructions
+#endif
     int tm, tn, bz;
     if (g.tile_magic_ok)
         tile_coords_batched_fast(blockIdx.x, g.nblocks, g.tiles_m, g.tiles_n, g.magic_tiles, g.magic_group, bz, tm, tn);
@@ -275,10 +305,41 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = (g.K + BK - 1) / BK;
     // which requantisation formula applies was decided on the device when the per-column constants were digested
+    // (a scalar load: as a vector load its wait would also wait for every direct-to-LDS load issued before it)
     int qflag = 1;
     if (EPI == EPI_FIXEDPOINT && u_fl != 0)
-        qflag = __builtin_amdgcn_readfirstlane(*(global_i32)u_fl);
+        qflag = *(const __attribute__((address_space(4))) int32_t *)u_fl;
     const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
+
+    // per-column epilogue constants of this block: fetched now by the consumer waves (before their share of the start-up
+    // loads, so that waiting for those covers these too), parked in registers, staged in LDS after the loop
+    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
+    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
+    int32_t       par_reg[PPT > 0 ? PPT : 1];
+    if (fast && wave < NW)
+    {
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            const int idx = tid + t * NW * 64;
+            par_reg[t]    = 0;
+            if (idx < NPAR * BN)
+            {
+                const int par = idx / BN, col = idx % BN;
+                par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
+                                         : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
+            }
+        }
+    }
+    if constexpr (SPREAD)
+    {
+        PanelProducer<BM, BN, BK, NALL, NS, CONV> first;
+        first.init(g, m0, n0, bz, wave, lane, lds0);
+#pragma unroll
+        for (int s = 0; s < NS - 1; ++s)
+            if (s < nk)
+                first.issue(s, s % NS);
+    }
 
     // Barrier protocol (b = number of barriers a wave has executed): consumer group 0 reads stage kt between barriers
     // 2kt and 2kt+1 and multiplies it between 2kt+1 and 2kt+2; group 1 does the same one barrier later. Producers make
@@ -289,14 +350,20 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
         // ================= producer: global -> LDS =================
         PanelProducer<BM, BN, BK, NP, NS, CONV> prod;
         prod.init(g, m0, n0, bz, wave - NW, lane, lds0);
+        MI355_PHASE(1); // producer: addresses set up
+        if constexpr (!SPREAD)
+        {
 #pragma unroll
-        for (int s = 0; s < NS - 1; ++s)
-            if (s < nk)
-                prod.issue(s, s % NS);
+            for (int s = 0; s < NS - 1; ++s)
+                if (s < nk)
+                    prod.issue(s, s % NS);
+        }
+        MI355_PHASE(2); // producer: the first NS-1 stages issued
         if (nk >= NS - 1)
-            wait_vmcnt<(NS - 2) * LPP>(); // stage 0 complete, the NS-2 younger stages may still be in flight
+            wait_vmcnt<(NS - 2) * (SPREAD ? LPW : LPP)>(); // stage 0 complete, the NS-2 younger stages may still be in flight
         else
             wait_vmcnt<0>();
+        MI355_PHASE(3); // producer: its part of stage 0 has landed
         block_barrier(); // barrier 0
         for (int kt = 0; kt < nk; ++kt)
         {
@@ -316,6 +383,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
             block_barrier(); // barrier 2kt+2
         }
         block_barrier(); // barrier 2nk+1
+        MI355_PHASE(4); // producer: K loop over
         if (fast)
         {
             __syncthreads(); // the consumers' staging of the epilogue constants
@@ -330,26 +398,6 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     const int wq    = wave % GW;
     const int row_w = group * (BM / 2) + (wq / GWN) * TM; // this wave's sub-tile inside the block tile
     const int col_w = (wq % GWN) * TN;
-
-    // per-column epilogue constants of this block: fetched now, parked in registers, staged in LDS after the loop
-    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
-    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
-    int32_t       par_reg[PPT > 0 ? PPT : 1];
-    if (fast)
-    {
-#pragma unroll
-        for (int t = 0; t < PPT; ++t)
-        {
-            const int idx = tid + t * NW * 64;
-            par_reg[t]    = 0;
-            if (idx < NPAR * BN)
-            {
-                const int par = idx / BN, col = idx % BN;
-                par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
-                                         : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
-            }
-        }
-    }
 
     v4i acc[RS][QS];
 #pragma unroll
@@ -382,7 +430,17 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
                              (uint32_t)(((lane % CPR) ^ swz<CPR>(wave * RPU + lane / CPR)) * 16);
     const uint32_t cb_lds  = lds0 + (uint32_t)(AU + wave) * 1024u;
 
+    MI355_PHASE(1); // consumer: set-up done, waiting for stage 0
+    if constexpr (SPREAD)
+    {
+        // this wave's units of stage 0 (and the epilogue constants before them)
+        if (nk >= NS - 1)
+            wait_vmcnt<(NS - 2) * LPW>();
+        else
+            wait_vmcnt<0>();
+    }
     block_barrier(); // barrier 0: stage 0 is in LDS
+    MI355_PHASE(2); // consumer: stage 0 is in LDS
     if (group == 1 && !INPHASE)
         block_barrier(); // group 1 runs one slot behind group 0
 
@@ -446,6 +504,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
         wait_vmcnt<0>();
     if (group == 0 || INPHASE)
         block_barrier(); // barrier 2nk+1; every operand read of every wave is complete beyond this point
+    MI355_PHASE(3); // consumer: K loop over
 
     if (fast)
     {
@@ -483,6 +542,7 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     }
     else
         epilogue_store_t<EPI, RS, QS>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
+    MI355_PHASE(4); // consumer: epilogue done (stores issued)
 }
 
 // ---- instantiation table -------------------------------------------------------------------------------------------
@@ -578,3 +638,11 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);
 }
 } // namespace mi355
+
+#ifdef MI355_PHASE_CLOCKS
+// 6 rows (first / middle / last workgroup x consumer wave 0, producer wave 0) of 8 clock readings, of the last launch
+extern "C" int mi355_phase_clocks_read(long long *out)
+{
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mi355::phase_clocks), sizeof(long long) * 48);
+}
+#endif

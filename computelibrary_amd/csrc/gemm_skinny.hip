@@ -417,16 +417,19 @@ struct OnceArgs
     float          scale, act_min, act_max;
     int32_t        has_offsets, accumulate, act_twice;
 };
-template <int EPI, bool FLIP_A, int PER, bool MULTI>
+// R16: up to 16 rows (all rows of the matrix instruction carry data, all 64 lanes hold results) instead of up to 8
+template <int EPI, bool FLIP_A, int PER, bool MULTI, bool R16>
 __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g)
 {
-    constexpr int SLICE = PER * 64, PITCH = SLICE + 64; // bytes of a row of A per wave; the pitch spreads 8 rows over the banks
-    constexpr int NA    = 8 * SLICE / 1024 > 0 ? 8 * SLICE / 1024 : 1; // 1 KiB loads that cover 8 rows of a slice
-    constexpr int LPR   = SLICE / 16;                                  // lanes per row
-    constexpr int RPL   = 64 / LPR > 8 ? 8 : 64 / LPR;                 // rows per load
-    __shared__ __attribute__((aligned(16))) int32_t red[2][ONCE_WAVES][32][4];
+    constexpr int ROWS  = R16 ? 16 : 8;   // rows of A that are staged
+    constexpr int RL    = R16 ? 64 : 32;  // lanes of a wave that hold results
+    constexpr int SLICE = PER * 64, PITCH = SLICE + 64; // bytes of a row of A per wave; the pitch spreads the rows over the banks
+    constexpr int NA    = ROWS * SLICE / 1024 > 0 ? ROWS * SLICE / 1024 : 1; // 1 KiB loads that cover the rows of a slice
+    constexpr int LPR   = SLICE / 16;                                        // lanes per row
+    constexpr int RPL   = 64 / LPR > ROWS ? ROWS : 64 / LPR;                 // rows per load
+    __shared__ __attribute__((aligned(16))) int32_t red[2][ONCE_WAVES][RL][4];
     __shared__ int32_t                              par[4][64]; // [vector][group * 16 + column]; row vector: [3][row]
-    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][8][PITCH]
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][ROWS][PITCH]
 
     // Everything is pinned in registers here, so that it is all fetched before this point. A pointer that went through the
     // asm as an integer is a generic pointer no more: it comes back as a pointer to global memory (generic loads would
@@ -474,11 +477,11 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
                                           : v == 1 ? (EPI == EPI_FIXEDPOINT ? g_mult : (EPI == EPI_F32 && has_bias ? g_bias : g_colvec))
                                           : v == 2 ? (EPI == EPI_FIXEDPOINT ? g_shift : g_colvec)
                                                    : g_rowvec;
-        par_v                           = vec[v == 3 ? min(lane & 7, g.M - 1) : j];
+        par_v                           = vec[v == 3 ? min(lane & (ROWS - 1), g.M - 1) : j];
     }
 
     // this wave's slice of A: rows past M re-read row M-1 into staging rows whose results are never stored
-    char *a_lds = a_stage + wave * 8 * PITCH;
+    char *a_lds = a_stage + wave * ROWS * PITCH;
     v4i   ta[NA];
     const int a_sr = lane / LPR, a_sc = (lane % LPR) * 16;
     {
@@ -509,18 +512,18 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
     {
         if (FLIP_A)
             ta[i] ^= (int)0x80808080;
-        if (i * RPL + a_sr < 8 && a_sr < RPL)
+        if (i * RPL + a_sr < ROWS && a_sr < RPL)
             *(v4i *)(a_lds + (i * RPL + a_sr) * PITCH + a_sc) = ta[i];
     }
     par[wave & 3][lane] = par_v; // read behind the first group's barrier
-    // operand blocks of A: lane -> row lane % 16 (rows 8..15 are zero), 16 bytes at k offset (lane / 16) * 16
+    // operand blocks of A: lane -> row lane % 16 (rows from ROWS on are zero), 16 bytes at k offset (lane / 16) * 16
     const int arow = lane & 15, akc = (lane >> 4) * 16;
     v4i       fa[PER];
 #pragma unroll
     for (int u = 0; u < PER; ++u)
     {
         fa[u] = (v4i){0, 0, 0, 0};
-        if (busy && arow < 8 && kb0 + u < KB)
+        if (busy && arow < ROWS && kb0 + u < KB)
             fa[u] = *(const v4i *)(a_lds + arow * PITCH + u * 64 + akc);
     }
 
@@ -549,18 +552,18 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
             if (gi + 2 < MINE)
                 load_b(gi & 1, gi + 2);
             // accumulator r of lane l is row 4 * (l / 16) + r, column l % 16: lanes 32..63 hold rows 8..15
-            if (lane < 32)
+            if (R16 || lane < 32)
                 *(v4i *)&red[gi & 1][wave][lane][0] = acc0;
             __syncthreads();
-            if (t < 128)
+            if (t < ROWS * 16)
             {
                 const int      j = ((int)blockIdx.x + gi * G) * 16 + ecol;
                 const int32_t *r = &red[gi & 1][0][(erow >> 2) * 16 + ecol][erow & 3];
                 int32_t        sum = 0;
 #pragma unroll
                 for (int w = 0; w < ONCE_WAVES; ++w)
-                    sum += r[w * 32 * 4];
-                const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & 7];
+                    sum += r[w * RL * 4];
+                const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & (ROWS - 1)];
                 if (j < g.N && erow < g.M)
                 {
                     const int64_t idx = (int64_t)erow * g.ldd + j;
@@ -659,21 +662,21 @@ int device_cus()
     return n;
 }
 
-template <int PER, bool MULTI>
-static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
+template <int PER, bool MULTI, bool R16>
+static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
     static const void *const fns[3][2] = {
-        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI>,
-         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI>},
-        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI>,
-         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI>},
-        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI>,
-         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI>}};
+        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI, R16>,
+         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI, R16>},
+        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI, R16>,
+         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI, R16>},
+        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI, R16>,
+         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI, R16>}};
     // the kernel fetches these without asking
     if (a.epi.colvec == nullptr || a.epi.rowvec == nullptr || (epi == EPI_FIXEDPOINT && (a.epi.mult == nullptr || a.epi.shift == nullptr)))
         return (int)hipErrorInvalidValue;
     static std::atomic<uint32_t> lds_raised[3][2];
-    const size_t                 lds = (size_t)ONCE_WAVES * 8 * (PER * 64 + 64);
+    const size_t                 lds = (size_t)ONCE_WAVES * (R16 ? 16 : 8) * (PER * 64 + 64);
     const void                  *fn  = fns[epi][flip_a ? 1 : 0];
     // 16 KiB of static LDS on top: declare the dynamic part whatever its size
     const int e = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
@@ -685,6 +688,13 @@ static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int gri
                p.has_offsets, p.accumulate, p.act_twice};
     void *kargs[] = {&o};
     return (int)hipLaunchKernel(fn, dim3(grid), dim3(ONCE_WAVES * 64), kargs, lds, s);
+}
+
+template <int PER, bool MULTI>
+static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
+{
+    return a.M > 8 ? skinny_once_launch_r<PER, MULTI, true>(epi, flip_a, a, grid, s)
+                   : skinny_once_launch_r<PER, MULTI, false>(epi, flip_a, a, grid, s);
 }
 
 // Environment overrides for experiments, read once: MI355_SKINNY_WAVES (4 or 8; anything else is ignored),
@@ -715,13 +725,14 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     const int KB     = (int)(args.Kp / 64);
     // Up to 8 rows every wave copies its K slice of A (at most 1 KiB per row) into LDS once and takes its operands
     // from there; that needs nothing to guard
-    const bool stage_ok = args.M <= 8 && args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 &&
-                          ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
+    const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
+    const bool stage_ok = args.M <= 8 && align_ok;
+    const bool once_ok  = args.M <= 16 && align_ok; // the stage-once form also takes a full block of 16 rows
     // Up to 4096 of K the stage-once form: one workgroup per column group while there are no more groups than compute
     // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
     // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside
     // the first on a compute unit: one workgroup of 8 waves per group below. Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
-    if (stage_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    if (once_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0 && (groups <= cus || groups >= 2 * cus))

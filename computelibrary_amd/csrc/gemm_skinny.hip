@@ -417,19 +417,34 @@ struct OnceArgs
     float          scale, act_min, act_max;
     int32_t        has_offsets, accumulate, act_twice;
 };
-// R16: up to 16 rows (all rows of the matrix instruction carry data, all 64 lanes hold results) instead of up to 8
-template <int EPI, bool FLIP_A, int PER, bool MULTI, bool R16>
+// bytes from one staged row of A to the next: 8 / 16 rows keep the pitch they were tuned with; 32 rows take the smallest
+// pitch that still spreads the rows over the banks (an odd number of 16-byte pieces), or the slices would not fit
+__host__ __device__ constexpr int once_pitch(int rows, int per)
+{
+    return per * 64 + (rows > 16 ? 16 : 64);
+}
+
+// ROWS: rows of A that are staged - 8 (half of the matrix instruction's rows are padding), 16, or 32 (two blocks of 16
+// rows: two matrix instructions per B operand block)
+template <int EPI, bool FLIP_A, int PER, bool MULTI, int ROWS>
 __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g)
 {
-    constexpr int ROWS  = R16 ? 16 : 8;   // rows of A that are staged
-    constexpr int RL    = R16 ? 64 : 32;  // lanes of a wave that hold results
-    constexpr int SLICE = PER * 64, PITCH = SLICE + 64; // bytes of a row of A per wave; the pitch spreads the rows over the banks
+    static_assert(ROWS == 8 || ROWS == 16 || ROWS == 32, "rows");
+    constexpr int RB    = ROWS > 16 ? 2 : 1;   // blocks of 16 rows
+    constexpr int RL    = ROWS == 8 ? 32 : 64; // lanes of a wave that hold results (per block of rows)
+    constexpr int SLICE = PER * 64, PITCH = once_pitch(ROWS, PER); // bytes of a row of A per wave
     constexpr int NA    = ROWS * SLICE / 1024 > 0 ? ROWS * SLICE / 1024 : 1; // 1 KiB loads that cover the rows of a slice
     constexpr int LPR   = SLICE / 16;                                        // lanes per row
     constexpr int RPL   = 64 / LPR > ROWS ? ROWS : 64 / LPR;                 // rows per load
-    __shared__ __attribute__((aligned(16))) int32_t red[2][ONCE_WAVES][RL][4];
+    // partial results [2][wave][block of rows][lane][4]: for 32 rows they take over the staging area once every wave
+    // has its operands of A in registers (the two together would not fit)
+    constexpr bool RED_IN_STAGE = RB > 1;
+    __shared__ __attribute__((aligned(16))) int32_t red_own[RED_IN_STAGE ? 1 : 2 * ONCE_WAVES * RB * RL * 4];
     __shared__ int32_t                              par[4][64]; // [vector][group * 16 + column]; row vector: [3][row]
     extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][ROWS][PITCH]
+    // (the launch sizes the dynamic area for the larger of the two)
+    int32_t *const red = RED_IN_STAGE ? (int32_t *)a_stage : red_own;
+    // red[((buf * ONCE_WAVES + wave) * RB + rb) * RL + lane][4]
 
     // Everything is pinned in registers here, so that it is all fetched before this point. A pointer that went through the
     // asm as an integer is a generic pointer no more: it comes back as a pointer to global memory (generic loads would
@@ -518,14 +533,18 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
     par[wave & 3][lane] = par_v; // read behind the first group's barrier
     // operand blocks of A: lane -> row lane % 16 (rows from ROWS on are zero), 16 bytes at k offset (lane / 16) * 16
     const int arow = lane & 15, akc = (lane >> 4) * 16;
-    v4i       fa[PER];
+    v4i       fa[RB][PER];
 #pragma unroll
-    for (int u = 0; u < PER; ++u)
-    {
-        fa[u] = (v4i){0, 0, 0, 0};
-        if (busy && arow < ROWS && kb0 + u < KB)
-            fa[u] = *(const v4i *)(a_lds + arow * PITCH + u * 64 + akc);
-    }
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            fa[rb][u] = (v4i){0, 0, 0, 0};
+            if (busy && rb * 16 + arow < ROWS && kb0 + u < KB)
+                fa[rb][u] = *(const v4i *)(a_lds + (rb * 16 + arow) * PITCH + u * 64 + akc);
+        }
+    if (RED_IN_STAGE)
+        __syncthreads(); // every wave has its operands: the staging area becomes the partial results' area
 
     // The groups of a workgroup, written out for each possible count: with the count a run-time value the fetch of
     // group gi + 2 sits behind a condition, the compiler loses count of the loads in flight, and the matrix instructions
@@ -536,7 +555,10 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
 #pragma unroll
         for (int gi = 0; gi < MINE; ++gi)
         {
-            v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+            v4i acc0[RB], acc1[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+                acc0[rb] = (v4i){0, 0, 0, 0}, acc1[rb] = (v4i){0, 0, 0, 0};
             if (busy)
             {
                 // The two chains are added and the sum is held back for 32 issue slots in the same basic block as the
@@ -545,24 +567,43 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
                 // branch it came 3 slots after the instruction and read the last register of the result too early.
 #pragma unroll
                 for (int u = 0; u < PER; ++u)
-                    (u & 1 ? acc1 : acc0) = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fb[gi & 1][u], u & 1 ? acc1 : acc0, 0, 0, 0);
-                acc0 += acc1;
-                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0));
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb)
+                        (u & 1 ? acc1[rb] : acc0[rb]) =
+                            __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[gi & 1][u], u & 1 ? acc1[rb] : acc0[rb], 0, 0, 0);
+                if (RB == 1)
+                {
+                    acc0[0] += acc1[0];
+                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]));
+                }
+                else
+                {
+                    // (the wait first: the sums below are the first readers of the results)
+                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc1[0]), "+v"(acc0[RB - 1]), "+v"(acc1[RB - 1]));
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb)
+                        acc0[rb] += acc1[rb];
+                }
             }
             if (gi + 2 < MINE)
                 load_b(gi & 1, gi + 2);
             // accumulator r of lane l is row 4 * (l / 16) + r, column l % 16: lanes 32..63 hold rows 8..15
-            if (R16 || lane < 32)
-                *(v4i *)&red[gi & 1][wave][lane][0] = acc0;
+            if (RL == 64 || lane < 32)
+            {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    *(v4i *)&red[((((gi & 1) * ONCE_WAVES + wave) * RB + rb) * RL + lane) * 4] = acc0[rb];
+            }
             __syncthreads();
             if (t < ROWS * 16)
             {
+                // output (erow, ecol): block of rows erow / 16, there accumulator erow % 4 of lane (erow % 16 / 4) * 16 + ecol
                 const int      j = ((int)blockIdx.x + gi * G) * 16 + ecol;
-                const int32_t *r = &red[gi & 1][0][(erow >> 2) * 16 + ecol][erow & 3];
+                const int32_t *r = &red[((((gi & 1) * ONCE_WAVES) * RB + (erow >> 4)) * RL + ((erow & 15) >> 2) * 16 + ecol) * 4 + (erow & 3)];
                 int32_t        sum = 0;
 #pragma unroll
                 for (int w = 0; w < ONCE_WAVES; ++w)
-                    sum += r[w * RL * 4];
+                    sum += r[w * RB * RL * 4];
                 const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & (ROWS - 1)];
                 if (j < g.N && erow < g.M)
                 {
@@ -662,21 +703,22 @@ int device_cus()
     return n;
 }
 
-template <int PER, bool MULTI, bool R16>
+template <int PER, bool MULTI, int ROWS>
 static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
     static const void *const fns[3][2] = {
-        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI, R16>,
-         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI, R16>},
-        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI, R16>,
-         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI, R16>},
-        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI, R16>,
-         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI, R16>}};
+        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI, ROWS>,
+         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI, ROWS>},
+        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI, ROWS>,
+         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI, ROWS>},
+        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI, ROWS>,
+         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI, ROWS>}};
     // the kernel fetches these without asking
     if (a.epi.colvec == nullptr || a.epi.rowvec == nullptr || (epi == EPI_FIXEDPOINT && (a.epi.mult == nullptr || a.epi.shift == nullptr)))
         return (int)hipErrorInvalidValue;
     static std::atomic<uint32_t> lds_raised[3][2];
-    const size_t                 lds = (size_t)ONCE_WAVES * (R16 ? 16 : 8) * (PER * 64 + 64);
+    // staged rows of A; with 32 rows the partial results (2 x 16 waves x 2 blocks x 64 lanes x 16 bytes) share the area
+    const size_t                 lds = std::max((size_t)ONCE_WAVES * ROWS * once_pitch(ROWS, PER), ROWS > 16 ? (size_t)65536 : (size_t)0);
     const void                  *fn  = fns[epi][flip_a ? 1 : 0];
     // 16 KiB of static LDS on top: declare the dynamic part whatever its size
     const int e = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
@@ -693,8 +735,9 @@ static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int gri
 template <int PER, bool MULTI>
 static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
-    return a.M > 8 ? skinny_once_launch_r<PER, MULTI, true>(epi, flip_a, a, grid, s)
-                   : skinny_once_launch_r<PER, MULTI, false>(epi, flip_a, a, grid, s);
+    return a.M > 16  ? skinny_once_launch_r<PER, MULTI, 32>(epi, flip_a, a, grid, s)
+           : a.M > 8 ? skinny_once_launch_r<PER, MULTI, 16>(epi, flip_a, a, grid, s)
+                     : skinny_once_launch_r<PER, MULTI, 8>(epi, flip_a, a, grid, s);
 }
 
 // Environment overrides for experiments, read once: MI355_SKINNY_WAVES (4 or 8; anything else is ignored),
@@ -727,7 +770,7 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     // from there; that needs nothing to guard
     const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
     const bool stage_ok = args.M <= 8 && align_ok;
-    const bool once_ok  = args.M <= 16 && align_ok; // the stage-once form also takes a full block of 16 rows
+    const bool once_ok  = args.M <= 32 && align_ok; // the stage-once form also takes one or two full blocks of 16 rows
     // Up to 4096 of K the stage-once form: one workgroup per column group while there are no more groups than compute
     // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
     // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside

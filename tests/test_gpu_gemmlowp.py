@@ -276,10 +276,11 @@ def test_skinny_kernel_with_staged_a(M):
         np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16])
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16, 17, 25, 32])
 def test_skinny_stage_once_kernel(M):
-    """Up to 16 rows (two builds: up to 8, where half of the matrix instruction's rows are padding, and 9 to 16) and K <= 4096 (whole 64-byte blocks, 16-byte aligned rows) one workgroup of 16 waves per compute unit
-    walks several column groups with A staged once: K picks 1, 2 or 4 k blocks per wave, with the last busy wave short
+    """Up to 32 rows (three builds: up to 8, where half of the matrix instruction's rows are padding, 9 to 16, and 17 to
+    32 as two blocks of rows) and K <= 4096 (whole 64-byte blocks, 16-byte aligned rows): one workgroup of 16 waves per
+    compute unit walks several column groups with A staged once: K picks 1, 2 or 4 k blocks per wave, with the last busy wave short
     (K = 2112, 3136) or waves without any k block (K = 64, 640); N covers a single ragged group, fewer groups than compute
     units, 2 to 3 groups per workgroup and more than four times the compute units; every epilogue, signed and unsigned
     A, a non-zero B offset (row vector) and accumulation."""

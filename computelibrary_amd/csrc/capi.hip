@@ -194,7 +194,10 @@ struct GemmCore
             // that the pipelined kernel would leave most compute units without a tile
             // (a batch of small products runs the streaming kernel once per entry: the tiled kernels would spend a 64-row
             // tile, mostly padding, on each)
-            path = (M <= 32 || (batch == 1 && M <= SKINNY_MAX_M && N < 8192)) ? MI355_PATH_SKINNY : MI355_PATH_MFMA;
+            // (and up to 64 rows whenever K <= 4096 is a whole number of 64-byte blocks: the form of the streaming
+            // kernel that keeps the operand blocks of A in registers for its whole run then applies)
+            path = (M <= 32 || (batch == 1 && M <= SKINNY_MAX_M && (N < 8192 || (K <= 4096 && K % 64 == 0)))) ? MI355_PATH_SKINNY
+                                                                                                         : MI355_PATH_MFMA;
         if (path == MI355_PATH_SKINNY && M > SKINNY_MAX_M)
             return fail("skinny path needs M <= %d", SKINNY_MAX_M);
         if (path == MI355_PATH_SIMPLE)

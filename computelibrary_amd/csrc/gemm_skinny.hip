@@ -424,13 +424,18 @@ __host__ __device__ constexpr int once_pitch(int rows, int per)
     return per * 64 + (rows > 16 ? 16 : 64);
 }
 
-// ROWS: rows of A that are staged - 8 (half of the matrix instruction's rows are padding), 16, or 32 (two blocks of 16
-// rows: two matrix instructions per B operand block)
-template <int EPI, bool FLIP_A, int PER, bool MULTI, int ROWS>
-__global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g)
+// ROWS: rows of A - 8 (half of the matrix instruction's rows are padding), 16, 32 (two blocks of 16 rows: two matrix
+// instructions per B operand block) or 64 (four blocks). Up to 32 rows a workgroup has 16 waves and every wave stages
+// its K slice of A in LDS; 64 rows x 4096 bytes would not fit there, and need not: the operand blocks of A stay in
+// registers for the whole kernel, so with 64 rows a workgroup has 8 waves (256 registers each: 128 of them hold A) and
+// gathers the blocks straight from global memory, once.
+template <int EPI, bool FLIP_A, int PER, bool MULTI, int ROWS, int WAVES = ONCE_WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g)
 {
-    static_assert(ROWS == 8 || ROWS == 16 || ROWS == 32, "rows");
-    constexpr int RB    = ROWS > 16 ? 2 : 1;   // blocks of 16 rows
+    static_assert(ROWS == 8 || ROWS == 16 || ROWS == 32 || ROWS == 64, "rows");
+    static_assert((ROWS == 64) == (WAVES == 8) && (WAVES == 8 || WAVES == ONCE_WAVES), "waves");
+    constexpr bool A_GLOBAL = ROWS == 64;      // operand blocks of A straight from global memory
+    constexpr int RB    = ROWS / 16 > 0 ? ROWS / 16 : 1; // blocks of 16 rows
     constexpr int RL    = ROWS == 8 ? 32 : 64; // lanes of a wave that hold results (per block of rows)
     constexpr int SLICE = PER * 64, PITCH = once_pitch(ROWS, PER); // bytes of a row of A per wave
     constexpr int NA    = ROWS * SLICE / 1024 > 0 ? ROWS * SLICE / 1024 : 1; // 1 KiB loads that cover the rows of a slice
@@ -439,12 +444,12 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
     // partial results [2][wave][block of rows][lane][4]: for 32 rows they take over the staging area once every wave
     // has its operands of A in registers (the two together would not fit)
     constexpr bool RED_IN_STAGE = RB > 1;
-    __shared__ __attribute__((aligned(16))) int32_t red_own[RED_IN_STAGE ? 1 : 2 * ONCE_WAVES * RB * RL * 4];
+    __shared__ __attribute__((aligned(16))) int32_t red_own[RED_IN_STAGE ? 1 : 2 * WAVES * RB * RL * 4];
     __shared__ int32_t                              par[4][64]; // [vector][group * 16 + column]; row vector: [3][row]
-    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][ROWS][PITCH]
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [WAVES][ROWS][PITCH] (nothing staged with 64 rows)
     // (the launch sizes the dynamic area for the larger of the two)
     int32_t *const red = RED_IN_STAGE ? (int32_t *)a_stage : red_own;
-    // red[((buf * ONCE_WAVES + wave) * RB + rb) * RL + lane][4]
+    // red[((buf * WAVES + wave) * RB + rb) * RL + lane][4]
 
     // Everything is pinned in registers here, so that it is all fetched before this point. A pointer that went through the
     // asm as an integer is a generic pointer no more: it comes back as a pointer to global memory (generic loads would
@@ -483,7 +488,7 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
     // wait for A wait for B too); the host passes every vector (replicated scalars, a zero row vector) and only the
     // float bias may be missing, in which case the column term stands in. Every wave leaves its dword in LDS (four
     // waves write the same value to the same place) for the epilogue threads.
-    const int t = (int)threadIdx.x, erow = t >> 4, ecol = t & 15;
+    const int t = (int)threadIdx.x;
     int32_t   par_v;
     {
         const int                   v   = wave & 3;
@@ -499,6 +504,10 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
     char *a_lds = a_stage + wave * ROWS * PITCH;
     v4i   ta[NA];
     const int a_sr = lane / LPR, a_sc = (lane % LPR) * 16;
+    // operand blocks of A: lane -> row lane % 16 of a block of rows, 16 bytes at k offset (lane / 16) * 16
+    const int arow = lane & 15, akc = (lane >> 4) * 16;
+    v4i       fa[RB][PER];
+    if constexpr (!A_GLOBAL)
     {
         // lanes past the end of K (last busy wave) re-read the slice's first 16 bytes into columns nobody reads; waves
         // without k blocks re-read the last k block
@@ -508,43 +517,74 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
             ta[i] = *(const MI355_GLOBAL v4i *)(gA + (int64_t)min(i * RPL + a_sr, g.M - 1) * g.lda + (int64_t)min(kb0, KB - 1) * 64 + col);
     }
     const MI355_GLOBAL int8_t *bp = gB + ((int64_t)min(kb0, KB - 1) * 64 + lane) * 16; // (waves without k blocks re-read the last one)
-    v4i           fb[2][PER];
-    auto load_b = [&](int slot, int gi)
+    // B operand blocks: two groups' worth in flight per wave - or, with 64 rows (half the registers hold A), one group's
+    // worth, refilled half by half as the matrix instructions release them
+    constexpr int H0 = PER / 2; // k blocks of the first half
+    v4i           fb[A_GLOBAL ? 1 : 2][PER];
+    auto load_b_part = [&](int slot, int gi, auto u0c, auto u1c)
     {
         const int grp = min((int)blockIdx.x + gi * G, NGT - 1);
 #pragma unroll
-        for (int u = 0; u < PER; ++u) // k blocks past KB (last busy wave, K not a multiple of 64 * PER) re-read the last one
+        for (int u = decltype(u0c)::value; u < decltype(u1c)::value; ++u) // k blocks past KB (last busy wave) re-read the last one
             fb[slot][u] = __builtin_nontemporal_load((const MI355_GLOBAL v4i *)(bp + ((int64_t)grp * KB + max(min(u, KB - 1 - kb0), 0)) * 1024));
     };
+    auto load_b = [&](int slot, int gi) { load_b_part(slot, gi, std::integral_constant<int, 0>{}, std::integral_constant<int, PER>{}); };
     // MULTI: every workgroup has at least two groups. Nothing between here and the wait for A may sit behind a branch:
     // the compiler would no longer know how many loads are in flight and would make the wait for A wait for B as well
     // (loads return in order) - hence also the unconditional fetches of the epilogue constants below.
     load_b(0, 0);
-    if (MULTI)
+    if (MULTI && !A_GLOBAL)
         load_b(1, 1);
-#pragma unroll
-    for (int i = 0; i < NA; ++i)
+    // (with nothing to stage, A is fetched behind the first B blocks: the first matrix instruction needs both anyway,
+    // and the stream of B starts that much earlier)
+    if constexpr (A_GLOBAL)
     {
-        if (FLIP_A)
-            ta[i] ^= (int)0x80808080;
-        if (i * RPL + a_sr < ROWS && a_sr < RPL)
-            *(v4i *)(a_lds + (i * RPL + a_sr) * PITCH + a_sc) = ta[i];
+        // rows past M re-read row M-1 (never stored), k blocks past KB the last one (set to zero below)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int u = 0; u < PER; ++u)
+                fa[rb][u] = *(const MI355_GLOBAL v4i *)(gA + (int64_t)min(rb * 16 + arow, g.M - 1) * g.lda +
+                                                        (int64_t)min(kb0 + u, KB - 1) * 64 + akc);
     }
-    par[wave & 3][lane] = par_v; // read behind the first group's barrier
-    // operand blocks of A: lane -> row lane % 16 (rows from ROWS on are zero), 16 bytes at k offset (lane / 16) * 16
-    const int arow = lane & 15, akc = (lane >> 4) * 16;
-    v4i       fa[RB][PER];
+    if constexpr (A_GLOBAL)
+    {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int u = 0; u < PER; ++u)
+            for (int u = 0; u < PER; ++u)
+            {
+                if (FLIP_A)
+                    fa[rb][u] ^= (int)0x80808080;
+                if (!(busy && kb0 + u < KB))
+                    fa[rb][u] = (v4i){0, 0, 0, 0};
+            }
+        par[wave & 3][lane] = par_v; // read behind the first group's barrier
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
         {
-            fa[rb][u] = (v4i){0, 0, 0, 0};
-            if (busy && rb * 16 + arow < ROWS && kb0 + u < KB)
-                fa[rb][u] = *(const v4i *)(a_lds + (rb * 16 + arow) * PITCH + u * 64 + akc);
+            if (FLIP_A)
+                ta[i] ^= (int)0x80808080;
+            if (i * RPL + a_sr < ROWS && a_sr < RPL)
+                *(v4i *)(a_lds + (i * RPL + a_sr) * PITCH + a_sc) = ta[i];
         }
-    if (RED_IN_STAGE)
-        __syncthreads(); // every wave has its operands: the staging area becomes the partial results' area
+        par[wave & 3][lane] = par_v; // read behind the first group's barrier
+        // (rows from ROWS on are zero)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int u = 0; u < PER; ++u)
+            {
+                fa[rb][u] = (v4i){0, 0, 0, 0};
+                if (busy && rb * 16 + arow < ROWS && kb0 + u < KB)
+                    fa[rb][u] = *(const v4i *)(a_lds + (rb * 16 + arow) * PITCH + u * 64 + akc);
+            }
+        if (RED_IN_STAGE)
+            __syncthreads(); // every wave has its operands: the staging area becomes the partial results' area
+    }
 
     // The groups of a workgroup, written out for each possible count: with the count a run-time value the fetch of
     // group gi + 2 sits behind a condition, the compiler loses count of the loads in flight, and the matrix instructions
@@ -555,54 +595,80 @@ __global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_once_kernel(OnceA
 #pragma unroll
         for (int gi = 0; gi < MINE; ++gi)
         {
-            v4i acc0[RB], acc1[RB];
+            v4i acc0[RB], acc1[RB < 4 ? RB : 1];
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
-                acc0[rb] = (v4i){0, 0, 0, 0}, acc1[rb] = (v4i){0, 0, 0, 0};
+                acc0[rb] = (v4i){0, 0, 0, 0}, acc1[RB < 4 ? rb : 0] = (v4i){0, 0, 0, 0};
             if (busy)
             {
                 // The two chains are added and the sum is held back for 32 issue slots in the same basic block as the
                 // matrix instructions: their results may not be read by another instruction type for about a dozen
                 // slots, and the compiler only pads that distance inside a block - with the first reader behind a taken
                 // branch it came 3 slots after the instruction and read the last register of the result too early.
-#pragma unroll
-                for (int u = 0; u < PER; ++u)
-#pragma unroll
-                    for (int rb = 0; rb < RB; ++rb)
-                        (u & 1 ? acc1[rb] : acc0[rb]) =
-                            __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[gi & 1][u], u & 1 ? acc1[rb] : acc0[rb], 0, 0, 0);
-                if (RB == 1)
+                if constexpr (RB == 4)
                 {
-                    acc0[0] += acc1[0];
-                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]));
+                    // four blocks of rows are four independent chains: one accumulator each. The B blocks of the next
+                    // group are asked for as soon as their registers are free, half by half.
+#pragma unroll
+                    for (int u = 0; u < H0; ++u)
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            acc0[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc0[rb], 0, 0, 0);
+                    if (gi + 1 < MINE)
+                        load_b_part(0, gi + 1, std::integral_constant<int, 0>{}, std::integral_constant<int, H0>{});
+#pragma unroll
+                    for (int u = H0; u < PER; ++u)
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            acc0[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc0[rb], 0, 0, 0);
+                    if (gi + 1 < MINE)
+                        load_b_part(0, gi + 1, std::integral_constant<int, H0>{}, std::integral_constant<int, PER>{});
+                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]));
                 }
                 else
                 {
-                    // (the wait first: the sums below are the first readers of the results)
-                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc1[0]), "+v"(acc0[RB - 1]), "+v"(acc1[RB - 1]));
 #pragma unroll
-                    for (int rb = 0; rb < RB; ++rb)
-                        acc0[rb] += acc1[rb];
+                    for (int u = 0; u < PER; ++u)
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            (u & 1 ? acc1[rb] : acc0[rb]) =
+                                __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[gi & 1][u], u & 1 ? acc1[rb] : acc0[rb], 0, 0, 0);
+                    if (RB == 1)
+                    {
+                        acc0[0] += acc1[0];
+                        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]));
+                    }
+                    else
+                    {
+                        // (the wait first: the sums below are the first readers of the results)
+                        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc1[0]), "+v"(acc0[RB - 1]), "+v"(acc1[RB - 1]));
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            acc0[rb] += acc1[rb];
+                    }
                 }
             }
-            if (gi + 2 < MINE)
+            if (!A_GLOBAL && gi + 2 < MINE)
                 load_b(gi & 1, gi + 2);
             // accumulator r of lane l is row 4 * (l / 16) + r, column l % 16: lanes 32..63 hold rows 8..15
             if (RL == 64 || lane < 32)
             {
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb)
-                    *(v4i *)&red[((((gi & 1) * ONCE_WAVES + wave) * RB + rb) * RL + lane) * 4] = acc0[rb];
+                    *(v4i *)&red[((((gi & 1) * WAVES + wave) * RB + rb) * RL + lane) * 4] = acc0[rb];
             }
             __syncthreads();
-            if (t < ROWS * 16)
+            // one output per thread and pass (with 64 rows the 512 threads make two passes)
+#pragma unroll
+            for (int o = t; o < ROWS * 16; o += WAVES * 64)
             {
                 // output (erow, ecol): block of rows erow / 16, there accumulator erow % 4 of lane (erow % 16 / 4) * 16 + ecol
+                const int      erow = o >> 4, ecol = o & 15;
                 const int      j = ((int)blockIdx.x + gi * G) * 16 + ecol;
-                const int32_t *r = &red[((((gi & 1) * ONCE_WAVES) * RB + (erow >> 4)) * RL + ((erow & 15) >> 2) * 16 + ecol) * 4 + (erow & 3)];
+                const int32_t *r = &red[((((gi & 1) * WAVES) * RB + (erow >> 4)) * RL + ((erow & 15) >> 2) * 16 + ecol) * 4 + (erow & 3)];
                 int32_t        sum = 0;
 #pragma unroll
-                for (int w = 0; w < ONCE_WAVES; ++w)
+                for (int w = 0; w < WAVES; ++w)
                     sum += r[w * RB * RL * 4];
                 const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & (ROWS - 1)];
                 if (j < g.N && erow < g.M)
@@ -706,19 +772,21 @@ int device_cus()
 template <int PER, bool MULTI, int ROWS>
 static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
+    constexpr int WAVES = ROWS == 64 ? 8 : ONCE_WAVES;
     static const void *const fns[3][2] = {
-        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI, ROWS>,
-         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI, ROWS>},
-        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI, ROWS>,
-         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI, ROWS>},
-        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI, ROWS>,
-         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI, ROWS>}};
+        {(const void *)gemm_skinny_once_kernel<EPI_S32, false, PER, MULTI, ROWS, WAVES>,
+         (const void *)gemm_skinny_once_kernel<EPI_S32, true, PER, MULTI, ROWS, WAVES>},
+        {(const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, false, PER, MULTI, ROWS, WAVES>,
+         (const void *)gemm_skinny_once_kernel<EPI_FIXEDPOINT, true, PER, MULTI, ROWS, WAVES>},
+        {(const void *)gemm_skinny_once_kernel<EPI_F32, false, PER, MULTI, ROWS, WAVES>,
+         (const void *)gemm_skinny_once_kernel<EPI_F32, true, PER, MULTI, ROWS, WAVES>}};
     // the kernel fetches these without asking
     if (a.epi.colvec == nullptr || a.epi.rowvec == nullptr || (epi == EPI_FIXEDPOINT && (a.epi.mult == nullptr || a.epi.shift == nullptr)))
         return (int)hipErrorInvalidValue;
     static std::atomic<uint32_t> lds_raised[3][2];
     // staged rows of A; with 32 rows the partial results (2 x 16 waves x 2 blocks x 64 lanes x 16 bytes) share the area
-    const size_t                 lds = std::max((size_t)ONCE_WAVES * ROWS * once_pitch(ROWS, PER), ROWS > 16 ? (size_t)65536 : (size_t)0);
+    const size_t                 lds = ROWS == 64 ? (size_t)65536 // nothing staged: only the partial results (2 x 8 waves x 4 blocks)
+                                                  : std::max((size_t)ONCE_WAVES * ROWS * once_pitch(ROWS, PER), ROWS > 16 ? (size_t)65536 : (size_t)0);
     const void                  *fn  = fns[epi][flip_a ? 1 : 0];
     // 16 KiB of static LDS on top: declare the dynamic part whatever its size
     const int e = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
@@ -729,7 +797,7 @@ static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int gri
                a.N,    (int32_t)(a.Kp / 64), grid, p.result_offset, p.stage, p.lo, p.hi, p.scale, p.act_min, p.act_max,
                p.has_offsets, p.accumulate, p.act_twice};
     void *kargs[] = {&o};
-    return (int)hipLaunchKernel(fn, dim3(grid), dim3(ONCE_WAVES * 64), kargs, lds, s);
+    return (int)hipLaunchKernel(fn, dim3(grid), dim3(WAVES * 64), kargs, lds, s);
 }
 
 template <int PER, bool MULTI>
@@ -775,6 +843,22 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
     // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside
     // the first on a compute unit: one workgroup of 8 waves per group below. Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
+    // 33 to 64 rows: the same with 8 waves, each holding the operand blocks of its 1, 2, 4 or 8 k blocks of all 64 rows
+    if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    {
+        const int cus = device_cus();
+        if (cus > 0 && (groups <= cus || groups >= 2 * cus))
+        {
+            const bool multi = groups >= 2 * cus;
+            const int  grid  = multi ? std::max(cus, (groups + ONCE_MAX_GROUPS - 1) / ONCE_MAX_GROUPS) : groups;
+            const int  per   = KB <= 8 ? 1 : (KB <= 16 ? 2 : (KB <= 32 ? 4 : 8));
+#define MI355_ONCE64(P_)                                                                        \
+    (multi ? skinny_once_launch_r<P_, true, 64>(epi, flip_a, args, grid, s)                     \
+           : skinny_once_launch_r<P_, false, 64>(epi, flip_a, args, grid, s))
+            return per == 1 ? MI355_ONCE64(1) : per == 2 ? MI355_ONCE64(2) : per == 4 ? MI355_ONCE64(4) : MI355_ONCE64(8);
+#undef MI355_ONCE64
+        }
+    }
     if (once_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();

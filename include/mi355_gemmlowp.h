@@ -65,7 +65,8 @@ typedef enum mi355_epilogue
 
 typedef enum mi355_path
 {
-    MI355_PATH_AUTO   = 0, /* MFMA tiled kernel, or the skinny kernel for small M (<= 32, or <= 64 with N < 8192) */
+    MI355_PATH_AUTO   = 0, /* MFMA tiled kernel, or the skinny kernel for small M (<= 32; <= 64 with N < 8192 or with
+                            * K <= 4096 a multiple of 64) */
     MI355_PATH_SIMPLE = 1, /* one thread per output; for cross-checking only */
     MI355_PATH_MFMA   = 2,
     MI355_PATH_SKINNY = 3

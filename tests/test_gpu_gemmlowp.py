@@ -276,7 +276,7 @@ def test_skinny_kernel_with_staged_a(M):
         np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16, 17, 25, 32])
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16, 17, 25, 32, 33, 50, 64])
 def test_skinny_stage_once_kernel(M):
     """Up to 32 rows (three builds: up to 8, where half of the matrix instruction's rows are padding, 9 to 16, and 17 to
     32 as two blocks of rows) and K <= 4096 (whole 64-byte blocks, 16-byte aligned rows): one workgroup of 16 waves per

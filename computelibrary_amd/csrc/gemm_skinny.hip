@@ -528,11 +528,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
         for (int u = decltype(u0c)::value; u < decltype(u1c)::value; ++u) // k blocks past KB (last busy wave) re-read the last one
             fb[slot][u] = __builtin_nontemporal_load((const MI355_GLOBAL v4i *)(bp + ((int64_t)grp * KB + max(min(u, KB - 1 - kb0), 0)) * 1024));
     };
-    auto load_b = [&](int slot, int gi) { load_b_part(slot, gi, std::integral_constant<int, 0>{}, std::integral_constant<int, PER>{}); };
+    auto load_b = [&](int slot, int gi)
+    {
+        const int grp = min((int)blockIdx.x + gi * G, NGT - 1);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            fb[slot][u] = __builtin_nontemporal_load((const MI355_GLOBAL v4i *)(bp + ((int64_t)grp * KB + max(min(u, KB - 1 - kb0), 0)) * 1024));
+    };
     // MULTI: every workgroup has at least two groups. Nothing between here and the wait for A may sit behind a branch:
     // the compiler would no longer know how many loads are in flight and would make the wait for A wait for B as well
     // (loads return in order) - hence also the unconditional fetches of the epilogue constants below.
     load_b(0, 0);
+    __builtin_amdgcn_sched_barrier(0); // group 0 goes out whole before group 1: the first wait then covers group 0 only
     if (MULTI && !A_GLOBAL)
         load_b(1, 1);
     // (with nothing to stage, A is fetched behind the first B blocks: the first matrix instruction needs both anyway,

@@ -177,6 +177,9 @@ class Gemm:
     def set_strides_3d(self, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride, a_plane_stride, d_plane_stride):
         _check(lib().mi355_gemmlowp_set_strides_3d(self._h, lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride,
                                                    a_plane_stride, d_plane_stride))
+        d = self.desc
+        d.lda, d.ldb, d.ldd, d.a_batch_stride, d.b_batch_stride, d.d_batch_stride = lda, ldb, ldd, a_batch_stride, b_batch_stride, d_batch_stride
+        d.a_plane_stride, d.d_plane_stride = a_plane_stride, d_plane_stride
 
     def update_quant(self, a_offset, b_offset, rq, scale=1.0, stream=None):
         _check(lib().mi355_gemmlowp_update_quant(self._h, a_offset, b_offset, C.byref(rq) if rq else None, scale,
@@ -190,6 +193,7 @@ class Gemm:
             else b_batch_stride
         _check(lib().mi355_gemmlowp_set_strides(self._h, lda, ldb, ldd, a_bs, b_bs, d_bs))
         d.lda, d.ldb, d.ldd, d.a_batch_stride, d.b_batch_stride, d.d_batch_stride = lda, ldb, ldd, a_bs, b_bs, d_bs
+        d.a_plane_stride, d.d_plane_stride = d.a_plane_rows * lda, d.d_plane_rows * ldd  # the library closes the gaps
 
     def run(self, A, D, bias_f32=None, stream=None):
         _check(lib().mi355_gemmlowp_run(self._h, ptr(A), ptr(bias_f32), ptr(D), stream))

@@ -101,3 +101,39 @@ def test_set_strides_checks_what_create_checks():
     with pytest.raises(capi.Mi355Error, match="stride is smaller"):
         c.set_strides(8, 16, 8)
     c.close()
+
+
+def test_strides_of_outer_dimensions_are_checked_without_a_gpu():
+    """Strides of dimensions 2 and 3 of convolution tensors and the plane strides of 3D-reinterpreted GEMM matrices: every
+    stride has to step over what lies below it, at create and when set later; 0 stands for 'no gap'."""
+    import pytest
+    # NHWC 1x6x5x16 -> 8 channels, 3x3 pad 1: src rows of 5 pixels x 20 bytes = 100, images of 6 rows
+    ok = capi.conv_desc(1, 6, 5, 16, 8, 3, 3, pad=(1, 1, 1, 1), pixel_strides=(20, 0, 0), outer_strides=((120, 900), (0, 0), (0, 0)))
+    capi.Conv(ok).close()
+    for bad in (((99, 0), (0, 0), (0, 0)),       # src row stride below 5 pixels x 20 bytes
+                ((120, 700), (0, 0), (0, 0)),    # src image stride below 6 rows x 120 bytes
+                ((0, 0), (40, 0), (0, 0)),       # weights: a row of 3 taps x 16 bytes needs 48
+                ((0, 0), (0, 0), (39, 0))):      # dst: a row of 5 pixels x 8 bytes needs 40
+        with pytest.raises(capi.Mi355Error, match="stride is smaller"):
+            capi.Conv(capi.conv_desc(1, 6, 5, 16, 8, 3, 3, pad=(1, 1, 1, 1), pixel_strides=(20, 0, 0), outer_strides=bad))
+    c = capi.Conv(capi.conv_desc(2, 6, 5, 16, 8, 3, 3, pad=(1, 1, 1, 1), layout=capi.NCHW))
+    c.set_strides_nd((7, 50, 900), (0, 0, 0), (5, 30, 0))   # NCHW: rows of 5 (+2), planes of 6 rows (+8 bytes), images of 16 planes
+    with pytest.raises(capi.Mi355Error, match="stride is smaller"):
+        c.set_strides_nd((4, 0, 0), (0, 0, 0), (0, 0, 0))
+    with pytest.raises(capi.Mi355Error, match="stride is smaller"):
+        c.set_strides_nd((7, 41, 0), (0, 0, 0), (0, 0, 0))
+    c.close()
+    # GEMM: 12 rows as 3 planes of 4 rows
+    g = capi.Gemm(12, 8, 16, capi.S8, capi.S8, capi.S32, capi.EPI_S32, batch=2, lda=20, ldd=8, a_planes=(4, 100), d_planes=(4, 40),
+                  a_batch_stride=300, d_batch_stride=120)
+    g.set_strides_3d(24, 8, 9, 400, 0, 200, 120, 50)
+    assert (g.desc.a_plane_stride, g.desc.d_plane_stride) == (120, 50)
+    g.set_strides(20, 8, 8, a_batch_stride=240, d_batch_stride=96)  # planes without a gap again
+    assert (g.desc.a_plane_stride, g.desc.d_plane_stride) == (80, 32)
+    with pytest.raises(capi.Mi355Error, match="plane stride"):
+        g.set_strides_3d(24, 8, 9, 400, 0, 200, 80, 50)     # 3 rows x 24 + 16 bytes do not fit 80
+    with pytest.raises(capi.Mi355Error, match="batch stride"):
+        g.set_strides_3d(24, 8, 9, 300, 0, 200, 120, 50)    # 2 planes x 120 + 3 x 24 + 16 > 300
+    g.close()
+    with pytest.raises(capi.Mi355Error, match="plane_rows"):
+        capi.Gemm(12, 8, 16, capi.S8, capi.S8, capi.S32, capi.EPI_S32, a_planes=(5, 100), a_batch_stride=400)

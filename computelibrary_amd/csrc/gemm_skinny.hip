@@ -417,6 +417,34 @@ struct OnceArgs
     float          scale, act_min, act_max;
     int32_t        has_offsets, accumulate, act_twice;
 };
+// One output of the stage-once kernels: the reduced sum, its column term c, multiplier (or float bias bits) m, shift sh
+// and row term rv through epilogue EPI into element idx of D
+#define MI355_GLOBAL __attribute__((address_space(1)))
+template <int EPI>
+__device__ __forceinline__ void once_store_output(MI355_GLOBAL char *gD, int64_t idx, int32_t sum, int32_t c, int32_t m, int32_t sh,
+                                                  int32_t rv, bool has_bias, const EpiParams &p)
+{
+    if (EPI == EPI_S32)
+        ((MI355_GLOBAL int32_t *)gD)[idx] =
+            (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv + (p.accumulate ? (uint32_t)((MI355_GLOBAL int32_t *)gD)[idx] : 0u));
+    else if (EPI == EPI_FIXEDPOINT)
+    {
+        const int32_t v = (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv);
+        int32_t       q;
+        if (p.stage == 0 && m >= 0 && sh > -32 && sh < 32)
+            // the branch-free form of the same arithmetic (see fast_requant), its constants derived here
+            q = fast_requant(v, (int32_t)((uint32_t)m << 1), (uint32_t)m >= 0x40000000u ? -1 : 0, sh < 0 ? -sh : 0, sh > 1 ? sh - 1 : 0,
+                             sh > 0 ? 1 : 0, p.result_offset, p.lo, p.hi);
+        else
+            q = epi_fixedpoint(sum, c, rv, m, sh, p);
+        ((MI355_GLOBAL int8_t *)gD)[idx] = (int8_t)q;
+    }
+    else
+        ((MI355_GLOBAL float *)gD)[idx] = epi_f32(sum, (int32_t)((uint32_t)c + (uint32_t)rv), __int_as_float(m), has_bias, p,
+                                                  p.accumulate ? ((MI355_GLOBAL float *)gD)[idx] : 0.f);
+}
+#undef MI355_GLOBAL
+
 // bytes from one staged row of A to the next: 8 / 16 rows keep the pitch they were tuned with; 32 rows take the smallest
 // pitch that still spreads the rows over the banks (an odd number of 16-byte pieces), or the slices would not fit
 __host__ __device__ constexpr int once_pitch(int rows, int per)
@@ -679,27 +707,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
                     sum += r[w * RB * RL * 4];
                 const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & (ROWS - 1)];
                 if (j < g.N && erow < g.M)
-                {
-                    const int64_t idx = (int64_t)erow * g.ldd + j;
-                    if (EPI == EPI_S32)
-                        ((MI355_GLOBAL int32_t *)gD)[idx] = (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv +
-                                                                      (p.accumulate ? (uint32_t)((MI355_GLOBAL int32_t *)gD)[idx] : 0u));
-                    else if (EPI == EPI_FIXEDPOINT)
-                    {
-                        const int32_t v = (int32_t)((uint32_t)sum + (uint32_t)c + (uint32_t)rv);
-                        int32_t       q;
-                        if (p.stage == 0 && m >= 0 && sh > -32 && sh < 32)
-                            // the branch-free form of the same arithmetic (see fast_requant), its constants derived here
-                            q = fast_requant(v, (int32_t)((uint32_t)m << 1), (uint32_t)m >= 0x40000000u ? -1 : 0, sh < 0 ? -sh : 0,
-                                             sh > 1 ? sh - 1 : 0, sh > 0 ? 1 : 0, p.result_offset, p.lo, p.hi);
-                        else
-                            q = epi_fixedpoint(sum, c, rv, m, sh, p);
-                        ((MI355_GLOBAL int8_t *)gD)[idx] = (int8_t)q;
-                    }
-                    else
-                        ((MI355_GLOBAL float *)gD)[idx] = epi_f32(sum, (int32_t)((uint32_t)c + (uint32_t)rv), __int_as_float(m), has_bias,
-                                                                  p, p.accumulate ? ((MI355_GLOBAL float *)gD)[idx] : 0.f);
-                }
+                    once_store_output<EPI>(gD, (int64_t)erow * g.ldd + j, sum, c, m, sh, rv, has_bias, p);
             }
         }
     };
@@ -714,6 +722,167 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
 }
 static_assert(ONCE_MAX_GROUPS == 4, "the group loop is written out for 1 to 4 groups");
 
+#undef MI355_GLOBAL
+
+// ---- the stage-once form for deep K: up to 8 rows, 4096 < K <= 16384 -------------------------------------------------
+// (the down projection of a transformer's feed-forward block is this shape: few rows, K = 11008 / 14336)
+// The same plan - one workgroup of 16 waves per compute unit, every wave stages its K slice of A once and walks the
+// column groups - but a wave's slice is NCH chunks of 4 k blocks now, and registers for all of it would leave none for
+// B in flight: the operand blocks of A are read from LDS again for every chunk (16 KiB of LDS reads per group and
+// workgroup, nothing beside the stream), and B moves in units of one chunk, two units in flight per wave.
+#define MI355_GLOBAL __attribute__((address_space(1)))
+template <int EPI, bool FLIP_A, int NCH, bool MULTI>
+__global__ __launch_bounds__(ONCE_WAVES * 64) void gemm_skinny_deepk_kernel(OnceArgs g)
+{
+    constexpr int CH = 4, PER = CH * NCH;       // k blocks per chunk / per wave
+    constexpr int PPR = PER * 4;                // 16-byte pieces per staged row
+    constexpr int PITCH = PER * 64 + 16;        // an odd number of pieces: the 8 rows of an operand read spread over the banks
+    constexpr int NA = 8 * PPR / 64;            // staging loads per lane (8 rows)
+    __shared__ __attribute__((aligned(16))) int32_t red[2][ONCE_WAVES][32][4];
+    __shared__ int32_t                              par[4][64];
+    extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [ONCE_WAVES][8][PITCH]
+
+    uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_d = (uintptr_t)g.D, u_cv = (uintptr_t)g.colvec, u_rv = (uintptr_t)g.rowvec,
+              u_mu = (uintptr_t)g.mult, u_sh = (uintptr_t)g.shift, u_bf = (uintptr_t)g.bias_f32;
+    asm volatile(""
+                 : "+s"(g.result_offset), "+s"(g.stage), "+s"(g.lo), "+s"(g.hi), "+s"(g.scale), "+s"(g.act_min), "+s"(g.act_max),
+                   "+s"(g.has_offsets), "+s"(g.accumulate), "+s"(g.act_twice), "+s"(g.lda), "+s"(g.ldd), "+s"(g.M), "+s"(g.N),
+                   "+s"(g.KB), "+s"(g.grid), "+s"(u_a), "+s"(u_b), "+s"(u_d), "+s"(u_cv), "+s"(u_rv), "+s"(u_mu), "+s"(u_sh),
+                   "+s"(u_bf));
+    const MI355_GLOBAL int8_t *const  gA = (const MI355_GLOBAL int8_t *)u_a, *const gB = (const MI355_GLOBAL int8_t *)u_b;
+    MI355_GLOBAL char *const          gD = (MI355_GLOBAL char *)u_d;
+    const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_rowvec = (const MI355_GLOBAL int32_t *)u_rv,
+                                     *const g_mult = (const MI355_GLOBAL int32_t *)u_mu, *const g_shift = (const MI355_GLOBAL int32_t *)u_sh,
+                                     *const g_bias = (const MI355_GLOBAL int32_t *)u_bf;
+    const bool has_bias = u_bf != 0;
+    EpiParams  p{};
+    p.result_offset = g.result_offset, p.stage = g.stage, p.lo = g.lo, p.hi = g.hi;
+    p.scale = g.scale, p.act_min = g.act_min, p.act_max = g.act_max;
+    p.has_offsets = g.has_offsets, p.accumulate = g.accumulate, p.act_twice = g.act_twice;
+
+    const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int KB = g.KB, NGT = (g.N + 15) / 16, G = g.grid;
+    const int mine = (NGT - (int)blockIdx.x + G - 1) / G; // column groups of this workgroup, 1..ONCE_MAX_GROUPS
+    const int kb0  = wave * PER;
+    const int nb   = min(max(KB - kb0, 0), PER); // k blocks of this wave (the last busy wave may be short, later ones have none)
+
+    // epilogue constants: as in the stage-once kernel (one dword per lane, vector wave % 4, no conditions)
+    int32_t par_v;
+    {
+        const int                   v   = wave & 3;
+        const int                   j   = min(((int)blockIdx.x + (lane >> 4) * G) * 16 + (lane & 15), g.N - 1);
+        const MI355_GLOBAL int32_t *vec = v == 0   ? g_colvec
+                                          : v == 1 ? (EPI == EPI_FIXEDPOINT ? g_mult : (EPI == EPI_F32 && has_bias ? g_bias : g_colvec))
+                                          : v == 2 ? (EPI == EPI_FIXEDPOINT ? g_shift : g_colvec)
+                                                   : g_rowvec;
+        par_v                           = vec[v == 3 ? min(lane & 7, g.M - 1) : j];
+    }
+    // this wave's slice of A, piece by piece: piece q of the slice is row q / PPR, 16-byte column q % PPR. Rows past M
+    // re-read row M-1, columns past the wave's k blocks its first column (neither is ever used)
+    char     *a_lds = a_stage + wave * 8 * PITCH;
+    v4i       ta[NA];
+    const int kbase = min(kb0, KB - 1) * 64;
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+    {
+        const int q = i * 64 + lane, row = q / PPR, pc = q - row * PPR;
+        ta[i]       = *(const MI355_GLOBAL v4i *)(gA + (int64_t)min(row, g.M - 1) * g.lda + kbase + (pc < nb * 4 ? pc * 16 : 0));
+    }
+    // B in units of one chunk of one group: unit c of group gi
+    const MI355_GLOBAL int8_t *bp = gB + ((int64_t)min(kb0, KB - 1) * 64 + lane) * 16;
+    v4i                        fb[2][CH];
+    auto load_unit = [&](int slot, int gi, int c)
+    {
+        const int grp = min((int)blockIdx.x + gi * G, NGT - 1);
+        // (addresses are formed here, unit by unit: hoisted above the dispatch on the number of groups - they are all
+        // invariant - the sixteen of them overflow the registers)
+        uintptr_t b = (uintptr_t)bp;
+        asm volatile("" : "+v"(b));
+#pragma unroll
+        for (int u = 0; u < CH; ++u) // k blocks past the wave's last re-read it
+            fb[slot][u] = __builtin_nontemporal_load(
+                (const MI355_GLOBAL v4i *)((const MI355_GLOBAL int8_t *)b + ((int64_t)grp * KB + max(min(c * CH + u, KB - 1 - kb0), 0)) * 1024));
+    };
+    load_unit(0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_unit(1, 0, 1); // NCH >= 2
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+    {
+        if (FLIP_A)
+            ta[i] ^= (int)0x80808080;
+        const int q = i * 64 + lane, row = q / PPR, pc = q - row * PPR;
+        *(v4i *)(a_lds + row * PITCH + pc * 16) = ta[i];
+    }
+    par[wave & 3][lane] = par_v; // read behind the first group's barrier
+    // operand blocks of A: lane -> row lane % 16 (rows 8..15 are zero), 16 bytes at k offset (lane / 16) * 16
+    const int  arow = lane & 15, akc = (lane >> 4) * 16;
+    const char *a_rd = a_lds + (arow & 7) * PITCH + akc;
+    auto read_a = [&](v4i (&fa)[CH], int c)
+    {
+#pragma unroll
+        for (int u = 0; u < CH; ++u)
+        {
+            fa[u] = *(const v4i *)(a_rd + (c * CH + u) * 64);
+            if (!(arow < 8 && c * CH + u < nb))
+                fa[u] = (v4i){0, 0, 0, 0};
+        }
+    };
+
+    const int erow = t >> 4, ecol = t & 15;
+    auto groups = [&](auto count)
+    {
+        constexpr int MINE = decltype(count)::value;
+        v4i fa[2][CH];
+        read_a(fa[0], 0);
+#pragma unroll
+        for (int gi = 0; gi < MINE; ++gi)
+        {
+            v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+            {
+                const int q = gi * NCH + c; // unit in flight order: slot q % 2
+                // the operand blocks of A for the next unit, while this unit's B blocks are awaited (read again for every
+                // group: without the clobber the compiler keeps all of a wave's blocks in registers, and spills)
+                asm volatile("" ::: "memory");
+                read_a(fa[(q + 1) & 1], (c + 1) % NCH);
+#pragma unroll
+                for (int u = 0; u < CH; ++u)
+                    (u & 1 ? acc1 : acc0) = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[q & 1][u], fb[q & 1][u], u & 1 ? acc1 : acc0, 0, 0, 0);
+                if (q + 2 < MINE * NCH)
+                    load_unit(q & 1, (q + 2) / NCH, (q + 2) % NCH);
+                __builtin_amdgcn_sched_barrier(0); // units stay apart: moved together, their operands overflow the registers
+            }
+            // (the sum is held back in the block of the matrix instructions: see the stage-once kernel)
+            acc0 += acc1;
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0));
+            if (lane < 32)
+                *(v4i *)&red[gi & 1][wave][lane][0] = acc0;
+            __syncthreads();
+            if (t < 128)
+            {
+                const int      j = ((int)blockIdx.x + gi * G) * 16 + ecol;
+                const int32_t *r = &red[gi & 1][0][(erow >> 2) * 16 + ecol][erow & 3];
+                int32_t        sum = 0;
+#pragma unroll
+                for (int w = 0; w < ONCE_WAVES; ++w)
+                    sum += r[w * 32 * 4];
+                const int32_t c = par[0][gi * 16 + ecol], m = par[1][gi * 16 + ecol], sh = par[2][gi * 16 + ecol], rv = par[3][erow & 7];
+                if (j < g.N && erow < g.M)
+                    once_store_output<EPI>(gD, (int64_t)erow * g.ldd + j, sum, c, m, sh, rv, has_bias, p);
+            }
+        }
+    };
+    if (!MULTI || mine == 1)
+        groups(std::integral_constant<int, 1>{});
+    else if (mine == 2)
+        groups(std::integral_constant<int, 2>{});
+    else if (mine == 3)
+        groups(std::integral_constant<int, 3>{});
+    else
+        groups(std::integral_constant<int, 4>{});
+}
 #undef MI355_GLOBAL
 
 // A kernel that needs more than 48 KiB of dynamic LDS has to be told so once per device
@@ -807,6 +976,34 @@ static int skinny_once_launch_r(int epi, bool flip_a, const GemmArgs &a, int gri
     return (int)hipLaunchKernel(fn, dim3(grid), dim3(WAVES * 64), kargs, lds, s);
 }
 
+// (built for one column group per workgroup only: with the group loop written out for 2 to 4 groups as well, the
+// compiler's register allocation spills the B blocks as they arrive)
+template <int NCH>
+static int skinny_deepk_launch(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
+{
+    constexpr bool MULTI = false;
+    static const void *const fns[3][2] = {
+        {(const void *)gemm_skinny_deepk_kernel<EPI_S32, false, NCH, MULTI>, (const void *)gemm_skinny_deepk_kernel<EPI_S32, true, NCH, MULTI>},
+        {(const void *)gemm_skinny_deepk_kernel<EPI_FIXEDPOINT, false, NCH, MULTI>,
+         (const void *)gemm_skinny_deepk_kernel<EPI_FIXEDPOINT, true, NCH, MULTI>},
+        {(const void *)gemm_skinny_deepk_kernel<EPI_F32, false, NCH, MULTI>, (const void *)gemm_skinny_deepk_kernel<EPI_F32, true, NCH, MULTI>}};
+    // the kernel fetches these without asking
+    if (a.epi.colvec == nullptr || a.epi.rowvec == nullptr || (epi == EPI_FIXEDPOINT && (a.epi.mult == nullptr || a.epi.shift == nullptr)))
+        return (int)hipErrorInvalidValue;
+    static std::atomic<uint32_t> lds_raised[3][2];
+    const size_t                 lds = (size_t)ONCE_WAVES * 8 * (NCH * 4 * 64 + 16);
+    const void                  *fn  = fns[epi][flip_a ? 1 : 0];
+    const int                    e   = raise_lds_limit(fn, lds, lds_raised[epi][flip_a ? 1 : 0]);
+    if (e)
+        return e;
+    const EpiParams &p = a.epi;
+    OnceArgs         o{a.A,    a.Bp,   a.D,    p.colvec, p.rowvec,  p.mult,    p.shift,       p.bias_f32,   a.lda,       a.ldd,        a.M,
+               a.N,    (int32_t)(a.Kp / 64), grid, p.result_offset, p.stage, p.lo, p.hi, p.scale, p.act_min, p.act_max,
+               p.has_offsets, p.accumulate, p.act_twice};
+    void *kargs[] = {&o};
+    return (int)hipLaunchKernel(fn, dim3(grid), dim3(ONCE_WAVES * 64), kargs, lds, s);
+}
+
 template <int PER, bool MULTI>
 static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
@@ -850,6 +1047,18 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
     // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside
     // the first on a compute unit: one workgroup of 8 waves per group below. Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
+    // up to 8 rows and 4096 < K <= 16384: the stage-once form for deep K (2, 3 or 4 chunks of 4 k blocks per wave)
+    if (stage_ok && KB > 4 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    {
+        const int cus = device_cus();
+        if (cus > 0 && groups <= cus) // one column group per workgroup
+        {
+            const int nch = (KB + 4 * ONCE_WAVES - 1) / (4 * ONCE_WAVES);
+            return nch == 2   ? skinny_deepk_launch<2>(epi, flip_a, args, groups, s)
+                   : nch == 3 ? skinny_deepk_launch<3>(epi, flip_a, args, groups, s)
+                              : skinny_deepk_launch<4>(epi, flip_a, args, groups, s);
+        }
+    }
     // 33 to 64 rows: the same with 8 waves, each holding the operand blocks of its 1, 2, 4 or 8 k blocks of all 64 rows
     if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {

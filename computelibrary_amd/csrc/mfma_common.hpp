@@ -411,35 +411,85 @@ __device__ __forceinline__ void epilogue_store_wave32(const v4i (&acc)[RS][QS], 
     const int32_t   *rowvec = p.rowvec ? p.rowvec + (int64_t)bz * p.rowvec_batch_stride : nullptr;
     char            *D      = (char *)g.D + (int64_t)bz * g.d_batch_stride * 4;
     const int        rr = lane / LPR, cc = lane % LPR;
+    // Everything the loop below needs from global memory is fetched before its first store goes out: a wait for a load
+    // issued after a store also waits for that store to reach memory, and one such wait per block of 16 x 16 outputs
+    // made the epilogue as slow as its slowest store, sixteen times over.
+    v4i     cvq[QS];
+    float   bfq[QS][4];
+    int32_t rvs[RS];
+    const bool has_bias = EPI == EPI_F32 && p.bias_f32 != nullptr;
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs)
+    {
+        const int j0 = col0 + qs * 16 + 4 * lh; // inside the padded vectors
+        cvq[qs]      = *(const v4i *)(colvec + j0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            bfq[qs][t] = (has_bias && j0 + t < g.N) ? p.bias_f32[j0 + t] : 0.f;
+    }
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs)
     {
-        const int     i  = row0 + rs * 16 + lr;
-        const int32_t rv = (rowvec && i < g.M) ? rowvec[i] : 0;
+        const int i = row0 + rs * 16 + lr;
+        rvs[rs]     = (rowvec && i < g.M) ? rowvec[i] : 0;
+    }
+    // The common F32 case (no bias, zero offsets) and tiles that lie inside the matrix get straight-line code: the general
+    // form spends about 25 vector instructions per output on conditions that are the same for the whole launch, and with
+    // two consumer waves per SIMD that, not the stores, set the length of the epilogue.
+    const bool plain    = EPI == EPI_F32 && !has_bias && !p.has_offsets;
+    const bool interior = __builtin_amdgcn_readfirstlane(row0) + RS * 16 <= g.M && __builtin_amdgcn_readfirstlane(col0) + QS * 16 <= g.N;
+    char         *dp    = D + ((int64_t)(row0 + rr) * g.ldd + col0 + cc * 4) * 4; // this lane's segment of the first row
+    const int64_t step  = (int64_t)RPI * g.ldd * 4;
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs)
+    for (int rs = 0; rs < RS; ++rs)
+    {
+        const int32_t rv = rvs[rs];
+        if (plain)
         {
-            const int c  = qs * 16 + 4 * lh;
-            const int j0 = col0 + c; // inside the padded vectors
-            const v4i cv = *(const v4i *)(colvec + j0);
-            v4i       o;
-            if (EPI == EPI_S32)
+#pragma clang fp contract(off)
+#pragma unroll
+            for (int qs = 0; qs < QS; ++qs)
             {
+                v4i o;
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv);
+                    o[t] = __float_as_int(fminf(fmaxf((float)acc[rs][qs][t] * p.scale, p.act_min), p.act_max));
+                *(v4i *)(stage + lr * PITCH + (qs * 16 + 4 * lh) * 4) = o;
             }
-            else
-            {
+        }
+        else
+        {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+            for (int qs = 0; qs < QS; ++qs)
+            {
+                const int c  = qs * 16 + 4 * lh;
+                const v4i cv = cvq[qs];
+                v4i       o;
+                if (EPI == EPI_S32)
                 {
-                    const float bf = (p.bias_f32 && j0 + t < g.N) ? p.bias_f32[j0 + t] : 0.f;
-                    o[t] = __float_as_int(epi_f32(acc[rs][qs][t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bf,
-                                                  p.bias_f32 != nullptr, p));
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv);
                 }
+                else
+                {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        o[t] = __float_as_int(epi_f32(acc[rs][qs][t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bfq[qs][t], has_bias, p));
+                }
+                *(v4i *)(stage + lr * PITCH + c * 4) = o;
             }
-            *(v4i *)(stage + lr * PITCH + c * 4) = o;
+        }
+        if (interior)
+        {
+#pragma unroll
+            for (int it = 0; it < 16 / RPI; ++it)
+            {
+                const v4i val = *(const v4i *)(stage + (it * RPI + rr) * PITCH + cc * 16);
+                __builtin_nontemporal_store(val, (v4i *)dp);
+                dp += step;
+            }
+            continue;
         }
 #pragma unroll
         for (int it = 0; it < 16 / RPI; ++it)

@@ -186,4 +186,22 @@ __device__ __forceinline__ float epi_f32(int32_t acc, int32_t off, float bias, b
     }
     return fminf(fmaxf(r, p.act_min), p.act_max);
 }
+// epi_f32 without accumulation, with the launch-wide conditions as template arguments: a tile's epilogue picks one of the
+// instances once instead of testing the flags for every output.
+template <bool BIAS, bool OFFS, bool TWICE>
+__device__ __forceinline__ float epi_f32_static(int32_t acc, int32_t off, float bias, float scale, float lo, float hi)
+{
+#pragma clang fp contract(off)
+    float r = (float)acc * scale;
+    if (BIAS)
+        r = r + bias;
+    if (OFFS)
+    {
+        if (TWICE)
+            r = fminf(fmaxf(r, lo), hi);
+        const float scaled = (float)off * scale;
+        r                  = r + scaled;
+    }
+    return fminf(fmaxf(r, lo), hi);
+}
 } // namespace mi355

@@ -1,5 +1,6 @@
 // Pieces shared by the matrix-core GEMM kernels: LDS swizzle, tile -> workgroup mapping, accumulator epilogue.
 #pragma once
+#include <type_traits>
 #include "internal.hpp"
 
 namespace mi355
@@ -433,81 +434,94 @@ __device__ __forceinline__ void epilogue_store_wave32(const v4i (&acc)[RS][QS], 
         const int i = row0 + rs * 16 + lr;
         rvs[rs]     = (rowvec && i < g.M) ? rowvec[i] : 0;
     }
-    // The common F32 case (no bias, zero offsets) and tiles that lie inside the matrix get straight-line code: the general
-    // form spends about 25 vector instructions per output on conditions that are the same for the whole launch, and with
-    // two consumer waves per SIMD that, not the stores, set the length of the epilogue.
-    const bool plain    = EPI == EPI_F32 && !has_bias && !p.has_offsets;
+    // The conditions that are the same for the whole launch (bias, offsets, second clamp) and for the whole tile (inside
+    // the matrix or on its edge) are decided once, here, and the loop over the outputs is instantiated for each answer:
+    // tested per output they cost about 25 vector instructions each, and with two consumer waves per SIMD that, not the
+    // stores, set the length of the epilogue. Inside the matrix a store is a running row pointer and nothing else.
     const bool interior = __builtin_amdgcn_readfirstlane(row0) + RS * 16 <= g.M && __builtin_amdgcn_readfirstlane(col0) + QS * 16 <= g.N;
-    char         *dp    = D + ((int64_t)(row0 + rr) * g.ldd + col0 + cc * 4) * 4; // this lane's segment of the first row
-    const int64_t step  = (int64_t)RPI * g.ldd * 4;
-#pragma unroll
-    for (int rs = 0; rs < RS; ++rs)
+    auto tile = [&](auto bias_c, auto offs_c, auto twice_c, auto inside_c)
     {
-        const int32_t rv = rvs[rs];
-        if (plain)
+        constexpr bool BIAS = decltype(bias_c)::value, OFFS = decltype(offs_c)::value, TWICE = decltype(twice_c)::value;
+        constexpr bool INSIDE = decltype(inside_c)::value;
+        char         *dp   = D + ((int64_t)(row0 + rr) * g.ldd + col0 + cc * 4) * 4; // this lane's segment of the first row
+        const int64_t step = (int64_t)RPI * g.ldd * 4;
+        const float   scale = p.scale, lo = p.act_min, hi = p.act_max;
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
         {
-#pragma clang fp contract(off)
+            const int32_t rv = rvs[rs];
 #pragma unroll
             for (int qs = 0; qs < QS; ++qs)
             {
-                v4i o;
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    o[t] = __float_as_int(fminf(fmaxf((float)acc[rs][qs][t] * p.scale, p.act_min), p.act_max));
-                *(v4i *)(stage + lr * PITCH + (qs * 16 + 4 * lh) * 4) = o;
-            }
-        }
-        else
-        {
-#pragma unroll
-            for (int qs = 0; qs < QS; ++qs)
-            {
-                const int c  = qs * 16 + 4 * lh;
                 const v4i cv = cvq[qs];
                 v4i       o;
-                if (EPI == EPI_S32)
-                {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)cv[t] + (uint32_t)rv);
-                }
-                else
+                for (int t = 0; t < 4; ++t)
                 {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = __float_as_int(epi_f32(acc[rs][qs][t], (int32_t)((uint32_t)cv[t] + (uint32_t)rv), bfq[qs][t], has_bias, p));
+                    const int32_t off = (int32_t)((uint32_t)cv[t] + (uint32_t)rv);
+                    if (EPI == EPI_S32)
+                        o[t] = (int32_t)((uint32_t)acc[rs][qs][t] + (uint32_t)off);
+                    else
+                        o[t] = __float_as_int(epi_f32_static<BIAS, OFFS, TWICE>(acc[rs][qs][t], off, bfq[qs][t], scale, lo, hi));
                 }
-                *(v4i *)(stage + lr * PITCH + c * 4) = o;
+                *(v4i *)(stage + lr * PITCH + (qs * 16 + 4 * lh) * 4) = o;
             }
-        }
-        if (interior)
-        {
 #pragma unroll
             for (int it = 0; it < 16 / RPI; ++it)
             {
-                const v4i val = *(const v4i *)(stage + (it * RPI + rr) * PITCH + cc * 16);
-                __builtin_nontemporal_store(val, (v4i *)dp);
-                dp += step;
-            }
-            continue;
-        }
-#pragma unroll
-        for (int it = 0; it < 16 / RPI; ++it)
-        {
-            const int r  = it * RPI + rr;
-            const int gi = row0 + rs * 16 + r, j0 = col0 + cc * 4;
-            if (gi >= g.M || j0 >= g.N)
-                continue;
-            const v4i     val = *(const v4i *)(stage + r * PITCH + cc * 16);
-            const int64_t idx = ((int64_t)gi * g.ldd + j0) * 4;
-            if (j0 + 3 < g.N)
-                __builtin_nontemporal_store(val, (v4i *)(D + idx));
-            else
-            {
-                for (int t = 0; t < g.N - j0; ++t)
-                    *(int32_t *)(D + idx + 4 * t) = val[t];
+                const int r   = it * RPI + rr;
+                const v4i val = *(const v4i *)(stage + r * PITCH + cc * 16);
+                if (INSIDE)
+                {
+                    __builtin_nontemporal_store(val, (v4i *)dp);
+                    dp += step;
+                    continue;
+                }
+                const int gi = row0 + rs * 16 + r, j0 = col0 + cc * 4;
+                if (gi >= g.M || j0 >= g.N)
+                    continue;
+                const int64_t idx = ((int64_t)gi * g.ldd + j0) * 4;
+                if (j0 + 3 < g.N)
+                    __builtin_nontemporal_store(val, (v4i *)(D + idx));
+                else
+                {
+                    for (int t = 0; t < g.N - j0; ++t)
+                        *(int32_t *)(D + idx + 4 * t) = val[t];
+                }
             }
         }
+    };
+    using yes = std::true_type;
+    using no  = std::false_type;
+    auto edge_or_not = [&](auto bias_c, auto offs_c, auto twice_c)
+    {
+        if (interior)
+            tile(bias_c, offs_c, twice_c, yes{});
+        else
+            tile(bias_c, offs_c, twice_c, no{});
+    };
+    if (EPI == EPI_S32)
+        edge_or_not(no{}, no{}, no{});
+    else if (!p.has_offsets)
+    {
+        if (has_bias)
+            edge_or_not(yes{}, no{}, no{});
+        else
+            edge_or_not(no{}, no{}, no{});
+    }
+    else if (p.act_twice)
+    {
+        if (has_bias)
+            edge_or_not(yes{}, yes{}, yes{});
+        else
+            edge_or_not(no{}, yes{}, yes{});
+    }
+    else
+    {
+        if (has_bias)
+            edge_or_not(yes{}, yes{}, no{});
+        else
+            edge_or_not(no{}, yes{}, no{});
     }
 }
 } // namespace mi355

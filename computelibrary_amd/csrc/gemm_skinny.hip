@@ -1031,6 +1031,20 @@ struct SkinnyEnv
     }
 };
 
+// Workgroups of the stage-once kernels for `groups` column groups on `cus` compute units: one per group while they all
+// fit at once; from two groups per unit on, the smallest whole number of workgroups per compute unit that keeps every
+// workgroup within ONCE_MAX_GROUPS groups (a grid just above the number of units would leave most of them idle behind
+// the first round); in between, half as many workgroups as groups, so that every workgroup still has two (one of them
+// three when the count is odd) and no compute unit gets a second workgroup behind its first.
+static int once_grid(int groups, int cus)
+{
+    if (groups <= cus)
+        return groups;
+    if (groups < 2 * cus)
+        return groups / 2;
+    return cus * ((groups + ONCE_MAX_GROUPS * cus - 1) / (ONCE_MAX_GROUPS * cus));
+}
+
 int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
 {
     if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
@@ -1043,10 +1057,8 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
     const bool stage_ok = args.M <= 8 && align_ok;
     const bool once_ok  = args.M <= 32 && align_ok; // the stage-once form also takes one or two full blocks of 16 rows
-    // Up to 4096 of K the stage-once form: one workgroup per column group while there are no more groups than compute
-    // units; from two groups per compute unit on, one workgroup per compute unit (or as many as keep every workgroup
-    // within ONCE_MAX_GROUPS groups) with at least two groups each. In between, a second workgroup would not fit beside
-    // the first on a compute unit: one workgroup of 8 waves per group below. Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
+    // Up to 4096 of K and ONCE_MAX_GROUPS column groups per compute unit the stage-once form (grid: once_grid above).
+    // Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
     // up to 8 rows and 4096 < K <= 16384: the stage-once form for deep K (2, 3 or 4 chunks of 4 k blocks per wave)
     if (stage_ok && KB > 4 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
@@ -1063,10 +1075,10 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
-        if (cus > 0 && (groups <= cus || groups >= 2 * cus))
+        if (cus > 0)
         {
-            const bool multi = groups >= 2 * cus;
-            const int  grid  = multi ? std::max(cus, (groups + ONCE_MAX_GROUPS - 1) / ONCE_MAX_GROUPS) : groups;
+            const bool multi = groups > cus;
+            const int  grid  = once_grid(groups, cus);
             const int  per   = KB <= 8 ? 1 : (KB <= 16 ? 2 : (KB <= 32 ? 4 : 8));
 #define MI355_ONCE64(P_)                                                                        \
     (multi ? skinny_once_launch_r<P_, true, 64>(epi, flip_a, args, grid, s)                     \
@@ -1078,10 +1090,10 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     if (once_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
-        if (cus > 0 && (groups <= cus || groups >= 2 * cus))
+        if (cus > 0)
         {
-            const bool multi = groups >= 2 * cus;
-            const int  grid  = multi ? std::max(cus, (groups + ONCE_MAX_GROUPS - 1) / ONCE_MAX_GROUPS) : groups;
+            const bool multi = groups > cus;
+            const int  grid  = once_grid(groups, cus);
             const int  per   = KB <= ONCE_WAVES ? 1 : (KB <= 2 * ONCE_WAVES ? 2 : 4);
             if (multi)
                 return per == 1   ? skinny_once_launch_v<1, true>(epi, flip_a, args, grid, s)

@@ -282,8 +282,10 @@ def test_skinny_stage_once_kernel(M):
     32 as two blocks of rows) and K <= 4096 (whole 64-byte blocks, 16-byte aligned rows): one workgroup of 16 waves per
     compute unit walks several column groups with A staged once: K picks 1, 2 or 4 k blocks per wave, with the last busy wave short
     (K = 2112, 3136) or waves without any k block (K = 64, 640); N covers a single ragged group, fewer groups than compute
-    units, 2 to 3 groups per workgroup and more than four times the compute units; every epilogue, signed and unsigned
-    A, a non-zero B offset (row vector) and accumulation."""
+    units, between one and two groups per compute unit (N = 4100, 5000: half as many workgroups as groups, one of them
+    with three when the count is odd), 2 to 3 groups per workgroup, and more than four times the compute units (N = 16400,
+    70000: several workgroups per unit); every epilogue, signed and unsigned A, a non-zero B offset (row vector) and
+    accumulation."""
     rng = np.random.default_rng(3300 + M)
     for once in (True,):
         for (N, K) in [(7, 64), (300, 640), (8200, 1024), (11008, 4096), (5000, 2112), (4100, 3136), (70000, 256),

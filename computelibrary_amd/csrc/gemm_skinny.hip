@@ -1034,7 +1034,7 @@ struct SkinnyEnv
 // Workgroups of the stage-once kernels for `groups` column groups on `cus` compute units: one per group while they all
 // fit at once; from two groups per unit on, the smallest whole number of workgroups per compute unit that keeps every
 // workgroup within ONCE_MAX_GROUPS groups (a grid just above the number of units would leave most of them idle behind
-// the first round); in between, half as many workgroups as groups, so that every workgroup still has two (one of them
+// the first round) - or fewer workgroups with equal shares, see below; in between, half as many workgroups as groups, so that every workgroup still has two (one of them
 // three when the count is odd) and no compute unit gets a second workgroup behind its first.
 static int once_grid(int groups, int cus)
 {
@@ -1042,6 +1042,11 @@ static int once_grid(int groups, int cus)
         return groups;
     if (groups < 2 * cus)
         return groups / 2;
+    // a last round that would occupy an eighth to half of the compute units: the same number of groups for every
+    // workgroup, on fewer units, measured 2-7 % faster (a fuller last round, or just a few groups: 0-1 % slower)
+    const int r = (groups + cus - 1) / cus, last = groups - (r - 1) * cus;
+    if (r <= ONCE_MAX_GROUPS && last >= cus / 8 && last <= cus / 2)
+        return (groups + r - 1) / r;
     return cus * ((groups + ONCE_MAX_GROUPS * cus - 1) / (ONCE_MAX_GROUPS * cus));
 }
 

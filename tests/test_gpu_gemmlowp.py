@@ -283,13 +283,14 @@ def test_skinny_stage_once_kernel(M):
     compute unit walks several column groups with A staged once: K picks 1, 2 or 4 k blocks per wave, with the last busy wave short
     (K = 2112, 3136) or waves without any k block (K = 64, 640); N covers a single ragged group, fewer groups than compute
     units, between one and two groups per compute unit (N = 4100, 5000: half as many workgroups as groups, one of them
-    with three when the count is odd), 2 to 3 groups per workgroup, and more than four times the compute units (N = 16400,
-    70000: several workgroups per unit); every epilogue, signed and unsigned A, a non-zero B offset (row vector) and
+    with three when the count is odd), 2 to 3 groups per workgroup, a sparse last round (N = 9300: fewer workgroups than
+    compute units, three groups each), and more than four times the compute units (N = 16400, 70000: several workgroups
+    per unit); every epilogue, signed and unsigned A, a non-zero B offset (row vector) and
     accumulation."""
     rng = np.random.default_rng(3300 + M)
     for once in (True,):
         for (N, K) in [(7, 64), (300, 640), (8200, 1024), (11008, 4096), (5000, 2112), (4100, 3136), (70000, 256),
-                       (16400, 2048)]:
+                       (16400, 2048), (9300, 512)]:
             a_dt = np.uint8 if (N + K) % 3 == 0 else np.int8
             A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
             B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)

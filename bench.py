@@ -453,38 +453,39 @@ def main():
             for f in fg3:
                 f.close()
 
-        # a deep-K decode shape (the down projection of a feed-forward block: few rows, K = 11008; not a BASELINE
-        # configuration), B rotated over ROT packed copies like the legs above
-        Md, Nd, Kd = 8, 4096, 11008
-        Adh, Bdh, biasdh, multdh, shiftdh = synth_config2(Md, Nd, Kd, seed=7)
-        Add = torch.from_numpy(Adh).cuda()
-        Ddd = torch.zeros((Md, Nd), dtype=torch.int8, device="cuda")
-        keepd = [torch.from_numpy(x).cuda() for x in (biasdh, multdh, shiftdh)]
-        hd = []
-        for r in range(ROT):
-            h = capi.Gemm(Md, Nd, Kd, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
-            h.prepare(torch.from_numpy(np.roll(Bdh, r, axis=1) if r else Bdh).cuda(), *keepd, stream)
-            hd.append(h)
-        torch.cuda.synchronize()
-        stepsd = max(args.steps, 10 * ROT) // ROT * ROT
-        for _ in range(max(args.warmup // ROT, 2)):
-            for h in hd:
-                h.run(Add, Ddd, None, stream)
-        graph_d = time_graph(torch, [(lambda cs, h=h: h.run(Add, Ddd, None, cs)) for h in hd], stepsd)
-        okd = None
-        if check:
+        # two more decode shapes (not BASELINE configurations), B rotated over ROT packed copies like the legs above: a deep K
+        # (the down projection of a feed-forward block: few rows, K = 11008) and a wide N (four column groups per compute
+        # unit, where the fixed part of a launch weighs least)
+        for leg, Md, Nd, Kd in (("decode_deep_k", 8, 4096, 11008), ("decode_wide_n", 8, 16384, 4096)):
+            Adh, Bdh, biasdh, multdh, shiftdh = synth_config2(Md, Nd, Kd, seed=7)
+            Add = torch.from_numpy(Adh).cuda()
+            Ddd = torch.zeros((Md, Nd), dtype=torch.int8, device="cuda")
+            keepd = [torch.from_numpy(x).cuda() for x in (biasdh, multdh, shiftdh)]
+            hd = []
+            for r in range(ROT):
+                h = capi.Gemm(Md, Nd, Kd, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq)
+                h.prepare(torch.from_numpy(np.roll(Bdh, r, axis=1) if r else Bdh).cuda(), *keepd, stream)
+                hd.append(h)
             torch.cuda.synchronize()
-            fgd = oracle.FastGemm(np.roll(Bdh, ROT - 1, axis=1))
-            okd = bool(np.array_equal(Ddd.cpu().numpy(), fgd.run(Adh, biasdh, -3, 0, multdh, shiftdh, -5, -128, 127, np.int8)))
-            fgd.close()
-        bytes_d = Nd * Kd + Md * Kd + Md * Nd + 3 * 4 * Nd
-        out["secondary"]["decode_deep_k"] = {
-            "workload": "M=8 N=4096 K=11008 s8 x per-channel s8 -> s8", "kernel": hd[0].kernel_name, "bytes": bytes_d,
-            "kernel_us": round(graph_d * 1e6, 3), "achieved_GBs": round(bytes_d / graph_d / 1e9, 1),
-            "frac_hbm": round(bytes_d / graph_d / 1e9 / HBM_PEAK_GBS, 4), "bit_exact_vs_cpu": okd}
-        for h in hd:
-            h.close()
-        del hd, Add, Ddd, keepd
+            stepsd = max(args.steps, 10 * ROT) // ROT * ROT
+            for _ in range(max(args.warmup // ROT, 2)):
+                for h in hd:
+                    h.run(Add, Ddd, None, stream)
+            graph_d = time_graph(torch, [(lambda cs, h=h: h.run(Add, Ddd, None, cs)) for h in hd], stepsd)
+            okd = None
+            if check:
+                torch.cuda.synchronize()
+                fgd = oracle.FastGemm(np.roll(Bdh, ROT - 1, axis=1))
+                okd = bool(np.array_equal(Ddd.cpu().numpy(), fgd.run(Adh, biasdh, -3, 0, multdh, shiftdh, -5, -128, 127, np.int8)))
+                fgd.close()
+            bytes_d = Nd * Kd + Md * Kd + Md * Nd + 3 * 4 * Nd
+            out["secondary"][leg] = {
+                "workload": "M=%d N=%d K=%d s8 x per-channel s8 -> s8" % (Md, Nd, Kd), "kernel": hd[0].kernel_name, "bytes": bytes_d,
+                "kernel_us": round(graph_d * 1e6, 3), "achieved_GBs": round(bytes_d / graph_d / 1e9, 1),
+                "frac_hbm": round(bytes_d / graph_d / 1e9 / HBM_PEAK_GBS, 4), "bit_exact_vs_cpu": okd}
+            for h in hd:
+                h.close()
+            del hd, Add, Ddd, keepd
 
         # config 4: NHWC 3x3 convolution as an implicit GEMM (M = 32*56*56, N = 64, K = 576), near the roofline ridge
         rng = np.random.default_rng(4)

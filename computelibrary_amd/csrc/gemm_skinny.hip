@@ -471,7 +471,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
     constexpr int RPL   = 64 / LPR > ROWS ? ROWS : 64 / LPR;                 // rows per load
     // partial results [2][wave][block of rows][lane][4]: for 32 rows they take over the staging area once every wave
     // has its operands of A in registers (the two together would not fit)
-    constexpr bool RED_IN_STAGE = RB > 1;
+    constexpr bool RED_IN_STAGE = RB > 1 || (ROWS == 16 && PER == 8); // (16 rows of 8 k blocks per wave fill LDS as well)
     __shared__ __attribute__((aligned(16))) int32_t red_own[RED_IN_STAGE ? 1 : 2 * WAVES * RB * RL * 4];
     __shared__ int32_t                              par[4][64]; // [vector][group * 16 + column]; row vector: [3][row]
     extern __shared__ __attribute__((aligned(16))) char a_stage[]; // [WAVES][ROWS][PITCH] (nothing staged with 64 rows)
@@ -502,7 +502,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
     p.has_offsets = g.has_offsets, p.accumulate = g.accumulate, p.act_twice = g.act_twice;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // (8 k blocks per wave: the wave index as a scalar, so that the addresses of the B blocks are a scalar base plus one
+    // per-lane offset - as per-lane 64-bit addresses, all computed ahead, they pushed the B blocks out of the registers)
+    const int wave = (PER == 8 && ROWS < 64) ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : (int)(threadIdx.x >> 6);
     const int KB   = g.KB;
     const int NGT  = (g.N + 15) / 16;
     const int G    = g.grid; // == gridDim.x
@@ -547,8 +549,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
     const MI355_GLOBAL int8_t *bp = gB + ((int64_t)min(kb0, KB - 1) * 64 + lane) * 16; // (waves without k blocks re-read the last one)
     // B operand blocks: two groups' worth in flight per wave - or, with 64 rows (half the registers hold A), one group's
     // worth, refilled half by half as the matrix instructions release them
-    constexpr int H0 = PER / 2; // k blocks of the first half
-    v4i           fb[A_GLOBAL ? 1 : 2][PER];
+    constexpr int  H0       = PER / 2;               // k blocks of the first half
+    constexpr bool ONE_SLOT = A_GLOBAL || PER == 8; // (8 k blocks per wave: two groups' worth would not fit the registers)
+    v4i            fb[ONE_SLOT ? 1 : 2][PER];
     auto load_b_part = [&](int slot, int gi, auto u0c, auto u1c)
     {
         const int grp = min((int)blockIdx.x + gi * G, NGT - 1);
@@ -568,7 +571,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
     // (loads return in order) - hence also the unconditional fetches of the epilogue constants below.
     load_b(0, 0);
     __builtin_amdgcn_sched_barrier(0); // group 0 goes out whole before group 1: the first wait then covers group 0 only
-    if (MULTI && !A_GLOBAL)
+    if (MULTI && !ONE_SLOT)
         load_b(1, 1);
     // (with nothing to stage, A is fetched behind the first B blocks: the first matrix instruction needs both anyway,
     // and the stream of B starts that much earlier)
@@ -640,25 +643,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
                 // matrix instructions: their results may not be read by another instruction type for about a dozen
                 // slots, and the compiler only pads that distance inside a block - with the first reader behind a taken
                 // branch it came 3 slots after the instruction and read the last register of the result too early.
-                if constexpr (RB == 4)
+                if constexpr (ONE_SLOT)
                 {
-                    // four blocks of rows are four independent chains: one accumulator each. The B blocks of the next
-                    // group are asked for as soon as their registers are free, half by half.
+                    // The B blocks of the next group are asked for as soon as their registers are free, half by half.
+                    // Four blocks of rows are four independent chains, one accumulator each; fewer blocks alternate
+                    // between two accumulators per block like the two-slot form below.
+                    auto half = [&](auto u0c, auto u1c)
+                    {
 #pragma unroll
-                    for (int u = 0; u < H0; ++u)
+                        for (int u = decltype(u0c)::value; u < decltype(u1c)::value; ++u)
 #pragma unroll
-                        for (int rb = 0; rb < RB; ++rb)
-                            acc0[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc0[rb], 0, 0, 0);
+                            for (int rb = 0; rb < RB; ++rb)
+                            {
+                                if (RB == 4 || !(u & 1))
+                                    acc0[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc0[rb], 0, 0, 0);
+                                else
+                                    acc1[RB < 4 ? rb : 0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc1[RB < 4 ? rb : 0], 0, 0, 0);
+                            }
+                    };
+                    half(std::integral_constant<int, 0>{}, std::integral_constant<int, H0>{});
                     if (gi + 1 < MINE)
                         load_b_part(0, gi + 1, std::integral_constant<int, 0>{}, std::integral_constant<int, H0>{});
-#pragma unroll
-                    for (int u = H0; u < PER; ++u)
-#pragma unroll
-                        for (int rb = 0; rb < RB; ++rb)
-                            acc0[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[rb][u], fb[0][u], acc0[rb], 0, 0, 0);
+                    half(std::integral_constant<int, H0>{}, std::integral_constant<int, PER>{});
                     if (gi + 1 < MINE)
                         load_b_part(0, gi + 1, std::integral_constant<int, H0>{}, std::integral_constant<int, PER>{});
-                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]));
+                    if constexpr (RB == 4)
+                        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]));
+                    else if constexpr (RB == 1)
+                    {
+                        acc0[0] += acc1[0];
+                        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]));
+                    }
+                    else
+                    {
+                        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc0[0]), "+v"(acc1[0]), "+v"(acc0[RB - 1]), "+v"(acc1[RB - 1]));
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            acc0[rb] += acc1[RB < 4 ? rb : 0];
+                    }
                 }
                 else
                 {
@@ -683,7 +705,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
                     }
                 }
             }
-            if (!A_GLOBAL && gi + 2 < MINE)
+            if (!ONE_SLOT && gi + 2 < MINE)
                 load_b(gi & 1, gi + 2);
             // accumulator r of lane l is row 4 * (l / 16) + r, column l % 16: lanes 32..63 hold rows 8..15
             if (RL == 64 || lane < 32)
@@ -724,7 +746,7 @@ static_assert(ONCE_MAX_GROUPS == 4, "the group loop is written out for 1 to 4 gr
 
 #undef MI355_GLOBAL
 
-// ---- the stage-once form for deep K: up to 8 rows, 4096 < K <= 16384 -------------------------------------------------
+// ---- the stage-once form for deep K: up to 8 rows, 8192 < K <= 16384 -------------------------------------------------
 // (the down projection of a transformer's feed-forward block is this shape: few rows, K = 11008 / 14336)
 // The same plan - one workgroup of 16 waves per compute unit, every wave stages its K slice of A once and walks the
 // column groups - but a wave's slice is NCH chunks of 4 k blocks now, and registers for all of it would leave none for
@@ -1004,6 +1026,13 @@ static int skinny_deepk_launch(int epi, bool flip_a, const GemmArgs &a, int grid
     return (int)hipLaunchKernel(fn, dim3(grid), dim3(ONCE_WAVES * 64), kargs, lds, s);
 }
 
+// 8 k blocks per wave (4096 < K <= 8192): up to 16 rows, whose slices still fit LDS
+template <bool MULTI>
+static int skinny_once_launch_v8(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
+{
+    return a.M > 8 ? skinny_once_launch_r<8, MULTI, 16>(epi, flip_a, a, grid, s) : skinny_once_launch_r<8, MULTI, 8>(epi, flip_a, a, grid, s);
+}
+
 template <int PER, bool MULTI>
 static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int grid, hipStream_t s)
 {
@@ -1062,18 +1091,17 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
     const bool stage_ok = args.M <= 8 && align_ok;
     const bool once_ok  = args.M <= 32 && align_ok; // the stage-once form also takes one or two full blocks of 16 rows
-    // Up to 4096 of K and ONCE_MAX_GROUPS column groups per compute unit the stage-once form (grid: once_grid above).
-    // Each of the 16 waves owns PER = 1, 2 or 4 k blocks.
-    // up to 8 rows and 4096 < K <= 16384: the stage-once form for deep K (2, 3 or 4 chunks of 4 k blocks per wave)
-    if (stage_ok && KB > 4 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    // Up to 4096 of K the stage-once form (grid: once_grid above), each of the 16 waves owning PER = 1, 2 or 4 k blocks;
+    // up to 16 rows it also takes 4096 < K <= 8192 with 8 k blocks per wave (one group's worth of B in flight per wave,
+    // refilled half by half - the same bytes as two groups of 4 k blocks).
+    // up to 8 rows and 8192 < K <= 16384: the stage-once form for deep K (3 or 4 chunks of 4 k blocks per wave)
+    if (stage_ok && KB > 8 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0 && groups <= cus) // one column group per workgroup
         {
             const int nch = (KB + 4 * ONCE_WAVES - 1) / (4 * ONCE_WAVES);
-            return nch == 2   ? skinny_deepk_launch<2>(epi, flip_a, args, groups, s)
-                   : nch == 3 ? skinny_deepk_launch<3>(epi, flip_a, args, groups, s)
-                              : skinny_deepk_launch<4>(epi, flip_a, args, groups, s);
+            return nch == 3 ? skinny_deepk_launch<3>(epi, flip_a, args, groups, s) : skinny_deepk_launch<4>(epi, flip_a, args, groups, s);
         }
     }
     // 33 to 64 rows: the same with 8 waves, each holding the operand blocks of its 1, 2, 4 or 8 k blocks of all 64 rows
@@ -1092,14 +1120,16 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
 #undef MI355_ONCE64
         }
     }
-    if (once_ok && KB <= 4 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    if (once_ok && (KB <= 4 * ONCE_WAVES || (KB <= 8 * ONCE_WAVES && args.M <= 16)) && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0)
         {
             const bool multi = groups > cus;
             const int  grid  = once_grid(groups, cus);
-            const int  per   = KB <= ONCE_WAVES ? 1 : (KB <= 2 * ONCE_WAVES ? 2 : 4);
+            const int  per   = KB <= ONCE_WAVES ? 1 : (KB <= 2 * ONCE_WAVES ? 2 : (KB <= 4 * ONCE_WAVES ? 4 : 8));
+            if (per == 8)
+                return multi ? skinny_once_launch_v8<true>(epi, flip_a, args, grid, s) : skinny_once_launch_v8<false>(epi, flip_a, args, grid, s);
             if (multi)
                 return per == 1   ? skinny_once_launch_v<1, true>(epi, flip_a, args, grid, s)
                        : per == 2 ? skinny_once_launch_v<2, true>(epi, flip_a, args, grid, s)

@@ -321,14 +321,48 @@ def test_skinny_stage_once_kernel(M):
                                               oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
 
 
+@pytest.mark.parametrize("M", [1, 8, 9, 16])
+def test_skinny_stage_once_kernel_with_8_k_blocks_per_wave(M):
+    """Up to 16 rows and 4096 < K <= 8192: the stage-once kernel with 8 k blocks per wave and one group's worth of B per
+    wave, refilled half by half. K = 4160 leaves one wave with a single k block and seven without any, 5120 and 6656 a
+    whole number of waves, 8192 all sixteen; N covers one workgroup per group, half as many workgroups as groups, one per
+    compute unit with 2 to 3 groups, and equal shares on fewer units; every epilogue, both signs, accumulation."""
+    rng = np.random.default_rng(5500 + M)
+    for (N, K) in [(300, 4160), (5120, 5120), (8200, 8192), (9300, 6656), (4100, 8192)]:
+        a_dt = np.uint8 if (N + K) % 3 == 0 else np.int8
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
+        lda = K + (0 if K % 128 else 16)
+        announce("skinny 8 k blocks per wave", (M, N, K), "lda", lda, a_dt.__name__)
+        want = oracle.gemmlowp_s32(A, B, ao, bo)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_AUTO, device=True, lda=lda, ldd=N + 3)
+        assert name.startswith("skinny"), name
+        np.testing.assert_array_equal(got, want)
+        prev = rng.integers(-10**6, 10**6, size=(M, N), dtype=np.int32)
+        got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, device=True, lda=lda, prev=prev, flags=capi.GEMM_ACCUMULATE)
+        np.testing.assert_array_equal(got, (want.astype(np.int64) + prev).astype(np.int32))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, 0, bias, mult, shift, off, lo, hi, device=True, lda=lda)
+        np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, off, lo, hi, a_dt))
+        if a_dt == np.int8:
+            biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, device=True, lda=lda)
+            np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
+
+
 @pytest.mark.parametrize("M", [1, 5, 8])
 def test_skinny_stage_once_kernel_deep_k(M):
-    """Up to 8 rows, 4096 < K <= 16384 and no more column groups than compute units (the down projection of a feed-forward
-    block): every wave stages 2, 3 or 4 chunks of 4 k blocks of A and re-reads them per chunk; K picks each chunk count,
-    with a short last busy wave (K = 11008: 172 k blocks over waves of 12), waves without k blocks, and a single k block
-    more than the shallow form takes; N a ragged single group up to 256 groups; every epilogue, both signs."""
+    """Up to 8 rows, 8192 < K <= 16384 and no more column groups than compute units (the down projection of a feed-forward
+    block): every wave stages 3 or 4 chunks of 4 k blocks of A and re-reads them per chunk; K picks both chunk counts,
+    with a short last busy wave (K = 11008: 172 k blocks over waves of 12) and waves without k blocks (K = 8256: one k
+    block more than the shallower form takes); N a ragged single group up to 256 groups; every epilogue, both signs.
+    (K = 4160, 6400 and 8192 run the shallower form with one workgroup per group.)"""
     rng = np.random.default_rng(4400 + M)
-    for (N, K) in [(4096, 11008), (40, 4160), (1000, 8192), (300, 12288), (2500, 16384), (777, 14336), (4096, 6400)]:
+    for (N, K) in [(4096, 11008), (40, 4160), (1000, 8192), (300, 12288), (2500, 16384), (777, 14336), (4096, 6400), (520, 8256)]:
         a_dt = np.uint8 if (N + K) % 3 == 0 else np.int8
         A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
         B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)

@@ -168,7 +168,8 @@ struct GemmCore
     bool    has_narrow = false; // Bn holds the narrow kernel's image of B
     bool    pt_vectors = false; // streaming path, per-tensor requantisation: mult / shift hold the scalars, replicated
     std::string kname;
-    DevBuf  Bp, Bs, Bn, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros;
+    DevBuf  Bp, Bs, Bn, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros, parts, zerocol;
+    int     splitk = 1; // K slices of the pipelined kernel (decided in prepare(), where the device is known)
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -182,7 +183,7 @@ struct GemmCore
     void release()
     {
         Bp.release(), Bs.release(), Bn.release(), colsum.release(), colvec.release(), rowvec.release(), mult.release();
-        shift.release(), bias.release(), Ap.release(), fill.release(), qp.release(), zeros.release();
+        shift.release(), bias.release(), Ap.release(), fill.release(), qp.release(), zeros.release(), parts.release(), zerocol.release();
     }
 
     int choose_kernel()
@@ -313,6 +314,32 @@ struct GemmCore
             // the streaming kernel fetches its per-row vector without asking whether there is one
             TRY(zeros.ensure(sizeof(int32_t) * SKINNY_MAX_M));
             HIP_TRY(fill_i32_launch(zeros.as<int32_t>(), 0, SKINNY_MAX_M, s));
+        }
+        // A deep K under few output tiles: the pipelined kernel would leave most compute units idle, each of the others
+        // walking the whole K. The K range is cut into slices that run as the batch entries of one S32 launch (the slice
+        // offset is the batch stride of A and of the packed B alike), and a second kernel sums the planes and applies the
+        // epilogue. Slices are whole k steps of the tile shape, so no slice but the matrix' own end has a tail.
+        splitk = 1;
+        static const bool no_splitk = getenv("MI355_NO_SPLITK") != nullptr;
+        if (path == MI355_PATH_MFMA && dma_idx >= 0 && batch == 1 && !no_splitk && K >= 2048)
+        {
+            const MfmaConfig c     = dma_config(dma_idx);
+            const int64_t    tiles = (int64_t)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN);
+            const int        cus   = device_cus();
+            if (cus > 0 && tiles * 2 <= cus)
+            {
+                int sl = (int)std::min<int64_t>(std::min<int64_t>(cus / tiles, K / 1024), 8);
+                while (sl > 1 && K % (sl * c.BK) != 0)
+                    --sl;
+                splitk = sl;
+            }
+        }
+        if (splitk > 1)
+        {
+            const size_t ldp = ((size_t)N + 3) & ~(size_t)3;
+            TRY(parts.ensure(sizeof(int32_t) * (size_t)splitk * M * ldp));
+            TRY(zerocol.ensure(sizeof(int32_t) * (size_t)Np));
+            HIP_TRY(fill_i32_launch(zerocol.as<int32_t>(), 0, Np, s));
         }
         TRY(refresh_colvec(s));
         TRY(refresh_qparams(s));
@@ -501,6 +528,22 @@ struct GemmCore
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;
                 g.tiles_n          = (g.N + c.BN - 1) / c.BN;
                 kname              = kprefix + kname_dma;
+                if (splitk > 1 && !conv && batch == 1 && g.K == K && K % (splitk * c.BK) == 0)
+                {
+                    const int     ldp = (N + 3) & ~3;
+                    const int64_t kc  = K / splitk;
+                    GemmArgs      gp  = g;
+                    gp.epi                     = EpiParams{};
+                    gp.epi.colvec              = zerocol.as<int32_t>();
+                    gp.epi.colvec_batch_stride = 0;
+                    gp.epi.vec_store           = 1;
+                    gp.D = parts.as<int32_t>(), gp.ldd = ldp, gp.d_batch_stride = (int64_t)M * ldp;
+                    gp.K = (int)kc, gp.a_batch_stride = kc, gp.bp_batch_stride = kc;
+                    kname += "_splitk" + std::to_string(splitk);
+                    HIP_TRY(dma_launch(dma_idx, EPI_S32, flip_in_loader, false, gp, splitk, s));
+                    HIP_TRY(splitk_finish_launch(epi, g, parts.as<int32_t>(), (int64_t)M * ldp, ldp, splitk, s));
+                    return 0;
+                }
                 HIP_TRY(dma_launch(dma_idx, epi, flip_in_loader, conv, g, batch, s));
             }
             else

@@ -131,6 +131,8 @@ int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t
 int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int32_t b_off, int32_t *rowvec, hipStream_t s);
 int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                         int N, const EpiParams &epi, hipStream_t s);
+// sum of `splits` S32 planes (M rows of ldp words, `plane` words apart) through epilogue `epi` of g into g.D
+int splitk_finish_launch(int epi, const GemmArgs &g, const int32_t *parts, int64_t plane, int ldp, int splits, hipStream_t s);
 int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,
                             int N, const EpiParams &epi, hipStream_t s);
 // [batch][R][C] bytes -> [batch][C][R]

@@ -32,6 +32,80 @@ int fill_i32_launch(int32_t *p, int32_t v, int64_t n, hipStream_t s)
     return launch_status();
 }
 
+// ---- split K: the partial products of `splits` K slices (S32 planes of M rows of ldp words, `plane` words apart) summed
+// and put through the epilogue the fused kernel would have applied. One thread per 4 consecutive columns of a row.
+// Same arithmetic as epilogue_store_t: the sum of the slices is the accumulator of the whole K
+// (what CpuGemmLowpOffsetContributionOutputStageKernel, src/cpu/kernels/CpuGemmLowpOffsetContributionOutputStageKernel.cpp:
+// 830-940, is handed by the matrix multiply before it).
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const int32_t *__restrict__ parts, int64_t plane, int ldp, int splits,
+                                                            GemmArgs g)
+{
+    typedef int   v4i __attribute__((ext_vector_type(4)));
+    const EpiParams &p  = g.epi;
+    const int        n4 = (g.N + 3) / 4;
+    const int64_t    t  = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (int64_t)g.M * n4)
+        return;
+    const int i = (int)(t / n4), j0 = (int)(t % n4) * 4;
+    v4i       acc = {0, 0, 0, 0};
+    for (int sl = 0; sl < splits; ++sl) // (columns from N on hold whatever the allocation held: never used below)
+        acc += *(const v4i *)(parts + (int64_t)sl * plane + (int64_t)i * ldp + j0);
+    const int32_t rv  = p.rowvec ? p.rowvec[i] : 0;
+    const int64_t idx = (int64_t)i * g.ldd + j0;
+    const bool    vec = p.vec_store && j0 + 3 < g.N;
+    char         *D   = (char *)g.D;
+    v4i           o   = {0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+    {
+        const int j = j0 + c;
+        if (j >= g.N)
+            continue;
+        const int32_t cv = p.colvec[j];
+        if (EPI == EPI_FIXEDPOINT)
+            o[c] = epi_fixedpoint(acc[c], cv, rv, p.mult ? p.mult[j] : p.mult_s, p.shift ? p.shift[j] : p.shift_s, p);
+        else if (EPI == EPI_S32)
+            o[c] = (int32_t)((uint32_t)acc[c] + (uint32_t)cv + (uint32_t)rv + (p.accumulate ? (uint32_t)((int32_t *)D)[idx + c] : 0u));
+        else
+            o[c] = __float_as_int(epi_f32(acc[c], (int32_t)((uint32_t)cv + (uint32_t)rv), p.bias_f32 ? p.bias_f32[j] : 0.f,
+                                          p.bias_f32 != nullptr, p, p.accumulate ? ((float *)D)[idx + c] : 0.f));
+    }
+    if (EPI == EPI_FIXEDPOINT)
+    {
+        if (vec)
+            *(uint32_t *)(D + idx) = ((uint32_t)o[0] & 0xFFu) | (((uint32_t)o[1] & 0xFFu) << 8) | (((uint32_t)o[2] & 0xFFu) << 16) |
+                                     (((uint32_t)o[3] & 0xFFu) << 24);
+        else
+            for (int c = 0; c < 4 && j0 + c < g.N; ++c)
+                D[idx + c] = (char)o[c];
+    }
+    else
+    {
+        if (vec)
+            *(v4i *)((int32_t *)D + idx) = o;
+        else
+            for (int c = 0; c < 4 && j0 + c < g.N; ++c)
+                ((int32_t *)D)[idx + c] = o[c];
+    }
+}
+int splitk_finish_launch(int epi, const GemmArgs &g, const int32_t *parts, int64_t plane, int ldp, int splits, hipStream_t s)
+{
+    if (g.M < 1 || g.N < 1 || splits < 1 || ldp % 4 != 0 || plane % 4 != 0 || ((uintptr_t)parts & 15) != 0 || g.epi.colvec == nullptr)
+        return (int)hipErrorInvalidValue;
+    const int64_t  n = (int64_t)g.M * ((g.N + 3) / 4);
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (epi == EPI_FIXEDPOINT)
+        splitk_finish_kernel<EPI_FIXEDPOINT><<<dim3(blocks), dim3(256), 0, s>>>(parts, plane, ldp, splits, g);
+    else if (epi == EPI_S32)
+        splitk_finish_kernel<EPI_S32><<<dim3(blocks), dim3(256), 0, s>>>(parts, plane, ldp, splits, g);
+    else if (epi == EPI_F32)
+        splitk_finish_kernel<EPI_F32><<<dim3(blocks), dim3(256), 0, s>>>(parts, plane, ldp, splits, g);
+    else
+        return (int)hipErrorInvalidValue;
+    return launch_status();
+}
+
 // ---- P1: B[K][ldb] -> Bp[Np][Kp] (transpose to K-contiguous, optional sign flip, zero padding) + column sums ----------
 // Replaces pretranspose_B_array (src/cpu/operators/internal/CpuGemmAssemblyDispatch.cpp:594-617) / CpuGemmTranspose1xWKernel and
 // CpuGemmLowpMatrixBReductionKernel (src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:273-446) in one pass over B.

@@ -239,7 +239,7 @@ def test_every_pipelined_configuration(cfg, monkeypatch):
         got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_MFMA, device=True)
         kp = -(-K // 128) * 128
         if cfg != 5 or kp % 256 == 0:
-            assert name == PIPELINED_CONFIGS[cfg], name
+            assert name.split("_splitk")[0] == PIPELINED_CONFIGS[cfg], name  # (K = 2048 under one tile runs as two K slices)
         np.testing.assert_array_equal(got, oracle.gemmlowp_s32(A, B, ao, bo))
         bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
         reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
@@ -319,6 +319,43 @@ def test_skinny_stage_once_kernel(M):
                 got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, device=True, lda=lda)
                 np.testing.assert_array_equal(got.view(np.uint32),
                                               oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
+
+
+def test_pipelined_kernel_with_k_slices():
+    """Few output tiles under a deep K: the K range runs as 2 to 8 slices (batch entries of one S32 launch) and a second
+    kernel sums the planes and applies the epilogue. Shapes pick 2, 4 and 8 slices, ragged M and N (a plane pitch padded to
+    4 columns), both signs of A, offsets on both sides (row and column terms applied once, by the second kernel), every
+    epilogue, per-channel and per-tensor constants, accumulation into S32 and F32; a K that no slice count divides stays
+    one launch."""
+    rng = np.random.default_rng(6600)
+    for (M, N, K, slices) in [(100, 512, 4096, 4), (200, 302, 8192, 8), (130, 200, 2560, 2), (70, 1000, 2049 + 63, 1)]:
+        a_dt = np.uint8 if K % 3 == 0 else np.int8
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
+        announce("k slices", (M, N, K), slices, a_dt.__name__)
+        want = oracle.gemmlowp_s32(A, B, ao, bo)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_MFMA, device=True, ldd=N + 5)
+        assert ("_splitk%d" % slices in name) if slices > 1 else ("_splitk" not in name), name
+        np.testing.assert_array_equal(got, want)
+        prev = rng.integers(-10**6, 10**6, size=(M, N), dtype=np.int32)
+        got, _ = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_MFMA, device=True, prev=prev, flags=capi.GEMM_ACCUMULATE)
+        np.testing.assert_array_equal(got, (want.astype(np.int64) + prev).astype(np.int32))
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+        got, name = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, bo, bias, mult, shift, off, lo, hi, path=capi.PATH_MFMA, device=True)
+        assert ("_splitk%d" % slices in name) if slices > 1 else ("_splitk" not in name), name
+        np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, bo, mult, shift, off, lo, hi, a_dt))
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, 0, bias, [int(mult[0])], [int(shift[0])], off, lo, hi,
+                          path=capi.PATH_MFMA, device=True, ldd=N + 16)
+        np.testing.assert_array_equal(
+            got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, [int(mult[0])], [int(shift[0])], off, lo, hi, a_dt))
+        if a_dt == np.int8:
+            biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, path=capi.PATH_MFMA, device=True)
+            np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
 
 
 @pytest.mark.parametrize("M", [1, 8, 9, 16])

@@ -321,6 +321,31 @@ def test_skinny_stage_once_kernel(M):
                                               oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
 
 
+def test_streaming_kernels_across_their_grid_rules():
+    """The stage-once kernels pick their grid from the number of column groups per compute unit (one workgroup per group,
+    half as many workgroups as groups, one per unit, equal shares on fewer units, whole rounds beyond four groups per
+    unit) and their build from M and K (1, 2, 4 or 8 k blocks per wave; 8, 16, 32 or 64 rows; the deep-K form). A seeded
+    sample of shapes on both sides of every boundary, raw S32 products against a float64 matrix product (exact: the sums
+    stay far below 2^53), with one requantised case per shape class elsewhere in this file."""
+    _, cus = capi.device_info()
+    rng = np.random.default_rng(8800)
+    group_counts = [cus - 1, cus, cus + 1, cus + cus // 2 + 1, 2 * cus - 1, 2 * cus, 2 * cus + 1, 2 * cus + cus // 8 - 1,
+                    2 * cus + cus // 8, 2 * cus + cus // 2, 2 * cus + cus // 2 + 1, 3 * cus + cus // 4, 4 * cus, 4 * cus + 1, 5 * cus + 3]
+    depths = [1024, 2112, 4096, 4160, 5120, 8192, 8256]
+    rows = [3, 8, 12, 16, 20, 32, 40, 64]
+    cases = [(rows[int(rng.integers(len(rows)))], group_counts[int(rng.integers(len(group_counts)))] * 16 - int(rng.integers(0, 16)),
+              depths[int(rng.integers(len(depths)))]) for _ in range(40)]
+    cases += [(8, (2 * cus + cus // 8) * 16, 8192), (16, (cus + 1) * 16, 8192), (8, 4 * cus * 16 + 1, 4096), (64, (cus + 3) * 16, 4096)]
+    for (M, N, K) in cases:
+        A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+        announce("streaming grid rules", (M, N, K), "groups per unit %.2f" % ((N + 15) // 16 / cus))
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, 0, 0, path=capi.PATH_SKINNY, device=True)
+        assert name.startswith("skinny"), name
+        want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.int64)
+        np.testing.assert_array_equal(got.astype(np.int64), want)
+
+
 def test_pipelined_kernel_with_k_slices():
     """Few output tiles under a deep K: the K range runs as 2 to 8 slices (batch entries of one S32 launch) and a second
     kernel sums the planes and applies the epilogue. Shapes pick 2, 4 and 8 slices, ragged M and N (a plane pitch padded to

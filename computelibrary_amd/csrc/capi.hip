@@ -169,7 +169,9 @@ struct GemmCore
     bool    pt_vectors = false; // streaming path, per-tensor requantisation: mult / shift hold the scalars, replicated
     std::string kname;
     DevBuf  Bp, Bs, Bn, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros, parts, zerocol;
-    int     splitk = 1; // K slices of the pipelined kernel (decided in prepare(), where the device is known)
+    int     splitk = 1;      // K slices of the pipelined kernel
+    int     splitk_plan = 1; // what the cost model chose with the tile shape (create()); prepare() checks it and allocates
+    bool    conv_core = false; // the GEMM inside a convolution handle: its implicit loader takes no K slices
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -232,26 +234,36 @@ struct GemmCore
             // barrier-separated slots of the consumer groups (about 1000 clocks per 128 bytes of K, whatever the tile);
             // every tile adds a fixed start-up plus an epilogue proportional to its outputs, which co-resident
             // workgroups overlap. Ties go to the deeper ring (more loads in flight when B comes from HBM).
+            // A single dense GEMM may also run its K range as 2, 4 or 8 slices (see prepare()): the tiles of all slices
+            // share the chip, every slice has 1/S of the K steps, and a second kernel reads the S planes of partial
+            // sums back (measured: about 2.5 bytes per clock and compute unit of the whole chip, plus a launch).
             auto pick_dma = [&]() -> int
             {
                 int    best = -1, best_lds = 0;
                 double best_cost = 0;
+                static const bool no_splitk = getenv("MI355_NO_SPLITK") != nullptr;
                 for (int i = 0; i < dma_num_configs(); ++i)
                 {
                     const MfmaConfig c = dma_config(i);
                     if ((N <= 64 && c.BN > 64) || Kp % c.BK != 0)
                         continue;
                     const double tiles   = (double)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN) * batch;
-                    const double per_cu  = std::ceil(tiles / cus);
                     const int    occ_lds = (160 * 1024) / c.lds_bytes, occ_wav = 32 / c.waves;
                     const double occ     = std::max(1, std::min(occ_lds, occ_wav));
                     const double nk      = (double)((K + c.BK - 1) / c.BK);
                     const double step    = std::max({(double)(c.BM + c.BN) * c.BK / 44.0, (double)c.BM * c.BN * c.BK / 4096.0,
                                                      1000.0 * c.BK / 128.0});
                     const double fixed   = 6000.0 + (double)c.BM * c.BN / 4.4;
-                    const double cost    = per_cu * nk * step + std::ceil(per_cu / occ) * fixed;
-                    if (best < 0 || cost < best_cost || (cost == best_cost && c.lds_bytes > best_lds))
-                        best = i, best_cost = cost, best_lds = c.lds_bytes;
+                    for (int sl = 1; sl <= 8; sl *= 2)
+                    {
+                        if (sl > 1 && (no_splitk || conv_core || batch != 1 || K % (sl * c.BK) != 0 || K / sl < 1024))
+                            break;
+                        const double per_cu = std::ceil(tiles * sl / cus);
+                        const double finish = sl > 1 ? 4000.0 + (double)sl * M * N * 4.0 / (2.5 * cus) : 0.0;
+                        const double cost   = per_cu * (nk / sl) * step + std::ceil(per_cu / occ) * fixed + finish;
+                        if (best < 0 || cost < best_cost || (cost == best_cost && sl == 1 && c.lds_bytes > best_lds))
+                            best = i, best_cost = cost, best_lds = c.lds_bytes, splitk_plan = sl;
+                    }
                 }
                 return best;
             };
@@ -260,8 +272,20 @@ struct GemmCore
             const char *f1 = getenv("MI355_GEMM_CFG"), *f2 = getenv("MI355_DMA_CFG");
             if (f1 && atoi(f1) >= 0 && atoi(f1) < mfma_num_configs())
                 cfg_idx = atoi(f1);
-            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs() && Kp % dma_config(atoi(f2)).BK == 0)
-                dma_idx = atoi(f2);
+            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs() && Kp % dma_config(atoi(f2)).BK == 0 && dma_idx != atoi(f2))
+            {
+                // a forced tile shape: as many slices as fill the chip once, at least 1024 deep
+                dma_idx = atoi(f2), splitk_plan = 1;
+                const MfmaConfig c     = dma_config(dma_idx);
+                const int64_t    tiles = (int64_t)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN);
+                if (batch == 1 && !conv_core && tiles * 2 <= cus && K >= 2048 && !getenv("MI355_NO_SPLITK"))
+                {
+                    int sl = (int)std::min<int64_t>(std::min<int64_t>(cus / tiles, K / 1024), 8);
+                    while (sl > 1 && K % (sl * c.BK) != 0)
+                        --sl;
+                    splitk_plan = sl;
+                }
+            }
             if (getenv("MI355_NO_DMA") || K < 16)
                 dma_idx = -1;
             kname_mfma = mfma_config(cfg_idx).name;
@@ -320,20 +344,8 @@ struct GemmCore
         // offset is the batch stride of A and of the packed B alike), and a second kernel sums the planes and applies the
         // epilogue. Slices are whole k steps of the tile shape, so no slice but the matrix' own end has a tail.
         splitk = 1;
-        static const bool no_splitk = getenv("MI355_NO_SPLITK") != nullptr;
-        if (path == MI355_PATH_MFMA && dma_idx >= 0 && batch == 1 && !no_splitk && K >= 2048)
-        {
-            const MfmaConfig c     = dma_config(dma_idx);
-            const int64_t    tiles = (int64_t)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN);
-            const int        cus   = device_cus();
-            if (cus > 0 && tiles * 2 <= cus)
-            {
-                int sl = (int)std::min<int64_t>(std::min<int64_t>(cus / tiles, K / 1024), 8);
-                while (sl > 1 && K % (sl * c.BK) != 0)
-                    --sl;
-                splitk = sl;
-            }
-        }
+        if (path == MI355_PATH_MFMA && dma_idx >= 0 && batch == 1 && splitk_plan > 1 && K % (splitk_plan * dma_config(dma_idx).BK) == 0)
+            splitk = splitk_plan;
         if (splitk > 1)
         {
             const size_t ldp = ((size_t)N + 3) & ~(size_t)3;
@@ -1170,7 +1182,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         delete h;
         return fail("convolution too large");
     }
-    c.M = (int)M64, c.N = d.OFM, c.K = (int)K64, c.batch = 1;
+    c.M = (int)M64, c.N = d.OFM, c.K = (int)K64, c.batch = 1, c.conv_core = true;
     c.epi = f32 ? EPI_F32 : EPI_FIXEDPOINT, c.dst_dtype = d.dst_dtype;
     c.flip_a = d.src_dtype == MI355_U8, c.flip_b = d.weights_dtype == MI355_U8;
     c.a_offset = d.src_offset, c.b_offset = d.weights_offset;

@@ -440,7 +440,7 @@ def main():
             "note": "B rotated over 9 packed copies (405 MB) so reads come from HBM; kernel_us from graph replays "
                     "of the 9 rotating launches, eager_us from back-to-back host launches"}}
 
-        # the same weights with larger decode batches (not BASELINE configurations; B rotated the same way)
+        # the same weights with larger decode batches (not among the five benchmark configurations; B rotated the same way)
         out["secondary"]["decode_batches"] = {}
         for Mb in (16, 32, 64):
             Abh = np.random.default_rng(30 + Mb).integers(-128, 128, size=(Mb, K3), dtype=np.int8)
@@ -453,7 +453,7 @@ def main():
             for f in fg3:
                 f.close()
 
-        # two more decode shapes (not BASELINE configurations), B rotated over ROT packed copies like the legs above: a deep K
+        # two more decode shapes (not among the five benchmark configurations), B rotated over ROT packed copies like the legs above: a deep K
         # (the down projection of a feed-forward block: few rows, K = 11008) and a wide N (four column groups per compute
         # unit, where the fixed part of a launch weighs least)
         for leg, Md, Nd, Kd in (("decode_deep_k", 8, 4096, 11008), ("decode_wide_n", 8, 16384, 4096)):

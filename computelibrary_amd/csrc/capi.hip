@@ -642,6 +642,8 @@ struct mi355_conv_handle
     DevBuf          denseSrc, denseW, denseDst; // tensors that came with gaps, without them
     DevBuf          biasF;                   // F32 destination: the float bias
     bool            has_bias_f32 = false;
+    int             c_pad = 0;               // > 0: the kernels see this many channels (source and weights padded, see create)
+    DevBuf          padSrc, padW;
     PtrKind         kindSrc, kindDst; // host or device memory, per argument of run()
 };
 
@@ -1175,8 +1177,30 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     h->d = d;
     conv_geom(d, h->geom);
     GemmCore     &c  = h->core;
+    // A channel count that is not a multiple of 16 (the RGB of a first layer, 24, 40 ...): the implicit loaders move
+    // 16-byte pieces of one tap, and the fallback that looks up every byte runs at a few percent of what the bytes
+    // allow. With weights whose offset is zero in the kernels' signed form (QSYMM8, or QASYMM8 around 128) channels can
+    // be added for nothing: source pixels and weight taps are copied into buffers with the channels padded to the next
+    // multiple of 16, the added weights are zero in that form, so no sum changes - and neither does any offset term,
+    // all of which multiply sums over the weights. (With a weights offset the added source bytes would enter the row
+    // sums: that case keeps the fallback.)
+    {
+        const bool flip_b = d.weights_dtype == MI355_U8;
+        const int32_t b_eff = (int32_t)((uint32_t)d.weights_offset + (flip_b ? 128u : 0u));
+        static const bool no_cpad = getenv("MI355_NO_CHANNEL_PAD") != nullptr;
+        if (d.path == 0 && d.C % 16 != 0 && b_eff == 0 && !no_cpad)
+        {
+            mi355_conv_desc dp = d;
+            dp.C               = round_up(d.C, 16);
+            ConvGeom gp;
+            conv_geom(dp, gp);
+            if (conv_fast_div_ok(dp, gp) && (int64_t)d.batch * d.H * d.W * dp.C < ((int64_t)1 << 31))
+                h->c_pad = dp.C, h->geom = gp;
+        }
+    }
+    const int     c_eff = h->c_pad ? h->c_pad : d.C;
     const int64_t M64 = (int64_t)d.batch * h->geom.OH * h->geom.OW;
-    const int64_t K64 = (int64_t)d.KH * d.KW * d.C;
+    const int64_t K64 = (int64_t)d.KH * d.KW * c_eff;
     if (M64 > INT32_MAX || K64 > INT32_MAX)
     {
         delete h;
@@ -1201,7 +1225,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     // The patch matrix is only materialised on request (path 1) or where the loaders' reciprocal divisions would not be
     // exact. Channel counts that are not a multiple of 16 take the register-staged kernel, whose loader then looks up
     // every byte; a weights offset adds a pass over the source for the patches' row sums.
-    h->implicit      = d.path == 0 && conv_fast_div_ok(d, h->geom);
+    h->implicit      = d.path == 0 && (h->c_pad > 0 || conv_fast_div_ok(d, h->geom));
     h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
     if (h->implicit)
         c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
@@ -1247,6 +1271,13 @@ int mi355_conv_prepare(mi355_conv_handle *h, const void *weights, const void *bi
         HIP_TRY(transpose_bytes_launch(wd, h->nhwcW.p, c.N, h->d.C, h->d.KH * h->d.KW, s));
         wd = h->nhwcW.p;
     }
+    if (h->c_pad)
+    {
+        // taps of C weights -> taps of c_pad weights; the added ones are zero once the packing has put them in signed form
+        TRY(h->padW.ensure((size_t)c.N * c.K));
+        HIP_TRY(channel_pad_launch(wd, h->padW.p, (int64_t)c.N * h->d.KH * h->d.KW, h->d.C, h->c_pad, c.flip_b ? 0x80 : 0x00, s));
+        wd = h->padW.p;
+    }
     TRY(to_device(bias, sizeof(int32_t) * c.N, h->stageBias, s, &biasd));
     TRY(to_device(c.rq.per_channel ? mult : nullptr, sizeof(int32_t) * c.N, h->stageMult, s, &multd));
     TRY(to_device(c.rq.per_channel ? shift : nullptr, sizeof(int32_t) * c.N, h->stageShift, s, &shiftd));
@@ -1272,6 +1303,10 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
     TRY(check_requant(*requant, c.dst_dtype));
     if ((requant->per_channel != 0) != (c.rq.per_channel != 0))
         return fail("update cannot switch between per-tensor and per-channel requantisation");
+    if (h->c_pad && (int32_t)((uint32_t)weights_offset + (c.flip_b ? 128u : 0u)) != 0)
+        return fail("this handle pads %d channels to %d, which needs weights whose offset is zero in signed form (0 for "
+                    "QSYMM8 / QASYMM8_SIGNED, -128 for QASYMM8): create a new handle for the new weights offset",
+                    h->d.C, h->c_pad);
     h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
     c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
     h->implicit      = h->d.path == 0 && conv_fast_div_ok(h->d, h->geom);
@@ -1367,6 +1402,14 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         srcd = h->nhwcSrc.p;
         Dd   = h->nhwcDst.p;
     }
+    if (h->c_pad)
+    {
+        // pixels of C channels -> pixels of c_pad channels (what the added ones hold meets zero weights; the padding value
+        // keeps them in range of the source type)
+        TRY(h->padSrc.ensure((size_t)d.batch * d.H * d.W * h->c_pad));
+        HIP_TRY(channel_pad_launch(srcd, h->padSrc.p, (int64_t)d.batch * d.H * d.W, d.C, h->c_pad, (uint8_t)(d.pad_value & 0xFF), s));
+        srcd = h->padSrc.p;
+    }
     if (h->implicit)
     {
         GemmArgs g{};
@@ -1425,7 +1468,7 @@ void mi355_conv_destroy(mi355_conv_handle *h)
     h->stageSrc.release(), h->stageW.release(), h->stageDst.release(), h->stageBias.release();
     h->stageMult.release(), h->stageShift.release(), h->cols.release();
     h->nhwcSrc.release(), h->nhwcW.release(), h->nhwcDst.release(), h->biasF.release();
-    h->denseSrc.release(), h->denseW.release(), h->denseDst.release();
+    h->denseSrc.release(), h->denseW.release(), h->denseDst.release(), h->padSrc.release(), h->padW.release();
     delete h;
 }
 

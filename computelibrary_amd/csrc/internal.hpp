@@ -138,6 +138,8 @@ int output_stage_s16_launch(const int32_t *src, int64_t ld_src, const int32_t *b
 // [batch][R][C] bytes -> [batch][C][R]
 int transpose_bytes_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
 int transpose_words_launch(const void *src, void *dst, int batch, int R, int C, hipStream_t s);
+// `runs` runs of C bytes -> runs of Cp bytes (Cp a multiple of 16): the first C copied, the rest set to `fill`
+int channel_pad_launch(const void *src, void *dst, int64_t runs, int C, int Cp, uint8_t fill, hipStream_t s);
 // dst[s * dst_stride + c] = src[s * src_stride + c] for s < segments, c < seg (bytes)
 // dense F32 [batch][M][N] -> F16 destination (row stride ldh, batch stride, in elements), optionally added to its
 // previous contents in half arithmetic and clamped

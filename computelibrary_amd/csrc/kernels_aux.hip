@@ -780,4 +780,46 @@ int simple_gemm_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hi
         simple_gemm_kernel<EPI_F32><<<grid, block, 0, s>>>(args, f);
     return launch_status();
 }
+// ---- runs of C bytes -> runs of Cp >= C bytes (the first C copied, the rest set to `fill`): pixels of an NHWC image or
+// taps of OHWI weights whose channel count the 16-byte loaders cannot take, padded to the next multiple of 16. The
+// channels added meet weights that are zero in the kernels' signed form, so they change no sum. One thread per
+// 16 bytes of output.
+__global__ __launch_bounds__(256) void channel_pad_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t runs, int C,
+                                                          int Cp, uint32_t fill)
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const int     per = Cp / 16;
+    const int64_t t   = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= runs * per)
+        return;
+    const int64_t  r  = t / per;
+    const int      c0 = (int)(t - r * per) * 16;
+    const uint8_t *in = src + r * C + c0;
+    uint32_t       w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        w[q] = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+        {
+            const int c = c0 + q * 4 + b;
+            w[q] |= (uint32_t)(c < C ? in[q * 4 + b] : (uint8_t)fill) << (8 * b);
+        }
+    }
+    *(v4i *)(dst + r * Cp + c0) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+}
+int channel_pad_launch(const void *src, void *dst, int64_t runs, int C, int Cp, uint8_t fill, hipStream_t s)
+{
+    if (runs <= 0)
+        return 0;
+    if (C < 1 || Cp < C || Cp % 16 != 0 || ((uintptr_t)dst & 15) != 0)
+        return (int)hipErrorInvalidValue;
+    const int64_t n = runs * (Cp / 16);
+    if ((n + 255) / 256 > 0x7fffffff)
+        return (int)hipErrorInvalidValue;
+    channel_pad_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>((const uint8_t *)src, (uint8_t *)dst, runs, C, Cp, fill);
+    return launch_status();
+}
+
 } // namespace mi355

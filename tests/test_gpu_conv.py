@@ -169,9 +169,54 @@ def test_conv_few_output_channels_kernel():
             got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
 
 
+def test_conv_channel_counts_padded_to_16():
+    """A channel count that is not a multiple of 16 under weights whose offset is zero in signed form (QSYMM8, QASYMM8
+    around 128): pixels and taps are copied with the channels padded to the next multiple of 16 and the fast implicit
+    kernels run (never the byte-wise fallback), with identical results - the RGB of a first layer (7 x 7 stride 2, 3 x 3
+    stride 2), 1, 4, 8, 24 and 40 channels, few and many output channels, both source signs with non-zero source offsets
+    and padding values, asymmetric padding, dilation, both layouts, per-channel and per-tensor requantisation. A later
+    change to a weights offset that padding cannot take is refused."""
+    rng = np.random.default_rng(99)
+    cases = [
+        # (src shape, weights shape, stride, pad, dilation, src dtype, weights dtype / zero point, layout)
+        ((2, 30, 28, 3), (64, 7, 7, 3), (2, 2), (3, 3, 3, 3), (1, 1), np.uint8, 0, capi.NHWC),
+        ((1, 17, 19, 3), (32, 3, 3, 3), (2, 2), (1, 1, 1, 1), (1, 1), np.int8, 128, capi.NHWC),
+        ((2, 9, 9, 1), (5, 3, 3, 1), (1, 1), (1, 0, 1, 2), (1, 1), np.uint8, 0, capi.NHWC),
+        ((1, 12, 10, 4), (70, 5, 5, 4), (1, 2), (2, 2, 2, 2), (1, 1), np.int8, 0, capi.NCHW),
+        ((2, 8, 8, 8), (16, 3, 3, 8), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8, 128, capi.NHWC),
+        ((1, 14, 14, 24), (64, 3, 3, 24), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, 0, capi.NHWC),
+        ((3, 7, 7, 40), (120, 1, 1, 40), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, 0, capi.NCHW),
+    ]
+    for (shape, wshape, stride, pad, dil, dt, w_zp, layout) in cases:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w_dt = np.uint8 if w_zp else np.int8
+        w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        for per_channel in (True, False):
+            reals = rng.uniform(0.5, 2.0, wshape[0] if per_channel else 1) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert 0.1 < ((want > lo) & (want < hi)).mean()
+            announce("conv padded channels", shape, wshape, stride, pad, dil, dt.__name__, "w_zp", w_zp, "layout", layout, per_channel)
+            got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil, layout=layout)
+            assert name.startswith("implicit_") and "mfma" not in name, name
+            np.testing.assert_array_equal(got, want)
+    # a handle that pads refuses a weights offset that is not zero in signed form
+    cv = capi.Conv(capi.conv_desc(1, 6, 6, 3, 8, 3, 3, src_dtype=capi.S8, weights_dtype=capi.S8, dst_dtype=capi.S8,
+                                  rq=capi.requant(1 << 30, 1, 0, -128, 127)))
+    with pytest.raises(capi.Mi355Error, match="pads 3 channels to 16"):
+        cv.update_quant(0, 7, 0, capi.requant(1 << 30, 1, 0, -128, 127))
+    cv.update_quant(-3, 0, 3, capi.requant(1 << 30, 2, 1, -128, 127))
+    cv.close()
+
+
 def test_conv_weights_offset_and_odd_channels_on_the_fly():
     """QASYMM8 weights with a non-zero offset need the row sums of the patch matrix (a pass over the source, padding
-    included), channel counts that are not a multiple of 16 the byte-wise loader: neither materialises the patches.
+    included); channel counts that are not a multiple of 16 take the byte-wise loader when the weights offset rules out
+    padding the channels (otherwise the padded form above): neither materialises the patches.
     Few and many output channels (both kernels), unsigned and signed sources."""
     rng = np.random.default_rng(88)
     for (shape, wshape, stride, pad, dil, dt, w_zp) in [
@@ -405,14 +450,16 @@ def test_conv_random_geometry_sweep():
 def test_conv_with_f32_destination(device):
     """QASYMM8_SIGNED input and weights, F32 destination (src/cpu/operators/CpuGemmConv2d.cpp:297-305 of the reference):
     the same on-the-fly lowering as the 8-bit destination with the dequantising epilogue (few output channels: the
-    LDS-resident-weights kernel; 5 input channels: the byte-wise loader; a weights offset: row sums of the patches);
+    LDS-resident-weights kernel; 5 input channels under a weights offset: the byte-wise loader and row sums of the patches;
+    3 input channels under symmetric weights: channels padded to 16);
     checked against the oracle's im2col + F32 GEMM, identical bits"""
     import torch
     rng = np.random.default_rng(91)
     for (B_, H, W, C, OFM, KH, KW, stride, pad, in_zp, w_zp, act, twice) in [
             (2, 9, 8, 16, 24, 3, 3, (1, 1), (1, 1, 1, 1), 4, 0, (-np.inf, np.inf), False),
             (1, 7, 6, 5, 9, 3, 2, (2, 1), (0, 1, 1, 0), -3, 6, (0.0, np.inf), True),
-            (3, 5, 5, 32, 64, 1, 1, (1, 1), (0, 0, 0, 0), 0, 0, (0.0, 6.0), True)]:
+            (3, 5, 5, 32, 64, 1, 1, (1, 1), (0, 0, 0, 0), 0, 0, (0.0, 6.0), True),
+            (2, 8, 7, 3, 12, 3, 3, (1, 1), (1, 1, 1, 1), 5, 0, (-np.inf, np.inf), False)]:
         src = rng.integers(-128, 128, size=(B_, H, W, C), dtype=np.int8)
         w = rng.integers(-127, 128, size=(OFM, KH, KW, C), dtype=np.int8)
         bias = rng.normal(0.0, 2.0, size=OFM).astype(np.float32)

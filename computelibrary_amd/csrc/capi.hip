@@ -172,6 +172,7 @@ struct GemmCore
     int     splitk = 1;      // K slices of the pipelined kernel
     int     splitk_plan = 1; // what the cost model chose with the tile shape (create()); prepare() checks it and allocates
     bool    conv_core = false; // the GEMM inside a convolution handle: its implicit loader takes no K slices
+    int     k_const = 0;       // > 0: the K of the constant term a_offset * b_offset * K, where the kernels' K counts padded channels
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -365,7 +366,7 @@ struct GemmCore
         for (int b = 0; b < nb(); ++b)
             HIP_TRY(colvec_launch(colsum.as<int32_t>() + (size_t)b * Np,
                                   (has_bias && epi == EPI_FIXEDPOINT) ? bias.as<int32_t>() : nullptr, a_off_eff(),
-                                  b_off_eff(), K, N, colvec.as<int32_t>() + (size_t)b * Np, s));
+                                  b_off_eff(), k_const > 0 ? k_const : K, N, colvec.as<int32_t>() + (size_t)b * Np, s));
         return 0;
     }
 
@@ -643,6 +644,7 @@ struct mi355_conv_handle
     DevBuf          biasF;                   // F32 destination: the float bias
     bool            has_bias_f32 = false;
     int             c_pad = 0;               // > 0: the kernels see this many channels (source and weights padded, see create)
+    ConvGeom        geom_true;               // ... and the geometry with the caller's channel count, for the patches' row sums
     DevBuf          padSrc, padW;
     PtrKind         kindSrc, kindDst; // host or device memory, per argument of run()
 };
@@ -1179,22 +1181,21 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     GemmCore     &c  = h->core;
     // A channel count that is not a multiple of 16 (the RGB of a first layer, 24, 40 ...): the implicit loaders move
     // 16-byte pieces of one tap, and the fallback that looks up every byte runs at a few percent of what the bytes
-    // allow. With weights whose offset is zero in the kernels' signed form (QSYMM8, or QASYMM8 around 128) channels can
-    // be added for nothing: source pixels and weight taps are copied into buffers with the channels padded to the next
-    // multiple of 16, the added weights are zero in that form, so no sum changes - and neither does any offset term,
-    // all of which multiply sums over the weights. (With a weights offset the added source bytes would enter the row
-    // sums: that case keeps the fallback.)
+    // allow. Channels can be added for nothing: source pixels and weight taps are copied into buffers with the channels
+    // padded to the next multiple of 16, the added weights are zero in the kernels' signed form, so no dot product
+    // changes and neither do the column sums of the weights. The two other offset terms are kept on the caller's
+    // channel count: the row sums of the patches (needed under a weights offset) are taken from the unpadded source,
+    // and the constant a_offset * b_offset * K uses the unpadded K.
+    h->geom_true = h->geom;
     {
-        const bool flip_b = d.weights_dtype == MI355_U8;
-        const int32_t b_eff = (int32_t)((uint32_t)d.weights_offset + (flip_b ? 128u : 0u));
-        static const bool no_cpad = getenv("MI355_NO_CHANNEL_PAD") != nullptr;
-        if (d.path == 0 && d.C % 16 != 0 && b_eff == 0 && !no_cpad)
+        const bool no_cpad = getenv("MI355_NO_CHANNEL_PAD") != nullptr; // (read at every create: tests switch it)
+        if (d.path == 0 && d.C % 16 != 0 && !no_cpad)
         {
             mi355_conv_desc dp = d;
             dp.C               = round_up(d.C, 16);
             ConvGeom gp;
             conv_geom(dp, gp);
-            if (conv_fast_div_ok(dp, gp) && (int64_t)d.batch * d.H * d.W * dp.C < ((int64_t)1 << 31))
+            if (conv_fast_div_ok(dp, gp) && conv_fast_div_ok(d, h->geom) && (int64_t)d.batch * d.H * d.W * dp.C < ((int64_t)1 << 31))
                 h->c_pad = dp.C, h->geom = gp;
         }
     }
@@ -1207,6 +1208,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
         return fail("convolution too large");
     }
     c.M = (int)M64, c.N = d.OFM, c.K = (int)K64, c.batch = 1, c.conv_core = true;
+    c.k_const = h->c_pad ? d.KH * d.KW * d.C : 0;
     c.epi = f32 ? EPI_F32 : EPI_FIXEDPOINT, c.dst_dtype = d.dst_dtype;
     c.flip_a = d.src_dtype == MI355_U8, c.flip_b = d.weights_dtype == MI355_U8;
     c.a_offset = d.src_offset, c.b_offset = d.weights_offset;
@@ -1303,10 +1305,6 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
     TRY(check_requant(*requant, c.dst_dtype));
     if ((requant->per_channel != 0) != (c.rq.per_channel != 0))
         return fail("update cannot switch between per-tensor and per-channel requantisation");
-    if (h->c_pad && (int32_t)((uint32_t)weights_offset + (c.flip_b ? 128u : 0u)) != 0)
-        return fail("this handle pads %d channels to %d, which needs weights whose offset is zero in signed form (0 for "
-                    "QSYMM8 / QASYMM8_SIGNED, -128 for QASYMM8): create a new handle for the new weights offset",
-                    h->d.C, h->c_pad);
     h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
     c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
     h->implicit      = h->d.path == 0 && conv_fast_div_ok(h->d, h->geom);
@@ -1402,6 +1400,7 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         srcd = h->nhwcSrc.p;
         Dd   = h->nhwcDst.p;
     }
+    const void *src_true = srcd; // the caller's channel count
     if (h->c_pad)
     {
         // pixels of C channels -> pixels of c_pad channels (what the added ones hold meets zero weights; the padding value
@@ -1416,10 +1415,10 @@ int mi355_conv_run(mi355_conv_handle *h, const void *src, void *dst, void *strea
         c.fill_epi(g.epi, h->has_bias_f32 ? h->biasF.as<float>() : nullptr);
         if (c.b_off_eff() != 0)
         {
-            ConvGeom gr = h->geom;
+            ConvGeom gr = h->c_pad ? h->geom_true : h->geom;
             gr.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
             TRY(c.rowvec.ensure(sizeof(int32_t) * (size_t)c.M));
-            HIP_TRY(conv_rowsum_launch(srcd, gr, c.M, c.flip_a, c.b_off_eff(), c.rowvec.as<int32_t>(), s));
+            HIP_TRY(conv_rowsum_launch(h->c_pad ? src_true : srcd, gr, c.M, c.flip_a, c.b_off_eff(), c.rowvec.as<int32_t>(), s));
             g.epi.rowvec = c.rowvec.as<int32_t>();
         }
         g.A = (const int8_t *)srcd, g.lda = 0, g.a_batch_stride = 0;

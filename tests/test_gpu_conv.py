@@ -169,27 +169,30 @@ def test_conv_few_output_channels_kernel():
             got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
 
 
-def test_conv_channel_counts_padded_to_16():
-    """A channel count that is not a multiple of 16 under weights whose offset is zero in signed form (QSYMM8, QASYMM8
-    around 128): pixels and taps are copied with the channels padded to the next multiple of 16 and the fast implicit
-    kernels run (never the byte-wise fallback), with identical results - the RGB of a first layer (7 x 7 stride 2, 3 x 3
-    stride 2), 1, 4, 8, 24 and 40 channels, few and many output channels, both source signs with non-zero source offsets
-    and padding values, asymmetric padding, dilation, both layouts, per-channel and per-tensor requantisation. A later
-    change to a weights offset that padding cannot take is refused."""
+def test_conv_channel_counts_padded_to_16(monkeypatch):
+    """A channel count that is not a multiple of 16: pixels and taps are copied with the channels padded to the next
+    multiple of 16 and the fast implicit kernels run (never the byte-wise fallback), with identical results - the RGB of
+    a first layer (7 x 7 stride 2, 3 x 3 stride 2), 1, 4, 5, 8, 24 and 40 channels, few and many output channels, both
+    source signs with non-zero source offsets and padding values, symmetric weights and weights with an offset (the row
+    sums of the patches then come from the unpadded source and the constant term from the unpadded K), asymmetric
+    padding, dilation, both layouts, per-channel and per-tensor requantisation, a later change of both offsets. With the
+    padding switched off the byte-wise loader gives the same bits."""
     rng = np.random.default_rng(99)
     cases = [
-        # (src shape, weights shape, stride, pad, dilation, src dtype, weights dtype / zero point, layout)
-        ((2, 30, 28, 3), (64, 7, 7, 3), (2, 2), (3, 3, 3, 3), (1, 1), np.uint8, 0, capi.NHWC),
-        ((1, 17, 19, 3), (32, 3, 3, 3), (2, 2), (1, 1, 1, 1), (1, 1), np.int8, 128, capi.NHWC),
-        ((2, 9, 9, 1), (5, 3, 3, 1), (1, 1), (1, 0, 1, 2), (1, 1), np.uint8, 0, capi.NHWC),
-        ((1, 12, 10, 4), (70, 5, 5, 4), (1, 2), (2, 2, 2, 2), (1, 1), np.int8, 0, capi.NCHW),
-        ((2, 8, 8, 8), (16, 3, 3, 8), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8, 128, capi.NHWC),
-        ((1, 14, 14, 24), (64, 3, 3, 24), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, 0, capi.NHWC),
-        ((3, 7, 7, 40), (120, 1, 1, 40), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, 0, capi.NCHW),
+        # (src shape, weights shape, stride, pad, dilation, src dtype, weights dtype, weights zero point, layout)
+        ((2, 30, 28, 3), (64, 7, 7, 3), (2, 2), (3, 3, 3, 3), (1, 1), np.uint8, np.int8, 0, capi.NHWC),
+        ((1, 17, 19, 3), (32, 3, 3, 3), (2, 2), (1, 1, 1, 1), (1, 1), np.int8, np.uint8, 128, capi.NHWC),
+        ((2, 9, 9, 1), (5, 3, 3, 1), (1, 1), (1, 0, 1, 2), (1, 1), np.uint8, np.int8, 0, capi.NHWC),
+        ((1, 12, 10, 4), (70, 5, 5, 4), (1, 2), (2, 2, 2, 2), (1, 1), np.int8, np.int8, 0, capi.NCHW),
+        ((2, 8, 8, 8), (16, 3, 3, 8), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8, np.uint8, 128, capi.NHWC),
+        ((1, 14, 14, 24), (64, 3, 3, 24), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, np.int8, 0, capi.NHWC),
+        ((3, 7, 7, 40), (120, 1, 1, 40), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, np.int8, 0, capi.NCHW),
+        ((3, 6, 6, 5), (9, 1, 1, 5), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, np.uint8, 7, capi.NHWC),
+        ((2, 9, 8, 3), (20, 3, 3, 3), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, np.int8, -4, capi.NHWC),
+        ((1, 11, 9, 20), (70, 2, 3, 20), (1, 2), (0, 1, 1, 0), (2, 1), np.uint8, np.uint8, 131, capi.NCHW),
     ]
-    for (shape, wshape, stride, pad, dil, dt, w_zp, layout) in cases:
+    for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp, layout) in cases:
         src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
-        w_dt = np.uint8 if w_zp else np.int8
         w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
         bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
         K = wshape[1] * wshape[2] * wshape[3]
@@ -200,23 +203,52 @@ def test_conv_channel_counts_padded_to_16():
             mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
             want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
             assert 0.1 < ((want > lo) & (want < hi)).mean()
-            announce("conv padded channels", shape, wshape, stride, pad, dil, dt.__name__, "w_zp", w_zp, "layout", layout, per_channel)
+            announce("conv padded channels", shape, wshape, stride, pad, dil, dt.__name__, w_dt.__name__, "w_zp", w_zp, "layout", layout,
+                     per_channel)
             got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil, layout=layout)
             assert name.startswith("implicit_") and "mfma" not in name, name
             np.testing.assert_array_equal(got, want)
-    # a handle that pads refuses a weights offset that is not zero in signed form
-    cv = capi.Conv(capi.conv_desc(1, 6, 6, 3, 8, 3, 3, src_dtype=capi.S8, weights_dtype=capi.S8, dst_dtype=capi.S8,
-                                  rq=capi.requant(1 << 30, 1, 0, -128, 127)))
-    with pytest.raises(capi.Mi355Error, match="pads 3 channels to 16"):
-        cv.update_quant(0, 7, 0, capi.requant(1 << 30, 1, 0, -128, 127))
-    cv.update_quant(-3, 0, 3, capi.requant(1 << 30, 2, 1, -128, 127))
+    # the byte-wise loader instead: the same bits
+    monkeypatch.setenv("MI355_NO_CHANNEL_PAD", "1")
+    for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp, layout) in cases[:2] + cases[7:9]:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multiplier(float(40.0 / ((wshape[1] * wshape[2] * wshape[3]) ** 0.5 * 74.0 * 74.0)))
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil)
+        announce("conv byte-wise loader", shape, wshape)
+        got, name = run_conv(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil, layout=layout)
+        assert name.startswith("implicit_mfma"), name
+        np.testing.assert_array_equal(got, want)
+    monkeypatch.delenv("MI355_NO_CHANNEL_PAD")
+    # a handle that pads, after a change of both offsets and of the padding value
+    src = rng.integers(-128, 128, size=(2, 7, 6, 3), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(8, 3, 3, 3), dtype=np.int8)
+    bias = rng.integers(-500, 500, size=8, dtype=np.int32)
+    mult, shift = oracle.calculate_quantized_multiplier(float(40.0 / (27 ** 0.5 * 74.0 * 74.0)))
+    cv = capi.Conv(capi.conv_desc(2, 7, 6, 3, 8, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.S8, -2, 0, 2,
+                                  capi.requant(mult, shift, 1, -128, 127)))
+    sd, wd, od = to_dev(src), to_dev(w), to_dev(np.zeros((2, 7, 6, 8), np.int8))
+    keep = to_dev(bias)
+    cv.prepare(wd, keep)
+    for (in_zp, w_zp) in ((2, 0), (-6, 9)):
+        if w_zp:
+            cv.update_quant(-in_zp, -w_zp, in_zp, capi.requant(mult, shift, 1, -128, 127))
+        cv.run(sd, od)
+        import torch
+        torch.cuda.synchronize()
+        announce("conv padded channels, offsets", in_zp, w_zp, cv.kernel_name)
+        np.testing.assert_array_equal(od.cpu().numpy(), oracle.conv_nhwc_direct(src, w, bias, in_zp, w_zp, [mult], [shift], 1, -128, 127,
+                                                                                  (1, 1), (1, 1, 1, 1), (1, 1)))
     cv.close()
 
 
 def test_conv_weights_offset_and_odd_channels_on_the_fly():
     """QASYMM8 weights with a non-zero offset need the row sums of the patch matrix (a pass over the source, padding
-    included); channel counts that are not a multiple of 16 take the byte-wise loader when the weights offset rules out
-    padding the channels (otherwise the padded form above): neither materialises the patches.
+    included); channel counts that are not a multiple of 16 run with their channels padded (the test above): neither
+    materialises the patches.
     Few and many output channels (both kernels), unsigned and signed sources."""
     rng = np.random.default_rng(88)
     for (shape, wshape, stride, pad, dil, dt, w_zp) in [

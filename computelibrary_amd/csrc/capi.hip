@@ -325,12 +325,13 @@ struct GemmCore
                 HIP_TRY(pack_b_skinny_launch(Bp.as<int8_t>() + (size_t)b * Np * Kp, Kp, Np, Bs.as<int8_t>() + (size_t)b * Np * Kp, s));
         }
         // few output columns and a short K: the image of the B panel the narrow kernel copies into LDS
-        has_narrow = path == MI355_PATH_MFMA && nb() == 1 && N <= 64 && narrow_panel_chunks(K) > 0;
+        has_narrow = path == MI355_PATH_MFMA && nb() == 1 && (N <= 64 || (N <= 256 && K <= 192)) && narrow_panel_chunks(K) > 0;
         if (has_narrow)
         {
             const int chunks = narrow_panel_chunks(K);
-            TRY(Bn.ensure((size_t)64 * (chunks + 1) * 16));
-            HIP_TRY(pack_b_narrow_launch(Bp.as<int8_t>(), Kp, Np, chunks, Bn.as<int8_t>(), s));
+            const int rows = round_up(N, 64); // panels of 64 columns (Np, a multiple of 256, covers them)
+            TRY(Bn.ensure((size_t)rows * (chunks + 1) * 16));
+            HIP_TRY(pack_b_narrow_launch(Bp.as<int8_t>(), Kp, Np, chunks, rows, Bn.as<int8_t>(), s));
         }
         TRY(fill.ensure(16));
         HIP_TRY(fill_i32_launch(fill.as<int32_t>(), (int32_t)(0x01010101u * fill_byte), 4, s));

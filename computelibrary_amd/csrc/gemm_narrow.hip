@@ -1,4 +1,6 @@
-// K5: implicit-GEMM convolution (and dense GEMM) with few output columns: N <= 64, K <= 1152.
+// K5: implicit-GEMM convolution (and dense GEMM) with few output columns: N <= 64, K <= 1152 - or, with K <= 192, up to
+// 256 columns as 2 to 4 panels of 64 (a 1 x 1 convolution that widens few channels: the patch of a wave stays in its
+// registers and goes against one panel after the other, every panel with its own epilogue).
 //
 // CpuGemmConv2d lowers a convolution with 64 output channels to a GEMM with M = batch * OH * OW rows and 64 columns
 // (src/cpu/operators/CpuGemmConv2d.cpp:923-1008); the work per output tile is then so small (K = KH * KW * C) that a
@@ -55,6 +57,8 @@ constexpr int NARROW_WAVES  = 4;
 constexpr int NARROW_ROWS   = 32;  // per wave
 constexpr int NARROW_BN     = 64;
 constexpr int NARROW_MAX_NB = 6;   // batches of 3 k blocks of 64: K <= 1152
+constexpr int NARROW_MAX_PANELS = 4; // panels of 64 columns with one batch (K <= 192): N <= 256 (8 panels fill LDS with one
+                                     // workgroup's weights and measured slower than the tiled kernel)
 
 // UNI: C % 64 == 0 - a k block of 64 lies inside one tap, so the tap of a load is decoded with scalar arithmetic
 template <int EPI, bool FLIP_A, bool CONV, bool UNI, int NB>
@@ -65,8 +69,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     constexpr int KBLK  = NB * 3;         // k blocks the loop covers (the B panel is zero beyond K)
     constexpr int PITCH = KBLK * 64 + 16; // bytes per B row in LDS
     constexpr int NPAR  = 1 + QP_COUNT;
-    extern __shared__ __attribute__((aligned(16))) char smem[]; // B panel [64][PITCH], then par[NPAR][64]
-    int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
+    extern __shared__ __attribute__((aligned(16))) char smem[]; // B panel [npan * 64][PITCH], then par[NPAR][npan * 64]
 
     // Everything the main part uses is fetched here in one batch of scalar loads and pinned in registers (left alone, the
     // compiler fetches kernel arguments where they are first used: a round trip to memory each time). Pointers go
@@ -78,11 +81,16 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     uint32_t  a_bytes = (uint32_t)(g.a_end - g.A); // bytes of A: what the range check of the A loads compares with
     int32_t   a_M = g.M, a_K = g.K, a_lda = (int32_t)g.lda, a_kp = (int32_t)g.Kp, a_qps = (int32_t)g.epi.qp_stride;
     int32_t   tail_start = g.tiles_m, tail_waves = g.tiles_n; // see narrow_launch
+    int32_t   a_npan = g.nblocks;                             // panels of 64 columns (more than one only with NB == 1)
     asm volatile(""
                  : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x), "+s"(cg.stride_y),
                    "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word), "+s"(cg.magic_C),
                    "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(cg.magic_OH), "+s"(a_M), "+s"(a_K), "+s"(a_lda), "+s"(a_kp),
-                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl), "+s"(a_bytes), "+s"(tail_start), "+s"(tail_waves));
+                   "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp), "+s"(u_fl), "+s"(a_bytes), "+s"(tail_start), "+s"(tail_waves),
+                   "+s"(a_npan));
+    const int npan = NB == 1 ? a_npan : 1; // (a constant for the deeper forms: their code does not change)
+    const int BNT  = npan * NARROW_BN;     // columns in LDS
+    int32_t  *par  = (int32_t *)(smem + BNT * PITCH);
     const MI355_GLOBAL int8_t *const gB = (const MI355_GLOBAL int8_t *)u_b;
     // raw buffer over A (stride 0, 32-bit elements untyped): loads at or past a_bytes - also "negative" offsets, which
     // are huge as unsigned - return zero
@@ -102,18 +110,33 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 
     // the epilogue's per-column constants (column term + the digested requantisation vectors), where they exist: 6 x 64
     // dwords, one or two per thread, fetched first and parked in LDS with the B panel
-    const bool have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
-    int32_t    tp[2]   = {0, 0};
+    const bool    have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
+    constexpr int TPN     = NB == 1 ? (NPAR * NARROW_BN * NARROW_MAX_PANELS + NARROW_WAVES * 64 - 1) / (NARROW_WAVES * 64) : 2; // dwords per thread
+    int32_t       tp[TPN];
+#pragma unroll
+    for (int i = 0; i < TPN; ++i)
+        tp[i] = 0;
     if (have_qp)
     {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < TPN; ++i)
         {
-            const int idx = min(tid + i * NARROW_WAVES * 64, NPAR * NARROW_BN - 1);
-            const int v = idx / NARROW_BN, col = idx - v * NARROW_BN;
+            if (NB == 1 && i * NARROW_WAVES * 64 >= NPAR * BNT) // (wave-uniform)
+                break;
+            const int idx = min(tid + i * NARROW_WAVES * 64, NPAR * BNT - 1);
+            const int v = idx / BNT, col = idx - v * BNT;
             tp[i]       = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
         }
     }
+    auto park_constants = [&]()
+    {
+        if (!have_qp)
+            return;
+#pragma unroll
+        for (int i = 0; i < TPN; ++i)
+            if (tid + i * NARROW_WAVES * 64 < NPAR * BNT)
+                par[tid + i * NARROW_WAVES * 64] = tp[i];
+    };
     int qflag = 1;
     if (have_qp && u_fl != 0)
         qflag = *(const MI355_GLOBAL int32_t *)u_fl;
@@ -125,29 +148,28 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     constexpr int  NDMA   = CHUNKS + 1;     // 64 rows x (CHUNKS + 1) pieces / 64 pieces per transfer
     constexpr int  DPW    = (NDMA + NARROW_WAVES - 1) / NARROW_WAVES;
     const uint32_t lds0   = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
-    int            my_dma = 0; // transfers this wave issues (wave-uniform)
-#pragma unroll
-    for (int i = 0; i < DPW; ++i)
+    if (NB == 1)
     {
-        const int ins = wave + i * NARROW_WAVES;
-        if (ins < NDMA)
-        {
+        // (any number of panels: a loop)
+        for (int ins = wave; ins < npan * NDMA; ins += NARROW_WAVES)
             narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
-            ++my_dma;
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < DPW; ++i)
+        {
+            const int ins = wave + i * NARROW_WAVES;
+            if (ins < NDMA)
+                narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
         }
     }
-    (void)my_dma;
 
     if (!active)
     {
         // this wave's share of the B panel and of the constants, then out
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (have_qp)
-        {
-            par[tid] = tp[0];
-            if (tid < NPAR * NARROW_BN - NARROW_WAVES * 64)
-                par[tid + NARROW_WAVES * 64] = tp[1];
-        }
+        park_constants();
         __syncthreads();
         return;
     }
@@ -251,22 +273,10 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * 3 * RS) : "memory");
     else
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * RS) : "memory");
-    if (have_qp)
-    {
-        par[tid] = tp[0];
-        if (tid < NPAR * NARROW_BN - NARROW_WAVES * 64)
-            par[tid + NARROW_WAVES * 64] = tp[1];
-    }
+    park_constants();
     qflag           = __builtin_amdgcn_readfirstlane(qflag);
     const bool fast = have_qp && (qflag & 1) == 0;
     __syncthreads();
-
-    v4i acc[RS][QS];
-#pragma unroll
-    for (int i = 0; i < RS; ++i)
-#pragma unroll
-        for (int j = 0; j < QS; ++j)
-            acc[i][j] = (v4i){0, 0, 0, 0};
 
     // The waves of a SIMD would otherwise share the matrix pipe evenly, finish together and then all queue for the vector
     // ALU with their epilogues: different priorities let one wave at a time through the matrix instructions, and its
@@ -279,13 +289,28 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
     case 2: __builtin_amdgcn_s_setprio(1); break;
     default: break;
     }
-    const char *b_rd = smem + lr * PITCH + lh * 16; // + q * 16 * PITCH + kb * 64
+    // one panel of 64 columns after the other against the same patch (more than one panel: NB == 1, the whole patch is
+    // in fa[0]); every panel has its own accumulators and epilogue
+    for (int np = 0; np < npan; ++np)
+    {
+    const int col0 = np * NARROW_BN;
+    v4i       acc[RS][QS];
+#pragma unroll
+    for (int i = 0; i < RS; ++i)
+#pragma unroll
+        for (int j = 0; j < QS; ++j)
+            acc[i][j] = (v4i){0, 0, 0, 0};
+    const char *b_rd = smem + (col0 + lr) * PITCH + lh * 16; // + q * 16 * PITCH + kb * 64
 #pragma unroll
     for (int b = 0; b < NB; ++b)
     {
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk)
         {
+            // (a single batch that K does not fill, K = 64 or 128 under many columns: the k blocks past K hold zeros in
+            // the panel - skip them, every panel would multiply them again)
+            if (NB == 1 && kk > 0 && kk * 64 >= a_K)
+                continue;
             v4i fb[QS];
 #pragma unroll
             for (int q = 0; q < QS; ++q)
@@ -332,14 +357,14 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
         {
             const int i = row0 + rb * 16 + lr;
             rv[rb]      = (rowvec && i < a_M) ? rowvec[i] : 0;
-            drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + 4 * lh;
+            drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + col0 + 4 * lh;
         }
 #pragma unroll
         for (int q = 0; q < QS; ++q)
         {
             const int c  = q * 16 + 4 * lh;
-            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * NARROW_BN + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * NARROW_BN + c);
-            const v4i cv = *(const v4i *)(par + c);
+            const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * BNT + col0 + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * BNT + col0 + c);
+            const v4i cv = *(const v4i *)(par + col0 + c);
 #pragma unroll
             for (int rb = 0; rb < RS; ++rb)
             {
@@ -354,15 +379,16 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
                 }
                 const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)o[1], (uint32_t)o[0], 0x0c0c0400u);
                 const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)o[3], (uint32_t)o[2], 0x0c0c0400u);
-                if (row0 + rb * 16 + lr < a_M && c < a_N)
+                if (row0 + rb * 16 + lr < a_M && col0 + c < a_N)
                     *(uint32_t *)(drow[rb] + q * 16) = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
             }
         }
     }
-    else if (fast)
+    else if (fast && npan == 1)
         epilogue_store_fast<RS, QS, NARROW_BN>(acc, g, par, row0, 0, 0, lane, 0);
     else
-        epilogue_store_t<EPI, RS, QS>(acc, g, row0, 0, lane, 0);
+        epilogue_store_t<EPI, RS, QS>(acc, g, row0, col0, lane, 0);
+    }
 #undef MI355_GLOBAL
 }
 
@@ -402,7 +428,9 @@ int narrow_panel_chunks(int K)
 
 bool narrow_applies(const GemmArgs &a, bool conv)
 {
-    if (a.N < 1 || a.N > NARROW_BN || a.K < 16 || a.K > NARROW_MAX_NB * 192 || a.K > a.Kp || a.Kp % 64 != 0 || a.M < 1)
+    if (a.N < 1 || a.N > NARROW_MAX_PANELS * NARROW_BN || a.K < 16 || a.K > NARROW_MAX_NB * 192 || a.K > a.Kp || a.Kp % 64 != 0 || a.M < 1)
+        return false;
+    if (a.N > NARROW_BN && a.K > 192) // several panels only while the whole patch stays in registers
         return false;
     if (conv)
     {
@@ -426,10 +454,11 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
                                               : narrow_fn_e<EPI_F32>(flip_a, conv, uni, nb);
     if (fn == nullptr)
         return (int)hipErrorInvalidValue;
-    const size_t lds = (size_t)NARROW_BN * (nb * 192 + 16) + (size_t)(1 + QP_COUNT) * NARROW_BN * sizeof(int32_t);
+    const int    npan = (args.N + NARROW_BN - 1) / NARROW_BN;
+    const size_t lds  = (size_t)npan * NARROW_BN * (nb * 192 + 16) + (size_t)(1 + QP_COUNT) * npan * NARROW_BN * sizeof(int32_t);
     if (lds > 48 * 1024)
     {
-        // once per kernel and device
+        // once per kernel and device (for the largest panel count the kernel may meet)
         static std::atomic<uint32_t> raised[3][2][2][2][NARROW_MAX_NB];
         std::atomic<uint32_t>       &done = raised[epi][flip_a ? 1 : 0][conv ? 1 : 0][uni ? 1 : 0][nb - 1];
         int                          dev  = 0;
@@ -437,13 +466,15 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
             return (int)hipErrorInvalidDevice;
         if ((done.load(std::memory_order_acquire) & (1u << dev)) == 0)
         {
-            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            const size_t most = nb == 1 ? (size_t)NARROW_MAX_PANELS * NARROW_BN * (192 + 16 + (1 + QP_COUNT) * sizeof(int32_t)) : lds;
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
             if (e != hipSuccess)
                 return (int)e;
             done.fetch_or(1u << dev, std::memory_order_release);
         }
     }
     GemmArgs a = args;
+    a.nblocks  = npan;
     // what the A loads' range check compares with
     if (conv)
     {

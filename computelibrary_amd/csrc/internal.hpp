@@ -117,7 +117,7 @@ int pack_bt_launch(const void *Bt, int64_t ldk, int K, int N, int Kp, int Np, bo
 // Bp [Np][Kp] -> operand order for the skinny kernel: [Np/16][Kp/64][64 lanes][16 bytes]
 int pack_b_skinny_launch(const int8_t *Bp, int Kp, int Np, int8_t *Bs, hipStream_t s);
 // rows 0..63 of Bp -> [64][chunks + 1] pieces of 16 bytes (the last one padding), zero beyond Kp
-int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int8_t *Bn, hipStream_t s);
+int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int rows, int8_t *Bn, hipStream_t s);
 // colvec[j] = a_off*colsum[j] + a_off*b_off*K (+ bias[j])
 int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int32_t b_off, int K, int N,
                   int32_t *colvec, hipStream_t s);

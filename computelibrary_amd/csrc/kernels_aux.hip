@@ -289,13 +289,13 @@ int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int
     return launch_status();
 }
 
-// The first 64 rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus one piece of
+// The first `rows` (a multiple of 64) rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus one piece of
 // padding, zero beyond Kp - the workgroups copy this image into LDS with plain linear transfers
-__global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__restrict__ Bp, int Kp, int chunks,
+__global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__restrict__ Bp, int Kp, int chunks, int rows,
                                                             int8_t *__restrict__ Bn)
 {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= 64 * (chunks + 1))
+    if (idx >= rows * (chunks + 1))
         return;
     const int r = idx / (chunks + 1), c = idx - r * (chunks + 1);
     v4i       v = {0, 0, 0, 0};
@@ -304,11 +304,11 @@ __global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__rest
     *(v4i *)(Bn + (int64_t)idx * 16) = v;
 }
 
-int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int8_t *Bn, hipStream_t s)
+int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int rows, int8_t *Bn, hipStream_t s)
 {
-    if (Kp % 16 || Np < 64 || chunks < 1)
+    if (Kp % 16 || rows < 64 || rows % 64 != 0 || Np < rows || chunks < 1)
         return (int)hipErrorInvalidValue;
-    pack_b_narrow_kernel<<<dim3((64 * (chunks + 1) + 255) / 256), dim3(256), 0, s>>>(Bp, Kp, chunks, Bn);
+    pack_b_narrow_kernel<<<dim3((rows * (chunks + 1) + 255) / 256), dim3(256), 0, s>>>(Bp, Kp, chunks, rows, Bn);
     return launch_status();
 }
 

@@ -119,8 +119,8 @@ def test_conv_few_output_channels_kernel():
     weights in LDS and reads the patches straight into the matrix cores' operand layout: 1 to 6 batches of 3 k blocks
     (K from 16 to 1152, with a last batch that is partly or mostly empty), C = 16 / 32 / 48 (a k block spans several
     taps) and 64 / 128 (one tap per k block), unsigned sources (flipped in the loader, non-zero padding value), strides,
-    dilation, asymmetric padding, ragged channel counts, and row counts that do not fill the last workgroup. Above
-    those limits the tiled kernels take over."""
+    dilation, asymmetric padding, ragged channel counts, and row counts that do not fill the last workgroup; with K <= 192
+    also 65 to 256 output channels as several panels of 64. Above those limits the tiled kernels take over."""
     rng = np.random.default_rng(77)
     cases = [
         # (src shape, weights shape, stride, pad, dilation, dtype)
@@ -137,6 +137,12 @@ def test_conv_few_output_channels_kernel():
         # workgroups, the very last of them ragged (33708 = 256 * 128 + 14 * 64 + 32 + 12 rows; 33800 rows, 7 columns)
         ((3, 106, 106, 16), (64, 1, 1, 16), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),
         ((2, 130, 130, 16), (7, 3, 3, 16), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8),
+        # K <= 192 and up to 256 output channels: 2 to 4 panels of 64 columns against the patch a wave keeps in registers
+        ((2, 20, 20, 64), (256, 1, 1, 64), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),     # 4 panels, K = 64
+        ((1, 15, 14, 32), (96, 1, 1, 32), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8),     # 2 panels, the second half empty
+        ((2, 9, 8, 16), (65, 3, 3, 16), (1, 1), (1, 1, 1, 1), (1, 1), np.uint8),       # K = 144, 65 columns: one in the second panel
+        ((1, 12, 12, 128), (130, 1, 1, 128), (2, 2), (0, 0, 0, 0), (1, 1), np.int8),   # K = 128, 3 panels, stride 2, N % 4 != 0
+        ((1, 10, 10, 192), (200, 1, 1, 192), (1, 1), (0, 0, 0, 0), (1, 1), np.int8),   # K = 192, the most one batch holds
     ]
     for (shape, wshape, stride, pad, dil, dt) in cases:
         src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)

@@ -382,6 +382,11 @@ def test_pipelined_kernel_with_k_slices():
             biasf = rng.normal(0.0, 1.0, size=N).astype(np.float32)
             got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, path=capi.PATH_MFMA, device=True)
             np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4).view(np.uint32))
+            prevf = rng.normal(0.0, 3.0, size=(M, N)).astype(np.float32)
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, bias_f32=biasf, act=(0.0, 6.0), path=capi.PATH_MFMA,
+                              device=True, prev=prevf, flags=capi.GEMM_ACCUMULATE)
+            np.testing.assert_array_equal(got.view(np.uint32),
+                                          oracle.gemmlowp_f32(A, B, biasf, ao, bo, 3e-4, 0.0, 6.0, prev=prevf).view(np.uint32))
 
 
 @pytest.mark.parametrize("M", [1, 8, 9, 16])

@@ -140,6 +140,28 @@ struct PanelProducer
         }
     }
 
+    // The same for a dense tile that lies inside the matrix (no row of it beyond M) and a K step that lies inside K:
+    // nothing to decide per load, so the loads go out back to back. (The general form below spends three branches and a
+    // dozen scalar instructions on every load; with 12 loads per producer wave and K step that was most of the step.)
+    __device__ __forceinline__ void issue_inside(int kt, int slot) const
+    {
+        static_assert(!CONV, "dense tiles only");
+        const uint32_t base = lds0 + (uint32_t)slot * STAGE;
+        const int8_t  *a_k  = a_base + (int64_t)kt * BK;
+        const int8_t  *b_k  = b_base + (int64_t)kt * BK;
+        static_assert(AU % NP == 0, "which panel a load belongs to must not depend on the wave");
+#pragma unroll
+        for (int i = 0; i < LPP; ++i)
+        {
+            const int      u   = pw + i * NP; // wave-uniform
+            const uint32_t dst = base + (uint32_t)u * 1024u;
+            if (i >= AU / NP)
+                dma16s(b_k + (int64_t)(u - AU) * RPU * Kp, lane_b, dst);
+            else
+                dma16s(a_k + (int64_t)u * RPU * lda, lane_a, dst);
+        }
+    }
+
     // K step kt of the tile into ring slot `slot`: loads [I0, I1) of this wave's LPP
     template <int I0 = 0, int I1 = LPP>
     __device__ __forceinline__ void issue(int kt, int slot) const
@@ -545,6 +567,299 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     MI355_PHASE(4); // consumer: epilogue done (stores issued)
 }
 
+// The 256 x 128 x 128 tile of a dense GEMM in another division of labour: 4 consumer waves, one per SIMD, in a 2 x 2
+// arrangement (wave tile 128 x 64: 8 + 4 operand blocks per 64 of K for 32 matrix instructions, a quarter fewer LDS reads
+// than 64 x 64 wave tiles), and 4 producer waves, one per SIMD, that issue every direct-to-LDS load of the block.
+// A consumer multiplies one half of a K step (64 deep) out of one register set while the operand reads of the next half
+// land in the other set; the reads are interleaved with the first matrix instructions of the half, one read behind each
+// instruction, so that after the workgroup barrier - which lets all waves go in the same clock - no wave queues its
+// reads in front of its matrix instructions (issued as a block, the reads of all waves kept the matrix pipes empty for
+// about 250 clocks per barrier). ONE barrier per K step, in the middle of the step: it opens stage kt+1 to its readers and
+// hands the ring slot of stage kt-1 to the producers. Measured against the 8 + 4 wave form above on 2048 x 4096 x 4096:
+// 1190 instead of 1640 clocks per K step.
+template <int BM, int BN, int BK, int NS, int EPI, bool FLIP_A>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
+{
+    GemmArgs g = g_in;
+    asm volatile(""
+                 : "+s"(g.tiles_m), "+s"(g.tiles_n), "+s"(g.magic_tiles), "+s"(g.magic_group), "+s"(g.tile_magic_ok), "+s"(g.lda),
+                   "+s"(g.a_batch_stride), "+s"(g.Kp), "+s"(g.bp_batch_stride), "+s"(g.M), "+s"(g.N), "+s"(g.K),
+                   "+s"(g.epi.qp_stride), "+s"(g.epi.colvec_batch_stride), "+s"(g.nblocks));
+    typedef const __attribute__((address_space(1))) int32_t *global_i32;
+    uintptr_t u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp, u_fl = (uintptr_t)g.epi.qp_flag;
+    asm volatile("" : "+s"(u_cv), "+s"(u_qp), "+s"(u_fl));
+
+    constexpr int NW = 4, NP = 4, NALL = NW + NP;
+    constexpr int CPR = BK / 16, RPU = 1024 / BK;
+    constexpr int AU = BM / RPU, BU = BN / RPU;
+    constexpr int LPP = (AU + BU) / NP;   // loads per producer wave per stage
+    constexpr int LPW = (AU + BU) / NALL; // loads per wave per start-up stage (all 8 waves issue those)
+    constexpr int TM = BM / 2, TN = BN / 2;
+    constexpr int RS = TM / 16, QS = TN / 16;
+    constexpr int NM = RS * QS, NR = RS + QS; // matrix instructions / operand reads per half step
+    constexpr int STAGE = (BM + BN) * BK;
+    static_assert(BK == 128, "a K step is two halves of 64");
+    static_assert((AU + BU) % NALL == 0 && (NS - 1) * LPW < 64 && (NS - 2) * LPP < 64 && NS >= 3, "staging shape");
+    static_assert(NW * 16 * (QS * 64 + 16) <= NS * STAGE, "the 32-bit epilogue stages through the ring's memory");
+    static_assert(NM >= NR, "one operand read behind each of the first matrix instructions");
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef MI355_PHASE_CLOCKS
+    const int phase_blk = blockIdx.x == 0 ? 0 : ((int)blockIdx.x == g.nblocks / 2 ? 1 : ((int)blockIdx.x == g.nblocks - 1 ? 2 : -1));
+    const int phase_row = phase_blk < 0 ? -1 : (wave == 0 ? phase_blk * 2 : (wave == NW ? phase_blk * 2 + 1 : -1));
+    MI355_PHASE(0);
+#endif
+    int tm, tn, bz;
+    if (g.tile_magic_ok)
+        tile_coords_batched_fast(blockIdx.x, g.nblocks, g.tiles_m, g.tiles_n, g.magic_tiles, g.magic_group, bz, tm, tn);
+    else
+        tile_coords_batched(blockIdx.x, g.nblocks, g.tiles_m, g.tiles_n, bz, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int nk = (g.K + BK - 1) / BK;
+    const bool inside = m0 + BM <= g.M; // no row of this tile lies beyond the matrix
+    int qflag = 1;
+    if (EPI == EPI_FIXEDPOINT && u_fl != 0)
+        qflag = *(const __attribute__((address_space(4))) int32_t *)u_fl;
+    const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
+
+    // per-column epilogue constants: fetched by the consumer waves before their share of the start-up loads
+    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
+    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
+    int32_t       par_reg[PPT > 0 ? PPT : 1];
+    if (fast && wave < NW)
+    {
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            const int idx = tid + t * NW * 64;
+            par_reg[t]    = 0;
+            if (idx < NPAR * BN)
+            {
+                const int par = idx / BN, col = idx % BN;
+                par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
+                                         : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
+            }
+        }
+    }
+    {
+        // the first NS-1 stages: unit u to wave u % 8, stage 0 first
+        PanelProducer<BM, BN, BK, NALL, NS, false> first;
+        first.init(g, m0, n0, bz, wave, lane, lds0);
+#pragma unroll
+        for (int s = 0; s < NS - 1; ++s)
+            if (s < nk)
+            {
+                if (inside && (s + 1) * BK <= g.K)
+                    first.issue_inside(s, s % NS);
+                else
+                    first.issue(s, s % NS);
+            }
+    }
+
+    // Barriers: barrier 0 opens stage 0; barrier kt+1 sits in the middle of K step kt, after every wave's reads of the
+    // first half of stage kt were issued ... and completed long before (their data fed the instructions in front of the
+    // barrier); it opens stage kt+1 and frees the ring slot of stage kt-1, whose last reads fed matrix instructions that
+    // every consumer issued before barrier kt. Every wave executes nk + 2 barriers (+ those of the epilogue).
+    if (wave >= NW)
+    {
+        PanelProducer<BM, BN, BK, NP, NS, false> prod;
+        prod.init(g, m0, n0, bz, wave - NW, lane, lds0);
+        MI355_PHASE(1);
+        MI355_PHASE(2);
+        if (nk >= NS - 1)
+            wait_vmcnt<(NS - 2) * LPW>();
+        else
+            wait_vmcnt<0>();
+        MI355_PHASE(3);
+        block_barrier(); // barrier 0
+        // stage kt+NS-1 goes into the slot of stage kt-1: free since barrier kt. A loop of its own for the steps that
+        // need no decisions (tile inside the matrix, K step inside K): sharing a loop with the general form, the loads
+        // of this one sat between reloads of spilled scalars, and the 12 loads of a producer are the longest chain of a
+        // K step.
+        int kt = 0;
+        if (inside)
+        {
+            const int n_lean = g.K / BK - NS + 1; // steps kt whose stage kt+NS-1 is a whole K step
+            for (; kt < n_lean; ++kt)
+            {
+                prod.issue_inside(kt + NS - 1, (kt + NS - 1) % NS);
+                wait_vmcnt<(NS - 2) * LPP>(); // this wave's part of stage kt+1 has landed
+                block_barrier();              // barrier kt+1
+            }
+        }
+        for (; kt < nk; ++kt)
+        {
+            if (kt + NS - 1 < nk)
+            {
+                prod.issue(kt + NS - 1, (kt + NS - 1) % NS);
+                wait_vmcnt<(NS - 2) * LPP>();
+            }
+            else
+                wait_vmcnt<0>();
+            block_barrier(); // barrier kt+1
+        }
+        block_barrier(); // barrier nk+1: every consumer is past its last operand read
+        MI355_PHASE(4);
+        if (fast)
+        {
+            __syncthreads(); // the consumers' staging of the epilogue constants
+            if (g.epi.vec_store16)
+                __syncthreads(); // ... and of the output tile
+        }
+        return;
+    }
+
+    // ================= consumers =================
+    const int row_w = (wave >> 1) * TM, col_w = (wave & 1) * TN;
+    v4i       acc[RS][QS];
+#pragma unroll
+    for (int i = 0; i < RS; ++i)
+#pragma unroll
+        for (int j = 0; j < QS; ++j)
+            acc[i][j] = (v4i){0, 0, 0, 0};
+    // operand read offsets inside a stage, for the two halves of a K step: lane -> (row lane%16, 16-byte column lane/16)
+    const int lr = lane & 15, lh = lane >> 4;
+    int       a_rd[2][RS], b_rd[2][QS];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+    {
+#pragma unroll
+        for (int f = 0; f < RS; ++f)
+        {
+            const int row = row_w + f * 16 + lr;
+            a_rd[kk][f]   = row * BK + (((kk * 4 + lh) ^ swz<CPR>(row)) << 4);
+        }
+#pragma unroll
+        for (int f = 0; f < QS; ++f)
+        {
+            const int row = col_w + f * 16 + lr;
+            b_rd[kk][f]   = BM * BK + row * BK + (((kk * 4 + lh) ^ swz<CPR>(row)) << 4);
+        }
+    }
+    MI355_PHASE(1);
+    if (nk >= NS - 1)
+        wait_vmcnt<(NS - 2) * LPW>(); // this wave's units of stage 0 (and the epilogue constants before them)
+    else
+        wait_vmcnt<0>();
+    block_barrier(); // barrier 0: stage 0 is in LDS
+    MI355_PHASE(2);
+    v4i fa0[RS], fb0[QS], fa1[RS], fb1[QS];
+#pragma unroll
+    for (int f = 0; f < RS; ++f)
+        fa0[f] = *(const v4i *)(smem + a_rd[0][f]);
+#pragma unroll
+    for (int f = 0; f < QS; ++f)
+        fb0[f] = *(const v4i *)(smem + b_rd[0][f]);
+    for (int kt = 0; kt < nk; ++kt)
+    {
+        const char *s  = smem + (kt % NS) * STAGE;
+        const char *s2 = smem + ((kt + 1) % NS) * STAGE; // beyond the last step: whatever the slot holds, never used
+        // ---- first half of step kt; the operands of its second half arrive meanwhile ----
+#pragma unroll
+        for (int f = 0; f < RS; ++f)
+            fa1[f] = *(const v4i *)(s + a_rd[1][f]);
+#pragma unroll
+        for (int f = 0; f < QS; ++f)
+            fb1[f] = *(const v4i *)(s + b_rd[1][f]);
+        if (FLIP_A)
+        {
+#pragma unroll
+            for (int f = 0; f < RS; ++f)
+                fa0[f] ^= (int)0x80808080;
+        }
+#pragma unroll
+        for (int i = 0; i < RS; ++i)
+#pragma unroll
+            for (int j = 0; j < QS; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb0[j], fa0[i], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one matrix instruction
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // the reads above (second half of stage kt) were issued a dozen matrix instructions ago; they must have left the
+        // LDS before the barrier after this one hands their slot to the producers - waiting here costs nothing
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); // (vmcnt: this wave's share of the start-up stages)
+        block_barrier(); // barrier kt+1: stage kt+1 is in LDS
+        // ---- second half of step kt; the operands of the first half of step kt+1 arrive meanwhile ----
+#pragma unroll
+        for (int f = 0; f < RS; ++f)
+            fa0[f] = *(const v4i *)(s2 + a_rd[0][f]);
+#pragma unroll
+        for (int f = 0; f < QS; ++f)
+            fb0[f] = *(const v4i *)(s2 + b_rd[0][f]);
+        if (FLIP_A)
+        {
+#pragma unroll
+            for (int f = 0; f < RS; ++f)
+                fa1[f] ^= (int)0x80808080;
+        }
+#pragma unroll
+        for (int i = 0; i < RS; ++i)
+#pragma unroll
+            for (int j = 0; j < QS; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb1[j], fa1[i], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // the reads issued in the last half step (into fa0 / fb0) are never used, but like every other wave's last operand
+    // reads they must have left the LDS before the epilogue writes there
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    block_barrier(); // barrier nk+1
+    MI355_PHASE(3);
+
+    if (fast)
+    {
+        int32_t *par = (int32_t *)smem;
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            const int idx = tid + t * NW * 64;
+            if (idx < NPAR * BN)
+                par[idx] = par_reg[t];
+        }
+        __syncthreads();
+        if (EPI == EPI_FIXEDPOINT)
+        {
+            char      *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
+            const bool rowv  = g.epi.rowvec != nullptr;
+            if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0 && !rowv)
+                epilogue_store_staged<true, false, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                       [] { __syncthreads(); });
+            else if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0)
+                epilogue_store_staged<true, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                      [] { __syncthreads(); });
+            else if (g.epi.vec_store16)
+                epilogue_store_staged<false, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
+                                                                       [] { __syncthreads(); });
+            else
+                epilogue_store_fast<RS, QS, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+        }
+    }
+    else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store && !g.epi.accumulate)
+    {
+        if constexpr (EPI != EPI_FIXEDPOINT)
+            epilogue_store_wave32<EPI, RS, QS>(acc, g, smem + wave * 16 * (QS * 64 + 16), m0 + row_w, n0 + col_w, lane, bz);
+    }
+    else
+        epilogue_store_t<EPI, RS, QS>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
+    MI355_PHASE(4);
+}
+
 // ---- instantiation table -------------------------------------------------------------------------------------------
 struct DmaEntry
 {
@@ -552,6 +867,7 @@ struct DmaEntry
     int         threads;
     int         lds_bytes;
     const void *fn[3][2][2]; // [epi][flip][conv]
+    int         threads_dense = 0; // workgroup size of the dense (non-convolution) kernels when it differs
 };
 
 #define MI355_DFN(BM, BN, BK, WM, WN, NS, E, F, C) (const void *)gemm_dma_kernel<BM, BN, BK, WM, WN, NS, E, F, C>
@@ -568,8 +884,23 @@ struct DmaEntry
         }                                                                                                            \
     }
 
+#define MI355_WFN(BM, BN, BK, NS, E, F) (const void *)gemm_wide_kernel<BM, BN, BK, NS, E, F>
+// dense: the 4 + 4 wave kernel; convolution: the 8 + 4 wave kernel
+#define MI355_WCFG(NAME, BM, BN, BK, WM, WN, NS)                                                                     \
+    {                                                                                                                \
+        {NAME, BM, BN, BK}, WM *WN * 192, NS * (BM + BN) * BK,                                                        \
+        {                                                                                                            \
+            {{MI355_WFN(BM, BN, BK, NS, 0, false), nullptr}, {MI355_WFN(BM, BN, BK, NS, 0, true), nullptr}},          \
+                {{MI355_WFN(BM, BN, BK, NS, 1, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, true)},            \
+                 {MI355_WFN(BM, BN, BK, NS, 1, true), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, true)}},             \
+                {{MI355_WFN(BM, BN, BK, NS, 2, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, true)},            \
+                 {MI355_WFN(BM, BN, BK, NS, 2, true), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, true, true)}},             \
+        },                                                                                                           \
+            512                                                                                                      \
+    }
+
 static const DmaEntry g_dma[] = {
-    MI355_DCFG("pp_256x128x128_s3", 256, 128, 128, 2, 2, 3),
+    MI355_WCFG("pp_256x128x128_s3", 256, 128, 128, 2, 2, 3),
     MI355_DCFG("pp_128x128x128_s3", 128, 128, 128, 2, 2, 3),
     MI355_DCFG("pp_128x64x128_s3", 128, 64, 128, 2, 2, 3),
     MI355_DCFG("pp_64x64x128_s3", 64, 64, 128, 1, 2, 3),
@@ -634,7 +965,7 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     a.magic_group = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_group) + 1u : 0u;
     a.nblocks     = (int32_t)nblocks;
     void    *kargs[] = {&a};
-    dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block(c.threads);
+    dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block((!conv && c.threads_dense) ? c.threads_dense : c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);
 }
 } // namespace mi355

@@ -23,9 +23,21 @@ sys.path.insert(0, ROOT)
 
 INT8_DENSE_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix rate (5.0 POP/s)
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
-# HBM-side bytes of one launch of the config-2 kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the
-# same counters read for a plain copy (profiles/gemm_kernels_hbm_traffic_and_lds_counters.txt holds the runs)
-CFG2_MEASURED_TRAFFIC_BYTES = int((33131.3 * (262144.0 / 131086.8) + 8192.0) * 1024)  # 76.2 MB: 67.8 read + 8.4 written
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_kernels_hbm_traffic_and_lds_counters.txt")
+
+
+def cfg2_measured_traffic_bytes():
+    """HBM-side bytes of one launch of the config-2 kernel: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the
+    same counters read for a plain copy. Not measured by this run: it is read from the tracked summary of the counter
+    runs (its line `config2_traffic_bytes_per_launch: N`); None when that file is not there."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("config2_traffic_bytes_per_launch:"):
+                    return int(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def quantized_multipliers(scales):
@@ -222,8 +234,8 @@ def run_phase_clocks(torch, capi, args):
     import ctypes
     from computelibrary_amd import build as _build
     if not os.path.exists(_build.PHASES_LIB):
-        print("%s is missing: run `python -m computelibrary_amd.build`" % _build.PHASES_LIB, file=sys.stderr)
-        sys.exit(2)
+        print("building %s (only this mode uses it)" % _build.PHASES_LIB, file=sys.stderr)
+        _build.build_phases(verbose=False)
     capi.LIB_PATH = _build.PHASES_LIB  # before the first call into the library
     stream = torch.cuda.current_stream().cuda_stream
     M, N, K = 2048, 4096, 4096
@@ -353,7 +365,8 @@ def main():
         "config": {"workload": "gemmlowp s8 x per-channel s8 -> s8, M=2048 N=4096 K=4096, fused offset + "
                                "FIXEDPOINT requant", "kernel": g.kernel_name, "prepare_ms": round(prepare_ms, 3)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_DENSE_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved / INT8_DENSE_PEAK_TOPS, 4), "traffic": CFG2_MEASURED_TRAFFIC_BYTES,
+                     "frac": round(achieved / INT8_DENSE_PEAK_TOPS, 4), "traffic": cfg2_measured_traffic_bytes(),
+                     "traffic_source": "profiles/gemm_kernels_hbm_traffic_and_lds_counters.txt (rocprofv3 --pmc runs, not this run)",
                      "kernel_us": round(kern_s * 1e6, 3), "eager_us": round(evt / args.steps * 1e6, 3)},
     }
     if clock_mhz:
@@ -410,7 +423,7 @@ def main():
                 st["i"] += 1
 
             steps3 = max(args.steps, 10 * ROT) // ROT * ROT
-            _, evt_rot = time_launches(torch, rotated, steps3, args.warmup // ROT * ROT)
+            _, evt_rot = time_launches(torch, rotated, steps3, max(ROT, -(-args.warmup // ROT) * ROT))  # whole rotations, at least one
             graph_s = time_graph(torch, [(lambda cs, h=h: h.run(Ab, Db, None, cs)) for h in hs], steps3)
             # the last launch of either loop used the last handle: bias/multipliers are not rolled, only B's columns
             ok = None

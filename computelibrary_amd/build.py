@@ -1,6 +1,7 @@
 """Builds libmi355gemmlowp.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-    python -m computelibrary_amd.build            # rebuild everything
+    python -m computelibrary_amd.build            # the product library and the measurement-only kernels
+    python -m computelibrary_amd.build --phases   # also the instrumented build for `bench.py --phase-clocks`
 The shared library lands in computelibrary_amd/lib/ (git-ignored; it travels with the tree to the GPU box).
 """
 import os
@@ -37,24 +38,40 @@ def _compile(src, extra=(), suffix=""):
     return obj
 
 
+def _link(lib, members, verbose):
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + members
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stdout)
+    if verbose:
+        print("built", lib)
+
+
 def build(verbose=True):
+    """The product library and the measurement-only kernels (a library of their own)."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        objs = list(ex.map(_compile, SOURCES + CEILINGS_SOURCES))
+    _link(LIB, objs[:len(SOURCES)], verbose)
+    _link(CEILINGS_LIB, objs[len(SOURCES):], verbose)
+    return LIB
+
+
+def build_phases(verbose=True):
+    """The instrumented build `bench.py --phase-clocks` runs on: only made when that is asked for."""
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=4) as ex:
         phases = ex.submit(_compile, "gemm_dma.hip", ("-DMI355_PHASE_CLOCKS",), "_phases")
-        objs = list(ex.map(_compile, SOURCES + CEILINGS_SOURCES))
-        phases_obj = phases.result()
-    phases_members = [phases_obj if os.path.basename(o) == "gemm_dma.o" else o for o in objs[:len(SOURCES)]]
-    for lib, members in ((LIB, objs[:len(SOURCES)]), (CEILINGS_LIB, objs[len(SOURCES):]), (PHASES_LIB, phases_members)):
-        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + members
-        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("link failed:\n" + r.stdout)
-        if verbose:
-            print("built", lib)
-    return LIB
+        objs = list(ex.map(_compile, [x for x in SOURCES if x != "gemm_dma.hip"]))
+        objs.append(phases.result())
+    _link(PHASES_LIB, objs, verbose)
+    return PHASES_LIB
 
 
 if __name__ == "__main__":
     build()
+    if "--phases" in sys.argv[1:]:
+        build_phases()
     sys.exit(0)

@@ -11,6 +11,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355gemmlowp.so")
 U8, S8, S32, F32, S16, F16 = 0, 1, 2, 3, 4, 5
 EPI_S32, EPI_FIXEDPOINT, EPI_F32 = 0, 1, 2
 PATH_AUTO, PATH_SIMPLE, PATH_MFMA, PATH_SKINNY = 0, 1, 2, 3
+PATH_TILE = 16  # + n: the pipelined kernel's n-th tile configuration
+CONV_AUTO, CONV_EXPLICIT, CONV_IN_PLACE = 0, 1, 2
 GEMM_ACCUMULATE, GEMM_ACT_TWICE = 1, 2
 NHWC, NCHW = 0, 1
 

@@ -162,6 +162,7 @@ struct GemmCore
     float   scale = 1.f, act_min = -INFINITY, act_max = INFINITY;
     bool    accumulate = false, act_twice = false;
     int     path = MI355_PATH_AUTO, cfg_idx = 0, dma_idx = -1;
+    int     force_tile = -1; // >= 0: the pipelined kernel's tile configuration the caller asked for (MI355_PATH_TILE + n)
     int     Kp = 0, Np = 0;
     bool    b_shared = true; // one B for all batches
     bool    has_bias = false, has_pc = false, prepared = false;
@@ -175,9 +176,23 @@ struct GemmCore
     int     k_const = 0;       // > 0: the K of the constant term a_offset * b_offset * K, where the kernels' K counts padded channels
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
+    // The names a run can report, composed when the choice is made (create, prepare, update): a run only points at one
+    // of them - it must not touch the host heap
+    std::string        kname_narrow, kname_dma_full, kname_splitk, kname_mfma_full;
+    const char        *kname_static = nullptr; // the streaming kernel names its forms itself
+    const std::string *kname_run = nullptr; // what the last run took (nullptr: no run yet, kname is what create announced)
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
     void   *ext_ws = nullptr; // set around a run that must not allocate: see run_dense
     size_t  ext_ws_bytes = 0;
+
+    void refresh_names()
+    {
+        kname_narrow    = kprefix + "narrow_32x64";
+        kname_dma_full  = kprefix + kname_dma;
+        kname_splitk    = kname_dma_full + "_splitk" + std::to_string(splitk);
+        kname_mfma_full = kprefix + kname_mfma;
+    }
+    const char *name() const { return kname_static ? kname_static : (kname_run ? kname_run->c_str() : kname.c_str()); }
 
     int32_t a_off_eff() const { return (int32_t)((uint32_t)a_offset + (flip_a ? 128u : 0u)); }
     int32_t b_off_eff() const { return (int32_t)((uint32_t)b_offset + (flip_b ? 128u : 0u)); }
@@ -193,6 +208,14 @@ struct GemmCore
     {
         Kp = round_up(K, PACK_K_ALIGN);
         Np = round_up(N, PACK_N_ALIGN);
+        if (path >= MI355_PATH_TILE)
+        {
+            if (path - MI355_PATH_TILE >= dma_num_configs())
+                return fail("path %d names tile configuration %d; there are %d", path, path - MI355_PATH_TILE, dma_num_configs());
+            force_tile = path - MI355_PATH_TILE, path = MI355_PATH_MFMA;
+        }
+        else if (path < 0 || path > MI355_PATH_SKINNY)
+            return fail("unknown path %d", path);
         if (path == MI355_PATH_AUTO)
             // measured: up to 32 rows the streaming kernel always wins; up to 64 rows only while N is small enough
             // that the pipelined kernel would leave most compute units without a tile
@@ -207,7 +230,7 @@ struct GemmCore
         if (path == MI355_PATH_SIMPLE)
             kname = "simple";
         else if (path == MI355_PATH_SKINNY)
-            kname = "skinny_16xN_splitk";
+            kname = "skinny";
         else
         {
             const int cus = num_cus();
@@ -242,7 +265,6 @@ struct GemmCore
             {
                 int    best = -1, best_lds = 0;
                 double best_cost = 0;
-                static const bool no_splitk = getenv("MI355_NO_SPLITK") != nullptr;
                 for (int i = 0; i < dma_num_configs(); ++i)
                 {
                     const MfmaConfig c = dma_config(i);
@@ -257,7 +279,7 @@ struct GemmCore
                     const double fixed   = 6000.0 + (double)c.BM * c.BN / 4.4;
                     for (int sl = 1; sl <= 8; sl *= 2)
                     {
-                        if (sl > 1 && (no_splitk || conv_core || batch != 1 || K % (sl * c.BK) != 0 || K / sl < 1024))
+                        if (sl > 1 && (conv_core || batch != 1 || K % (sl * c.BK) != 0 || K / sl < 1024))
                             break;
                         const double per_cu = std::ceil(tiles * sl / cus);
                         const double finish = sl > 1 ? 4000.0 + (double)sl * M * N * 4.0 / (2.5 * cus) : 0.0;
@@ -270,16 +292,13 @@ struct GemmCore
             };
             cfg_idx = pick(mfma_num_configs(), mfma_config, nullptr);
             dma_idx = pick_dma();
-            const char *f1 = getenv("MI355_GEMM_CFG"), *f2 = getenv("MI355_DMA_CFG");
-            if (f1 && atoi(f1) >= 0 && atoi(f1) < mfma_num_configs())
-                cfg_idx = atoi(f1);
-            if (f2 && atoi(f2) >= 0 && atoi(f2) < dma_num_configs() && Kp % dma_config(atoi(f2)).BK == 0 && dma_idx != atoi(f2))
+            if (force_tile >= 0 && Kp % dma_config(force_tile).BK == 0 && dma_idx != force_tile)
             {
-                // a forced tile shape: as many slices as fill the chip once, at least 1024 deep
-                dma_idx = atoi(f2), splitk_plan = 1;
+                // a tile shape named by the caller: as many slices as fill the chip once, at least 1024 deep
+                dma_idx = force_tile, splitk_plan = 1;
                 const MfmaConfig c     = dma_config(dma_idx);
                 const int64_t    tiles = (int64_t)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN);
-                if (batch == 1 && !conv_core && tiles * 2 <= cus && K >= 2048 && !getenv("MI355_NO_SPLITK"))
+                if (batch == 1 && !conv_core && tiles * 2 <= cus && K >= 2048)
                 {
                     int sl = (int)std::min<int64_t>(std::min<int64_t>(cus / tiles, K / 1024), 8);
                     while (sl > 1 && K % (sl * c.BK) != 0)
@@ -287,12 +306,13 @@ struct GemmCore
                     splitk_plan = sl;
                 }
             }
-            if (getenv("MI355_NO_DMA") || K < 16)
+            if (K < 16)
                 dma_idx = -1;
             kname_mfma = mfma_config(cfg_idx).name;
             kname_dma  = dma_idx >= 0 ? dma_config(dma_idx).name : "";
             kname      = dma_idx >= 0 ? kname_dma : kname_mfma;
         }
+        refresh_names();
         return 0;
     }
 
@@ -357,6 +377,7 @@ struct GemmCore
         }
         TRY(refresh_colvec(s));
         TRY(refresh_qparams(s));
+        refresh_names();
         prepared = true;
         return 0;
     }
@@ -511,7 +532,7 @@ struct GemmCore
                 gb.epi.colvec += (int64_t)b * g.epi.colvec_batch_stride;
                 if (g.epi.rowvec != zeros.as<int32_t>() && g.epi.rowvec != nullptr)
                     gb.epi.rowvec += (int64_t)b * g.epi.rowvec_batch_stride;
-                HIP_TRY(skinny_launch(epi, flip_in_loader, gb, s));
+                HIP_TRY(skinny_launch(epi, flip_in_loader, gb, s, &kname_static));
             }
         }
         else
@@ -527,11 +548,10 @@ struct GemmCore
                                             g.conv.H * g.conv.W * g.conv.C
                                       : (int64_t)g.lda * 256 + g.K;
             // few output columns and a short K: every wave for itself, weights resident in LDS (gemm_narrow.hip)
-            static const bool no_narrow = getenv("MI355_NO_NARROW") != nullptr;
-            if (!no_narrow && has_narrow && batch == 1 && conv && !g.epi.accumulate && span < ((int64_t)1 << 31) &&
+            if (has_narrow && batch == 1 && conv && !g.epi.accumulate && span < ((int64_t)1 << 31) &&
                 narrow_applies(g, conv))
             {
-                kname           = kprefix + "narrow_32x64";
+                kname_run       = &kname_narrow;
                 g.Bp            = Bn.as<int8_t>();
                 g.conv.pad_word = 0x01010101u * fill_byte; // as in the image: the kernel flips what it loads
                 HIP_TRY(narrow_launch(epi, flip_in_loader, conv, g, s));
@@ -541,7 +561,7 @@ struct GemmCore
                 const MfmaConfig c = dma_config(dma_idx);
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;
                 g.tiles_n          = (g.N + c.BN - 1) / c.BN;
-                kname              = kprefix + kname_dma;
+                kname_run          = &kname_dma_full;
                 if (splitk > 1 && !conv && batch == 1 && g.K == K && K % (splitk * c.BK) == 0)
                 {
                     const int     ldp = (N + 3) & ~3;
@@ -553,7 +573,7 @@ struct GemmCore
                     gp.epi.vec_store           = 1;
                     gp.D = parts.as<int32_t>(), gp.ldd = ldp, gp.d_batch_stride = (int64_t)M * ldp;
                     gp.K = (int)kc, gp.a_batch_stride = kc, gp.bp_batch_stride = kc;
-                    kname += "_splitk" + std::to_string(splitk);
+                    kname_run = &kname_splitk;
                     HIP_TRY(dma_launch(dma_idx, EPI_S32, flip_in_loader, false, gp, splitk, s));
                     HIP_TRY(splitk_finish_launch(epi, g, parts.as<int32_t>(), (int64_t)M * ldp, ldp, splitk, s));
                     return 0;
@@ -565,7 +585,7 @@ struct GemmCore
                 const MfmaConfig c = mfma_config(cfg_idx);
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;
                 g.tiles_n          = (g.N + c.BN - 1) / c.BN;
-                kname              = kprefix + kname_mfma;
+                kname_run          = &kname_mfma_full;
                 if (conv)
                     g.conv.pad_word = (0x01010101u * fill_byte) ^ (flip_in_loader ? 0x80808080u : 0u);
                 HIP_TRY(mfma_launch(cfg_idx, epi, flip_in_loader, conv, g, batch, s));
@@ -985,7 +1005,7 @@ void mi355_gemmlowp_destroy(mi355_gemm_handle *h)
 
 const char *mi355_gemmlowp_kernel_name(const mi355_gemm_handle *h)
 {
-    return h ? h->core.kname.c_str() : "";
+    return h ? h->core.name() : "";
 }
 
 int mi355_output_stage_run(const mi355_output_stage_desc *desc, const int32_t *src, const int32_t *bias, void *dst,
@@ -1152,6 +1172,8 @@ static int conv_check(const mi355_conv_desc &d)
         if ((d.flags & ~MI355_GEMM_ACT_TWICE) != 0)
             return fail("unknown flag bits 0x%x", d.flags);
     }
+    if (d.path < MI355_CONV_AUTO || d.path > MI355_CONV_IN_PLACE)
+        return fail("unknown convolution path %d", d.path);
     if (d.layout != MI355_NHWC && d.layout != MI355_NCHW)
         return fail("unknown layout %d", d.layout);
     ConvGeom g;
@@ -1189,8 +1211,7 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     // and the constant a_offset * b_offset * K uses the unpadded K.
     h->geom_true = h->geom;
     {
-        const bool no_cpad = getenv("MI355_NO_CHANNEL_PAD") != nullptr; // (read at every create: tests switch it)
-        if (d.path == 0 && d.C % 16 != 0 && !no_cpad)
+        if (d.path == MI355_CONV_AUTO && d.C % 16 != 0)
         {
             mi355_conv_desc dp = d;
             dp.C               = round_up(d.C, 16);
@@ -1228,12 +1249,13 @@ int mi355_conv_create(const mi355_conv_desc *desc, mi355_conv_handle **out)
     // The patch matrix is only materialised on request (path 1) or where the loaders' reciprocal divisions would not be
     // exact. Channel counts that are not a multiple of 16 take the register-staged kernel, whose loader then looks up
     // every byte; a weights offset adds a pass over the source for the patches' row sums.
-    h->implicit      = d.path == 0 && (h->c_pad > 0 || conv_fast_div_ok(d, h->geom));
+    h->implicit      = d.path != MI355_CONV_EXPLICIT && (h->c_pad > 0 || conv_fast_div_ok(d, h->geom));
     h->geom.pad_word = ((uint32_t)d.pad_value & 0xFFu) * 0x01010101u;
     if (h->implicit)
         c.fill_byte = (uint8_t)(d.pad_value & 0xFF);
     c.kprefix = h->implicit ? "implicit_" : "im2col+";
     c.kname   = c.kprefix + c.kname;
+    c.refresh_names();
     *out                = h;
     return 0;
 }
@@ -1308,10 +1330,11 @@ int mi355_conv_update_quant(mi355_conv_handle *h, int32_t src_offset, int32_t we
         return fail("update cannot switch between per-tensor and per-channel requantisation");
     h->d.src_offset = src_offset, h->d.weights_offset = weights_offset, h->d.pad_value = pad_value, h->d.requant = *requant;
     c.a_offset = src_offset, c.b_offset = weights_offset, c.rq = *requant;
-    h->implicit      = h->d.path == 0 && conv_fast_div_ok(h->d, h->geom);
+    h->implicit      = h->d.path != MI355_CONV_EXPLICIT && (h->c_pad > 0 || conv_fast_div_ok(h->d, h->geom));
     h->geom.pad_word = ((uint32_t)pad_value & 0xFFu) * 0x01010101u;
     c.fill_byte      = (uint8_t)(pad_value & 0xFF);
     c.kprefix        = h->implicit ? "implicit_" : "im2col+";
+    c.refresh_names();
     if (!c.prepared)
         return 0;
     if (c.rq.per_channel)
@@ -1474,7 +1497,7 @@ void mi355_conv_destroy(mi355_conv_handle *h)
 
 const char *mi355_conv_kernel_name(const mi355_conv_handle *h)
 {
-    return h ? h->core.kname.c_str() : "";
+    return h ? h->core.name() : "";
 }
 
 int mi355_im2col_nhwc_run(const mi355_conv_desc *desc, const void *src, void *dst, void *stream)

@@ -622,32 +622,14 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = (g.K + BK - 1) / BK;
     const bool inside = m0 + BM <= g.M; // no row of this tile lies beyond the matrix
+    // which requantisation formula applies was decided on the device when the per-column constants were digested; the
+    // word is asked for here and looked at after the first loads have gone out
     int qflag = 1;
     if (EPI == EPI_FIXEDPOINT && u_fl != 0)
         qflag = *(const __attribute__((address_space(4))) int32_t *)u_fl;
-    const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
-
-    // per-column epilogue constants: fetched by the consumer waves before their share of the start-up loads
-    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
-    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
-    int32_t       par_reg[PPT > 0 ? PPT : 1];
-    if (fast && wave < NW)
     {
-#pragma unroll
-        for (int t = 0; t < PPT; ++t)
-        {
-            const int idx = tid + t * NW * 64;
-            par_reg[t]    = 0;
-            if (idx < NPAR * BN)
-            {
-                const int par = idx / BN, col = idx % BN;
-                par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
-                                         : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
-            }
-        }
-    }
-    {
-        // the first NS-1 stages: unit u to wave u % 8, stage 0 first
+        // The first NS-1 stages before anything else - every clock before the first load goes out is a clock in which
+        // the whole chip waits for memory: unit u to wave u % 8, stage 0 first
         PanelProducer<BM, BN, BK, NALL, NS, false> first;
         first.init(g, m0, n0, bz, wave, lane, lds0);
 #pragma unroll
@@ -659,6 +641,26 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
                 else
                     first.issue(s, s % NS);
             }
+    }
+    const bool fast = EPI == EPI_FIXEDPOINT && (qflag & 1) == 0;
+
+    // per-column epilogue constants: fetched by the consumer waves behind their share of the start-up loads, parked in
+    // registers, staged in LDS after the loop
+    constexpr int NPAR = (EPI == EPI_FIXEDPOINT) ? 1 + QP_COUNT : 0;
+    constexpr int PPT  = (NPAR * BN + NW * 64 - 1) / (NW * 64);
+    static_assert((NS - 2) * LPW + PPT < 64, "vmcnt range");
+    int32_t       par_reg[PPT > 0 ? PPT : 1];
+    if (fast && wave < NW)
+    {
+#pragma unroll
+        for (int t = 0; t < PPT; ++t)
+        {
+            // (every lane loads: the count of loads in flight must not depend on the lane)
+            const int idx = min(tid + t * NW * 64, NPAR * BN - 1);
+            const int par = idx / BN, col = idx % BN;
+            par_reg[t]    = par == 0 ? ((global_i32)u_cv)[(int64_t)bz * g.epi.colvec_batch_stride + n0 + col]
+                                     : ((global_i32)u_qp)[(int64_t)(par - 1) * g.epi.qp_stride + n0 + col];
+        }
     }
 
     // Barriers: barrier 0 opens stage 0; barrier kt+1 sits in the middle of K step kt, after every wave's reads of the
@@ -742,10 +744,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
         }
     }
     MI355_PHASE(1);
-    if (nk >= NS - 1)
-        wait_vmcnt<(NS - 2) * LPW>(); // this wave's units of stage 0 (and the epilogue constants before them)
-    else
+    // this wave's units of stage 0: behind them, stage 1 and the epilogue constants may still be in flight
+    if (nk < NS - 1)
         wait_vmcnt<0>();
+    else if (fast)
+        wait_vmcnt<(NS - 2) * LPW + PPT>();
+    else
+        wait_vmcnt<(NS - 2) * LPW>();
     block_barrier(); // barrier 0: stage 0 is in LDS
     MI355_PHASE(2);
     v4i fa0[RS], fb0[QS], fa1[RS], fb1[QS];

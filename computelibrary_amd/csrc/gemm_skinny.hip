@@ -1041,25 +1041,6 @@ static int skinny_once_launch_v(int epi, bool flip_a, const GemmArgs &a, int gri
                      : skinny_once_launch_r<PER, MULTI, 8>(epi, flip_a, a, grid, s);
 }
 
-// Environment overrides for experiments, read once: MI355_SKINNY_WAVES (4 or 8; anything else is ignored),
-// MI355_SKINNY_NG (column groups per workgroup), MI355_SKINNY_NO_STAGE (A operands straight from global memory),
-// MI355_SKINNY_NO_ONCE (one workgroup per column group also where the stage-once form applies)
-struct SkinnyEnv
-{
-    int  waves = 0, ng = 0;
-    bool no_stage = false, no_once = false;
-    SkinnyEnv()
-    {
-        const char *w = getenv("MI355_SKINNY_WAVES"), *n = getenv("MI355_SKINNY_NG");
-        if (w && (atoi(w) == 4 || atoi(w) == 8))
-            waves = atoi(w);
-        if (n && atoi(n) >= 1 && atoi(n) <= 4)
-            ng = atoi(n);
-        no_stage = getenv("MI355_SKINNY_NO_STAGE") != nullptr;
-        no_once  = getenv("MI355_SKINNY_NO_ONCE") != nullptr;
-    }
-};
-
 // Workgroups of the stage-once kernels for `groups` column groups on `cus` compute units: one per group while they all
 // fit at once; from two groups per unit on, the smallest whole number of workgroups per compute unit that keeps every
 // workgroup within ONCE_MAX_GROUPS groups (a grid just above the number of units would leave most of them idle behind
@@ -1079,37 +1060,41 @@ static int once_grid(int groups, int cus)
     return cus * ((groups + ONCE_MAX_GROUPS * cus - 1) / (ONCE_MAX_GROUPS * cus));
 }
 
-int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, const char **variant)
 {
+    const char *unused;
+    const char *&form = variant ? *variant : unused;
+    form = "skinny_stream";
     if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
         return (int)hipErrorInvalidValue;
-    static const SkinnyEnv env;
     const int groups = (args.N + 15) / 16;
     const int KB     = (int)(args.Kp / 64);
     // Up to 8 rows every wave copies its K slice of A (at most 1 KiB per row) into LDS once and takes its operands
     // from there; that needs nothing to guard
-    const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 && !env.no_stage;
+    const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0;
     const bool stage_ok = args.M <= 8 && align_ok;
     const bool once_ok  = args.M <= 32 && align_ok; // the stage-once form also takes one or two full blocks of 16 rows
     // Up to 4096 of K the stage-once form (grid: once_grid above), each of the 16 waves owning PER = 1, 2 or 4 k blocks;
     // up to 16 rows it also takes 4096 < K <= 8192 with 8 k blocks per wave (one group's worth of B in flight per wave,
     // refilled half by half - the same bytes as two groups of 4 k blocks).
     // up to 8 rows and 8192 < K <= 16384: the stage-once form for deep K (3 or 4 chunks of 4 k blocks per wave)
-    if (stage_ok && KB > 8 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    if (stage_ok && KB > 8 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0 && groups <= cus) // one column group per workgroup
         {
+            form          = "skinny_deepk";
             const int nch = (KB + 4 * ONCE_WAVES - 1) / (4 * ONCE_WAVES);
             return nch == 3 ? skinny_deepk_launch<3>(epi, flip_a, args, groups, s) : skinny_deepk_launch<4>(epi, flip_a, args, groups, s);
         }
     }
     // 33 to 64 rows: the same with 8 waves, each holding the operand blocks of its 1, 2, 4 or 8 k blocks of all 64 rows
-    if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0)
         {
+            form             = "skinny_once_64rows";
             const bool multi = groups > cus;
             const int  grid  = once_grid(groups, cus);
             const int  per   = KB <= 8 ? 1 : (KB <= 16 ? 2 : (KB <= 32 ? 4 : 8));
@@ -1120,11 +1105,12 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
 #undef MI355_ONCE64
         }
     }
-    if (once_ok && (KB <= 4 * ONCE_WAVES || (KB <= 8 * ONCE_WAVES && args.M <= 16)) && !env.no_once && epi >= EPI_S32 && epi <= EPI_F32)
+    if (once_ok && (KB <= 4 * ONCE_WAVES || (KB <= 8 * ONCE_WAVES && args.M <= 16)) && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0)
         {
+            form             = "skinny_once";
             const bool multi = groups > cus;
             const int  grid  = once_grid(groups, cus);
             const int  per   = KB <= ONCE_WAVES ? 1 : (KB <= 2 * ONCE_WAVES ? 2 : (KB <= 4 * ONCE_WAVES ? 4 : 8));
@@ -1142,23 +1128,21 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
     // The kernel lives on loads in flight: 8 waves per workgroup while each of them still has at least one whole
     // step of 8 k blocks and all workgroups are resident together (24 waves of this size per compute unit), 4 otherwise
     int waves = (groups >= 512 && !(stage_ok && KB >= 64 && (int64_t)groups * 8 <= 24 * 256)) ? 4 : 8;
-    if (env.waves)
-        waves = env.waves;
     const int  per   = (KB + waves - 1) / waves;
     const bool stage = stage_ok && per * 64 <= sk_a_slice(waves);
     // more than 8 rows: per-step staging (dword-aligned rows are enough: the staging loads are plain 16-byte loads)
-    const bool step = args.M > 8 && args.lda % 4 == 0 && ((uintptr_t)args.A & 3) == 0 && !env.no_stage;
+    const bool step = args.M > 8 && args.lda % 4 == 0 && ((uintptr_t)args.A & 3) == 0;
     // (17..24 rows: the gathers of the unstaged variants below re-read row M-1 for the missing rows of the second
     // block, which costs less than staging 32 rows)
     if (args.M > 24 && step)
     {
         // LDS: 8.25 KiB per wave and block of 16 rows; a workgroup covers 2 column groups when there are many
-        const int ng     = env.ng ? (env.ng >= 2 ? 2 : 1) : (groups >= 512 ? 2 : 1);
+        const int ng     = groups >= 512 ? 2 : 1;
         const int blocks = (groups + ng - 1) / ng;
         if (args.M > 32)
             return ng == 2 ? skinny_launch_v<2, 4, 8, false, 4, true>(epi, flip_a, args, s)
                            : skinny_launch_v<1, 4, 8, false, 4, true>(epi, flip_a, args, s);
-        const int w = env.waves ? env.waves : (blocks >= 320 ? 4 : 8);
+        const int w = blocks >= 320 ? 4 : 8;
         if (ng == 2)
             return w == 4 ? skinny_launch_v<2, 4, 8, false, 2, true>(epi, flip_a, args, s)
                           : skinny_launch_v<2, 8, 8, false, 2, true>(epi, flip_a, args, s);
@@ -1171,11 +1155,9 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
         // the B stream unless a block covers several column groups - as many as still leave a few hundred blocks.
         const int mr = args.M > 32 ? 4 : 2;
         int       ng = groups >= 1024 ? 4 : (groups >= 512 ? 2 : 1);
-        if (env.ng)
-            ng = env.ng;
         ng = ng >= 4 && mr == 4 ? 4 : (ng >= 2 ? 2 : 1);
         const int blocks = (groups + ng - 1) / ng;
-        const int w      = env.waves ? env.waves : (blocks >= 320 ? 4 : 8);
+        const int w      = blocks >= 320 ? 4 : 8;
 #define MI355_SKV(NG_, MR_)                                                                          \
     (w == 4 ? skinny_launch_v<NG_, 4, 2, false, MR_>(epi, flip_a, args, s)                           \
             : skinny_launch_v<NG_, 8, 2, false, MR_>(epi, flip_a, args, s))
@@ -1185,7 +1167,7 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s)
 #undef MI355_SKV
     }
     // the waves of the unstaged / per-step variants follow the old rule
-    const int w1 = env.waves ? env.waves : (groups >= 512 ? 4 : 8);
+    const int w1 = groups >= 512 ? 4 : 8;
     if (step) // 9..16 rows
         return w1 == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, s)
                        : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, s);

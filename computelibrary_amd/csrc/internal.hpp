@@ -105,7 +105,8 @@ int  narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStr
 
 // gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 64;
-int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s);
+// *variant (when given): a static string naming the form of the kernel that ran
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, const char **variant = nullptr);
 
 // kernels_aux.hip
 // B [K][ldb] (row-major, N contiguous) -> Bp [Np][Kp] int8 (flip: xor 0x80), colsum[Np] (sums of the packed int8 values)

@@ -270,47 +270,58 @@ namespace quantization
 {
 namespace
 {
-constexpr int64_t one_q31 = (1LL << 31);
-constexpr float   epsilon = 0.00001f;
+// A real multiplier as mantissa * 2^(exponent - 31) with |mantissa| in [2^30, 2^31) (or 0): the form the fixed-point
+// output stage multiplies by. frexp gives the fraction in [0.5, 1); a fraction so close to 1 that it rounds up to 2^31
+// is renormalised to 2^30 with the exponent one higher.
+struct Q31
+{
+    int64_t mantissa;
+    int     exponent;
+};
+
+Q31 to_q31(float real)
+{
+    int          exponent = 0;
+    const double fraction = std::frexp(static_cast<double>(real), &exponent);
+    int64_t      mantissa = std::llround(std::ldexp(fraction, 31)); // halves away from zero, like std::round
+    if (mantissa == (int64_t{1} << 31))
+    {
+        mantissa >>= 1;
+        ++exponent;
+    }
+    return {mantissa, exponent};
+}
 } // namespace
 
+// Semantics of src/core/utils/quantization/AsymmHelpers.cpp:43-115: (multiplier, shift) with shift > 0 a rounding right
+// shift after the multiply and shift < 0 a left shift before it; real multipliers of 1 and above take the left-shift form.
 Status calculate_quantized_multiplier(float multiplier, int32_t *quant_multiplier, int32_t *shift, bool ignore_epsilon)
 {
-    if (multiplier >= 1.f)
-    {
-        Status status = calculate_quantized_multiplier_greater_than_one(multiplier, quant_multiplier, shift);
-        *shift *= -1;
-        return status;
-    }
-    return calculate_quantized_multiplier_less_than_one(multiplier, quant_multiplier, shift, ignore_epsilon);
+    if (multiplier < 1.f)
+        return calculate_quantized_multiplier_less_than_one(multiplier, quant_multiplier, shift, ignore_epsilon);
+    int32_t      left   = 0;
+    const Status status = calculate_quantized_multiplier_greater_than_one(multiplier, quant_multiplier, &left);
+    if (shift != nullptr)
+        *shift = -left;
+    return status;
 }
 
 Status calculate_quantized_multiplier_less_than_one(float multiplier, int32_t *quant_multiplier, int32_t *right_shift,
                                                     bool ignore_epsilon)
 {
-    const float eps = ignore_epsilon ? 0.0f : epsilon;
     ARM_COMPUTE_RETURN_ERROR_ON(quant_multiplier == nullptr);
     ARM_COMPUTE_RETURN_ERROR_ON(right_shift == nullptr);
-    ARM_COMPUTE_RETURN_ERROR_ON(multiplier < -eps);
-    ARM_COMPUTE_RETURN_ERROR_ON(multiplier > 1.0f + eps);
-    int          exponent = 0;
-    const double q        = std::frexp(multiplier, &exponent);
-    *right_shift          = -exponent;
-    int64_t q_fixed       = static_cast<int64_t>(std::round(q * one_q31));
-    ARM_COMPUTE_RETURN_ERROR_ON(q_fixed > one_q31);
-    if (q_fixed == one_q31)
-    {
-        q_fixed /= 2;
-        --*right_shift;
-    }
-    if (ignore_epsilon && *right_shift > 31)
-    {
-        *right_shift = 0;
-        q_fixed      = 0;
-    }
-    ARM_COMPUTE_RETURN_ERROR_ON(*right_shift < 0);
-    ARM_COMPUTE_RETURN_ERROR_ON(q_fixed > std::numeric_limits<int32_t>::max());
-    *quant_multiplier = static_cast<int32_t>(q_fixed);
+    // the reference tolerates values a hair outside [0, 1] unless told not to
+    const float slack = ignore_epsilon ? 0.f : 0.00001f;
+    ARM_COMPUTE_RETURN_ERROR_ON(multiplier < -slack);
+    ARM_COMPUTE_RETURN_ERROR_ON(multiplier > 1.f + slack);
+    Q31 q     = to_q31(multiplier);
+    int right = -q.exponent;
+    if (ignore_epsilon && right > 31)
+        q.mantissa = 0, right = 0; // too small to leave a trace in 32 bits
+    ARM_COMPUTE_RETURN_ERROR_ON(right < 0);
+    *quant_multiplier = static_cast<int32_t>(q.mantissa);
+    *right_shift      = right;
     return Status{};
 }
 
@@ -320,45 +331,32 @@ Status calculate_quantized_multiplier_greater_than_one(float multiplier, int32_t
     ARM_COMPUTE_RETURN_ERROR_ON(quantized_multiplier == nullptr);
     ARM_COMPUTE_RETURN_ERROR_ON(left_shift == nullptr);
     ARM_COMPUTE_RETURN_ERROR_ON(multiplier < 1.f);
-    int          exponent = 0;
-    const double q        = std::frexp(multiplier, &exponent);
-    *left_shift           = exponent;
-    int64_t q_fixed       = static_cast<int64_t>(std::round(q * one_q31));
-    ARM_COMPUTE_RETURN_ERROR_ON(q_fixed > one_q31);
-    if (q_fixed == one_q31)
-    {
-        q_fixed /= 2;
-        ++*left_shift;
-    }
-    ARM_COMPUTE_RETURN_ERROR_ON(*left_shift < 0);
-    ARM_COMPUTE_RETURN_ERROR_ON(q_fixed > std::numeric_limits<int32_t>::max());
-    *quantized_multiplier = static_cast<int32_t>(q_fixed);
+    const Q31 q = to_q31(multiplier);
+    ARM_COMPUTE_RETURN_ERROR_ON(q.exponent < 0);
+    *quantized_multiplier = static_cast<int32_t>(q.mantissa);
+    *left_shift           = q.exponent;
     return Status{};
 }
 
+// One (multiplier, shift) per weight scale from input_scale * weight_scale / output_scale
+// (src/core/utils/quantization/AsymmHelpers.cpp:117-152). Per-channel vectors get 32 spare zero entries at the end:
+// callers written against the reference size their buffers that way.
 Status calculate_quantized_multipliers(const QuantizationInfo &iq_info, const QuantizationInfo &wq_info,
                                        const QuantizationInfo &oq_info, GEMMLowpOutputStageInfo &stage_info)
 {
     ARM_COMPUTE_RETURN_ERROR_ON(iq_info.scale().empty());
     ARM_COMPUTE_RETURN_ERROR_ON(wq_info.scale().empty());
     ARM_COMPUTE_RETURN_ERROR_ON(oq_info.scale().empty());
-    // callers written against the reference expect 32 spare entries behind a per-channel vector
-    const size_t size   = wq_info.scale().size();
-    const size_t padded = (size == 1) ? 1 : size + 32;
-    stage_info.gemmlowp_multipliers.assign(padded, 0);
-    stage_info.gemmlowp_shifts.assign(padded, 0);
-    const float i_scale = iq_info.scale().at(0);
-    const float o_scale = oq_info.scale().at(0);
-    for (size_t i = 0; i < size; ++i)
-    {
-        const float multiplier = i_scale * wq_info.scale()[i] / o_scale;
-        int32_t     qm = 0, qs = 0;
-        ARM_COMPUTE_RETURN_ON_ERROR(calculate_quantized_multiplier(multiplier, &qm, &qs));
-        stage_info.gemmlowp_multipliers[i] = qm;
-        stage_info.gemmlowp_shifts[i]      = qs;
-    }
-    stage_info.gemmlowp_shift      = stage_info.gemmlowp_shifts[0];
-    stage_info.gemmlowp_multiplier = stage_info.gemmlowp_multipliers[0];
+    const std::vector<float> &w_scales = wq_info.scale();
+    const size_t              channels = w_scales.size();
+    const float               in_scale = iq_info.scale().front(), out_scale = oq_info.scale().front();
+    std::vector<int32_t> &mults = stage_info.gemmlowp_multipliers, &shifts = stage_info.gemmlowp_shifts;
+    mults.assign(channels == 1 ? 1 : channels + 32, 0);
+    shifts.assign(mults.size(), 0);
+    for (size_t ch = 0; ch < channels; ++ch)
+        ARM_COMPUTE_RETURN_ON_ERROR(calculate_quantized_multiplier(in_scale * w_scales[ch] / out_scale, &mults[ch], &shifts[ch]));
+    stage_info.gemmlowp_multiplier = mults.front();
+    stage_info.gemmlowp_shift      = shifts.front();
     return Status{};
 }
 

@@ -63,13 +63,19 @@ typedef enum mi355_epilogue
                                * previous half values are widened, added in float, and the sum rounded once). */
 } mi355_epilogue;
 
+/* Which kernel family runs the product. The reference chooses among its kernels the same way: a method table that the
+ * caller may narrow with arm_gemm::GemmConfig (method / filter, src/cpu/kernels/assembly/arm_gemm/arm_gemm.hpp:94-130;
+ * table in src/core/NEON/kernels/arm_gemm/gemm_qint8.cpp:75-250), with CpuGemmLowpMatrixMultiplyKernel as the plain
+ * fallback (src/cpu/operators/CpuGemmLowpMatrixMultiplyCore.cpp:216-263). */
 typedef enum mi355_path
 {
-    MI355_PATH_AUTO   = 0, /* MFMA tiled kernel, or the skinny kernel for small M (<= 32; <= 64 with N < 8192 or with
-                            * K <= 4096 a multiple of 64) */
-    MI355_PATH_SIMPLE = 1, /* one thread per output; for cross-checking only */
-    MI355_PATH_MFMA   = 2,
-    MI355_PATH_SKINNY = 3
+    MI355_PATH_AUTO   = 0, /* pipelined matrix-core kernel, or the streaming kernel for small M (<= 32; <= 64 with
+                            * N < 8192 or with K <= 4096 a multiple of 64) */
+    MI355_PATH_SIMPLE = 1, /* one thread per output, no matrix cores: the plain fallback (any alignment, any shape) */
+    MI355_PATH_MFMA   = 2, /* a tiled matrix-core kernel whatever M is */
+    MI355_PATH_SKINNY = 3, /* the streaming kernel (M <= 64) */
+    MI355_PATH_TILE   = 16 /* MI355_PATH_TILE + n: the pipelined kernel with its n-th tile configuration (n counts the
+                            * rows of its table, 256x128x128 first) wherever that configuration can take the shape */
 } mi355_path;
 
 typedef enum mi355_stage
@@ -229,6 +235,15 @@ typedef enum mi355_conv_layout
     MI355_NCHW = 1
 } mi355_conv_layout;
 
+typedef enum mi355_conv_path
+{
+    MI355_CONV_AUTO     = 0, /* implicit GEMM where the shape allows; channel counts that are not a multiple of 16 are
+                              * padded to one (one pass over the source) so that the 16-byte loaders apply */
+    MI355_CONV_EXPLICIT = 1, /* CpuIm2ColKernel's way: the patch matrix is written out, then a dense GEMM */
+    MI355_CONV_IN_PLACE = 2  /* implicit GEMM on the caller's channel count: no padded copy of the source; channel counts
+                              * that are not a multiple of 16 take the loader that gathers single bytes */
+} mi355_conv_path;
+
 /* Quantized NHWC convolution lowered to GEMM. Replaces CpuGemmConv2d::{configure,prepare,run}
  * (src/cpu/operators/CpuGemmConv2d.cpp:461-651, :1011-1101, :923-1008): CpuIm2ColKernel + CpuWeightsReshapeKernel
  * + CpuGemmLowpMatrixMultiplyCore. src is [batch][H][W][C], weights [OFM][KH][KW][C], dst [batch][OH][OW][OFM].
@@ -243,7 +258,7 @@ typedef struct mi355_conv_desc
     int32_t       src_offset, weights_offset;
     int32_t       pad_value;
     mi355_requant requant;
-    int32_t       path; /* 0 auto (implicit GEMM where the shape allows), 1 force explicit im2col + GEMM */
+    int32_t       path; /* mi355_conv_path */
     int32_t       layout; /* mi355_conv_layout of src, weights and dst */
     /* Bytes from one pixel (one tap of the weights) to the next when the tensors carry padding along the channel
      * dimension, as the reference's own fixtures give them (add_padding_x, tests/validation/Helpers.cpp:335-357;

@@ -1419,57 +1419,92 @@ static void test_error_paths()
     EXPECT(threw);
 }
 
+// Every case has a name so that the runner (tests/test_host_api.py) can start each one in a process of its own and
+// report it on its own: --list-cpu / --list-gpu print the names, --case NAME runs one, --cpu / --gpu run a whole group.
+struct Case
+{
+    const char *name;
+    bool        gpu;
+    void (*fn)();
+};
+
+static const Case g_cases[] = {
+    {"tensor_info", false, [] { test_tensor_info(); }},
+    {"quant_helpers", false, [] { test_quant_helpers(); }},
+    {"validate_tables", false, [] { test_validate_tables(); }},
+    {"fully_connected_validate", false, [] { test_fully_connected_validate(); }},
+    {"gemm_conv2d_validate", false, [] { test_gemm_conv2d_validate(); }},
+    {"error_paths", false, [] { test_error_paths(); }},
+    {"gemmlowp_fused_u8_host", true, [] { test_gemmlowp_fused_u8(false); }},
+    {"gemmlowp_fused_u8_device", true, [] { test_gemmlowp_fused_u8(true); }},
+    {"gemmlowp_s32_batched", true, [] { test_gemmlowp_s32_batched(); }},
+    {"reference_small_datasets", true, [] { test_reference_small_datasets(); }},
+    {"gemmlowp_accumulate_and_3d", true, [] { test_gemmlowp_accumulate_and_3d(); }},
+    {"gemmlowp_dynamic_qinfo", true, [] { test_gemmlowp_dynamic_qinfo(); }},
+    {"gemmlowp_per_channel_and_update", true, [] { test_gemmlowp_per_channel_and_update(); }},
+    {"gemmlowp_f32", true, [] { test_gemmlowp_f32(); }},
+    {"output_stage", true, [] { test_output_stage(); }},
+    {"quantize_down_scale", true, [] { test_quantize_down_scale(); }},
+    {"convolution_s8_per_channel_64", true, [] { test_convolution(DataType::QASYMM8_SIGNED, true, 64, ActivationLayerInfo()); }},
+    {"convolution_s8_relu_16", true,
+     [] { test_convolution(DataType::QASYMM8_SIGNED, false, 16, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU)); }},
+    {"convolution_u8_6", true, [] { test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo()); }},
+    {"convolution_u8_per_channel_bounded_relu_32", true,
+     [] {
+         test_convolution(DataType::QASYMM8, true, 32, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
+     }},
+    {"convolution_s8_per_channel_32_variant1", true, [] { test_convolution(DataType::QASYMM8_SIGNED, true, 32, ActivationLayerInfo(), 1); }},
+    {"convolution_u8_relu_6_variant1", true,
+     [] { test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), 1); }},
+    {"convolution_s8_per_channel_16_variant2", true, [] { test_convolution(DataType::QASYMM8_SIGNED, true, 16, ActivationLayerInfo(), 2); }},
+    {"convolution_u8_6_variant2", true, [] { test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(), 2); }},
+    {"gemm_conv2d", true, [] { test_gemm_conv2d(); }},
+    {"stateless_operator", true, [] { test_stateless_operator(); }},
+    {"stateless_operators_padded_after_configure", true, [] { test_stateless_operators_padded_after_configure(); }},
+    {"convolution_nchw_and_stateless", true, [] { test_convolution_nchw_and_stateless(); }},
+    {"convolution_f32_destination", true, [] { test_convolution_f32_destination(); }},
+    {"fully_connected_s8_after_fc", true, [] { test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc); }},
+    {"fully_connected_u8_after_fc", true, [] { test_fully_connected(DataType::QASYMM8, FcCase::AfterFc); }},
+    {"fully_connected_s8_after_conv_nhwc", true, [] { test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc); }},
+    {"fully_connected_u8_after_conv_nchw", true, [] { test_fully_connected(DataType::QASYMM8, FcCase::AfterConvNchw); }},
+    {"fully_connected_s8_weights_reshaped", true, [] { test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::WeightsReshaped); }},
+};
+
 int main(int argc, char **argv)
 {
     const std::string mode = argc > 1 ? argv[1] : "--cpu";
+    const std::string want = argc > 2 ? argv[2] : "";
+    if (mode == "--list-cpu" || mode == "--list-gpu")
+    {
+        for (const Case &c : g_cases)
+            if (c.gpu == (mode == "--list-gpu"))
+                std::printf("%s\n", c.name);
+        return 0;
+    }
+    if (mode != "--cpu" && mode != "--gpu" && mode != "--case")
+    {
+        std::printf("usage: %s --cpu | --gpu | --case NAME | --list-cpu | --list-gpu\n", argv[0]);
+        return 2;
+    }
+    int ran = 0;
     try
     {
-        if (mode == "--cpu")
-        {
-            test_tensor_info();
-            test_quant_helpers();
-            test_validate_tables();
-            test_fully_connected_validate();
-            test_gemm_conv2d_validate();
-            test_error_paths();
-        }
-        else
-        {
-            test_gemmlowp_fused_u8(false);
-            test_gemmlowp_fused_u8(true);
-            test_gemmlowp_s32_batched();
-            test_reference_small_datasets();
-            test_gemmlowp_accumulate_and_3d();
-            test_gemmlowp_dynamic_qinfo();
-            test_gemmlowp_per_channel_and_update();
-            test_gemmlowp_f32();
-            test_output_stage();
-            test_quantize_down_scale();
-            test_convolution(DataType::QASYMM8_SIGNED, true, 64, ActivationLayerInfo());
-            test_convolution(DataType::QASYMM8_SIGNED, false, 16, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU));
-            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo());
-            test_convolution(DataType::QASYMM8, true, 32,
-                             ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::BOUNDED_RELU, 20.f));
-            test_convolution(DataType::QASYMM8_SIGNED, true, 32, ActivationLayerInfo(), 1);
-            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(ActivationLayerInfo::ActivationFunction::RELU), 1);
-            test_convolution(DataType::QASYMM8_SIGNED, true, 16, ActivationLayerInfo(), 2);
-            test_convolution(DataType::QASYMM8, false, 6, ActivationLayerInfo(), 2);
-            test_gemm_conv2d();
-            test_stateless_operator();
-            test_stateless_operators_padded_after_configure();
-            test_convolution_nchw_and_stateless();
-            test_convolution_f32_destination();
-            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterFc);
-            test_fully_connected(DataType::QASYMM8, FcCase::AfterFc);
-            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::AfterConvNhwc);
-            test_fully_connected(DataType::QASYMM8, FcCase::AfterConvNchw);
-            test_fully_connected(DataType::QASYMM8_SIGNED, FcCase::WeightsReshaped);
-        }
+        for (const Case &c : g_cases)
+            if (mode == "--case" ? want == c.name : c.gpu == (mode == "--gpu"))
+            {
+                c.fn();
+                ++ran;
+            }
     }
     catch (const std::exception &e)
     {
         std::printf("FAILED: unexpected exception: %s\n", e.what());
         ++g_failures;
+    }
+    if (ran == 0)
+    {
+        std::printf("no such case: %s\n", want.c_str());
+        return 2;
     }
     std::printf("%d checks, %d failures\n", g_checks, g_failures);
     return g_failures == 0 ? 0 : 1;

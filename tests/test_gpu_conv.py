@@ -175,7 +175,7 @@ def test_conv_few_output_channels_kernel():
             got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
 
 
-def test_conv_channel_counts_padded_to_16(monkeypatch):
+def test_conv_channel_counts_padded_to_16():
     """A channel count that is not a multiple of 16: pixels and taps are copied with the channels padded to the next
     multiple of 16 and the fast implicit kernels run (never the byte-wise fallback), with identical results - the RGB of
     a first layer (7 x 7 stride 2, 3 x 3 stride 2), 1, 4, 5, 8, 24 and 40 channels, few and many output channels, both
@@ -214,8 +214,7 @@ def test_conv_channel_counts_padded_to_16(monkeypatch):
             got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil, layout=layout)
             assert name.startswith("implicit_") and "mfma" not in name, name
             np.testing.assert_array_equal(got, want)
-    # the byte-wise loader instead: the same bits
-    monkeypatch.setenv("MI355_NO_CHANNEL_PAD", "1")
+    # the byte-wise loader instead (the convolution on the caller's channel count, no padded copy): the same bits
     for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp, layout) in cases[:2] + cases[7:9]:
         src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
         w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
@@ -225,10 +224,10 @@ def test_conv_channel_counts_padded_to_16(monkeypatch):
         lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
         want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil)
         announce("conv byte-wise loader", shape, wshape)
-        got, name = run_conv(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil, layout=layout)
+        got, name = run_conv(src, w, bias, zp, w_zp, [mult], [shift], ozp, lo, hi, stride, pad, dil, layout=layout,
+                             path=capi.CONV_IN_PLACE)
         assert name.startswith("implicit_mfma"), name
         np.testing.assert_array_equal(got, want)
-    monkeypatch.delenv("MI355_NO_CHANNEL_PAD")
     # a handle that pads, after a change of both offsets and of the padding value
     src = rng.integers(-128, 128, size=(2, 7, 6, 3), dtype=np.int8)
     w = rng.integers(-127, 128, size=(8, 3, 3, 3), dtype=np.int8)

@@ -225,18 +225,18 @@ PIPELINED_CONFIGS = ["pp_256x128x128_s3", "pp_128x128x128_s3", "pp_128x64x128_s3
 
 
 @pytest.mark.parametrize("cfg", range(len(PIPELINED_CONFIGS)))
-def test_every_pipelined_configuration(cfg, monkeypatch):
-    """Each tile / ring-depth configuration of the pipelined kernel, forced through the environment override, on K of
+def test_every_pipelined_configuration(cfg):
+    """Each tile / ring-depth configuration of the pipelined kernel, asked for by name (MI355_PATH_TILE + n), on K of
     one to nine steps with and without a tail (the 256-byte-step configuration needs a packed K that is a multiple of
     256 and is otherwise replaced by the automatic choice)."""
-    monkeypatch.setenv("MI355_DMA_CFG", str(cfg))
+    tile = capi.PATH_TILE + cfg
     rng = np.random.default_rng(70 + cfg)
     for (M, N, K) in [(300, 200, 512), (70, 129, 100), (257, 64, 1100), (129, 300, 250), (64, 65, 2048)]:
         A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
         B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
         ao, bo = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
         announce("pipelined config", cfg, (M, N, K))
-        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=capi.PATH_MFMA, device=True)
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=tile, device=True)
         kp = -(-K // 128) * 128
         if cfg != 5 or kp % 256 == 0:
             assert name.split("_splitk")[0] == PIPELINED_CONFIGS[cfg], name  # (K = 2048 under one tile runs as two K slices)
@@ -244,10 +244,10 @@ def test_every_pipelined_configuration(cfg, monkeypatch):
         bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
         reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
         mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
-        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, 0, bias, mult, shift, -7, -128, 127, path=capi.PATH_MFMA,
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, 0, bias, mult, shift, -7, -128, 127, path=tile,
                           device=True)
         np.testing.assert_array_equal(got, oracle.gemmlowp_fixedpoint(A, B, bias, ao, 0, mult, shift, -7, -128, 127, np.int8))
-        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, path=capi.PATH_MFMA, device=True)
+        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, path=tile, device=True)
         np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
 
 

@@ -459,7 +459,12 @@ struct GemmCore
         int  k_valid        = K;
         const bool direct =
             path == MI355_PATH_SIMPLE || ((((uintptr_t)A | (uintptr_t)lda | (uintptr_t)a_bs) & 3) == 0);
-        const bool need_rowvec = b_off_eff() != 0;
+        // the per-row term b_offset * rowsum(A): the pipelined kernels sum the rows of A themselves while its tiles pass
+        // through them (dword-aligned rows, K a whole number of 16-byte columns, one launch); otherwise one pass over A
+        // in front of the GEMM leaves the sums in a vector
+        const bool rowsum_in_kernel = b_off_eff() != 0 && direct && path == MI355_PATH_MFMA && dma_idx >= 0 && K % 16 == 0 && K >= 16 &&
+                                      splitk == 1 && (int64_t)lda * 256 + K < ((int64_t)1 << 32);
+        const bool need_rowvec = b_off_eff() != 0 && !rowsum_in_kernel;
         // the two workspaces of a run: owned by the handle and grown on demand, or carved out of a buffer the caller of
         // this function brings (ext_ws != nullptr: nothing is allocated, sizes beyond ext_ws_bytes are an error)
         const size_t rv_bytes = need_rowvec ? ((sizeof(int32_t) * (size_t)M * batch + 255) & ~(size_t)255) : 0;
@@ -496,6 +501,8 @@ struct GemmCore
                 HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, nullptr, Kp, rv + (size_t)b * M,
                                          b_off_eff(), s));
         }
+        if (rowsum_in_kernel)
+            g.epi.rowsum_mul = b_off_eff();
         if (need_rowvec)
             g.epi.rowvec = rv;
         else if (path == MI355_PATH_SKINNY)

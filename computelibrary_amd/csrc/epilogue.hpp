@@ -46,6 +46,10 @@ struct EpiParams
     const int32_t *qp_flag;
     int32_t        accumulate; // EPI_S32 / EPI_F32: add the destination's previous contents (GEMMInfo::accumulate)
     int32_t        act_twice;  // EPI_F32: the activation clamp is also applied before the offset term is added
+    // != 0: the pipelined kernels sum the rows of A themselves while its tiles pass through their registers (what
+    // compute_row_sums does inside the reference's fused kernels, src/core/NEON/kernels/arm_gemm/quantized.cpp:802-838)
+    // and use rowsum_mul * rowsum(A)[i] as the per-row term; rowvec is not read then. Needs K % 16 == 0.
+    int32_t        rowsum_mul;
 };
 
 // Per-column constants of the branch-free requantisation used by the pipelined kernel's epilogue, valid for

@@ -253,7 +253,7 @@ __device__ long long phase_clocks[6][8];
 
 // GWM x GWN consumer waves per group, 2 groups stacked along M, plus NP = GWM*GWN producer waves
 template <int BM, int BN, int BK, int GWM, int GWN, int NS, int EPI, bool FLIP_A, bool CONV>
-__global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
+__global__ __launch_bounds__(GWM *GWN * 192) __attribute__((amdgpu_waves_per_eu(1, 6))) void gemm_dma_kernel(GemmArgs g_in)
 {
     // What a workgroup needs before its first loads go out is read here, in one batch of scalar loads, and pinned in
     // registers. Left alone, the compiler fetches kernel arguments where they are first used: five dependent round trips
@@ -466,6 +466,12 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     if (group == 1 && !INPHASE)
         block_barrier(); // group 1 runs one slot behind group 0
 
+    // row sums of A, taken from the operand blocks as they pass (dense tiles, on request)
+    const bool rowsum = !CONV && g.epi.rowsum_mul != 0;
+    int32_t    rsum[RS];
+#pragma unroll
+    for (int f = 0; f < RS; ++f)
+        rsum[f] = 0;
     v4i fa[KK][RS], fb[KK][QS];
     for (int kt = 0; kt < nk; ++kt)
     {
@@ -499,6 +505,14 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
                     fa[kk][f] ^= (int)0x80808080;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (rowsum)
+        {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+                for (int f = 0; f < RS; ++f)
+                    rsum[f] = sum_bytes(fa[kk][f], rsum[f]);
+        }
         // this wave's units of stage kt+1 have to be in LDS before the barrier that opens that stage to its first
         // reader; the NS-2 younger stages (the last of them just issued) may still be in flight
         if (CDMA)
@@ -527,6 +541,8 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
     if (group == 0 || INPHASE)
         block_barrier(); // barrier 2nk+1; every operand read of every wave is complete beyond this point
     MI355_PHASE(3); // consumer: K loop over
+    if (rowsum)
+        finish_row_sums<RS>(rsum, g.epi.rowsum_mul, FLIP_A ? nk * BK - g.K : 0);
 
     if (fast)
     {
@@ -542,28 +558,28 @@ __global__ __launch_bounds__(GWM *GWN * 192) void gemm_dma_kernel(GemmArgs g_in)
         if (EPI == EPI_FIXEDPOINT)
         {
             char *stage = smem + ((NPAR * BN * 4 + 15) & ~15);
-            const bool rowv = g.epi.rowvec != nullptr;
+            const bool rowv = g.epi.rowvec != nullptr || rowsum;
             if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0 && !rowv)
                 epilogue_store_staged<true, false, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
                                                                        [] { __syncthreads(); });
             else if (g.epi.vec_store16 && g.epi.qp_std && qflag == 0)
                 epilogue_store_staged<true, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
-                                                                      [] { __syncthreads(); });
+                                                                      [] { __syncthreads(); }, rsum, rowsum);
             else if (g.epi.vec_store16)
                 epilogue_store_staged<false, true, RS, QS, BM, BN, NW>(acc, g, par, stage, m0, n0, row_w, col_w, wave, lane, bz,
-                                                                       [] { __syncthreads(); });
+                                                                       [] { __syncthreads(); }, rsum, rowsum);
             else
-                epilogue_store_fast<RS, QS, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz);
+                epilogue_store_fast<RS, QS, BN>(acc, g, par, m0 + row_w, n0 + col_w, col_w, lane, bz, rsum, rowsum);
         }
     }
     else if ((EPI == EPI_S32 || EPI == EPI_F32) && g.epi.vec_store && !g.epi.accumulate)
     {
         // the ring is free beyond the last barrier: 16 x (QS*64 + 16) bytes per wave
         if constexpr (EPI != EPI_FIXEDPOINT)
-            epilogue_store_wave32<EPI, RS, QS>(acc, g, smem + wave * 16 * (QS * 64 + 16), m0 + row_w, n0 + col_w, lane, bz);
+            epilogue_store_wave32<EPI, RS, QS>(acc, g, smem + wave * 16 * (QS * 64 + 16), m0 + row_w, n0 + col_w, lane, bz, rsum, rowsum);
     }
     else
-        epilogue_store_t<EPI, RS, QS>(acc, g, m0 + row_w, n0 + col_w, lane, bz);
+        epilogue_store_t<EPI, RS, QS>(acc, g, m0 + row_w, n0 + col_w, lane, bz, rsum, rowsum);
     MI355_PHASE(4); // consumer: epilogue done (stores issued)
 }
 
@@ -777,6 +793,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
             for (int f = 0; f < RS; ++f)
                 fa0[f] ^= (int)0x80808080;
         }
+
 #pragma unroll
         for (int i = 0; i < RS; ++i)
 #pragma unroll
@@ -807,6 +824,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
             for (int f = 0; f < RS; ++f)
                 fa1[f] ^= (int)0x80808080;
         }
+
 #pragma unroll
         for (int i = 0; i < RS; ++i)
 #pragma unroll
@@ -904,6 +922,13 @@ struct DmaEntry
             512                                                                                                      \
     }
 
+// Row sums of A taken inside the kernel (EpiParams::rowsum_mul) are a run-time switch of the 8 + 4 wave kernel; the
+// 4 + 4 wave kernel has no registers left for them, so its tile shape falls back to the 8 + 4 wave form there: [epi][flip]
+static const void *const g_rowsum_256x128x128[3][2] = {
+    {MI355_DFN(256, 128, 128, 2, 2, 3, 0, false, false), MI355_DFN(256, 128, 128, 2, 2, 3, 0, true, false)},
+    {MI355_DFN(256, 128, 128, 2, 2, 3, 1, false, false), MI355_DFN(256, 128, 128, 2, 2, 3, 1, true, false)},
+    {MI355_DFN(256, 128, 128, 2, 2, 3, 2, false, false), MI355_DFN(256, 128, 128, 2, 2, 3, 2, true, false)}};
+
 static const DmaEntry g_dma[] = {
     MI355_WCFG("pp_256x128x128_s3", 256, 128, 128, 2, 2, 3),
     MI355_DCFG("pp_128x128x128_s3", 128, 128, 128, 2, 2, 3),
@@ -931,6 +956,14 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
         return (int)hipErrorInvalidValue;
     const DmaEntry &c  = g_dma[cfg_idx];
     const void     *fn = c.fn[epi][flip_a ? 1 : 0][conv ? 1 : 0];
+    int             fn_slot = conv ? 1 : 0; // which entry of the once-per-device table below
+    if (args.epi.rowsum_mul != 0)
+    {
+        if (conv || args.K % 16 != 0)
+            return (int)hipErrorInvalidValue;
+        if (c.threads_dense) // the 4 + 4 wave kernel's tile shape: see g_rowsum_256x128x128
+            fn = g_rowsum_256x128x128[epi][flip_a ? 1 : 0], fn_slot = 2;
+    }
     if (fn == nullptr || args.fill16 == nullptr)
         return (int)hipErrorInvalidValue;
     // shapes the kernel assumes: dword-aligned rows of at least one 16-byte column (whole columns of one tap for the
@@ -944,8 +977,8 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     if (c.lds_bytes > 48 * 1024)
     {
         // once per kernel and device
-        static std::atomic<uint32_t> raised[sizeof(g_dma) / sizeof(g_dma[0])][3][2][2];
-        std::atomic<uint32_t>       &done = raised[cfg_idx][epi][flip_a ? 1 : 0][conv ? 1 : 0];
+        static std::atomic<uint32_t> raised[sizeof(g_dma) / sizeof(g_dma[0])][3][2][3];
+        std::atomic<uint32_t>       &done = raised[cfg_idx][epi][flip_a ? 1 : 0][fn_slot];
         int                          dev  = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
             return (int)hipErrorInvalidDevice;
@@ -970,7 +1003,7 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     a.magic_group = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_group) + 1u : 0u;
     a.nblocks     = (int32_t)nblocks;
     void    *kargs[] = {&a};
-    dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block((!conv && c.threads_dense) ? c.threads_dense : c.threads);
+    dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block((fn_slot == 0 && c.threads_dense) ? c.threads_dense : c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);
 }
 } // namespace mi355

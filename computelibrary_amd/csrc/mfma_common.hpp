@@ -78,6 +78,31 @@ __device__ __forceinline__ void tile_coords_batched_fast(int bid, int nblocks, i
     tm = first + in_grp - tn * gsize;
 }
 
+// Row sums of A taken inside the pipelined kernels: a lane holds the 16-byte column lane/16 of row lane%16 of every
+// operand block of A it reads; sums[f] collects the bytes of block row f over the whole K loop (sdot4 with ones). The four
+// lanes of a row are added up here, the padding the loader flipped along with the data (K steps beyond K hold zeros;
+// a flipped zero counts -128) is taken out, and the sum is scaled: sums[f] becomes the per-row term of output row
+// f*16 + lane%16, in every lane of that row - the layout the epilogues above take their row terms in.
+template <int RS>
+__device__ __forceinline__ void finish_row_sums(int32_t (&sums)[RS], int32_t mul, int32_t flipped_pad_bytes)
+{
+#pragma unroll
+    for (int f = 0; f < RS; ++f)
+    {
+        int32_t v = sums[f];
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        sums[f] = (int32_t)((uint32_t)mul * (uint32_t)(v + 128 * flipped_pad_bytes));
+    }
+}
+__device__ __forceinline__ int32_t sum_bytes(v4i x, int32_t acc)
+{
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        acc = __builtin_amdgcn_sdot4(x[t], 0x01010101, acc, false);
+    return acc;
+}
+
 // Accumulator (fm, fn, r) of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 block.
 // (row0, col0) is the wave's top-left output coordinate.
 template <int EPI, int FM, int FN>
@@ -139,7 +164,7 @@ __device__ __forceinline__ void epilogue_store(const v16i (&acc)[FM][FN], const 
 // (row0, col0) is the wave's top-left output coordinate.
 template <int EPI, int RS, int QS>
 __device__ __forceinline__ void epilogue_store_t(const v4i (&acc)[RS][QS], const GemmArgs &g, int row0, int col0,
-                                                 int lane, int bz)
+                                                 int lane, int bz, const int32_t *rvk = nullptr, bool use_rvk = false)
 {
     const int        lr = lane & 15, lh = lane >> 4;
     const EpiParams &p      = g.epi;
@@ -151,7 +176,7 @@ __device__ __forceinline__ void epilogue_store_t(const v4i (&acc)[RS][QS], const
     for (int rs = 0; rs < RS; ++rs)
     {
         const int i = row0 + rs * 16 + lr;
-        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+        rv[rs]      = use_rvk ? rvk[rs] : ((rowvec && i < g.M) ? rowvec[i] : 0);
     }
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs)
@@ -263,7 +288,8 @@ __device__ __forceinline__ void epilogue_store_t(const v4i (&acc)[RS][QS], const
 // column inside the block tile. Same accumulator layout as epilogue_store_t.
 template <int RS, int QS, int BN>
 __device__ __forceinline__ void epilogue_store_fast(const v4i (&acc)[RS][QS], const GemmArgs &g, const int32_t *par,
-                                                    int row0, int col0, int col_in_tile, int lane, int bz)
+                                                    int row0, int col0, int col_in_tile, int lane, int bz,
+                                                    const int32_t *rvk = nullptr, bool use_rvk = false)
 {
     const int        lr = lane & 15, lh = lane >> 4;
     const EpiParams &p      = g.epi;
@@ -274,7 +300,7 @@ __device__ __forceinline__ void epilogue_store_fast(const v4i (&acc)[RS][QS], co
     for (int rs = 0; rs < RS; ++rs)
     {
         const int i = row0 + rs * 16 + lr;
-        rv[rs]      = (rowvec && i < g.M) ? rowvec[i] : 0;
+        rv[rs]      = use_rvk ? rvk[rs] : ((rowvec && i < g.M) ? rowvec[i] : 0);
     }
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs)
@@ -326,7 +352,8 @@ __device__ __forceinline__ void epilogue_store_fast(const v4i (&acc)[RS][QS], co
 template <bool STD, bool ROWV, int RS, int QS, int BM, int BN, int NW, typename Barrier>
 __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], const GemmArgs &g, const int32_t *par,
                                                       char *stage, int m0, int n0, int row_in_tile, int col_in_tile,
-                                                      int wave, int lane, int bz, Barrier barrier)
+                                                      int wave, int lane, int bz, Barrier barrier,
+                                                      const int32_t *rvk = nullptr, bool use_rvk = false)
 {
     constexpr int    PITCH = BN + 16;
     const int        lr = lane & 15, lh = lane >> 4;
@@ -338,7 +365,7 @@ __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], 
     for (int rs = 0; rs < RS; ++rs)
     {
         const int i = m0 + row_in_tile + rs * 16 + lr;
-        rv[rs]      = (ROWV && rowvec && i < g.M) ? rowvec[i] : 0;
+        rv[rs]      = !ROWV ? 0 : (use_rvk ? rvk[rs] : ((rowvec && i < g.M) ? rowvec[i] : 0));
     }
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs)
@@ -399,7 +426,7 @@ __device__ __forceinline__ void epilogue_store_staged(const v4i (&acc)[RS][QS], 
 // instead of 16-byte pieces of 16 different rows. Needs no synchronisation with other waves. Requires p.vec_store.
 template <int EPI, int RS, int QS>
 __device__ __forceinline__ void epilogue_store_wave32(const v4i (&acc)[RS][QS], const GemmArgs &g, char *stage, int row0,
-                                                      int col0, int lane, int bz)
+                                                      int col0, int lane, int bz, const int32_t *rvk = nullptr, bool use_rvk = false)
 {
     static_assert(EPI == EPI_S32 || EPI == EPI_F32, "32-bit outputs only");
     constexpr int    PITCH = QS * 64 + 16;
@@ -432,7 +459,7 @@ __device__ __forceinline__ void epilogue_store_wave32(const v4i (&acc)[RS][QS], 
     for (int rs = 0; rs < RS; ++rs)
     {
         const int i = row0 + rs * 16 + lr;
-        rvs[rs]     = (rowvec && i < g.M) ? rowvec[i] : 0;
+        rvs[rs]     = use_rvk ? rvk[rs] : ((rowvec && i < g.M) ? rowvec[i] : 0);
     }
     // The conditions that are the same for the whole launch (bias, offsets, second clamp) and for the whole tile (inside
     // the matrix or on its edge) are decided once, here, and the loop over the outputs is instantiated for each answer:

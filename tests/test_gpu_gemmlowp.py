@@ -251,6 +251,40 @@ def test_every_pipelined_configuration(cfg):
         np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
 
 
+@pytest.mark.parametrize("cfg", range(len(PIPELINED_CONFIGS)))
+def test_row_sums_taken_inside_the_pipelined_kernels(cfg):
+    """A non-zero B offset (or an unsigned B) needs b_offset * rowsum(A): with dword-aligned rows and K a multiple of 16
+    the pipelined kernels sum the rows of A themselves from the tiles that pass through them (one launch, no pass over A
+    in front). Every tile configuration; K with whole steps and with a last step that is mostly padding (which an
+    unsigned A turns into -128s that must not be counted); signed and unsigned A and B; a batch; a row stride with a
+    gap; every epilogue."""
+    tile = capi.PATH_TILE + cfg
+    rng = np.random.default_rng(900 + cfg)
+    for (M, N, K, a_dt, b_dt, batch) in [(300, 200, 512, np.int8, np.int8, 1), (257, 140, 400, np.uint8, np.uint8, 1),
+                                         (70, 129, 144, np.uint8, np.int8, 3), (520, 260, 1040, np.int8, np.uint8, 2)]:
+        shape_a = (batch, M, K) if batch > 1 else (M, K)
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=shape_a).astype(a_dt)
+        B = rng.integers(np.iinfo(b_dt).min, np.iinfo(b_dt).max + 1, size=(K, N)).astype(b_dt)
+        ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
+        lda = K + 16
+        announce("row sums in kernel", cfg, (batch, M, N, K), a_dt.__name__, b_dt.__name__, ao, bo)
+        As = A if batch > 1 else A[None]
+        want = np.stack([oracle.gemmlowp_s32(As[z], B, ao, bo) for z in range(batch)])
+        got, name = run_gemm(A, B, capi.EPI_S32, np.int32, ao, bo, path=tile, device=True, lda=lda)
+        np.testing.assert_array_equal(got if batch > 1 else got[None], want)
+        bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+        mult, shift = oracle.calculate_quantized_multiplier(float(128.0 / np.sqrt(K) * 2e-4))
+        lo, hi, off = (-128, 127, -7) if a_dt == np.int8 else (0, 255, 121)
+        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, a_dt, ao, bo, bias, [mult], [shift], off, lo, hi, path=tile, device=True,
+                          lda=lda)
+        wantq = np.stack([oracle.gemmlowp_fixedpoint(As[z], B, bias, ao, bo, [mult], [shift], off, lo, hi, a_dt)
+                          for z in range(batch)])
+        np.testing.assert_array_equal(got if batch > 1 else got[None], wantq)
+        if a_dt == np.int8 and b_dt == np.int8:
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, path=tile, device=True, lda=lda)
+            np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
+
+
 @pytest.mark.parametrize("M", [1, 5, 8, 9, 12, 16])
 def test_skinny_kernel_with_staged_a(M):
     """Up to 8 rows the streaming kernel copies each wave's K slice of A into LDS once, 9 to 16 rows it stages the 512

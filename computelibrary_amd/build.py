@@ -63,9 +63,10 @@ def build_phases(verbose=True):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=4) as ex:
-        phases = ex.submit(_compile, "gemm_dma.hip", ("-DMI355_PHASE_CLOCKS",), "_phases")
-        objs = list(ex.map(_compile, [x for x in SOURCES if x != "gemm_dma.hip"]))
-        objs.append(phases.result())
+        instrumented = ("gemm_dma.hip", "gemm_narrow.hip")
+        phases = [ex.submit(_compile, src, ("-DMI355_PHASE_CLOCKS",), "_phases") for src in instrumented]
+        objs = list(ex.map(_compile, [x for x in SOURCES if x not in instrumented]))
+        objs += [f.result() for f in phases]
     _link(PHASES_LIB, objs, verbose)
     return PHASES_LIB
 

@@ -178,7 +178,7 @@ struct GemmCore
     std::string kname_mfma, kname_dma, kprefix;
     // The names a run can report, composed when the choice is made (create, prepare, update): a run only points at one
     // of them - it must not touch the host heap
-    std::string        kname_narrow, kname_dma_full, kname_splitk, kname_mfma_full;
+    std::string        kname_narrow, kname_band, kname_dma_full, kname_splitk, kname_mfma_full;
     const char        *kname_static = nullptr; // the streaming kernel names its forms itself
     const std::string *kname_run = nullptr; // what the last run took (nullptr: no run yet, kname is what create announced)
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
@@ -188,6 +188,7 @@ struct GemmCore
     void refresh_names()
     {
         kname_narrow    = kprefix + "narrow_32x64";
+        kname_band      = kprefix + "band_32x64";
         kname_dma_full  = kprefix + kname_dma;
         kname_splitk    = kname_dma_full + "_splitk" + std::to_string(splitk);
         kname_mfma_full = kprefix + kname_mfma;
@@ -350,7 +351,7 @@ struct GemmCore
         {
             const int chunks = narrow_panel_chunks(K);
             const int rows = round_up(N, 64); // panels of 64 columns (Np, a multiple of 256, covers them)
-            TRY(Bn.ensure((size_t)rows * (chunks + 1) * 16));
+            TRY(Bn.ensure((size_t)rows * (chunks + NARROW_PAD_PIECES) * 16));
             HIP_TRY(pack_b_narrow_launch(Bp.as<int8_t>(), Kp, Np, chunks, rows, Bn.as<int8_t>(), s));
         }
         TRY(fill.ensure(16));
@@ -438,6 +439,7 @@ struct GemmCore
         const int32_t tlo = dst_dtype == MI355_S8 ? -128 : 0, thi = dst_dtype == MI355_S8 ? 127 : 255;
         p.lo                  = rq.min_bound > tlo ? rq.min_bound : tlo;
         p.hi                  = rq.max_bound < thi ? rq.max_bound : thi;
+        p.qp_pk16             = (p.qp_std && rq.result_offset >= -1024 && rq.result_offset <= 1024 && p.lo >= -1024 && p.hi <= 1024) ? 1 : 0;
         p.scale               = scale;
         p.act_min             = act_min;
         p.act_max             = act_max;
@@ -558,10 +560,11 @@ struct GemmCore
             if (has_narrow && batch == 1 && conv && !g.epi.accumulate && span < ((int64_t)1 << 31) &&
                 narrow_applies(g, conv))
             {
-                kname_run       = &kname_narrow;
                 g.Bp            = Bn.as<int8_t>();
                 g.conv.pad_word = 0x01010101u * fill_byte; // as in the image: the kernel flips what it loads
-                HIP_TRY(narrow_launch(epi, flip_in_loader, conv, g, s));
+                bool band       = false;
+                HIP_TRY(narrow_launch(epi, flip_in_loader, conv, g, s, &band));
+                kname_run = band ? &kname_band : &kname_narrow;
             }
             else if (dma_idx >= 0 && aligned && g.K >= 16 && span < ((int64_t)1 << 32))
             {

@@ -41,6 +41,7 @@ struct EpiParams
     const int32_t *qp;
     int64_t        qp_stride;
     int32_t        qp_std; // |result_offset| < 2^28: std_requant may be used where the flag word allows it
+    int32_t        qp_pk16; // ... and |result_offset|, |lo|, |hi| <= 1024: std_requant4_pk16 may be used instead
     // One word written together with qp: 0 when every column has a multiplier >= 2^30 and a shift in [2, 31]
     // (std_requant applies), bit 0 set when some multiplier is negative (then only the general formula applies)
     const int32_t *qp_flag;
@@ -92,6 +93,27 @@ __device__ __forceinline__ int32_t std_requant(int32_t v, int32_t s2, int32_t rs
 {
     const int32_t h = __mulhi(v, s2) + v;
     return clamp_med3(((h >> rsm1) + off2p1) >> 1, lo, hi);
+}
+
+// std_requant of 4 values at once, the 4 results' low bytes packed into one word. After the per-column shift the
+// values are narrowed to 16 bits with saturation and the constant, the halving and the clamp work on pairs
+// (2.75 vector-ALU slots per value instead of 3.75). Same results as std_requant while |off2p1| <= 2049 and
+// -1024 <= lo <= hi <= 1024: a value the narrowing saturates ends beyond +-15359 after the halving and is clamped
+// to lo or hi either way.
+typedef short pk16_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t std_requant4_pk16(const int32_t (&v)[4], const int32_t (&s2)[4], const int32_t (&rsm1)[4],
+                                                      pk16_t off2p1, pk16_t lo, pk16_t hi)
+{
+    int32_t x[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        x[t] = (__mulhi(v[t], s2[t]) + v[t]) >> rsm1[t];
+    pk16_t a = __builtin_amdgcn_cvt_pk_i16(x[0], x[1]), b = __builtin_amdgcn_cvt_pk_i16(x[2], x[3]);
+    a = __builtin_elementwise_add_sat(a, off2p1) >> (pk16_t){1, 1};
+    b = __builtin_elementwise_add_sat(b, off2p1) >> (pk16_t){1, 1};
+    a = __builtin_elementwise_min(__builtin_elementwise_max(a, lo), hi);
+    b = __builtin_elementwise_min(__builtin_elementwise_max(b, lo), hi);
+    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, a), 0x06040200u);
 }
 
 // (a * b * 2) >> 32 with the single saturating case, without 64-bit VALU arithmetic

@@ -21,6 +21,7 @@
 //   * no barrier after the one that publishes the B panel; 4 workgroups of 4 waves fit a compute unit.
 #include "mfma_common.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -31,6 +32,11 @@ namespace mi355
 __device__ __forceinline__ void narrow_dma16(const void *sbase, uint32_t voff, uint32_t lds_addr)
 {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+}
+// (one 64-bit address per lane)
+__device__ __forceinline__ void narrow_dma16_at(const void *from, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(from), "s"(lds_addr) : "memory");
 }
 
 // x / d with the reciprocal of ConvGeom::magic_* (0 stands for d == 1), without a branch on the reciprocal
@@ -67,7 +73,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 {
     constexpr int RS = NARROW_ROWS / 16, QS = NARROW_BN / 16;
     constexpr int KBLK  = NB * 3;         // k blocks the loop covers (the B panel is zero beyond K)
-    constexpr int PITCH = KBLK * 64 + 16; // bytes per B row in LDS
+    constexpr int PITCH = KBLK * 64 + NARROW_PAD_PIECES * 16; // bytes per B row in LDS
     constexpr int NPAR  = 1 + QP_COUNT;
     extern __shared__ __attribute__((aligned(16))) char smem[]; // B panel [npan * 64][PITCH], then par[NPAR][npan * 64]
 
@@ -142,10 +148,10 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
         qflag = *(const MI355_GLOBAL int32_t *)u_fl;
 
     // ---- B panel: straight into LDS (no registers), issued before the A loads, which are needed later. The host keeps
-    // the panel in global memory exactly as it lies in LDS (rows of CHUNKS pieces of 16 bytes plus one of padding,
+    // the panel in global memory exactly as it lies in LDS (rows of CHUNKS pieces of 16 bytes plus NARROW_PAD_PIECES of padding,
     // zero beyond Kp), so it moves as NDMA linear transfers of 1 KiB; wave w issues transfers w, w + 4, ... ----
     constexpr int  CHUNKS = KBLK * 4;       // 16-byte pieces of a row that hold data
-    constexpr int  NDMA   = CHUNKS + 1;     // 64 rows x (CHUNKS + 1) pieces / 64 pieces per transfer
+    constexpr int  NDMA   = CHUNKS + NARROW_PAD_PIECES; // 64 rows x that many pieces / 64 pieces per transfer
     constexpr int  DPW    = (NDMA + NARROW_WAVES - 1) / NARROW_WAVES;
     const uint32_t lds0   = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
     if (NB == 1)
@@ -392,6 +398,321 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 #undef MI355_GLOBAL
 }
 
+// ---- the same convolution for large images: the input rows a workgroup needs, staged once in LDS ---------------------
+// Above, every wave fetches its 32 patches tap by tap from global memory: KH * KW times the image crosses the compute
+// unit's vector-memory path (one 1 KiB load instruction every 20 clocks or so, whatever the caches hold), and with more
+// than a few tiles per compute unit that path, not the matrix cores, sets the time (config 4 of the benchmark: 327 KiB
+// per compute unit = 3 us of an 8.5 us kernel, and 1.9 us more for the B panel that each of its three workgroups
+// copies). Here ONE workgroup of 16 waves takes a band of output rows of one image: the window of input rows and
+// columns under the band (band + halo + padding) is copied into LDS once, next to the one B panel, by direct-to-LDS
+// loads - a lane of a transfer fetches 16 bytes of a pixel, or 16 bytes of the padding value where the window leaves the
+// image; the 16-byte pieces of a pixel are permuted so that the 16 pixels of an operand read fall into 16 bank groups -
+// and every wave forms the operand blocks of its 32 output pixels with per-lane LDS addresses: a tap is a shift of the
+// pixel index, no test. (With the tests and a select per tap and row the kernel was bound by the vector ALU, not by
+// the matrix cores or LDS: 700 issue slots per wave, a third of them in the k loop.)
+// Needs C a power of two >= 64 (a 64-byte k block then lies inside one tap and one pixel), N <= 64, K <= 1152.
+constexpr int HALO_WAVES = 16;
+
+// Measurement build only (-DMI355_PHASE_CLOCKS, a library of its own that the product never loads): the first lane of
+// wave 0 and of wave 12 of the first, the middle and the last workgroup leaves the 100 MHz real-time counter at the ends
+// of the kernel's parts.
+#ifdef MI355_PHASE_CLOCKS
+__device__ long long band_clocks[6][8];
+#define MI355_BAND_PHASE(i)                                   \
+    do                                                        \
+    {                                                         \
+        if (band_row >= 0 && lane == 0)                       \
+            band_clocks[band_row][i] = (long long)wall_clock64(); \
+    } while (0)
+#else
+#define MI355_BAND_PHASE(i) \
+    do                      \
+    {                       \
+    } while (0)
+#endif
+
+template <int EPI, bool FLIP_A, int NB>
+__global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_halo_kernel(GemmArgs g)
+{
+    constexpr int RS = NARROW_ROWS / 16, QS = NARROW_BN / 16;
+    constexpr int KBLK  = NB * 3;
+    constexpr int PITCH = KBLK * 64 + NARROW_PAD_PIECES * 16;
+    constexpr int NPAR  = 1 + QP_COUNT;
+    // LDS: B panel [64][PITCH] | par[NPAR][64] | (to the next KiB) the staged window
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+#define MI355_GLOBAL __attribute__((address_space(1)))
+    ConvGeom  cg = g.conv;
+    uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp,
+              u_fl = (uintptr_t)g.epi.qp_flag;
+    int32_t   a_qps = (int32_t)g.epi.qp_stride, wpi = g.tiles_m, rpw = g.tiles_n; // workgroups per image, output rows per workgroup
+    uint32_t  magic_wp = g.magic_tiles; // for the division by the staged window's width (see halo_plan)
+    uintptr_t u_fill   = (uintptr_t)g.fill16;
+    asm volatile("" : "+s"(magic_wp), "+s"(u_fill));
+    asm volatile(""
+                 : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KH), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x),
+                   "+s"(cg.stride_y), "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word),
+                   "+s"(cg.magic_C), "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp),
+                   "+s"(u_fl), "+s"(wpi), "+s"(rpw));
+    int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
+    const MI355_GLOBAL int8_t *const  gB = (const MI355_GLOBAL int8_t *)u_b;
+    const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lh = lane >> 4;
+#ifdef MI355_PHASE_CLOCKS
+    const int band_blk = blockIdx.x == 0 ? 0 : (blockIdx.x == gridDim.x / 2 ? 1 : (blockIdx.x == gridDim.x - 1 ? 2 : -1));
+    const int band_row = band_blk < 0 ? -1 : (wave == 0 ? band_blk * 2 : (wave == 12 ? band_blk * 2 + 1 : -1));
+#endif
+    MI355_BAND_PHASE(0); // arguments fetched
+
+    // this workgroup's band: output rows [oy0, oy1) of image n. Staged in LDS: the window of input rows and columns
+    // under it, padding included - rows iy_first .. iy_first + in_rows - 1, columns -pad_left .. -pad_left + Wp - 1,
+    // pixel (r, x) of the window at pixel index r * Wp + x - so that a tap is an address and nothing else
+    const int n = (int)blockIdx.x / wpi, part = (int)blockIdx.x - n * wpi;
+    const int oy0 = part * rpw, oy1 = min(cg.OH, oy0 + rpw);
+    const int P        = (oy1 - oy0) * cg.OW; // output pixels of the band (<= 16 tiles of 32)
+    const int Wp       = (cg.OW - 1) * cg.stride_x + (cg.KW - 1) * cg.dil_x + 1;
+    const int in_rows  = (oy1 - oy0 - 1) * cg.stride_y + (cg.KH - 1) * cg.dil_y + 1;
+    const int iy_first = oy0 * cg.stride_y - cg.pad_top;
+    const int staged   = in_rows * Wp;              // pixels
+    const int m_base   = (n * cg.OH + oy0) * cg.OW; // GEMM row of the band's first pixel
+    // pieces of 16 bytes per pixel and the permutation of a pixel's pieces: piece c of the pixel at LDS pixel index s
+    // (counted from the start of LDS: img_off is a multiple of the pixel size) lies at position
+    // c ^ (((s >> sw_sh) & sw_m) << 1). With lane l at pixel s + l % 16, piece l / 16 of a block of 4, each of the
+    // four batches of 16 lanes a ds_read_b128 is served in (see NARROW_PAD_PIECES) then has its 16 addresses distinct
+    // modulo 256 bytes for pixels of 4, 8 and 16 or more pieces (checked by enumeration for every start s).
+    const int cpr = cg.C >> 4, lcpr = 31 - __builtin_clz(cpr), lc = lcpr + 4;
+    const int sw_m = cpr >= 16 ? 7 : (cpr == 8 ? 3 : 1), sw_sh = cpr >= 16 ? 0 : (cpr == 8 ? 1 : 2);
+    const int sw_l = 5 - sw_sh, sw_mask = sw_m << 5; // the permutation as a byte offset: ((s << sw_l) & sw_mask) ^ piece * 16
+    const uint32_t lds0    = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const int      img_off = (NARROW_BN * PITCH + NPAR * NARROW_BN * 4 + 1023) & ~1023;
+    const int      s_img   = img_off >> lc; // LDS pixel index of the window's first pixel
+
+    // epilogue constants (one dword per thread: 6 x 64 of them), the flag word of the requantisation
+    const bool have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
+    int32_t    tp      = 0;
+    if (have_qp)
+    {
+        const int idx = min(tid, NPAR * NARROW_BN - 1);
+        const int v = idx / NARROW_BN, col = idx - v * NARROW_BN;
+        tp          = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
+    }
+    int qflag = 1;
+    if (have_qp && u_fl != 0)
+        qflag = *(const MI355_GLOBAL int32_t *)u_fl;
+
+    // ---- B panel and the staged window: transfers of 1 KiB, dealt out to the 16 waves. A lane of a window transfer
+    // fetches the piece its LDS position stands for from the image, or 16 bytes of the padding value ----
+    constexpr int   NDMA = KBLK * 4 + NARROW_PAD_PIECES;
+    const int       nimg = ((staged << lc) + 1023) >> 10;
+    const uintptr_t img  = u_a + (uintptr_t)((int64_t)n * cg.H * cg.W * cg.C);
+    for (int ins = wave; ins < NDMA + nimg; ins += HALO_WAVES)
+    {
+        if (ins < NDMA)
+            narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
+        else
+        {
+            const int q = (ins - NDMA) * 64 + lane; // position in the window, in pieces
+            const int s = q >> lcpr, c = (q & (cpr - 1)) ^ ((((s + s_img) >> sw_sh) & sw_m) << 1);
+            const int r = narrow_div(s, magic_wp), x = s - r * Wp;
+            const int iy = iy_first + r, ix = x - cg.pad_left;
+            // (lanes past the window's end fill LDS nobody looks at)
+            const bool      in   = (s < staged) & ((unsigned)iy < (unsigned)cg.H) & ((unsigned)ix < (unsigned)cg.W);
+            const uintptr_t from = in ? img + (uint32_t)(((iy * cg.W + ix) << lc) + c * 16) : u_fill;
+            narrow_dma16_at((const void *)from, lds0 + (uint32_t)img_off + (uint32_t)(ins - NDMA) * 1024u);
+        }
+    }
+
+    // ---- this wave's tile: 32 consecutive pixels of the band ----
+    const bool active = wave * NARROW_ROWS < P;
+    int32_t    s0[RS]; // LDS pixel index of the top-left tap of each of the tile's rows
+#pragma unroll
+    for (int rb = 0; rb < RS; ++rb)
+    {
+        const int lp = min(wave * NARROW_ROWS + rb * 16 + lr, P - 1);
+        const int ry = narrow_div(lp, cg.magic_OW), ox = lp - ry * cg.OW;
+        s0[rb]       = s_img + ry * cg.stride_y * Wp + ox * cg.stride_x;
+    }
+    MI355_BAND_PHASE(1); // transfers issued, addresses set up
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's transfers (and its constant)
+    MI355_BAND_PHASE(2); // this wave's transfers have landed
+    if (have_qp && tid < NPAR * NARROW_BN)
+        par[tid] = tp;
+    const int  qflag_u = __builtin_amdgcn_readfirstlane(qflag);
+    const bool fast    = have_qp && (qflag_u & 1) == 0;
+    __syncthreads();
+    MI355_BAND_PHASE(3); // everybody's transfers have landed
+    if (!active)
+        return;
+
+    // waves that share a SIMD (w, w + 4, w + 8, w + 12) get different priorities: one at a time goes through the matrix
+    // instructions and its epilogue then runs beside the matrix instructions of the next
+    switch ((wave >> 2) & 3)
+    {
+    case 0: __builtin_amdgcn_s_setprio(3); break;
+    case 1: __builtin_amdgcn_s_setprio(2); break;
+    case 2: __builtin_amdgcn_s_setprio(1); break;
+    default: break;
+    }
+    // (One instance of what follows for every wave: a second, for a last tile of 16 pixels or fewer, measured slower -
+    // the code is fetched once per workgroup, a path that one wave takes alone pays for its own instruction fetches.)
+    {
+        constexpr int RSX = RS;
+        v4i acc[RSX][QS];
+#pragma unroll
+        for (int i = 0; i < RSX; ++i)
+#pragma unroll
+            for (int j = 0; j < QS; ++j)
+                acc[i][j] = (v4i){0, 0, 0, 0};
+        const char *b_rd  = smem + lr * PITCH + lh * 16;
+        const int   nkb   = (g.K + 63) >> 6; // k blocks that hold data (the panel is zero beyond)
+        // operand blocks of k block kb: B from the panel, A from the staged window
+        auto read_ops = [&](int kb, v4i (&fa)[RSX], v4i (&fb)[QS])
+        {
+            // (scalar. K may end before the last batch of 3 k blocks does: those blocks meet zeros in the panel and read
+            // the first tap again)
+            const int kbe = kb < nkb ? kb : 0;
+            const int tap = narrow_div(kbe * 64, cg.magic_C), c64 = kbe * 64 - tap * cg.C;
+            const int ky = narrow_div(tap, cg.magic_KW), kx = tap - ky * cg.KW;
+            const int ds = ky * cg.dil_y * Wp + kx * cg.dil_x;
+            const int pc = c64 + lh * 16; // this lane's 16 bytes within the pixel
+#pragma unroll
+            for (int q = 0; q < QS; ++q)
+                fb[q] = *(const v4i *)(b_rd + q * 16 * PITCH + kb * 64);
+#pragma unroll
+            for (int rb = 0; rb < RSX; ++rb)
+            {
+                const int s = s0[rb] + ds;
+                // (C is a power of two: shifts, not a quarter-rate multiply)
+                fa[rb] = *(const v4i *)(smem + ((s << lc) + (((s << sw_l) & sw_mask) ^ pc)));
+            }
+        };
+        v4i fa[2][RSX], fb[2][QS];
+        read_ops(0, fa[0], fb[0]);
+        // Straight-line code over every k block the panel has (a wave-uniform branch per block made the compiler wait for
+        // the operands of the next block before the matrix instructions of this one). K may end before the last batch of 3
+        // blocks does: there the panel holds zeros.
+#pragma unroll
+        for (int kb = 0; kb < KBLK; ++kb)
+        {
+            if (kb + 1 < KBLK)
+                read_ops(kb + 1, fa[(kb + 1) & 1], fb[(kb + 1) & 1]);
+#pragma unroll
+            for (int rb = 0; rb < RSX; ++rb)
+            {
+                v4i a = fa[kb & 1][rb];
+                if (FLIP_A)
+                    a ^= (int)0x80808080;
+#pragma unroll
+                for (int q = 0; q < QS; ++q)
+                    acc[rb][q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[kb & 1][q], a, acc[rb][q], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_s_setprio(0);
+        MI355_BAND_PHASE(4); // matrix instructions issued
+
+        const int row0 = m_base + wave * NARROW_ROWS, a_M = m_base + P; // rows of the GEMM this tile covers, and where the band ends
+        if (fast && g.epi.qp_pk16 && (qflag_u & 3) == 0 && g.epi.vec_store && (g.N & 3) == 0)
+        {
+            // the short form of the requantisation, 4 columns at a time: lane l holds, for row rb * 16 + l % 16, the 4
+            // consecutive columns q * 16 + 4 * (l / 16) + {0..3}
+            const int16_t  o16 = (int16_t)(2 * g.epi.result_offset + 1), lo16 = (int16_t)g.epi.lo, hi16 = (int16_t)g.epi.hi;
+            const pk16_t   off2p1 = {o16, o16}, lo = {lo16, lo16}, hi = {hi16, hi16};
+            const int32_t *rowvec = g.epi.rowvec;
+            const int      a_N    = g.N;
+            int32_t        rv[RSX];
+            char          *drow[RSX];
+#pragma unroll
+            for (int rb = 0; rb < RSX; ++rb)
+            {
+                const int i = row0 + rb * 16 + lr;
+                rv[rb]      = (rowvec && i < a_M) ? rowvec[i] : 0;
+                drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + 4 * lh;
+            }
+#pragma unroll
+            for (int q = 0; q < QS; ++q)
+            {
+                const int c  = q * 16 + 4 * lh;
+                const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * NARROW_BN + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * NARROW_BN + c);
+                const v4i cv = *(const v4i *)(par + c);
+                const int32_t s2a[4] = {s2[0], s2[1], s2[2], s2[3]}, r1a[4] = {r1[0], r1[1], r1[2], r1[3]};
+#pragma unroll
+                for (int rb = 0; rb < RSX; ++rb)
+                {
+                    int32_t v[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        v[t] = (int32_t)((uint32_t)acc[rb][q][t] + (uint32_t)cv[t] + (uint32_t)rv[rb]);
+                    const uint32_t w = std_requant4_pk16(v, s2a, r1a, off2p1, lo, hi);
+                    if (row0 + rb * 16 + lr < a_M && c < a_N)
+                        *(uint32_t *)(drow[rb] + q * 16) = w;
+                }
+            }
+        }
+        else
+        {
+            // the general forms check rows against g.M: the band's end stands in for it
+            GemmArgs gl = g;
+            gl.M        = a_M;
+            if (fast)
+                epilogue_store_fast<RSX, QS, NARROW_BN>(acc, gl, par, row0, 0, 0, lane, 0);
+            else
+                epilogue_store_t<EPI, RSX, QS>(acc, gl, row0, 0, lane, 0);
+        }
+    }
+    MI355_BAND_PHASE(5); // stores issued
+#undef MI355_GLOBAL
+}
+
+template <int EPI, bool FLIP_A>
+static const void *halo_fn(int nb)
+{
+    switch (nb)
+    {
+    case 1: return (const void *)conv_halo_kernel<EPI, FLIP_A, 1>;
+    case 2: return (const void *)conv_halo_kernel<EPI, FLIP_A, 2>;
+    case 3: return (const void *)conv_halo_kernel<EPI, FLIP_A, 3>;
+    case 4: return (const void *)conv_halo_kernel<EPI, FLIP_A, 4>;
+    case 5: return (const void *)conv_halo_kernel<EPI, FLIP_A, 5>;
+    case 6: return (const void *)conv_halo_kernel<EPI, FLIP_A, 6>;
+    }
+    return nullptr;
+}
+
+// The band form for this convolution? Fills rows-per-workgroup / workgroups-per-image / LDS bytes when it applies: more
+// tiles of 32 pixels than 4 per compute unit, C a power of two from 64 on, one panel of columns, and a band whose pixels
+// (at most 16 tiles) and input window fit one workgroup; magic_wp: the reciprocal (see ConvGeom) of the window's width.
+static bool halo_plan(const GemmArgs &a, int epi, int cus, int &rpw, int &wpi, size_t &lds, uint32_t &magic_wp)
+{
+    const ConvGeom &c = a.conv;
+    if (cus <= 0 || (epi != EPI_FIXEDPOINT && epi != EPI_F32) || a.N > NARROW_BN || c.C < 64 || (c.C & (c.C - 1)) != 0 || c.C > 1024)
+        return false;
+    const int64_t images = (int64_t)a.M / ((int64_t)c.OH * c.OW);
+    if (images * c.OH * c.OW != a.M || (a.M + NARROW_ROWS - 1) / NARROW_ROWS <= (int64_t)NARROW_WAVES * cus)
+        return false;
+    if (c.OW > HALO_WAVES * NARROW_ROWS)
+        return false;
+    const int nb = (a.K + 191) / 192;
+    // as many workgroups as compute units where the images allow it, bands no longer than 16 tiles
+    const int most = HALO_WAVES * NARROW_ROWS / c.OW; // output rows whose pixels fit the 16 waves
+    int       parts = (int)std::max<int64_t>(1, ((int64_t)cus + images - 1) / images);
+    parts           = std::min(parts, c.OH);
+    rpw             = std::min(most, (c.OH + parts - 1) / parts);
+    wpi             = (c.OH + rpw - 1) / rpw;
+    // the staged window: band + halo + padding (see the kernel)
+    const int64_t in_rows = (int64_t)(rpw - 1) * c.stride_y + (int64_t)(c.KH - 1) * c.dil_y + 1;
+    const int64_t wp      = (int64_t)(c.OW - 1) * c.stride_x + (int64_t)(c.KW - 1) * c.dil_x + 1;
+    const int64_t img_off = ((int64_t)NARROW_BN * (nb * 192 + NARROW_PAD_PIECES * 16) + (1 + QP_COUNT) * NARROW_BN * 4 + 1023) & ~(int64_t)1023;
+    const int64_t bytes   = img_off + ((in_rows * wp * c.C + 1023) & ~(int64_t)1023);
+    if (bytes > 160 * 1024 || images * wpi > (int64_t)INT32_MAX)
+        return false;
+    magic_wp = wp == 1 ? 0u : (uint32_t)(0x100000000ull / (uint64_t)wp) + 1u; // (pixel indices stay far below 2^32 / wp)
+    lds = (size_t)bytes;
+    return true;
+}
+
 template <int EPI, bool FLIP_A, bool CONV, bool UNI>
 static const void *narrow_fn(int nb)
 {
@@ -443,19 +764,53 @@ bool narrow_applies(const GemmArgs &a, bool conv)
     return ((uintptr_t)a.A & 15) == 0 && a.lda % 16 == 0 && a.K % 16 == 0 && (int64_t)a.M * a.lda < ((int64_t)1 << 31);
 }
 
-int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s)
+int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s, bool *band)
 {
+    if (band)
+        *band = false;
     if (!narrow_applies(args, conv) || args.fill16 == nullptr || epi < 0 || epi > 2)
         return (int)hipErrorInvalidValue;
     const int   nb  = (args.K + 191) / 192;
     const bool  uni = conv && args.conv.C % 64 == 0;
+    if (conv)
+    {
+        int      rpw = 0, wpi = 0;
+        size_t   hl  = 0;
+        uint32_t mwp = 0;
+        if (halo_plan(args, epi, device_cus(), rpw, wpi, hl, mwp))
+        {
+            const void *hf = epi == EPI_FIXEDPOINT ? (flip_a ? halo_fn<EPI_FIXEDPOINT, true>(nb) : halo_fn<EPI_FIXEDPOINT, false>(nb))
+                                                   : (flip_a ? halo_fn<EPI_F32, true>(nb) : halo_fn<EPI_F32, false>(nb));
+            if (hf == nullptr)
+                return (int)hipErrorInvalidValue;
+            static std::atomic<uint32_t> raised_h[2][2][NARROW_MAX_NB];
+            std::atomic<uint32_t>       &done = raised_h[epi == EPI_F32 ? 1 : 0][flip_a ? 1 : 0][nb - 1];
+            int                          dev  = 0;
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
+                return (int)hipErrorInvalidDevice;
+            if ((done.load(std::memory_order_acquire) & (1u << dev)) == 0)
+            {
+                const hipError_t e = hipFuncSetAttribute(hf, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess)
+                    return (int)e;
+                done.fetch_or(1u << dev, std::memory_order_release);
+            }
+            GemmArgs a = args;
+            a.tiles_m = wpi, a.tiles_n = rpw, a.magic_tiles = mwp;
+            const int64_t images = (int64_t)args.M / ((int64_t)args.conv.OH * args.conv.OW);
+            void         *kargs[] = {&a};
+            if (band)
+                *band = true;
+            return (int)hipLaunchKernel(hf, dim3((unsigned)(images * wpi)), dim3(HALO_WAVES * 64), kargs, hl, s);
+        }
+    }
     const void *fn  = epi == EPI_S32 ? narrow_fn_e<EPI_S32>(flip_a, conv, uni, nb)
                       : epi == EPI_FIXEDPOINT ? narrow_fn_e<EPI_FIXEDPOINT>(flip_a, conv, uni, nb)
                                               : narrow_fn_e<EPI_F32>(flip_a, conv, uni, nb);
     if (fn == nullptr)
         return (int)hipErrorInvalidValue;
     const int    npan = (args.N + NARROW_BN - 1) / NARROW_BN;
-    const size_t lds  = (size_t)npan * NARROW_BN * (nb * 192 + 16) + (size_t)(1 + QP_COUNT) * npan * NARROW_BN * sizeof(int32_t);
+    const size_t lds  = (size_t)npan * NARROW_BN * (nb * 192 + NARROW_PAD_PIECES * 16) + (size_t)(1 + QP_COUNT) * npan * NARROW_BN * sizeof(int32_t);
     if (lds > 48 * 1024)
     {
         // once per kernel and device (for the largest panel count the kernel may meet)
@@ -504,3 +859,11 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
     return (int)hipLaunchKernel(fn, dim3(grid), dim3(NARROW_WAVES * 64), kargs, lds, s);
 }
 } // namespace mi355
+
+#ifdef MI355_PHASE_CLOCKS
+// 6 rows (first / middle / last workgroup x wave 0, wave 12) of 8 readings of the 100 MHz counter, of the last launch
+extern "C" int mi355_band_clocks_read(long long *out)
+{
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mi355::band_clocks), sizeof(long long) * 48);
+}
+#endif

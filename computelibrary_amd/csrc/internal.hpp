@@ -98,10 +98,16 @@ int         dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmA
 
 // gemm_narrow.hip — N <= 64, K <= 1152, 16-byte aligned operands: A straight from global memory into the matrix cores'
 // operand layout, B resident in LDS; dense or implicit convolution (C % 16 == 0). needs args.fill16
-// (args.Bp: the image written by pack_b_narrow_launch with narrow_panel_chunks(K) pieces per row)
+// (args.Bp: the image written by pack_b_narrow_launch with narrow_panel_chunks(K) + NARROW_PAD_PIECES pieces per row)
 int  narrow_panel_chunks(int K); // 0: K outside the kernel's range
+// Pieces of padding after each row of that image. A ds_read_b128 goes through LDS in four batches of 16 lanes - lanes
+// {0-3, 12-15, 20-23, 24-27}, {4-11, 16-19, 28-31} and the same of the upper half - and a batch is free of bank
+// conflicts when its 16 addresses differ modulo 256 bytes: with lane l at row l % 16, piece l / 16 that holds for a row
+// pitch of 32 modulo 64 bytes (measured: 2.8 clocks per instruction and compute unit against 4.6 with 16 modulo 64).
+constexpr int NARROW_PAD_PIECES = 2;
 bool narrow_applies(const GemmArgs &args, bool conv);
-int  narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s);
+// *band (when given): whether the launch took the form that stages a band of input rows in LDS (large images)
+int  narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStream_t s, bool *band = nullptr);
 
 // gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 64;

@@ -289,15 +289,16 @@ int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int
     return launch_status();
 }
 
-// The first `rows` (a multiple of 64) rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus one piece of
-// padding, zero beyond Kp - the workgroups copy this image into LDS with plain linear transfers
+// The first `rows` (a multiple of 64) rows of Bp as the narrow kernel keeps them in LDS: rows of `chunks` 16-byte pieces of data plus
+// NARROW_PAD_PIECES of padding, zero beyond Kp - the workgroups copy this image into LDS with plain linear transfers
 __global__ __launch_bounds__(256) void pack_b_narrow_kernel(const int8_t *__restrict__ Bp, int Kp, int chunks, int rows,
                                                             int8_t *__restrict__ Bn)
 {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= rows * (chunks + 1))
+    constexpr int PAD = NARROW_PAD_PIECES;
+    if (idx >= rows * (chunks + PAD))
         return;
-    const int r = idx / (chunks + 1), c = idx - r * (chunks + 1);
+    const int r = idx / (chunks + PAD), c = idx - r * (chunks + PAD);
     v4i       v = {0, 0, 0, 0};
     if (c < chunks && c * 16 < Kp)
         v = *(const v4i *)(Bp + (int64_t)r * Kp + c * 16);
@@ -308,7 +309,7 @@ int pack_b_narrow_launch(const int8_t *Bp, int Kp, int Np, int chunks, int rows,
 {
     if (Kp % 16 || rows < 64 || rows % 64 != 0 || Np < rows || chunks < 1)
         return (int)hipErrorInvalidValue;
-    pack_b_narrow_kernel<<<dim3((rows * (chunks + 1) + 255) / 256), dim3(256), 0, s>>>(Bp, Kp, chunks, rows, Bn);
+    pack_b_narrow_kernel<<<dim3((rows * (chunks + NARROW_PAD_PIECES) + 255) / 256), dim3(256), 0, s>>>(Bp, Kp, chunks, rows, Bn);
     return launch_status();
 }
 

@@ -175,6 +175,79 @@ def test_conv_few_output_channels_kernel():
             got, oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, -5, -128, 127, (1, 1), (4, 4, 4, 4), (1, 1)))
 
 
+def test_conv_few_output_channels_large_images_band_form():
+    """With more than 4 tiles of 32 output pixels per compute unit (and C a power of two from 64 on) the kernel above
+    gives way to the form in which one workgroup stages the window of input rows under a band of output rows in LDS -
+    padding included - and every tap is an LDS address: bands that do not divide the image height, a last tile of
+    a few pixels, signed and unsigned sources (non-zero padding values), asymmetric padding, strides, dilation, 40 and
+    33 output channels, C = 64 / 128 / 256, a 1 x 1 kernel whose K ends before its batch of k blocks does, weights with an
+    offset (row sums of the patches), requantisation constants outside the short form, and the F32 destination."""
+    rng = np.random.default_rng(707)
+    cases = [
+        # (src shape, weights shape, stride, pad, dilation, src dtype, weights dtype, weights zero point)
+        ((8, 72, 72, 64), (64, 3, 3, 64), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, np.int8, 0),
+        ((2, 150, 150, 64), (40, 3, 3, 64), (1, 1), (1, 0, 2, 1), (1, 1), np.uint8, np.int8, 0),
+        ((4, 200, 190, 64), (64, 3, 3, 64), (2, 2), (1, 1, 1, 1), (1, 1), np.int8, np.int8, 0),
+        ((2, 140, 140, 64), (33, 3, 3, 64), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8, np.int8, 0),
+        ((2, 132, 132, 128), (64, 3, 3, 128), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, np.int8, 0),
+        ((1, 190, 190, 256), (64, 1, 1, 256), (1, 1), (0, 0, 0, 0), (1, 1), np.int8, np.int8, 0),
+        ((1, 420, 170, 64), (64, 2, 3, 64), (1, 2), (0, 1, 1, 0), (1, 1), np.uint8, np.uint8, 131),
+    ]
+    for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp) in cases:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        for per_channel in (True, False):
+            reals = rng.uniform(0.5, 2.0, wshape[0] if per_channel else 1) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            if per_channel and shape[0] == 2:
+                mult[1], shift[1] = 1 << 29, -1   # a multiplier below 2^30 and a left shift: not the short form
+            want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert 0.1 < ((want > lo) & (want < hi)).mean()
+            announce("conv band form", shape, wshape, stride, pad, dil, dt.__name__, w_dt.__name__, w_zp, "per_channel", per_channel)
+            got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert name == "implicit_band_32x64", name
+            np.testing.assert_array_equal(got, want)
+    # a result offset beyond what the 16-bit tail of the short form takes: the general short form, same bits
+    src = rng.integers(-128, 128, size=(8, 72, 72, 64), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(64, 3, 3, 64), dtype=np.int8)
+    bias = rng.integers(-500, 500, size=64, dtype=np.int32)
+    mult, shift = oracle.calculate_quantized_multipliers(1.0, np.full(64, 40.0 / (24.0 * 74.0 * 74.0)), 1.0)
+    import torch
+    rq = capi.requant(0, 0, 3000, -32768, 32767, True)
+    cv = capi.Conv(capi.conv_desc(8, 72, 72, 64, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.S8, -5, 0, 5, rq))
+    sd, wd, od = to_dev(src), to_dev(w), to_dev(np.zeros((8, 72, 72, 64), np.int8))
+    keep = [to_dev(bias), to_dev(mult), to_dev(shift)]
+    cv.prepare(wd, *keep)
+    announce("conv band form, large result offset", cv.kernel_name)
+    cv.run(sd, od)
+    torch.cuda.synchronize()
+    assert cv.kernel_name == "implicit_band_32x64", cv.kernel_name
+    np.testing.assert_array_equal(od.cpu().numpy(),
+                                  oracle.conv_nhwc_direct(src, w, bias, 5, 0, mult, shift, 3000, -128, 127, (1, 1), (1, 1, 1, 1), (1, 1)))
+    cv.close()
+    # F32 destination
+    src = rng.integers(-128, 128, size=(2, 140, 130, 64), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(48, 3, 3, 64), dtype=np.int8)
+    bias_f = rng.normal(0.0, 2.0, size=48).astype(np.float32)
+    scale = float(np.float32(0.02) * np.float32(0.005))
+    cols = oracle.im2col_nhwc(src, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 4)
+    want = oracle.gemmlowp_f32(cols, oracle.weights_reshape(w), bias_f, -4, 0, scale, 0.0, 6.0, act_twice=False)
+    cv = capi.Conv(capi.conv_desc(2, 140, 130, 64, 48, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.F32, -4, 0, 4,
+                                  scale=scale, act=(0.0, 6.0)))
+    sd, wd, od, bd = to_dev(src), to_dev(w), to_dev(np.zeros((2, 140, 130, 48), np.float32)), to_dev(bias_f)
+    cv.prepare(wd, bd)
+    announce("conv band form, F32 destination", cv.kernel_name)
+    cv.run(sd, od)
+    torch.cuda.synchronize()
+    assert cv.kernel_name == "implicit_band_32x64", cv.kernel_name
+    assert np.array_equal(od.cpu().numpy().reshape(-1, 48).view(np.uint32), want.view(np.uint32))
+    cv.close()
+
+
 def test_conv_channel_counts_padded_to_16():
     """A channel count that is not a multiple of 16: pixels and taps are copied with the channels padded to the next
     multiple of 16 and the fast implicit kernels run (never the byte-wise fallback), with identical results - the RGB of

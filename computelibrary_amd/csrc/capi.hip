@@ -172,7 +172,7 @@ struct GemmCore
     DevBuf  Bp, Bs, Bn, colsum, colvec, rowvec, mult, shift, bias, Ap, fill, qp, zeros, parts, zerocol;
     int     splitk = 1;      // K slices of the pipelined kernel
     int     splitk_plan = 1; // what the cost model chose with the tile shape (create()); prepare() checks it and allocates
-    bool    conv_core = false; // the GEMM inside a convolution handle: its implicit loader takes no K slices
+    bool    conv_core = false; // the GEMM inside a convolution handle
     int     k_const = 0;       // > 0: the K of the constant term a_offset * b_offset * K, where the kernels' K counts padded channels
     bool    qp_on = false; // the digested requantisation vectors (and the flag word behind them) exist
     std::string kname_mfma, kname_dma, kprefix;
@@ -280,7 +280,7 @@ struct GemmCore
                     const double fixed   = 6000.0 + (double)c.BM * c.BN / 4.4;
                     for (int sl = 1; sl <= 8; sl *= 2)
                     {
-                        if (sl > 1 && (conv_core || batch != 1 || K % (sl * c.BK) != 0 || K / sl < 1024))
+                        if (sl > 1 && (batch != 1 || K % (sl * c.BK) != 0 || K / sl < 1024))
                             break;
                         const double per_cu = std::ceil(tiles * sl / cus);
                         const double finish = sl > 1 ? 4000.0 + (double)sl * M * N * 4.0 / (2.5 * cus) : 0.0;
@@ -299,7 +299,7 @@ struct GemmCore
                 dma_idx = force_tile, splitk_plan = 1;
                 const MfmaConfig c     = dma_config(dma_idx);
                 const int64_t    tiles = (int64_t)((M + c.BM - 1) / c.BM) * ((N + c.BN - 1) / c.BN);
-                if (batch == 1 && !conv_core && tiles * 2 <= cus && K >= 2048)
+                if (batch == 1 && tiles * 2 <= cus && K >= 2048)
                 {
                     int sl = (int)std::min<int64_t>(std::min<int64_t>(cus / tiles, K / 1024), 8);
                     while (sl > 1 && K % (sl * c.BK) != 0)
@@ -492,16 +492,12 @@ struct GemmCore
         if (!direct)
         {
             // rows not dword aligned: padded, sign-normalised copy (and the row sums in the same pass)
-            for (int b = 0; b < batch; ++b)
-                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, ap + (size_t)b * M * Kp, Kp,
-                                         need_rowvec ? rv + (size_t)b * M : nullptr, b_off_eff(), s));
+            HIP_TRY(a_prepass_launch(A, lda, a_bs, batch, M, K, flip_a, ap, Kp, need_rowvec ? rv : nullptr, b_off_eff(), s));
             A = ap, lda = Kp, a_bs = (int64_t)M * Kp, k_valid = Kp, flip_in_loader = false;
         }
         else if (need_rowvec)
         {
-            for (int b = 0; b < batch; ++b)
-                HIP_TRY(a_prepass_launch(A + (size_t)b * a_bs, lda, M, K, flip_a, nullptr, Kp, rv + (size_t)b * M,
-                                         b_off_eff(), s));
+            HIP_TRY(a_prepass_launch(A, lda, a_bs, batch, M, K, flip_a, nullptr, Kp, rv, b_off_eff(), s));
         }
         if (rowsum_in_kernel)
             g.epi.rowsum_mul = b_off_eff();
@@ -531,18 +527,28 @@ struct GemmCore
             HIP_TRY(simple_gemm_launch(epi, flip_in_loader, g, batch, s));
         else if (path == MI355_PATH_SKINNY)
         {
-            // one launch per batch entry, each with its own operands and per-column / per-row vectors
-            for (int b = 0; b < batch; ++b)
-            {
-                GemmArgs gb = g;
-                gb.A        = g.A + (int64_t)b * g.a_batch_stride;
-                gb.Bp       = Bs.as<int8_t>() + (b_shared ? 0 : (int64_t)b * Np * Kp);
-                gb.D        = (char *)g.D + (int64_t)b * g.d_batch_stride * (epi == EPI_FIXEDPOINT ? 1 : 4);
-                gb.epi.colvec += (int64_t)b * g.epi.colvec_batch_stride;
-                if (g.epi.rowvec != zeros.as<int32_t>() && g.epi.rowvec != nullptr)
-                    gb.epi.rowvec += (int64_t)b * g.epi.rowvec_batch_stride;
-                HIP_TRY(skinny_launch(epi, flip_in_loader, gb, s, &kname_static));
-            }
+            GemmArgs gb        = g;
+            gb.Bp              = Bs.as<int8_t>();
+            gb.bp_batch_stride = b_shared ? 0 : (int64_t)Np * Kp;
+            if (g.epi.rowvec == zeros.as<int32_t>() || g.epi.rowvec == nullptr)
+                gb.epi.rowvec_batch_stride = 0;
+            // A batch of small products (under 4 MiB of B each, where the launches themselves are what costs) goes out
+            // as one launch with the entries along the grid; larger ones one launch per entry, each free to take the
+            // form that stages its A once
+            if (batch > 1 && (int64_t)Np * Kp <= ((int64_t)4 << 20) && batch <= 65535)
+                HIP_TRY(skinny_launch(epi, flip_in_loader, gb, batch, s, &kname_static));
+            else
+                for (int b = 0; b < batch; ++b)
+                {
+                    GemmArgs ge = gb;
+                    ge.A        = gb.A + (int64_t)b * gb.a_batch_stride;
+                    ge.Bp       = gb.Bp + (int64_t)b * gb.bp_batch_stride;
+                    ge.D        = (char *)gb.D + (int64_t)b * gb.d_batch_stride * (epi == EPI_FIXEDPOINT ? 1 : 4);
+                    ge.epi.colvec += (int64_t)b * gb.epi.colvec_batch_stride;
+                    if (ge.epi.rowvec != nullptr)
+                        ge.epi.rowvec += (int64_t)b * gb.epi.rowvec_batch_stride;
+                    HIP_TRY(skinny_launch(epi, flip_in_loader, ge, 1, s, &kname_static));
+                }
         }
         else
         {
@@ -572,7 +578,7 @@ struct GemmCore
                 g.tiles_m          = (g.M + c.BM - 1) / c.BM;
                 g.tiles_n          = (g.N + c.BN - 1) / c.BN;
                 kname_run          = &kname_dma_full;
-                if (splitk > 1 && !conv && batch == 1 && g.K == K && K % (splitk * c.BK) == 0)
+                if (splitk > 1 && batch == 1 && g.K == K && K % (splitk * c.BK) == 0)
                 {
                     const int     ldp = (N + 3) & ~3;
                     const int64_t kc  = K / splitk;
@@ -582,9 +588,11 @@ struct GemmCore
                     gp.epi.colvec_batch_stride = 0;
                     gp.epi.vec_store           = 1;
                     gp.D = parts.as<int32_t>(), gp.ldd = ldp, gp.d_batch_stride = (int64_t)M * ldp;
-                    gp.K = (int)kc, gp.a_batch_stride = kc, gp.bp_batch_stride = kc;
+                    // (dense: a slice starts kc bytes into every row of A; convolution: kc values into every patch,
+                    // which the loader adds to the k it decodes)
+                    gp.K = (int)kc, gp.a_batch_stride = conv ? 0 : kc, gp.bp_batch_stride = kc, gp.k_slice = conv ? (int32_t)kc : 0;
                     kname_run = &kname_splitk;
-                    HIP_TRY(dma_launch(dma_idx, EPI_S32, flip_in_loader, false, gp, splitk, s));
+                    HIP_TRY(dma_launch(dma_idx, EPI_S32, flip_in_loader, conv, gp, splitk, s));
                     HIP_TRY(splitk_finish_launch(epi, g, parts.as<int32_t>(), (int64_t)M * ldp, ldp, splitk, s));
                     return 0;
                 }

@@ -100,6 +100,7 @@ struct PanelProducer
     int           c_iy0[CONV ? LPA : 1], c_ix0[CONV ? LPA : 1]; // conv: its input coordinates
     uint32_t      lds0;
     int           pw, K, lane_id;
+    int           k_base; // conv: first k of this launch entry's slice of the patch
     ConvGeom      conv;
 
     __device__ __forceinline__ void init(const GemmArgs &g, int m0, int n0, int bz, int producer_wave, int lane,
@@ -108,6 +109,7 @@ struct PanelProducer
         pw        = producer_wave;
         lds0      = lds_base;
         K         = g.K;
+        k_base    = CONV ? bz * g.k_slice : 0;
         conv      = g.conv;
         fill16    = g.fill16;
         a_end     = g.a_end;
@@ -177,7 +179,7 @@ struct PanelProducer
         uint32_t t_off = 0;
         if (CONV)
         {
-            const int k   = k0 + c16;
+            const int k   = k_base + k0 + c16; // within the whole patch
             const int tap = fast_div(k, conv.magic_C);
             const int c0  = k - tap * conv.C;
             const int ky  = fast_div(tap, conv.magic_KW);
@@ -185,7 +187,7 @@ struct PanelProducer
             t_dy          = ky * conv.dil_y;
             t_dx          = kx * conv.dil_x;
             t_off         = (uint32_t)((t_dy * conv.W + t_dx) * conv.C + c0);
-            t_in          = k < K;
+            t_in          = k0 + c16 < K;
         }
 #pragma unroll
         for (int i = I0; i < I1; ++i)
@@ -898,8 +900,8 @@ struct DmaEntry
     {                                                                                                                \
         {NAME, BM, BN, BK}, WM *WN * 192, NS * (BM + BN) * BK,                                                        \
         {                                                                                                            \
-            {{MI355_DFN(BM, BN, BK, WM, WN, NS, 0, false, false), nullptr},                                           \
-             {MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, false), nullptr}},                                           \
+            {{MI355_DFN(BM, BN, BK, WM, WN, NS, 0, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 0, false, true)}, \
+             {MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, true)}},  \
                 {{MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, true)}, \
                  {MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, true)}}, \
                 {{MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, true)}, \
@@ -913,7 +915,8 @@ struct DmaEntry
     {                                                                                                                \
         {NAME, BM, BN, BK}, WM *WN * 192, NS * (BM + BN) * BK,                                                        \
         {                                                                                                            \
-            {{MI355_WFN(BM, BN, BK, NS, 0, false), nullptr}, {MI355_WFN(BM, BN, BK, NS, 0, true), nullptr}},          \
+            {{MI355_WFN(BM, BN, BK, NS, 0, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 0, false, true)},                \
+             {MI355_WFN(BM, BN, BK, NS, 0, true), MI355_DFN(BM, BN, BK, WM, WN, NS, 0, true, true)}},                 \
                 {{MI355_WFN(BM, BN, BK, NS, 1, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, false, true)},            \
                  {MI355_WFN(BM, BN, BK, NS, 1, true), MI355_DFN(BM, BN, BK, WM, WN, NS, 1, true, true)}},             \
                 {{MI355_WFN(BM, BN, BK, NS, 2, false), MI355_DFN(BM, BN, BK, WM, WN, NS, 2, false, true)},            \
@@ -965,6 +968,9 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
             fn = g_rowsum_256x128x128[epi][flip_a ? 1 : 0], fn_slot = 2;
     }
     if (fn == nullptr || args.fill16 == nullptr)
+        return (int)hipErrorInvalidValue;
+    // K slices of a convolution: whole K steps, and K names one slice
+    if (args.k_slice != 0 && (!conv || args.K != args.k_slice || args.k_slice % c.cfg.BK != 0 || (int64_t)args.k_slice * batch > args.Kp))
         return (int)hipErrorInvalidValue;
     // shapes the kernel assumes: dword-aligned rows of at least one 16-byte column (whole columns of one tap for the
     // convolution), tiles that cover the output and stay inside the packed B panel

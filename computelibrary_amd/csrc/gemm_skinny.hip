@@ -36,6 +36,17 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
     __shared__ __attribute__((aligned(16))) int32_t red[SK_WAVES][NG][64][4];
     extern __shared__ __attribute__((aligned(16))) char a_stage[]; // STAGE_A: [SK_WAVES][M <= 8][sk_a_pitch(SK_WAVES)]
 
+    // entry blockIdx.y of a batch: every operand moves on by its batch stride (one launch covers the batch)
+    if (gridDim.y > 1)
+    {
+        const int64_t bz = blockIdx.y;
+        g.A += bz * g.a_batch_stride;
+        g.Bp += bz * g.bp_batch_stride;
+        g.D = (char *)g.D + bz * g.d_batch_stride * (EPI == EPI_FIXEDPOINT ? 1 : 4);
+        g.epi.colvec += bz * g.epi.colvec_batch_stride;
+        if (g.epi.rowvec)
+            g.epi.rowvec += bz * g.epi.rowvec_batch_stride;
+    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int ng0  = blockIdx.x * NG; // first of this block's NG groups of 16 columns
@@ -922,10 +933,10 @@ static int raise_lds_limit(const void *fn, size_t lds, std::atomic<uint32_t> &do
 }
 
 template <int NG, int WAVES, int UNROLL, bool STAGE_A, int MR = 1, bool STEP_A = false>
-static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, hipStream_t s)
+static int skinny_launch_v(int epi, bool flip_a, const GemmArgs &a, int batch, hipStream_t s)
 {
     const int    groups = (a.N + 15) / 16;
-    const dim3   grid((groups + NG - 1) / NG), block(WAVES * 64);
+    const dim3   grid((groups + NG - 1) / NG, batch), block(WAVES * 64);
     const size_t lds = STAGE_A ? (size_t)WAVES * 8 * sk_a_pitch(WAVES) : (STEP_A ? (size_t)WAVES * MR * 16 * ((MR == 4 ? 4 : 8) * 64 + 16) : 0);
     if (epi != EPI_S32 && epi != EPI_FIXEDPOINT && epi != EPI_F32)
         return (int)hipErrorInvalidValue;
@@ -1060,25 +1071,28 @@ static int once_grid(int groups, int cus)
     return cus * ((groups + ONCE_MAX_GROUPS * cus - 1) / (ONCE_MAX_GROUPS * cus));
 }
 
-int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, const char **variant)
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s, const char **variant)
 {
     const char *unused;
     const char *&form = variant ? *variant : unused;
     form = "skinny_stream";
-    if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp)
+    if (args.M < 1 || args.M > SKINNY_MAX_M || args.Kp % 64 != 0 || args.K > args.Kp || batch < 1 || batch > 65535)
         return (int)hipErrorInvalidValue;
     const int groups = (args.N + 15) / 16;
     const int KB     = (int)(args.Kp / 64);
     // Up to 8 rows every wave copies its K slice of A (at most 1 KiB per row) into LDS once and takes its operands
     // from there; that needs nothing to guard
-    const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0;
+    const bool align_ok = args.K == args.Kp && args.K % 64 == 0 && args.lda % 16 == 0 && ((uintptr_t)args.A & 15) == 0 &&
+                          (batch == 1 || args.a_batch_stride % 16 == 0);
+    // (a batch along the grid: the streaming form, whose workgroups need nothing from each other)
+    const bool align_ok1 = align_ok && batch == 1;
     const bool stage_ok = args.M <= 8 && align_ok;
-    const bool once_ok  = args.M <= 32 && align_ok; // the stage-once form also takes one or two full blocks of 16 rows
+    const bool once_ok  = args.M <= 32 && align_ok1; // the stage-once form also takes one or two full blocks of 16 rows
     // Up to 4096 of K the stage-once form (grid: once_grid above), each of the 16 waves owning PER = 1, 2 or 4 k blocks;
     // up to 16 rows it also takes 4096 < K <= 8192 with 8 k blocks per wave (one group's worth of B in flight per wave,
     // refilled half by half - the same bytes as two groups of 4 k blocks).
     // up to 8 rows and 8192 < K <= 16384: the stage-once form for deep K (3 or 4 chunks of 4 k blocks per wave)
-    if (stage_ok && KB > 8 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && epi >= EPI_S32 && epi <= EPI_F32)
+    if (stage_ok && batch == 1 && KB > 8 * ONCE_WAVES && KB <= 16 * ONCE_WAVES && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0 && groups <= cus) // one column group per workgroup
@@ -1089,7 +1103,7 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, con
         }
     }
     // 33 to 64 rows: the same with 8 waves, each holding the operand blocks of its 1, 2, 4 or 8 k blocks of all 64 rows
-    if (args.M > 32 && args.M <= 64 && align_ok && KB <= 8 * 8 && epi >= EPI_S32 && epi <= EPI_F32)
+    if (args.M > 32 && args.M <= 64 && align_ok1 && KB <= 8 * 8 && epi >= EPI_S32 && epi <= EPI_F32)
     {
         const int cus = device_cus();
         if (cus > 0)
@@ -1140,14 +1154,14 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, con
         const int ng     = groups >= 512 ? 2 : 1;
         const int blocks = (groups + ng - 1) / ng;
         if (args.M > 32)
-            return ng == 2 ? skinny_launch_v<2, 4, 8, false, 4, true>(epi, flip_a, args, s)
-                           : skinny_launch_v<1, 4, 8, false, 4, true>(epi, flip_a, args, s);
+            return ng == 2 ? skinny_launch_v<2, 4, 8, false, 4, true>(epi, flip_a, args, batch, s)
+                           : skinny_launch_v<1, 4, 8, false, 4, true>(epi, flip_a, args, batch, s);
         const int w = blocks >= 320 ? 4 : 8;
         if (ng == 2)
-            return w == 4 ? skinny_launch_v<2, 4, 8, false, 2, true>(epi, flip_a, args, s)
-                          : skinny_launch_v<2, 8, 8, false, 2, true>(epi, flip_a, args, s);
-        return w == 4 ? skinny_launch_v<1, 4, 8, false, 2, true>(epi, flip_a, args, s)
-                      : skinny_launch_v<1, 8, 8, false, 2, true>(epi, flip_a, args, s);
+            return w == 4 ? skinny_launch_v<2, 4, 8, false, 2, true>(epi, flip_a, args, batch, s)
+                          : skinny_launch_v<2, 8, 8, false, 2, true>(epi, flip_a, args, batch, s);
+        return w == 4 ? skinny_launch_v<1, 4, 8, false, 2, true>(epi, flip_a, args, batch, s)
+                      : skinny_launch_v<1, 8, 8, false, 2, true>(epi, flip_a, args, batch, s);
     }
     if (args.M > 16)
     {
@@ -1159,8 +1173,8 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, con
         const int blocks = (groups + ng - 1) / ng;
         const int w      = blocks >= 320 ? 4 : 8;
 #define MI355_SKV(NG_, MR_)                                                                          \
-    (w == 4 ? skinny_launch_v<NG_, 4, 2, false, MR_>(epi, flip_a, args, s)                           \
-            : skinny_launch_v<NG_, 8, 2, false, MR_>(epi, flip_a, args, s))
+    (w == 4 ? skinny_launch_v<NG_, 4, 2, false, MR_>(epi, flip_a, args, batch, s)                           \
+            : skinny_launch_v<NG_, 8, 2, false, MR_>(epi, flip_a, args, batch, s))
         if (mr == 2)
             return ng == 2 ? MI355_SKV(2, 2) : MI355_SKV(1, 2);
         return ng == 4 ? MI355_SKV(4, 4) : (ng == 2 ? MI355_SKV(2, 4) : MI355_SKV(1, 4));
@@ -1169,10 +1183,10 @@ int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, con
     // the waves of the unstaged / per-step variants follow the old rule
     const int w1 = groups >= 512 ? 4 : 8;
     if (step) // 9..16 rows
-        return w1 == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, s)
-                       : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, s);
+        return w1 == 4 ? skinny_launch_v<1, 4, 8, false, 1, true>(epi, flip_a, args, batch, s)
+                       : skinny_launch_v<1, 8, 8, false, 1, true>(epi, flip_a, args, batch, s);
     if (stage)
-        return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, s);
-    return w1 == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, s);
+        return waves == 4 ? skinny_launch_v<1, 4, 8, true>(epi, flip_a, args, batch, s) : skinny_launch_v<1, 8, 8, true>(epi, flip_a, args, batch, s);
+    return w1 == 4 ? skinny_launch_v<1, 4, 8, false>(epi, flip_a, args, batch, s) : skinny_launch_v<1, 8, 8, false>(epi, flip_a, args, batch, s);
 }
 } // namespace mi355

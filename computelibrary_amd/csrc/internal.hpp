@@ -51,6 +51,9 @@ struct GemmArgs
     uint32_t magic_tiles, magic_group;
     int32_t  tile_magic_ok;
     int32_t  nblocks; // workgroups of the launch (gridDim.x is a hidden argument behind this block: one more fetch)
+    // implicit convolution whose K range runs as slices (the batch entries of one launch): K values per slice, a whole
+    // number of K steps; entry z covers k in [z * k_slice, (z + 1) * k_slice) of the patch and K holds k_slice. 0: no slices
+    int32_t  k_slice;
 };
 
 struct MfmaConfig
@@ -112,7 +115,7 @@ int  narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStr
 // gemm_skinny.hip — M <= 64, B packed in matrix-core operand order (see pack_b_skinny)
 constexpr int SKINNY_MAX_M = 64;
 // *variant (when given): a static string naming the form of the kernel that ran
-int skinny_launch(int epi, bool flip_a, const GemmArgs &args, hipStream_t s, const char **variant = nullptr);
+int skinny_launch(int epi, bool flip_a, const GemmArgs &args, int batch, hipStream_t s, const char **variant = nullptr);
 
 // kernels_aux.hip
 // B [K][ldb] (row-major, N contiguous) -> Bp [Np][Kp] int8 (flip: xor 0x80), colsum[Np] (sums of the packed int8 values)
@@ -131,9 +134,10 @@ int colvec_launch(const int32_t *colsum, const int32_t *bias, int32_t a_off, int
 // (multiplier, shift) per column -> qp[QP_COUNT][Np]; *neg != 0 afterwards if any multiplier is negative
 int qparams_launch(const int32_t *mult, const int32_t *shift, int32_t mult_s, int32_t shift_s, int N, int Np,
                    int32_t *qp, int32_t *neg, hipStream_t s);
-// A pre-pass: optional padded + flipped copy Ap[M][Kp] and/or rowvec[i] = b_off * sum_k(flip(A[i][k]))
-int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
-                     int32_t b_off, hipStream_t s);
+// A pre-pass over `batch` matrices a_bs bytes apart, one launch: optional padded + flipped copies Ap[batch][M][Kp]
+// and/or rowvec[batch][M], rowvec[b][i] = b_off * sum_k(flip(A_b[i][k]))
+int a_prepass_launch(const void *A, int64_t lda, int64_t a_bs, int batch, int M, int K, bool flip, int8_t *Ap, int Kp,
+                     int32_t *rowvec, int32_t b_off, hipStream_t s);
 // rowvec[m] = b_off * (sum of the sign-normalised patch of output pixel m); g.pad_word = the raw padding byte, replicated
 int conv_rowsum_launch(const void *src, const ConvGeom &g, int M, bool flip, int32_t b_off, int32_t *rowvec, hipStream_t s);
 int output_stage_launch(const int32_t *src, int64_t ld_src, const int32_t *bias, void *dst, int64_t ld_dst, int M,

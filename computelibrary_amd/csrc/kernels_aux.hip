@@ -378,12 +378,13 @@ int qparams_launch(const int32_t *mult, const int32_t *shift, int32_t mult_s, in
 // aligned), optionally reduces it: rowvec[i] = b_off * sum_k flip(A[i][k])
 // (CpuGemmLowpMatrixAReductionKernel, src/cpu/kernels/CpuGemmLowpMatrixReductionKernel.cpp:133-204).
 template <int VEC>
-__global__ __launch_bounds__(256) void a_prepass_kernel(const uint8_t *__restrict__ A, int64_t lda, int K, uint8_t flip,
+__global__ __launch_bounds__(256) void a_prepass_kernel(const uint8_t *__restrict__ A, int64_t lda, int64_t a_bs, int K, uint8_t flip,
                                                         int8_t *__restrict__ Ap, int Kp, int32_t *__restrict__ rowvec,
                                                         uint32_t b_off)
 {
-    const int      row  = blockIdx.x;
-    const uint8_t *src  = A + (int64_t)row * lda;
+    // (grid: rows x batch entries; the copies and the sums of the entries lie one after the other)
+    const int      row  = blockIdx.y * gridDim.x + blockIdx.x;
+    const uint8_t *src  = A + (int64_t)blockIdx.y * a_bs + (int64_t)blockIdx.x * lda;
     const int      kmax = Ap ? Kp : K;
     int32_t        s    = 0;
     for (int k = threadIdx.x * VEC; k < kmax; k += 256 * VEC)
@@ -446,22 +447,24 @@ __global__ __launch_bounds__(256) void a_prepass_kernel(const uint8_t *__restric
     }
 }
 
-int a_prepass_launch(const void *A, int64_t lda, int M, int K, bool flip, int8_t *Ap, int Kp, int32_t *rowvec,
-                     int32_t b_off, hipStream_t s)
+int a_prepass_launch(const void *A, int64_t lda, int64_t a_bs, int batch, int M, int K, bool flip, int8_t *Ap, int Kp,
+                     int32_t *rowvec, int32_t b_off, hipStream_t s)
 {
-    if (M <= 0)
+    if (M <= 0 || batch <= 0)
         return 0;
-    const uintptr_t mix  = (uintptr_t)A | (uintptr_t)lda | (uintptr_t)K;
+    if (batch > 65535)
+        return (int)hipErrorInvalidValue;
+    const uintptr_t mix  = (uintptr_t)A | (uintptr_t)lda | (uintptr_t)K | (batch > 1 ? (uintptr_t)a_bs : 0);
     const uint8_t   f    = flip ? 0x80 : 0;
-    const dim3      grid(M), block(256);
+    const dim3      grid(M, batch), block(256);
     if ((mix & 15) == 0)
-        a_prepass_kernel<16><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+        a_prepass_kernel<16><<<grid, block, 0, s>>>((const uint8_t *)A, lda, a_bs, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
     else if ((mix & 7) == 0)
-        a_prepass_kernel<8><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+        a_prepass_kernel<8><<<grid, block, 0, s>>>((const uint8_t *)A, lda, a_bs, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
     else if ((mix & 3) == 0)
-        a_prepass_kernel<4><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+        a_prepass_kernel<4><<<grid, block, 0, s>>>((const uint8_t *)A, lda, a_bs, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
     else
-        a_prepass_kernel<1><<<grid, block, 0, s>>>((const uint8_t *)A, lda, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
+        a_prepass_kernel<1><<<grid, block, 0, s>>>((const uint8_t *)A, lda, a_bs, K, f, Ap, Kp, rowvec, (uint32_t)b_off);
     return launch_status();
 }
 

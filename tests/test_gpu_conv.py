@@ -248,6 +248,37 @@ def test_conv_few_output_channels_large_images_band_form():
     cv.close()
 
 
+def test_conv_deep_patches_under_few_tiles_run_as_k_slices():
+    """Few output tiles under a deep patch (the last 3 x 3 layers of a classifier: 14 x 14 or 7 x 7 pixels, 512 channels):
+    the K range of the on-the-fly loader runs as slices along the grid of one S32 launch and a second kernel sums the
+    planes and applies the epilogue, as for a dense product: strides, padding, dilation, both source signs, weights with
+    an offset (row sums of the patches), per-channel and per-tensor requantisation; the explicit lowering (patches
+    written out, then the dense product with its own slices) gives the same bits."""
+    rng = np.random.default_rng(4608)
+    for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp) in [
+            ((1, 14, 14, 512), (96, 3, 3, 512), (1, 1), (1, 1, 1, 1), (1, 1), np.int8, np.int8, 0),
+            ((2, 9, 7, 256), (130, 3, 3, 256), (1, 1), (2, 2, 2, 2), (2, 2), np.uint8, np.int8, 0),
+            ((1, 15, 15, 512), (200, 2, 2, 512), (2, 2), (0, 1, 1, 0), (1, 1), np.uint8, np.uint8, 131),
+            ((3, 7, 7, 2048), (80, 1, 1, 2048), (1, 1), (0, 0, 0, 0), (1, 1), np.int8, np.int8, 0)]:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        for per_channel in (True, False):
+            reals = rng.uniform(0.5, 2.0, wshape[0] if per_channel else 1) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert 0.1 < ((want > lo) & (want < hi)).mean()
+            for path in (capi.CONV_AUTO, capi.CONV_EXPLICIT):
+                announce("conv k slices", shape, wshape, stride, pad, dil, dt.__name__, w_dt.__name__, w_zp, "per_channel", per_channel,
+                         "path", path)
+                got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil, path=path)
+                assert "_splitk" in name and name.startswith("implicit" if path == capi.CONV_AUTO else "im2col"), name
+                np.testing.assert_array_equal(got, want)
+
+
 def test_conv_channel_counts_padded_to_16():
     """A channel count that is not a multiple of 16: pixels and taps are copied with the channels padded to the next
     multiple of 16 and the fast implicit kernels run (never the byte-wise fallback), with identical results - the RGB of

@@ -176,11 +176,14 @@ def test_f16_destination(device):
 
 def test_batched_small_products_take_the_streaming_kernel():
     """Batches of small products (tests/datasets/GEMMLowpFusedOffsetOutputDataset.h:142-162: up to 32 entries of a few
-    rows) run the streaming kernel once per entry instead of a mostly empty tile per entry: per-entry and shared B, a
-    B offset (row sums per entry), padded rows and batch strides, every epilogue."""
+    rows) run the streaming kernel instead of a mostly empty tile per entry - one launch with the entries along the grid
+    (and one more for the row sums of all entries), or, from 4 MiB of B per entry on, one launch per entry in the form
+    that stages A once: per-entry and shared B, a B offset (row sums per entry), padded rows and batch strides, every
+    epilogue."""
     rng = np.random.default_rng(4242)
     for (batch, M, N, K, b_batched) in [(3, 4, 5, 2, True), (3, 7, 29, 15, True), (32, 17, 5, 56, True), (32, 13, 19, 256, True),
-                                        (5, 8, 300, 1024, False), (4, 32, 130, 200, True)]:
+                                        (5, 8, 300, 1024, False), (4, 32, 130, 200, True), (3, 8, 64, 2048, True),
+                                        (2, 8, 1100, 4096, False)]:
         A = rng.integers(-128, 128, size=(batch, M, K), dtype=np.int8)
         B = rng.integers(-128, 128, size=(batch, K, N) if b_batched else (K, N), dtype=np.int8)
         ao, bo = int(rng.integers(-20, 20)), int(rng.integers(1, 20))
@@ -191,7 +194,8 @@ def test_batched_small_products_take_the_streaming_kernel():
         assert name.startswith("skinny"), name
         for z in range(batch):
             np.testing.assert_array_equal(got[z], oracle.gemmlowp_s32(A[z], B[z] if b_batched else B, ao, bo))
-        got, _ = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, bo, bias, [mult], [shift], -3, -128, 127, device=True)
+        got, name = run_gemm(A, B, capi.EPI_FIXEDPOINT, np.int8, ao, bo, bias, [mult], [shift], -3, -128, 127, device=True)
+        assert name == ("skinny_once" if N * K > (4 << 20) else "skinny_stream"), name
         for z in range(batch):
             np.testing.assert_array_equal(
                 got[z], oracle.gemmlowp_fixedpoint(A[z], B[z] if b_batched else B, bias, ao, bo, [mult], [shift], -3, -128, 127, np.int8))

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -61,9 +62,9 @@ bool is_device_ptr(const void *p)
     return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
-// What kind of memory an argument slot of a handle was last given. Device allocations live in an address range the
-// driver reserves for them, so a pointer value does not change sides while the process lives: asking once per value
-// and slot is enough, and a steady-state run() asks nothing.
+// What kind of memory an argument slot of a handle was last given: asked once per value and slot, so that a
+// steady-state run() asks nothing. The answer lives and dies with the handle. It is stale only if the address is freed
+// and handed out again by an allocation of the other kind between two runs of the same handle (the header says so).
 struct PtrKind
 {
     const void *p   = nullptr;
@@ -184,6 +185,8 @@ struct GemmCore
     uint8_t fill_byte = 0; // value of the 16 filler bytes (0, or the im2col pad value)
     void   *ext_ws = nullptr; // set around a run that must not allocate: see run_dense
     size_t  ext_ws_bytes = 0;
+    bool    ext_ws_busy = false; // the caller's workspace may still be read by kernels of another stream
+    bool    ext_ws_used = false; // set by run_dense: this run put something into the caller's workspace
 
     void refresh_names()
     {
@@ -475,6 +478,9 @@ struct GemmCore
         int8_t      *ap       = nullptr;
         if (ext_ws != nullptr)
         {
+            if (rv_bytes + ap_bytes > 0 && ext_ws_busy)
+                return fail("mi355_gemmlowp_run_noalloc: this GPU's workspace is still in use by a call on another stream");
+            ext_ws_used = rv_bytes + ap_bytes > 0;
             if (rv_bytes + ap_bytes > ext_ws_bytes)
                 return fail("this run needs %zu bytes of workspace (row sums %zu + padded copy of A %zu); the fixed "
                             "workspace holds %zu",
@@ -961,23 +967,36 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
     return 0;
 }
 
-// The address of this GPU's copy of the workspace array, asked once per device (with that device current)
-static int noalloc_scratch(void **out)
+// Per GPU: the address of its copy of the workspace array, asked once (with that device current), and an event behind
+// the last call's kernels, created in the same set-up step. Calls on one stream are ordered by the stream; a call that
+// arrives on another stream while the event is still pending would overwrite the workspace under running kernels and
+// is refused.
+struct NoallocState
 {
-    static void *ptrs[64];
-    int          dev = 0;
+    void       *ptr      = nullptr;
+    hipEvent_t  done     = nullptr;
+    hipStream_t last     = nullptr;
+    bool        recorded = false;
+};
+static std::mutex g_noalloc_mutex;
+static int noalloc_state(NoallocState **out)
+{
+    static NoallocState states[64];
+    int                 dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64)
         return fail("device index %d out of range", dev);
-    void *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
-    if (p == nullptr)
+    NoallocState &st = states[dev];
+    if (st.ptr == nullptr)
     {
+        void *p = nullptr;
         HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
         if (p == nullptr)
             return fail("hipGetSymbolAddress returned no address for the workspace");
-        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+        HIP_TRY(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
+        st.ptr = p;
     }
-    *out = p;
+    *out = &st;
     return 0;
 }
 
@@ -1003,11 +1022,37 @@ int mi355_gemmlowp_run_noalloc(mi355_gemm_handle *h, const void *A, const float 
         return fail("mi355_gemmlowp_run_noalloc does not take planes with gaps between them (they need dense copies)");
     if (!h->kindA.is_device(A) || !h->kindD.is_device(D) || (bias_f32 && !h->kindBiasF.is_device(bias_f32)))
         return fail("mi355_gemmlowp_run_noalloc takes device memory only");
-    void *ws = nullptr;
-    TRY(noalloc_scratch(&ws));
-    c.ext_ws = ws, c.ext_ws_bytes = MI355_NOALLOC_SCRATCH_BYTES;
-    const int rc = c.run_dense((const int8_t *)A, d.lda, d.a_batch_stride, D, d.ldd, d.d_batch_stride, bias_f32, s);
-    c.ext_ws = nullptr, c.ext_ws_bytes = 0;
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    NoallocState               *st = nullptr;
+    TRY(noalloc_state(&st));
+    // (a stream under graph capture records no event and is not checked: the graph's own order is the caller's)
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusActive;
+    }
+    const bool tracked = cap == hipStreamCaptureStatusNone;
+    if (tracked && st->recorded && st->last != s)
+    {
+        const hipError_t q = hipEventQuery(st->done);
+        if (q == hipErrorNotReady)
+        {
+            (void)hipGetLastError();
+            c.ext_ws_busy = true; // an error if this run needs the workspace at all
+        }
+        else
+            HIP_TRY(q);
+    }
+    c.ext_ws = st->ptr, c.ext_ws_bytes = MI355_NOALLOC_SCRATCH_BYTES, c.ext_ws_used = false;
+    const int  rc   = c.run_dense((const int8_t *)A, d.lda, d.a_batch_stride, D, d.ldd, d.d_batch_stride, bias_f32, s);
+    const bool used = c.ext_ws_used;
+    c.ext_ws = nullptr, c.ext_ws_bytes = 0, c.ext_ws_busy = false;
+    if (tracked && used && rc == 0)
+    {
+        HIP_TRY(hipEventRecord(st->done, s));
+        st->last = s, st->recorded = true;
+    }
     return rc;
 }
 

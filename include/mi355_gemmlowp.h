@@ -22,7 +22,10 @@
  *    hipPointerGetAttributes. Host buffers are staged through device memory owned by the
  *    handle (synchronous, like the reference's run()); device buffers are used in place and
  *    the call only enqueues work on `stream` (a hipStream_t passed as void*, NULL = default
- *    stream).
+ *    stream). A handle asks once per pointer value and argument: it remembers which kind the
+ *    value last given for A, D and the float bias was, until the handle is destroyed. If memory
+ *    of one kind is freed and the SAME address comes back from an allocation of the other kind
+ *    between two runs of one handle, pass a different address first or use a new handle.
  *  - All functions return 0 on success, non-zero on failure; mi355_last_error() then returns
  *    a thread-local message. No exception crosses this boundary.
  *  - A handle is single-caller: one call at a time per handle. Distinct handles may be used
@@ -196,9 +199,13 @@ int mi355_gemmlowp_run(mi355_gemm_handle *h, const void *A, const float *bias_f3
  * followed by the padded copy of A (batch * M * round_up(K, 128) bytes; needed when a row of A does not start on a
  * 4-byte boundary) - lives in one fixed array of mi355_gemmlowp_noalloc_workspace_bytes() (8 MiB) that each GPU holds
  * for the life of the process; a run that needs more is refused with an error, as is an F16 destination. The call
- * allocates and frees nothing and only enqueues kernels on `stream`. Every call on a GPU uses that GPU's one array
- * (nothing in it has to start at zero: the kernels overwrite what they read), so calls that overlap in time on one GPU
- * - different streams, different handles - race; serialise them. The handle must be prepared. */
+ * allocates and frees nothing and only enqueues kernels (and one event) on `stream`. Every call on a GPU uses that
+ * GPU's one array (nothing in it has to start at zero: the kernels overwrite what they read), so calls that overlap in
+ * time on one GPU - different streams, different handles - would race: calls on one stream are ordered by the stream;
+ * a call that needs the workspace while the kernels of a call on ANOTHER stream are still pending is refused with an
+ * error (synchronise, or keep to one stream). Under HIP graph capture nothing is recorded or checked: the order of the
+ * graphs that share the array is the caller's business. The array's address and the event are set up by the first call
+ * on each GPU. The handle must be prepared. */
 int    mi355_gemmlowp_run_noalloc(mi355_gemm_handle *h, const void *A, const float *bias_f32, void *D, void *stream);
 size_t mi355_gemmlowp_noalloc_workspace_bytes(void);
 

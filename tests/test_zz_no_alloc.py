@@ -11,8 +11,9 @@ from gpu_util import announce, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def _case(M, N, K, lda, a_dt, b_dt, b_off, seed):
-    """one handle, one input: (A on the device, handle, result of the allocating entry point, oracle result)"""
+def _case(M, N, K, lda, a_dt, b_dt, b_off, seed, run_first=True):
+    """one handle, one input: (A on the device, handle, result of the allocating entry point, oracle result); with
+    run_first False the handle is prepared but has never run"""
     import torch
     rng = np.random.default_rng(seed)
     A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(M, K)).astype(a_dt)
@@ -28,10 +29,13 @@ def _case(M, N, K, lda, a_dt, b_dt, b_off, seed):
     Ad = to_dev(Ah)
     keep = [to_dev(B), to_dev(bias)]
     g.prepare(keep[0], keep[1])
+    want = oracle.gemmlowp_fixedpoint(A, B, bias, -7, b_off, mult, shift, 5, lo, hi, a_dt)
+    if not run_first:
+        torch.cuda.synchronize()
+        return Ad, g, None, want, keep
     D_ref = torch.zeros((M, N), dtype=torch.int8 if a_dt == np.int8 else torch.uint8, device="cuda")
     g.run(Ad, D_ref)
     torch.cuda.synchronize()
-    want = oracle.gemmlowp_fixedpoint(A, B, bias, -7, b_off, mult, shift, 5, lo, hi, a_dt)
     return Ad, g, D_ref.cpu().numpy(), want, keep
 
 
@@ -86,3 +90,57 @@ def test_noalloc_rejects_what_does_not_fit_and_host_memory():
     g.run(Ad, Dd)  # the allocating entry point still takes it
     torch.cuda.synchronize()
     g.close()
+
+
+@pytest.mark.parametrize("lda_extra", [0, 3])
+def test_noalloc_on_a_handle_that_never_ran_allocates_nothing(lda_extra):
+    """The first run of a handle through the entry point that allocates nothing (the allocating one has not sized any
+    workspace for it), and the device's free memory before and after: unchanged."""
+    import torch
+    M, N, K = 260, 136, 400
+    # (a first handle takes whatever the first use of these kernels costs the process - code objects, the one-time set-up
+    # of the workspace - out of the measurement)
+    Ad, g, _, want, keep = _case(M, N, K, K + lda_extra, np.uint8, np.uint8, 9, 700, run_first=False)
+    D = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+    g.run_noalloc(Ad, D)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(D.cpu().numpy(), want)
+    g.close()
+    Ad, g, _, want, keep = _case(M, N, K, K + lda_extra, np.uint8, np.uint8, 9, 701, run_first=False)
+    D.fill_(3)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    announce("no-alloc, cold handle", (M, N, K), "lda +", lda_extra)
+    for _ in range(3):
+        g.run_noalloc(Ad, D)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    np.testing.assert_array_equal(D.cpu().numpy(), want)
+    g.close()
+
+
+def test_noalloc_refuses_a_second_stream_while_the_first_is_busy():
+    """One workspace per GPU: calls on one stream follow each other; a call on another stream while kernels of the first
+    are still queued is refused, and accepted once they are done. A run that needs no workspace (no B offset, aligned
+    rows) is never refused."""
+    import torch
+    M, N, K = 1024, 1024, 4000
+    Ad, g, ref, want, keep = _case(M, N, K, K + 3, np.int8, np.int8, 4, 800)  # (rows not dword aligned: a padded copy of A)
+    Ad0, g0, ref0, want0, keep0 = _case(64, 64, 256, 256, np.int8, np.int8, 0, 801)
+    D = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    D0 = torch.zeros((64, 64), dtype=torch.int8, device="cuda")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    announce("no-alloc, two streams")
+    for _ in range(400):  # several milliseconds of queued work on the first stream
+        g.run_noalloc(Ad, D, stream=s1.cuda_stream)
+    with pytest.raises(capi.Mi355Error, match="still in use"):
+        g.run_noalloc(Ad, D, stream=s2.cuda_stream)
+    g0.run_noalloc(Ad0, D0, stream=s2.cuda_stream)  # nothing of it lives in the workspace
+    torch.cuda.synchronize()
+    g.run_noalloc(Ad, D, stream=s2.cuda_stream)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(D.cpu().numpy(), ref)
+    np.testing.assert_array_equal(D0.cpu().numpy(), ref0)
+    g.close()
+    g0.close()

@@ -110,8 +110,9 @@ def ceilings_lib():
     l = C.CDLL(path)
     vp, i64 = C.c_void_p, C.c_int64
     l.mi355_ceiling_read.argtypes = [vp, i64, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp]
-    l.mi355_ceiling_mfma.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
-    l.mi355_ceiling_mfma_lds.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp]
+    l.mi355_ceiling_mfma.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]
+    l.mi355_ceiling_mfma_lds.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp]
+    l.mi355_ceiling_mfma_lds_pipelined.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
     l.mi355_ceiling_dma.argtypes = [vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]
     l.mi355_ceiling_clock.argtypes = [i64, i64, vp, vp]
     l.mi355_ceiling_lds_read.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp, vp]
@@ -167,23 +168,40 @@ def run_ceilings(torch, args):
     zero = torch.zeros(16 << 20, dtype=torch.int8, device="cuda")
     out["mfma_cfg2_instruction_count"] = []
 
-    def timed(name, fn, data):
+    spans = torch.zeros(256 * 4, dtype=torch.int64, device="cuda")
+
+    def timed(name, fn, data, waves):
+        """us: per launch over graph replays (launch to launch). span_us: from the first wave's start of its timed loop
+        to the last wave's end, over all workgroups of the last launch (100 MHz counter) - what the chip needs for the
+        instructions themselves; the loop of a single wave says little (the oldest wave of a SIMD is served first)."""
         s = time_graph(torch, [fn], args.steps)
         torch.cuda.synchronize()
-        t = ticks.cpu().numpy()
+        sp = spans.cpu().numpy().reshape(256, 4)
+        span = float(sp[:, 1].max() - sp[:, 0].min()) * 1e-8
+        mean_clocks = float(sp[:, 3].sum()) / (256 * waves)
+        wave_real = float((sp[:, 1] - sp[:, 0]).mean()) * 1e-8  # a workgroup's own span, averaged
         out["mfma_cfg2_instruction_count"].append({
             "what": name, "operands": data, "us": round(s * 1e6, 3), "TOPS": round(ops / s / 1e12, 1),
             "frac_of_5.0_POPs": round(ops / s / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
-            "loop_clocks": int(t[0]), "shader_MHz_in_loop": round(float(t[0]) / max(float(t[1]), 1.0) * 100.0, 1)})
+            "span_us": round(span * 1e6, 2), "span_TOPS": round(ops / span / 1e12, 1),
+            "span_frac_of_5.0_POPs": round(ops / span / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+            "workgroup_span_us_mean": round(wave_real * 1e6, 2),
+            "loop_clocks_mean_per_wave": int(mean_clocks), "loop_clocks_longest_wave": int(sp[:, 2].max()),
+            "shader_MHz_from_longest_wave": round(float(sp[:, 2].max()) / max(span * 1e6, 1e-9), 1)})
 
     for data, src in (("random", rnd), ("zero", zero)):
         for shape in (16, 32):
-            timed("registers only, v_mfma_i32_%dx%dx%d_i8" % (shape, shape, 64 if shape == 16 else 32),
+            timed("registers only, v_mfma_i32_%dx%dx%d_i8, 8 waves per compute unit" % (shape, shape, 64 if shape == 16 else 32),
                   lambda cs, shape=shape, src=src: cl.mi355_ceiling_mfma(src.data_ptr(), shape, 256, 1024, sink.data_ptr(),
-                                                                         ticks.data_ptr(), cs), data)
-        timed("operands read from LDS (64x64 wave tiles), 16x16x64",
-              lambda cs, src=src: cl.mi355_ceiling_mfma_lds(src.data_ptr(), 256, 32, sink.data_ptr(), ticks.data_ptr(), cs),
-              data)
+                                                                         ticks.data_ptr(), spans.data_ptr(), cs), data, 8)
+        timed("operands from LDS, 64x64 wave tiles, all reads then all matrix instructions then a barrier per K step",
+              lambda cs, src=src: cl.mi355_ceiling_mfma_lds(src.data_ptr(), 256, 32, sink.data_ptr(), ticks.data_ptr(),
+                                                            spans.data_ptr(), cs), data, 8)
+        for waves in (8, 4):
+            timed("operands from LDS, %s wave tiles, double-buffered in registers, reads interleaved, no barrier" %
+                  ("64x64" if waves == 8 else "128x64"),
+                  lambda cs, src=src, waves=waves: cl.mi355_ceiling_mfma_lds_pipelined(src.data_ptr(), 256, waves, 32, sink.data_ptr(),
+                                                                                      spans.data_ptr(), cs), data, waves)
     # LDS operand reads alone: 16 KiB per wave and step, 32 steps (config 2 reads 128 KiB per compute unit and step)
     out["lds_operand_reads"] = []
     sink2 = torch.zeros(256 * 1024, dtype=torch.int32, device="cuda")

@@ -4,7 +4,10 @@
 //
 //   mi355_ceiling_read        one streaming pass over a buffer (the skinny GEMM's B stream, without any arithmetic)
 //   mi355_ceiling_mfma        int8 matrix instructions out of registers only (no LDS, no global traffic)
-//   mi355_ceiling_mfma_lds    the same instruction count with every operand read from LDS first (64 x 64 wave tiles)
+//   mi355_ceiling_mfma_lds    the same instruction count with every operand read from LDS first (64 x 64 wave tiles),
+//                             the plain schedule: all reads of a K step, then its matrix instructions, then a barrier
+//   mi355_ceiling_mfma_lds_pipelined   the same with operands double-buffered in registers, reads interleaved with the
+//                             matrix instructions, no barrier; 64 x 64 or 128 x 64 wave tiles
 //   mi355_ceiling_lds_read    the operand reads of the pipelined GEMM alone (LDS bandwidth per compute unit)
 //   mi355_ceiling_dma         the pipelined GEMM's global -> LDS stream alone (direct-to-LDS loads, 3-slot ring)
 //   mi355_ceiling_clock       shader clock while other work runs: shader-clock ticks over a span of real time
@@ -16,6 +19,31 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace
 {
+// What one workgroup leaves behind for the host (4 x int64 per workgroup, overwritten by every launch): the earliest
+// start and the latest end of its waves' timed loops on the 100 MHz real-time counter, and the longest and the summed
+// loop duration in shader clocks. The host takes the minimum start and the maximum end over all workgroups: the span
+// in which the chip worked on the loops, which is what a rate has to be computed from - the scheduler favours the
+// oldest wave of a SIMD, so the loop of any single wave (the first of its workgroup least of all) says little.
+__device__ __forceinline__ void leave_span(int64_t *spans, int64_t r0, int64_t r1, int64_t clocks)
+{
+    __shared__ int64_t w_r0[16], w_r1[16], w_ck[16];
+    const int          wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    if ((threadIdx.x & 63) == 0)
+        w_r0[wave] = r0, w_r1[wave] = r1, w_ck[wave] = clocks;
+    __syncthreads();
+    if (threadIdx.x == 0 && spans)
+    {
+        int64_t a = w_r0[0], b = w_r1[0], mx = w_ck[0], sum = w_ck[0];
+        for (int w = 1; w < nw; ++w)
+        {
+            a = w_r0[w] < a ? w_r0[w] : a, b = w_r1[w] > b ? w_r1[w] : b;
+            mx = w_ck[w] > mx ? w_ck[w] : mx, sum += w_ck[w];
+        }
+        int64_t *o = spans + (int64_t)blockIdx.x * 4;
+        o[0] = a, o[1] = b, o[2] = mx, o[3] = sum;
+    }
+}
+
 // PATTERN 0: workgroup b owns the contiguous chunk b of the buffer and its waves split that chunk into contiguous
 // slices (what a kernel with one workgroup per group of output columns does). PATTERN 1: the whole grid reads one
 // contiguous window per iteration (wave w of the grid takes block it * waves + w), the DRAM-friendliest order.
@@ -60,8 +88,9 @@ __global__ __launch_bounds__(512) void read_kernel(const v4i *__restrict__ src, 
 // SHAPE 16: v_mfma_i32_16x16x64_i8, SHAPE 32: v_mfma_i32_32x32x32_i8 (the same multiply-accumulates per instruction
 // pair). Every wave issues `mfma16` instructions' worth of work (counted in 16x16x64 units) on operands it read once.
 template <int SHAPE>
-__global__ __launch_bounds__(512) void mfma_kernel(const v4i *__restrict__ src, int mfma16, int *sink, int64_t *ticks)
+__global__ __launch_bounds__(512) void mfma_kernel(const v4i *__restrict__ src, int mfma16, int *sink, int64_t *ticks, int64_t *spans)
 {
+    extern __shared__ char reserve[]; // (the host asks for more than half of LDS: one workgroup per compute unit)
     const int tid = blockIdx.x * blockDim.x + threadIdx.x;
     v4i       a[8], b[8];
 #pragma unroll
@@ -103,11 +132,12 @@ __global__ __launch_bounds__(512) void mfma_kernel(const v4i *__restrict__ src, 
     sink[tid] = s;
     if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
         ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+    leave_span(spans, r0, r1, t1 - t0);
 }
 
 // 8 waves per workgroup; per K step of 128 every wave reads the operands of a 64 x 64 wave tile (16 x ds_read_b128)
 // from a 48 KiB stage of random bytes and issues 32 matrix instructions; one barrier per step.
-__global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ src, int steps, int *sink, int64_t *ticks)
+__global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ src, int steps, int *sink, int64_t *ticks, int64_t *spans)
 {
     extern __shared__ __attribute__((aligned(1024))) char smem[]; // 3 x 48 KiB
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -150,6 +180,96 @@ __global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ s
     sink[blockIdx.x * blockDim.x + threadIdx.x] = sum;
     if (ticks && threadIdx.x == 0 && blockIdx.x == 100 % gridDim.x)
         ticks[0] = t1 - t0, ticks[1] = r1 - r0;
+    leave_span(spans, r0, r1, t1 - t0);
+}
+
+// The matrix instructions of the 256 x 128 x 128 tile with every operand read from LDS first, scheduled as well as this
+// file knows how: the stage holds static data, so nothing waits for a producer and there is no barrier; operands are
+// double-buffered in registers by halves of a K step (64 of K), and the reads of the next half are interleaved one by
+// one behind the first matrix instructions of this half (what the pipelined GEMM's consumer waves do). NW = 8: wave
+// tiles of 64 x 64 (8 reads per 16 matrix instructions); NW = 4: wave tiles of 128 x 64 (12 reads per 32). Rows of 128
+// bytes, 16-byte piece p of row r at position p ^ ((r >> 1) & 7): free of bank conflicts.
+template <int NW>
+__global__ __launch_bounds__(512) void mfma_lds_pipelined_kernel(const v4i *__restrict__ src, int steps, int *sink, int64_t *spans)
+{
+    constexpr int RS = NW == 8 ? 4 : 8, QS = 4;
+    extern __shared__ __attribute__((aligned(1024))) char smem[]; // 3 x 48 KiB
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 3 * 49152 / 16; i += blockDim.x)
+        ((v4i *)smem)[i] = src[(blockIdx.x * 9216 + i) & 0xFFFFF];
+    __syncthreads();
+    const int row = lane & 15, lh = lane >> 4;
+    uint32_t  offa[RS], offb[QS]; // byte offset of this lane's piece of every operand block, first half of a K step
+#pragma unroll
+    for (int f = 0; f < RS; ++f)
+    {
+        const int r = ((wave >> 1) * RS + f) * 16 + row;
+        offa[f]     = (uint32_t)(r * 128 + ((lh ^ ((r >> 1) & 7)) << 4));
+    }
+#pragma unroll
+    for (int f = 0; f < QS; ++f)
+    {
+        const int r = 256 + ((wave & 1) * QS + f) * 16 + row;
+        offb[f]     = (uint32_t)(r * 128 + ((lh ^ ((r >> 1) & 7)) << 4));
+    }
+    v4i acc[RS][QS];
+#pragma unroll
+    for (int i = 0; i < RS; ++i)
+#pragma unroll
+        for (int j = 0; j < QS; ++j)
+            acc[i][j] = (v4i){0, 0, 0, 0};
+    v4i fa[2][RS], fb[2][QS];
+    // (the second half of a K step lies 4 pieces on: position p ^ 4 of the same row)
+    auto read_half = [&](const char *stage, int half, v4i (&a)[RS], v4i (&b)[QS])
+    {
+#pragma unroll
+        for (int f = 0; f < QS; ++f)
+            b[f] = *(const v4i *)(stage + (offb[f] ^ (uint32_t)(half * 64)));
+#pragma unroll
+        for (int f = 0; f < RS; ++f)
+            a[f] = *(const v4i *)(stage + (offa[f] ^ (uint32_t)(half * 64)));
+    };
+    auto multiply = [&](const v4i (&a)[RS], const v4i (&b)[QS])
+    {
+#pragma unroll
+        for (int i = 0; i < RS; ++i)
+#pragma unroll
+            for (int j = 0; j < QS; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b[j], a[i], acc[i][j], 0, 0, 0);
+    };
+    auto interleave = [&]()
+    {
+        // one LDS read behind each of the first RS + QS matrix instructions, the rest of them after
+#pragma unroll
+        for (int i = 0; i < RS + QS; ++i)
+        {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, RS * QS - (RS + QS), 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const int64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    read_half(smem, 0, fa[0], fb[0]);
+    for (int kt = 0; kt < steps; ++kt)
+    {
+        const char *cur = smem + (kt % 3) * 49152, *nxt = smem + ((kt + 1) % 3) * 49152;
+        read_half(cur, 1, fa[1], fb[1]);
+        multiply(fa[0], fb[0]);
+        interleave();
+        read_half(nxt, 0, fa[0], fb[0]); // (after the last step: a read nobody uses)
+        multiply(fa[1], fb[1]);
+        interleave();
+    }
+    const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    int           sum = fa[0][0][0] + fb[0][0][0];
+#pragma unroll
+    for (int i = 0; i < RS; ++i)
+#pragma unroll
+        for (int j = 0; j < QS; ++j)
+            sum += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+    leave_span(spans, r0, r1, t1 - t0);
 }
 
 // LDS operand reads alone: `waves` waves per workgroup, each reading the 16 operand blocks of a 64 x 64 wave tile
@@ -275,19 +395,56 @@ int mi355_ceiling_read(const void *buf, int64_t kib, int pattern, int grid, int 
 
 // src: 16 MiB of operand bytes; grid workgroups of 8 waves, each wave issuing mfma16 (a multiple of 32) 16x16x64-sized
 // instructions; sink: grid * 512 ints; ticks: 2 x int64 (shader-clock ticks, 100 MHz ticks of one wave's loop) or null
-int mi355_ceiling_mfma(const void *src, int shape, int grid, int mfma16, int *sink, int64_t *ticks, void *stream)
+// spans: 4 x int64 per workgroup (see leave_span) or null. One workgroup per compute unit (96 KiB of LDS reserved).
+int mi355_ceiling_mfma(const void *src, int shape, int grid, int mfma16, int *sink, int64_t *ticks, int64_t *spans, void *stream)
 {
     if (!src || !sink || grid < 1 || mfma16 < 32 || mfma16 % 32 != 0 || (shape != 16 && shape != 32))
         return (int)hipErrorInvalidValue;
-    hipStream_t s = (hipStream_t)stream;
+    hipStream_t   s       = (hipStream_t)stream;
+    constexpr int RESERVE = 96 * 1024;
+    static bool   raised  = false;
+    if (!raised)
+    {
+        hipError_t e = hipFuncSetAttribute((const void *)mfma_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, RESERVE);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)mfma_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, RESERVE);
+        if (e != hipSuccess)
+            return (int)e;
+        raised = true;
+    }
     if (shape == 16)
-        hipLaunchKernelGGL(mfma_kernel<16>, dim3(grid), dim3(512), 0, s, (const v4i *)src, mfma16, sink, ticks);
+        hipLaunchKernelGGL(mfma_kernel<16>, dim3(grid), dim3(512), RESERVE, s, (const v4i *)src, mfma16, sink, ticks, spans);
     else
-        hipLaunchKernelGGL(mfma_kernel<32>, dim3(grid), dim3(512), 0, s, (const v4i *)src, mfma16, sink, ticks);
+        hipLaunchKernelGGL(mfma_kernel<32>, dim3(grid), dim3(512), RESERVE, s, (const v4i *)src, mfma16, sink, ticks, spans);
     return (int)hipGetLastError();
 }
 
-int mi355_ceiling_mfma_lds(const void *src, int grid, int steps, int *sink, int64_t *ticks, void *stream)
+// The pipelined form (see mfma_lds_pipelined_kernel): waves 8 (64 x 64 wave tiles) or 4 (128 x 64); every workgroup
+// issues steps * 256 * 128 * 128 multiply-accumulates
+int mi355_ceiling_mfma_lds_pipelined(const void *src, int grid, int waves, int steps, int *sink, int64_t *spans, void *stream)
+{
+    if (!src || !sink || grid < 1 || steps < 1 || (waves != 4 && waves != 8))
+        return (int)hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised)
+    {
+        hipError_t e = hipFuncSetAttribute((const void *)mfma_lds_pipelined_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)mfma_lds_pipelined_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
+        if (e != hipSuccess)
+            return (int)e;
+        raised = true;
+    }
+    if (waves == 8)
+        hipLaunchKernelGGL(mfma_lds_pipelined_kernel<8>, dim3(grid), dim3(512), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps,
+                           sink, spans);
+    else
+        hipLaunchKernelGGL(mfma_lds_pipelined_kernel<4>, dim3(grid), dim3(256), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps,
+                           sink, spans);
+    return (int)hipGetLastError();
+}
+
+int mi355_ceiling_mfma_lds(const void *src, int grid, int steps, int *sink, int64_t *ticks, int64_t *spans, void *stream)
 {
     if (!src || !sink || grid < 1 || steps < 1)
         return (int)hipErrorInvalidValue;
@@ -300,7 +457,7 @@ int mi355_ceiling_mfma_lds(const void *src, int grid, int steps, int *sink, int6
         raised = true;
     }
     hipLaunchKernelGGL(mfma_lds_kernel, dim3(grid), dim3(512), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps, sink,
-                       ticks);
+                       ticks, spans);
     return (int)hipGetLastError();
 }
 

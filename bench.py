@@ -245,6 +245,38 @@ def run_ceilings(torch, args):
     print(json.dumps(out))
 
 
+def run_tile_sweep(torch, capi, args):
+    """Config 2 on every configuration of the pipelined kernel (tile shape, K step, ring depth), chosen through the
+    descriptor's path field instead of the cost model: graph-replayed time per launch, bit-exact results checked against
+    the configuration the cost model picks."""
+    stream = torch.cuda.current_stream().cuda_stream
+    M, N, K = 2048, 4096, 4096
+    A, B, bias, mult, shift = synth_config2(M, N, K)
+    rq = capi.requant(0, 0, -5, -128, 127, per_channel=True)
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    keep = [torch.from_numpy(x).cuda() for x in (bias, mult, shift)]
+    rows, ref = [], None
+    for path in [capi.PATH_AUTO] + [capi.PATH_TILE + i for i in range(6)]:  # the 6 pipelined configurations
+        g = capi.Gemm(M, N, K, capi.S8, capi.S8, capi.S8, capi.EPI_FIXEDPOINT, -3, 0, rq, path=path)
+        Dd = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+        g.prepare(Bd, *keep, stream)
+        for _ in range(args.warmup):
+            g.run(Ad, Dd, None, stream)
+        torch.cuda.synchronize()
+        s = min(time_graph(torch, [lambda cs: g.run(Ad, Dd, None, cs)], args.steps) for _ in range(2))
+        torch.cuda.synchronize()
+        got = Dd.cpu().numpy()
+        if ref is None:
+            ref = got
+        rows.append({"path": "cost model" if path == capi.PATH_AUTO else "PATH_TILE + %d" % (path - capi.PATH_TILE),
+                     "kernel": g.kernel_name, "kernel_us": round(s * 1e6, 3),
+                     "frac_of_5.0_POPs": round(2.0 * M * N * K / s / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
+                     "same_bits_as_cost_model_choice": bool(np.array_equal(got, ref))})
+        g.close()
+    print(json.dumps({"tile_sweep": True, "workload": "config 2: M=2048 N=4096 K=4096 s8 -> s8", "launches": args.steps,
+                      "rows": rows}))
+
+
 def run_phase_clocks(torch, capi, args):
     """Config 2 on the instrumented build (a library of its own: the product library carries no instrumentation): shader
     clocks between the ends of the kernel's parts, read from the first lane of consumer wave 0 and producer wave 0 of
@@ -314,6 +346,8 @@ def main():
     ap.add_argument("--ceilings", action="store_true",
                     help="only run the measurement-only kernels (read stream, matrix instructions, LDS, direct-to-LDS "
                          "stream, vendor int8 GEMM) and print their figures as one JSON line")
+    ap.add_argument("--tile-sweep", action="store_true",
+                    help="only time config 2 on every configuration of the pipelined kernel (tile shape sweep) and exit")
     ap.add_argument("--phase-clocks", action="store_true",
                     help="only run config 2 on the build of the library whose pipelined kernel leaves clock readings at "
                          "the ends of its parts, and print start-up / K loop / epilogue clocks as one JSON line")
@@ -346,6 +380,10 @@ def main():
 
     if args.phase_clocks:
         run_phase_clocks(torch, capi, args)
+        return
+
+    if args.tile_sweep:
+        run_tile_sweep(torch, capi, args)
         return
 
     M, N, K = 2048, 4096, 4096

@@ -412,6 +412,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 // the matrix cores or LDS: 700 issue slots per wave, a third of them in the k loop.)
 // Needs C a power of two >= 64 (a 64-byte k block then lies inside one tap and one pixel), N <= 64, K <= 1152.
 constexpr int HALO_WAVES = 16;
+constexpr int HALO_DMA_WAVES = 8; // waves that issue the transfers
 
 // Measurement build only (-DMI355_PHASE_CLOCKS, a library of its own that the product never loads): the first lane of
 // wave 0 and of wave 12 of the first, the middle and the last workgroup leaves the 100 MHz real-time counter at the ends
@@ -508,8 +509,12 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     constexpr int   NDMA = KBLK * 4 + NARROW_PAD_PIECES;
     const int       nimg = ((staged << lc) + 1023) >> 10;
     const uintptr_t img  = u_a + (uintptr_t)((int64_t)n * cg.H * cg.W * cg.C);
-    for (int ins = wave; ins < NDMA + nimg; ins += HALO_WAVES)
+    // (by the first HALO_DMA_WAVES waves only: the waves of a workgroup start one after the other over most of a
+    // microsecond, and what the last ones still have to do before the barrier is what the barrier waits for)
+    for (int ins = wave; ins < NDMA + nimg; ins += HALO_DMA_WAVES)
     {
+        if (wave >= HALO_DMA_WAVES)
+            break;
         if (ins < NDMA)
             narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
         else

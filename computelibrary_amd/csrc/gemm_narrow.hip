@@ -455,6 +455,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
                    "+s"(cg.magic_C), "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp),
                    "+s"(u_fl), "+s"(wpi), "+s"(rpw));
     int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
+    static_assert(((NARROW_BN * PITCH + NPAR * NARROW_BN * 4) & 1023) != 0, "one more word (the flag) fits in front of the next KiB");
     const MI355_GLOBAL int8_t *const  gB = (const MI355_GLOBAL int8_t *)u_b;
     const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
 
@@ -492,16 +493,17 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const int      s_img   = img_off >> lc; // LDS pixel index of the window's first pixel
 
     // epilogue constants (one dword per thread: 6 x 64 of them), the flag word of the requantisation
+    // (fetched by the waves that start first - the threads of waves 0 to 5 hold one constant each, wave 0 the flag word -
+    // and handed on through LDS: the waves that start last then have nothing to wait for before the barrier)
     const bool have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
     int32_t    tp      = 0;
-    if (have_qp)
+    if (have_qp && tid < NPAR * NARROW_BN)
     {
-        const int idx = min(tid, NPAR * NARROW_BN - 1);
-        const int v = idx / NARROW_BN, col = idx - v * NARROW_BN;
+        const int v = tid / NARROW_BN, col = tid - v * NARROW_BN;
         tp          = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
     }
     int qflag = 1;
-    if (have_qp && u_fl != 0)
+    if (wave == 0 && have_qp && u_fl != 0)
         qflag = *(const MI355_GLOBAL int32_t *)u_fl;
 
     // ---- B panel and the staged window: transfers of 1 KiB, dealt out to the 16 waves. A lane of a window transfer
@@ -530,27 +532,37 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
     }
 
-    // ---- this wave's tile: 32 consecutive pixels of the band ----
+    // ---- this wave's tile: 32 consecutive pixels of the band (worked out in front of the barrier by the waves that
+    // have to wait there anyway, behind it by the others) ----
     const bool active = wave * NARROW_ROWS < P;
     int32_t    s0[RS]; // LDS pixel index of the top-left tap of each of the tile's rows
-#pragma unroll
-    for (int rb = 0; rb < RS; ++rb)
+    auto       tile_setup = [&]()
     {
-        const int lp = min(wave * NARROW_ROWS + rb * 16 + lr, P - 1);
-        const int ry = narrow_div(lp, cg.magic_OW), ox = lp - ry * cg.OW;
-        s0[rb]       = s_img + ry * cg.stride_y * Wp + ox * cg.stride_x;
-    }
+#pragma unroll
+        for (int rb = 0; rb < RS; ++rb)
+        {
+            const int lp = min(wave * NARROW_ROWS + rb * 16 + lr, P - 1);
+            const int ry = narrow_div(lp, cg.magic_OW), ox = lp - ry * cg.OW;
+            s0[rb]       = s_img + ry * cg.stride_y * Wp + ox * cg.stride_x;
+        }
+    };
+    if (wave < HALO_DMA_WAVES)
+        tile_setup();
     MI355_BAND_PHASE(1); // transfers issued, addresses set up
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's transfers (and its constant)
     MI355_BAND_PHASE(2); // this wave's transfers have landed
     if (have_qp && tid < NPAR * NARROW_BN)
         par[tid] = tp;
-    const int  qflag_u = __builtin_amdgcn_readfirstlane(qflag);
-    const bool fast    = have_qp && (qflag_u & 1) == 0;
+    if (tid == 0)
+        par[NPAR * NARROW_BN] = qflag; // (the area is padded to the next KiB: there is room)
     __syncthreads();
     MI355_BAND_PHASE(3); // everybody's transfers have landed
     if (!active)
         return;
+    if (wave >= HALO_DMA_WAVES)
+        tile_setup();
+    const int  qflag_u = __builtin_amdgcn_readfirstlane(par[NPAR * NARROW_BN]);
+    const bool fast    = have_qp && (qflag_u & 1) == 0;
 
     // waves that share a SIMD (w, w + 4, w + 8, w + 12) get different priorities: one at a time goes through the matrix
     // instructions and its epilogue then runs beside the matrix instructions of the next

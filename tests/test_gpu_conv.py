@@ -543,6 +543,48 @@ def test_conv_f32_destination_padded():
     assert (got[mask] == 7.5).all(), "padding of the destination was overwritten"
 
 
+def test_conv_band_form_random_geometry_sweep():
+    """10 seeded geometries on images large enough for the band form: kernel sizes, strides, asymmetric padding,
+    dilation, 64 / 128 channels, 1 to 64 output channels, both source signs, weights with and without an offset"""
+    rng = np.random.default_rng(1777)
+    done, bands = 0, 0
+    while done < 10:
+        C = int(rng.choice([64, 64, 128]))
+        KH, KW = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        if KH * KW * C > 1152:
+            continue
+        stride = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pad = tuple(int(x) for x in rng.integers(0, 3, size=4))
+        B_ = int(rng.integers(1, 4))
+        # about 36000 output pixels
+        OW = int(rng.integers(40, 180))
+        OH = max(8, 36000 // (B_ * OW) + int(rng.integers(0, 9)))
+        W = (OW - 1) * stride[0] + dil[0] * (KW - 1) + 1 - pad[0] - pad[2]
+        H = (OH - 1) * stride[1] + dil[1] * (KH - 1) + 1 - pad[1] - pad[3] + int(rng.integers(0, stride[1]))
+        if B_ * OH * OW <= 4 * 256 * 32 or W < 1 or H < 1:
+            continue
+        OFM = int(rng.choice([1, 7, 24, 40, 64, 64]))
+        dt = np.int8 if rng.integers(2) else np.uint8
+        w_dt = np.int8 if (dt == np.int8 or rng.integers(2)) else np.uint8
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=(B_, H, W, C)).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + (1 if w_dt == np.int8 else 0), np.iinfo(w_dt).max + 1, size=(OFM, KH, KW, C)).astype(w_dt)
+        bias = rng.integers(-800, 800, size=OFM, dtype=np.int32)
+        in_zp = int(rng.integers(-10, 10)) if dt == np.int8 else int(rng.integers(100, 150))
+        w_zp = 0 if w_dt == np.int8 else int(rng.integers(100, 150))
+        K = KH * KW * C
+        reals = rng.uniform(0.5, 2.0, OFM) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+        mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        want = oracle.conv_nhwc_direct(src, w, bias, in_zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+        announce("conv band sweep", done, src.shape, w.shape, stride, pad, dil, dt.__name__, w_dt.__name__, in_zp, w_zp)
+        got, name = run_conv(src, w, bias, in_zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+        np.testing.assert_array_equal(got, want)
+        bands += name == "implicit_band_32x64"
+        done += 1
+    assert bands >= 6, bands  # (an output row of more than 512 pixels or a window beyond LDS takes the other form)
+
+
 def test_conv_random_geometry_sweep():
     """40 seeded geometries: kernel sizes, strides, asymmetric padding, dilation, channel counts on and off the implicit
     loader's 16-byte granularity, both layouts, both signs, per-tensor and per-channel weights"""

@@ -170,15 +170,15 @@ def run_ceilings(torch, args):
 
     spans = torch.zeros(256 * 4, dtype=torch.int64, device="cuda")
 
-    def timed(name, fn, data, waves):
+    def timed(name, fn, data, waves, work=1.0):
         """us: per launch over graph replays (launch to launch). span_us: from the first wave's start of its timed loop
         to the last wave's end, over all workgroups of the last launch (100 MHz counter) - what the chip needs for the
         instructions themselves; the loop of a single wave says little (the oldest wave of a SIMD is served first)."""
-        s = time_graph(torch, [fn], args.steps)
+        s = time_graph(torch, [fn], args.steps) / work  # (work: this kernel's instruction count over config 2's)
         torch.cuda.synchronize()
         sp = spans.cpu().numpy().reshape(256, 4)
-        span = float(sp[:, 1].max() - sp[:, 0].min()) * 1e-8
-        mean_clocks = float(sp[:, 3].sum()) / (256 * waves)
+        span = float(sp[:, 1].max() - sp[:, 0].min()) * 1e-8 / work
+        mean_clocks = float(sp[:, 3].sum()) / (256 * waves) / work
         wave_real = float((sp[:, 1] - sp[:, 0]).mean()) * 1e-8  # a workgroup's own span, averaged
         out["mfma_cfg2_instruction_count"].append({
             "what": name, "operands": data, "us": round(s * 1e6, 3), "TOPS": round(ops / s / 1e12, 1),
@@ -186,7 +186,7 @@ def run_ceilings(torch, args):
             "span_us": round(span * 1e6, 2), "span_TOPS": round(ops / span / 1e12, 1),
             "span_frac_of_5.0_POPs": round(ops / span / 1e12 / INT8_DENSE_PEAK_TOPS, 4),
             "workgroup_span_us_mean": round(wave_real * 1e6, 2),
-            "loop_clocks_mean_per_wave": int(mean_clocks), "loop_clocks_longest_wave": int(sp[:, 2].max()),
+            "loop_clocks_mean_per_wave": int(mean_clocks), "loop_clocks_longest_wave": int(sp[:, 2].max() / work),
             "shader_MHz_from_longest_wave": round(float(sp[:, 2].max()) / max(span * 1e6, 1e-9), 1)})
 
     for data, src in (("random", rnd), ("zero", zero)):
@@ -197,11 +197,14 @@ def run_ceilings(torch, args):
         timed("operands from LDS, 64x64 wave tiles, all reads then all matrix instructions then a barrier per K step",
               lambda cs, src=src: cl.mi355_ceiling_mfma_lds(src.data_ptr(), 256, 32, sink.data_ptr(), ticks.data_ptr(),
                                                             spans.data_ptr(), cs), data, 8)
-        for waves in (8, 4):
-            timed("operands from LDS, %s wave tiles, double-buffered in registers, reads interleaved, no barrier" %
-                  ("64x64" if waves == 8 else "128x64"),
-                  lambda cs, src=src, waves=waves: cl.mi355_ceiling_mfma_lds_pipelined(src.data_ptr(), 256, waves, 32, sink.data_ptr(),
-                                                                                      spans.data_ptr(), cs), data, waves)
+        for tile, waves, what in ((0, 8, "operands from LDS, 64x64 wave tiles"), (1, 4, "operands from LDS, 128x64 wave tiles"),
+                                  (2, 4, "operands from LDS, 64x128 wave tiles"),
+                                  (3, 4, "A from LDS, B straight from global memory in operand order, 128x64 wave tiles")):
+            # (33 K steps for the global-fed form: its loop is written out for multiples of 3; its figures are scaled back)
+            steps_k = 33 if tile == 3 else 32
+            timed(what + ", double-buffered in registers, reads interleaved, no barrier",
+                  lambda cs, src=src, tile=tile, steps_k=steps_k: cl.mi355_ceiling_mfma_lds_pipelined(
+                      src.data_ptr(), 256, tile, steps_k, sink.data_ptr(), spans.data_ptr(), cs), data, waves, steps_k / 32.0)
     # LDS operand reads alone: 16 KiB per wave and step, 32 steps (config 2 reads 128 KiB per compute unit and step)
     out["lds_operand_reads"] = []
     sink2 = torch.zeros(256 * 1024, dtype=torch.int32, device="cuda")

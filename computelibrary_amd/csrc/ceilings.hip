@@ -7,7 +7,8 @@
 //   mi355_ceiling_mfma_lds    the same instruction count with every operand read from LDS first (64 x 64 wave tiles),
 //                             the plain schedule: all reads of a K step, then its matrix instructions, then a barrier
 //   mi355_ceiling_mfma_lds_pipelined   the same with operands double-buffered in registers, reads interleaved with the
-//                             matrix instructions, no barrier; 64 x 64 or 128 x 64 wave tiles
+//                             matrix instructions, no barrier; 64 x 64, 128 x 64 or 64 x 128 wave tiles, or only A from LDS
+//                             and the B operand blocks straight from global memory
 //   mi355_ceiling_lds_read    the operand reads of the pipelined GEMM alone (LDS bandwidth per compute unit)
 //   mi355_ceiling_dma         the pipelined GEMM's global -> LDS stream alone (direct-to-LDS loads, 3-slot ring)
 //   mi355_ceiling_clock       shader clock while other work runs: shader-clock ticks over a span of real time
@@ -186,13 +187,17 @@ __global__ __launch_bounds__(512) void mfma_lds_kernel(const v4i *__restrict__ s
 // The matrix instructions of the 256 x 128 x 128 tile with every operand read from LDS first, scheduled as well as this
 // file knows how: the stage holds static data, so nothing waits for a producer and there is no barrier; operands are
 // double-buffered in registers by halves of a K step (64 of K), and the reads of the next half are interleaved one by
-// one behind the first matrix instructions of this half (what the pipelined GEMM's consumer waves do). NW = 8: wave
-// tiles of 64 x 64 (8 reads per 16 matrix instructions); NW = 4: wave tiles of 128 x 64 (12 reads per 32). Rows of 128
-// bytes, 16-byte piece p of row r at position p ^ ((r >> 1) & 7): free of bank conflicts.
-template <int NW>
+// one behind the first matrix instructions of this half (what the pipelined GEMM's consumer waves do). Wave tiles of
+// (RS * 16) x (QS * 16): 64 x 64 (8 waves, 8 reads per 16 matrix instructions), 128 x 64 or 64 x 128 (4 waves, 12 reads per
+// 32). Rows of 128 bytes, 16-byte piece p of row r at position p ^ ((r >> 1) & 7): free of bank conflicts.
+// BGLOBAL: the B operand blocks do not pass through LDS at all - they come straight from global memory in operand order
+// (1 KiB per block, the 64 lanes' 16 bytes one after the other: the layout the streaming kernel's packed B has), fetched
+// one half step ahead into registers; only A is read from LDS. Every workgroup walks its own 512 KiB of B (one of 32
+// column tiles of config 2), which the L2 holds.
+template <int RS, int QS, bool BGLOBAL>
 __global__ __launch_bounds__(512) void mfma_lds_pipelined_kernel(const v4i *__restrict__ src, int steps, int *sink, int64_t *spans)
 {
-    constexpr int RS = NW == 8 ? 4 : 8, QS = 4;
+    constexpr int WN = 128 / (QS * 16); // waves along the tile's columns; wave -> (wave / WN, wave % WN)
     extern __shared__ __attribute__((aligned(1024))) char smem[]; // 3 x 48 KiB
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < 3 * 49152 / 16; i += blockDim.x)
@@ -203,13 +208,13 @@ __global__ __launch_bounds__(512) void mfma_lds_pipelined_kernel(const v4i *__re
 #pragma unroll
     for (int f = 0; f < RS; ++f)
     {
-        const int r = ((wave >> 1) * RS + f) * 16 + row;
+        const int r = ((wave / WN) * RS + f) * 16 + row;
         offa[f]     = (uint32_t)(r * 128 + ((lh ^ ((r >> 1) & 7)) << 4));
     }
 #pragma unroll
     for (int f = 0; f < QS; ++f)
     {
-        const int r = 256 + ((wave & 1) * QS + f) * 16 + row;
+        const int r = 256 + ((wave % WN) * QS + f) * 16 + row;
         offb[f]     = (uint32_t)(r * 128 + ((lh ^ ((r >> 1) & 7)) << 4));
     }
     v4i acc[RS][QS];
@@ -250,19 +255,79 @@ __global__ __launch_bounds__(512) void mfma_lds_pipelined_kernel(const v4i *__re
         __builtin_amdgcn_sched_barrier(0);
     };
     const int64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
-    read_half(smem, 0, fa[0], fb[0]);
-    for (int kt = 0; kt < steps; ++kt)
+    int           extra = 0;
+    if constexpr (!BGLOBAL)
     {
-        const char *cur = smem + (kt % 3) * 49152, *nxt = smem + ((kt + 1) % 3) * 49152;
-        read_half(cur, 1, fa[1], fb[1]);
-        multiply(fa[0], fb[0]);
-        interleave();
-        read_half(nxt, 0, fa[0], fb[0]); // (after the last step: a read nobody uses)
-        multiply(fa[1], fb[1]);
-        interleave();
+        read_half(smem, 0, fa[0], fb[0]);
+        for (int kt = 0; kt < steps; ++kt)
+        {
+            const char *cur = smem + (kt % 3) * 49152, *nxt = smem + ((kt + 1) % 3) * 49152;
+            read_half(cur, 1, fa[1], fb[1]);
+            multiply(fa[0], fb[0]);
+            interleave();
+            read_half(nxt, 0, fa[0], fb[0]); // (after the last step: a read nobody uses)
+            multiply(fa[1], fb[1]);
+            interleave();
+        }
+        extra = fb[0][0][0];
+    }
+    else
+    {
+        // half steps between a B block's load and its use: 1 - two register sets, as many registers as the LDS-fed form
+        // (2 needs a third set: 256 registers and 10 of them spilled, at the 8 waves per compute unit of the product)
+        constexpr int BDIST = 1;
+        // half step i of the walk: blocks ((i * WN + wave % WN) * QS + q) of this workgroup's 512 KiB
+        // (src holds 16 MiB = 2^20 pieces: the index is taken modulo that, like the LDS fill above - 33 K steps of the last
+        // of the 32 column tiles would otherwise end 16 KiB beyond the buffer)
+        const size_t bbase = (size_t)(blockIdx.x & 31) * (512 * 1024 / 16) + lane;
+        v4i        gb[BDIST + 1][QS];
+        auto       load_b = [&](int i, v4i (&b)[QS])
+        {
+            const int ii = i < 2 * steps ? i : 0; // (beyond the end: a load nobody uses)
+#pragma unroll
+            for (int q = 0; q < QS; ++q)
+                b[q] = src[(bbase + (size_t)((ii * WN + wave % WN) * QS + q) * 64) & 0xFFFFF];
+        };
+        auto read_a = [&](const char *stage, int half, v4i (&a)[RS])
+        {
+#pragma unroll
+            for (int f = 0; f < RS; ++f)
+                a[f] = *(const v4i *)(stage + (offa[f] ^ (uint32_t)(half * 64)));
+        };
+        auto half_step = [&](const v4i (&a)[RS], const v4i (&b)[QS])
+        {
+            // this half's B blocks are the oldest loads in flight: BDIST younger half steps may stay out
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(BDIST * QS) : "memory");
+            multiply(a, b);
+#pragma unroll
+            for (int i = 0; i < RS; ++i)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, RS * QS - RS, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        static_assert(BDIST == 1, "the rotation below is written out for two register sets");
+        load_b(0, gb[0]);
+        read_a(smem, 0, fa[0]);
+        // 6 half steps per trip (3 K steps: the ring of stages comes round)
+        for (int i = 0; i < 2 * steps; i += 6)
+        {
+#pragma unroll
+            for (int u = 0; u < 6; ++u)
+            {
+                const int   h   = i + u; // half step: K step h / 2, half h % 2
+                const char *stg = smem + (((h + 1) / 2) % 3) * 49152;
+                load_b(h + 1, gb[(u + 1) & 1]);
+                read_a(stg, (h + 1) & 1, fa[(u + 1) & 1]);
+                half_step(fa[u & 1], gb[u & 1]);
+            }
+        }
+        extra = gb[0][0][0] + gb[1][0][0];
     }
     const int64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
-    int           sum = fa[0][0][0] + fb[0][0][0];
+    int           sum = fa[0][0][0] + extra;
 #pragma unroll
     for (int i = 0; i < RS; ++i)
 #pragma unroll
@@ -419,29 +484,29 @@ int mi355_ceiling_mfma(const void *src, int shape, int grid, int mfma16, int *si
     return (int)hipGetLastError();
 }
 
-// The pipelined form (see mfma_lds_pipelined_kernel): waves 8 (64 x 64 wave tiles) or 4 (128 x 64); every workgroup
-// issues steps * 256 * 128 * 128 multiply-accumulates
-int mi355_ceiling_mfma_lds_pipelined(const void *src, int grid, int waves, int steps, int *sink, int64_t *spans, void *stream)
+// The pipelined form (see mfma_lds_pipelined_kernel). tile: 0 = 64 x 64 wave tiles (8 waves), 1 = 128 x 64 (4 waves),
+// 2 = 64 x 128 (4 waves), 3 = 128 x 64 with the B operand blocks straight from global memory (src: at least 16 MiB);
+// steps: K steps of 128 (with tile 3 a multiple of 3); every workgroup issues steps * 256 * 128 * 128 multiply-accumulates
+int mi355_ceiling_mfma_lds_pipelined(const void *src, int grid, int tile, int steps, int *sink, int64_t *spans, void *stream)
 {
-    if (!src || !sink || grid < 1 || steps < 1 || (waves != 4 && waves != 8))
+    if (!src || !sink || grid < 1 || steps < 1 || tile < 0 || tile > 3 || (tile == 3 && steps % 3 != 0))
         return (int)hipErrorInvalidValue;
+    const void *fns[4] = {(const void *)mfma_lds_pipelined_kernel<4, 4, false>, (const void *)mfma_lds_pipelined_kernel<8, 4, false>,
+                          (const void *)mfma_lds_pipelined_kernel<4, 8, false>, (const void *)mfma_lds_pipelined_kernel<8, 4, true>};
     static bool raised = false;
     if (!raised)
     {
-        hipError_t e = hipFuncSetAttribute((const void *)mfma_lds_pipelined_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)mfma_lds_pipelined_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
-        if (e != hipSuccess)
-            return (int)e;
+        for (const void *f : fns)
+        {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 49152);
+            if (e != hipSuccess)
+                return (int)e;
+        }
         raised = true;
     }
-    if (waves == 8)
-        hipLaunchKernelGGL(mfma_lds_pipelined_kernel<8>, dim3(grid), dim3(512), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps,
-                           sink, spans);
-    else
-        hipLaunchKernelGGL(mfma_lds_pipelined_kernel<4>, dim3(grid), dim3(256), 3 * 49152, (hipStream_t)stream, (const v4i *)src, steps,
-                           sink, spans);
-    return (int)hipGetLastError();
+    const v4i *p       = (const v4i *)src;
+    void      *kargs[] = {(void *)&p, (void *)&steps, (void *)&sink, (void *)&spans};
+    return (int)hipLaunchKernel(fns[tile], dim3(grid), dim3(tile == 0 ? 512 : 256), kargs, 3 * 49152, (hipStream_t)stream);
 }
 
 int mi355_ceiling_mfma_lds(const void *src, int grid, int steps, int *sink, int64_t *ticks, int64_t *spans, void *stream)

@@ -144,3 +144,33 @@ def test_noalloc_refuses_a_second_stream_while_the_first_is_busy():
     np.testing.assert_array_equal(D0.cpu().numpy(), ref0)
     g.close()
     g0.close()
+
+
+def test_noalloc_captured_in_a_hip_graph_on_a_handle_that_never_ran():
+    """What the entry point is for: a handle that has only been prepared is run for the first time inside a stream
+    capture (rows that are not dword aligned: the padded copy of A and the row sums live in the fixed workspace), and
+    every replay - with eager work and synchronisations in between - reproduces the oracle's bytes. (The per-GPU set-up of
+    the workspace happened in an earlier call of this process, outside any capture.)"""
+    import torch
+    M, N, K = 300, 200, 528
+    Ad0, g0, _, want0, keep0 = _case(64, 64, 272, 275, np.uint8, np.uint8, 9, 900, run_first=False)
+    D0 = torch.zeros((64, 64), dtype=torch.uint8, device="cuda")
+    g0.run_noalloc(Ad0, D0)  # the set-up call
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(D0.cpu().numpy(), want0)
+    g0.close()
+    Ad, g, _, want, keep = _case(M, N, K, K + 3, np.uint8, np.uint8, 9, 901, run_first=False)
+    D = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    announce("no-alloc, graph capture of a cold handle", (M, N, K))
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        g.run_noalloc(Ad, D, stream=torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        D.fill_(77)  # eager work between replays
+        torch.cuda.synchronize()
+        announce("no-alloc, graph replay", rep)
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(D.cpu().numpy(), want)
+    g.close()

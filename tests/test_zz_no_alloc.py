@@ -132,8 +132,9 @@ def test_noalloc_refuses_a_second_stream_while_the_first_is_busy():
     s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
     torch.cuda.synchronize()
     announce("no-alloc, two streams")
-    for _ in range(400):  # several milliseconds of queued work on the first stream
-        g.run_noalloc(Ad, D, stream=s1.cuda_stream)
+    with torch.cuda.stream(s1):
+        torch.cuda._sleep(100_000_000)  # tens of milliseconds of queued work in front of the first stream's call
+    g.run_noalloc(Ad, D, stream=s1.cuda_stream)
     with pytest.raises(capi.Mi355Error, match="still in use"):
         g.run_noalloc(Ad, D, stream=s2.cuda_stream)
     g0.run_noalloc(Ad0, D0, stream=s2.cuda_stream)  # nothing of it lives in the workspace

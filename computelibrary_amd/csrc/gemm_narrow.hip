@@ -442,6 +442,9 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // LDS: B panel [64][PITCH] | par[NPAR][64] | (to the next KiB) the staged window
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 #define MI355_GLOBAL __attribute__((address_space(1)))
+#ifdef MI355_PHASE_CLOCKS
+    const long long t_entry = (long long)wall_clock64(); // before the first argument is asked for
+#endif
     ConvGeom  cg = g.conv;
     uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp,
               u_fl = (uintptr_t)g.epi.qp_flag;
@@ -468,6 +471,10 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const int band_row = band_blk < 0 ? -1 : (wave == 0 ? band_blk * 2 : (wave == 12 ? band_blk * 2 + 1 : -1));
 #endif
     MI355_BAND_PHASE(0); // arguments fetched
+#ifdef MI355_PHASE_CLOCKS
+    if (band_row >= 0 && lane == 0)
+        band_clocks[band_row][6] = t_entry;
+#endif
 
     // this workgroup's band: output rows [oy0, oy1) of image n. Staged in LDS: the window of input rows and columns
     // under it, padding included - rows iy_first .. iy_first + in_rows - 1, columns -pad_left .. -pad_left + Wp - 1,

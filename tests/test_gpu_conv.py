@@ -277,6 +277,24 @@ def test_conv_deep_patches_under_few_tiles_run_as_k_slices():
                 got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil, path=path)
                 assert "_splitk" in name and name.startswith("implicit" if path == capi.CONV_AUTO else "im2col"), name
                 np.testing.assert_array_equal(got, want)
+    # the dequantising (F32) destination through the same slices
+    import torch
+    src = rng.integers(-128, 128, size=(1, 14, 14, 512), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(96, 3, 3, 512), dtype=np.int8)
+    bias_f = rng.normal(0.0, 2.0, size=96).astype(np.float32)
+    scale = float(np.float32(0.02) * np.float32(0.005))
+    cols = oracle.im2col_nhwc(src, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 4)
+    want = oracle.gemmlowp_f32(cols, oracle.weights_reshape(w), bias_f, -4, 0, scale, 0.0, 6.0, act_twice=False)
+    cv = capi.Conv(capi.conv_desc(1, 14, 14, 512, 96, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), capi.S8, capi.S8, capi.F32, -4, 0, 4,
+                                  scale=scale, act=(0.0, 6.0)))
+    sd, wd, od, bd = to_dev(src), to_dev(w), to_dev(np.zeros((1, 14, 14, 96), np.float32)), to_dev(bias_f)
+    cv.prepare(wd, bd)
+    announce("conv k slices, F32 destination", cv.kernel_name)
+    cv.run(sd, od)
+    torch.cuda.synchronize()
+    assert "_splitk" in cv.kernel_name, cv.kernel_name
+    assert np.array_equal(od.cpu().numpy().reshape(-1, 96).view(np.uint32), want.view(np.uint32))
+    cv.close()
 
 
 def test_conv_channel_counts_padded_to_16():

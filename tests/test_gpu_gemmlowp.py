@@ -199,10 +199,11 @@ def test_batched_small_products_take_the_streaming_kernel():
         for z in range(batch):
             np.testing.assert_array_equal(
                 got[z], oracle.gemmlowp_fixedpoint(A[z], B[z] if b_batched else B, bias, ao, bo, [mult], [shift], -3, -128, 127, np.int8))
-        got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, device=False)
-        for z in range(batch):
-            np.testing.assert_array_equal(got[z].view(np.uint32),
-                                          oracle.gemmlowp_f32(A[z], B[z] if b_batched else B, None, ao, bo, 3e-4).view(np.uint32))
+        for device in (False, True):
+            got, _ = run_gemm(A, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, device=device)
+            for z in range(batch):
+                np.testing.assert_array_equal(got[z].view(np.uint32),
+                                              oracle.gemmlowp_f32(A[z], B[z] if b_batched else B, None, ao, bo, 3e-4).view(np.uint32))
 
 
 def test_f16_fixture(golden):

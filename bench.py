@@ -317,14 +317,16 @@ def run_phase_clocks(torch, capi, args):
         sys.exit(1)
     rows = []
     for r in range(6):
-        v = [int(buf[r * 8 + i]) for i in range(5)]
+        v = [int(buf[r * 8 + i]) for i in range(6)]
         who = ("first", "middle", "last")[r // 2] + " workgroup, " + ("consumer wave 0" if r % 2 == 0 else "producer wave 0")
+        # (entry: from the wave's first instruction to the first stamp - what it waits for its arguments)
         if r % 2 == 0:
-            parts = {"set_up": v[1] - v[0], "wait_for_stage_0": v[2] - v[1], "k_loop": v[3] - v[2], "epilogue": v[4] - v[3]}
+            parts = {"entry": v[0] - v[5], "set_up": v[1] - v[0], "wait_for_stage_0": v[2] - v[1], "k_loop": v[3] - v[2],
+                     "epilogue": v[4] - v[3]}
         else:
-            parts = {"set_up": v[1] - v[0], "issue_first_stages": v[2] - v[1], "wait_for_stage_0": v[3] - v[2],
+            parts = {"entry": v[0] - v[5], "set_up": v[1] - v[0], "issue_first_stages": v[2] - v[1], "wait_for_stage_0": v[3] - v[2],
                      "k_loop": v[4] - v[3]}
-        parts["total"] = v[4] - v[0]
+        parts["total"] = v[4] - v[5]
         rows.append({"wave": who, "clocks": parts})
     print(json.dumps({"phase_clocks": True, "workload": "config 2: M=2048 N=4096 K=4096 s8 -> s8", "kernel": g.kernel_name,
                       "kernel_us_instrumented_build": round(kern_s * 1e6, 3), "eager_us": round(evt / args.steps * 1e6, 3),

@@ -598,6 +598,9 @@ __global__ __launch_bounds__(GWM *GWN * 192) __attribute__((amdgpu_waves_per_eu(
 template <int BM, int BN, int BK, int NS, int EPI, bool FLIP_A>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
 {
+#ifdef MI355_PHASE_CLOCKS
+    const long long t_entry = (long long)__builtin_readcyclecounter(); // before the first argument is asked for
+#endif
     GemmArgs g = g_in;
     asm volatile(""
                  : "+s"(g.tiles_m), "+s"(g.tiles_n), "+s"(g.magic_tiles), "+s"(g.magic_group), "+s"(g.tile_magic_ok), "+s"(g.lda),
@@ -631,6 +634,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
     const int phase_blk = blockIdx.x == 0 ? 0 : ((int)blockIdx.x == g.nblocks / 2 ? 1 : ((int)blockIdx.x == g.nblocks - 1 ? 2 : -1));
     const int phase_row = phase_blk < 0 ? -1 : (wave == 0 ? phase_blk * 2 : (wave == NW ? phase_blk * 2 + 1 : -1));
     MI355_PHASE(0);
+    if (phase_row >= 0 && lane == 0)
+        phase_clocks[phase_row][5] = t_entry;
 #endif
     int tm, tn, bz;
     if (g.tile_magic_ok)

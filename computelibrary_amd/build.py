@@ -26,9 +26,14 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+# per file: the narrow-N convolution kernels' file asks for the first 2 dwords of a kernel's arguments to be preloaded into
+# scalar registers when a wave is launched (see conv_halo_kernel)
+FILE_FLAGS = {"gemm_narrow.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"]}
+
+
 def _compile(src, extra=(), suffix=""):
     obj = os.path.join(OBJDIR, src.replace(".hip", suffix + ".o"))
-    cmd = [HIPCC] + FLAGS + list(extra) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + FILE_FLAGS.get(src, []) + list(extra) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

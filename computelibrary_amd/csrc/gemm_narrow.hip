@@ -433,21 +433,34 @@ __device__ long long band_clocks[6][8];
 #endif
 
 template <int EPI, bool FLIP_A, int NB>
-__global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_halo_kernel(GemmArgs g)
+// (p_Bp: the panel image's address once more, in front of the argument block. This file is compiled with
+// -mllvm -amdgpu-kernarg-preload-count=2: a kernel's first two argument dwords arrive in scalar registers with the wave, so
+// the panel's transfers - more than half of all - go out while the block is still being fetched: 10 scalar loads over
+// 6 cache lines per wave, 0.25 us for the first wave of a workgroup and up to 1 us for the last.)
+__global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_halo_kernel(const int8_t *p_Bp, GemmArgs g)
 {
     constexpr int RS = NARROW_ROWS / 16, QS = NARROW_BN / 16;
     constexpr int KBLK  = NB * 3;
     constexpr int PITCH = KBLK * 64 + NARROW_PAD_PIECES * 16;
     constexpr int NPAR  = 1 + QP_COUNT;
+    constexpr int NDMA  = KBLK * 4 + NARROW_PAD_PIECES; // transfers of 1 KiB that make up the panel
     // LDS: B panel [64][PITCH] | par[NPAR][64] | (to the next KiB) the staged window
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 #define MI355_GLOBAL __attribute__((address_space(1)))
 #ifdef MI355_PHASE_CLOCKS
     const long long t_entry = (long long)wall_clock64(); // before the first argument is asked for
 #endif
+    {
+        // ---- the B panel: linear transfers of 1 KiB, by the first HALO_DMA_WAVES waves ----
+        const int      wv = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+        const uint32_t l0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
+        if (wv < HALO_DMA_WAVES)
+            for (int ins = wv; ins < NDMA; ins += HALO_DMA_WAVES)
+                narrow_dma16((const void *)((const MI355_GLOBAL int8_t *)p_Bp + ins * 1024), ((uint32_t)threadIdx.x & 63u) * 16u,
+                             l0 + (uint32_t)ins * 1024u);
+    }
     ConvGeom  cg = g.conv;
-    uintptr_t u_a = (uintptr_t)g.A, u_b = (uintptr_t)g.Bp, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp,
-              u_fl = (uintptr_t)g.epi.qp_flag;
+    uintptr_t u_a = (uintptr_t)g.A, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp, u_fl = (uintptr_t)g.epi.qp_flag;
     int32_t   a_qps = (int32_t)g.epi.qp_stride, wpi = g.tiles_m, rpw = g.tiles_n; // workgroups per image, output rows per workgroup
     uint32_t  magic_wp = g.magic_tiles; // for the division by the staged window's width (see halo_plan)
     uintptr_t u_fill   = (uintptr_t)g.fill16;
@@ -455,11 +468,10 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     asm volatile(""
                  : "+s"(cg.H), "+s"(cg.W), "+s"(cg.C), "+s"(cg.KH), "+s"(cg.KW), "+s"(cg.OW), "+s"(cg.OH), "+s"(cg.stride_x),
                    "+s"(cg.stride_y), "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word),
-                   "+s"(cg.magic_C), "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(a_qps), "+s"(u_a), "+s"(u_b), "+s"(u_cv), "+s"(u_qp),
+                   "+s"(cg.magic_C), "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(a_qps), "+s"(u_a), "+s"(u_cv), "+s"(u_qp),
                    "+s"(u_fl), "+s"(wpi), "+s"(rpw));
     int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
     static_assert(((NARROW_BN * PITCH + NPAR * NARROW_BN * 4) & 1023) != 0, "one more word (the flag) fits in front of the next KiB");
-    const MI355_GLOBAL int8_t *const  gB = (const MI355_GLOBAL int8_t *)u_b;
     const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
 
     const int tid  = threadIdx.x;
@@ -513,20 +525,15 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     if (wave == 0 && have_qp && u_fl != 0)
         qflag = *(const MI355_GLOBAL int32_t *)u_fl;
 
-    // ---- B panel and the staged window: transfers of 1 KiB, dealt out to the 16 waves. A lane of a window transfer
-    // fetches the piece its LDS position stands for from the image, or 16 bytes of the padding value ----
-    constexpr int   NDMA = KBLK * 4 + NARROW_PAD_PIECES;
+    // ---- the staged window: transfers of 1 KiB; a lane fetches the piece its LDS position stands for from the image, or
+    // 16 bytes of the padding value. (By the first HALO_DMA_WAVES waves only, like the panel's: the later a wave of the
+    // workgroup gets its arguments, the less it should have to do before the barrier - the barrier waits for it.) ----
     const int       nimg = ((staged << lc) + 1023) >> 10;
     const uintptr_t img  = u_a + (uintptr_t)((int64_t)n * cg.H * cg.W * cg.C);
-    // (by the first HALO_DMA_WAVES waves only: the waves of a workgroup start one after the other over most of a
-    // microsecond, and what the last ones still have to do before the barrier is what the barrier waits for)
-    for (int ins = wave; ins < NDMA + nimg; ins += HALO_DMA_WAVES)
+    for (int ins = NDMA + wave; ins < NDMA + nimg; ins += HALO_DMA_WAVES)
     {
         if (wave >= HALO_DMA_WAVES)
             break;
-        if (ins < NDMA)
-            narrow_dma16((const void *)(gB + ins * 1024), (uint32_t)lane * 16u, lds0 + (uint32_t)ins * 1024u);
-        else
         {
             const int q = (ins - NDMA) * 64 + lane; // position in the window, in pieces
             const int s = q >> lcpr, c = (q & (cpr - 1)) ^ ((((s + s_img) >> sw_sh) & sw_m) << 1);
@@ -822,7 +829,7 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
             GemmArgs a = args;
             a.tiles_m = wpi, a.tiles_n = rpw, a.magic_tiles = mwp;
             const int64_t images = (int64_t)args.M / ((int64_t)args.conv.OH * args.conv.OW);
-            void         *kargs[] = {&a};
+            void         *kargs[] = {&a.Bp, &a};
             if (band)
                 *band = true;
             return (int)hipLaunchKernel(hf, dim3((unsigned)(images * wpi)), dim3(HALO_WAVES * 64), kargs, hl, s);

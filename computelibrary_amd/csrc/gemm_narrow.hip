@@ -506,7 +506,9 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // modulo 256 bytes for pixels of 4, 8 and 16 or more pieces (checked by enumeration for every start s).
     const int cpr = cg.C >> 4, lcpr = 31 - __builtin_clz(cpr), lc = lcpr + 4;
     const int sw_m = cpr >= 16 ? 7 : (cpr == 8 ? 3 : 1), sw_sh = cpr >= 16 ? 0 : (cpr == 8 ? 1 : 2);
-    const int sw_l = 5 - sw_sh, sw_mask = sw_m << 5; // the permutation as a byte offset: ((s << sw_l) & sw_mask) ^ piece * 16
+    // the permutation as a byte offset: ((s << (5 - sw_sh)) & sw_mask) ^ piece * 16, or from the byte offset x = s << lc:
+    // ((x >> sw_r) & sw_mask) - the bits of x below the pixel size land below the mask
+    const int sw_mask = sw_m << 5, sw_r = lc - (5 - sw_sh);
     const uint32_t lds0    = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
     const int      img_off = (NARROW_BN * PITCH + NPAR * NARROW_BN * 4 + 1023) & ~1023;
     const int      s_img   = img_off >> lc; // LDS pixel index of the window's first pixel
@@ -549,7 +551,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // ---- this wave's tile: 32 consecutive pixels of the band (worked out in front of the barrier by the waves that
     // have to wait there anyway, behind it by the others) ----
     const bool active = wave * NARROW_ROWS < P;
-    int32_t    s0[RS]; // LDS pixel index of the top-left tap of each of the tile's rows
+    int32_t    s0[RS]; // LDS byte offset of the top-left tap of each of the tile's rows, plus this lane's 16 bytes of a 64-byte block
     auto       tile_setup = [&]()
     {
 #pragma unroll
@@ -557,7 +559,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         {
             const int lp = min(wave * NARROW_ROWS + rb * 16 + lr, P - 1);
             const int ry = narrow_div(lp, cg.magic_OW), ox = lp - ry * cg.OW;
-            s0[rb]       = s_img + ry * cg.stride_y * Wp + ox * cg.stride_x;
+            s0[rb]       = ((s_img + ry * cg.stride_y * Wp + ox * cg.stride_x) << lc) + lh * 16;
         }
     };
     if (wave < HALO_DMA_WAVES)
@@ -607,17 +609,19 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
             const int kbe = kb < nkb ? kb : 0;
             const int tap = narrow_div(kbe * 64, cg.magic_C), c64 = kbe * 64 - tap * cg.C;
             const int ky = narrow_div(tap, cg.magic_KW), kx = tap - ky * cg.KW;
-            const int ds = ky * cg.dil_y * Wp + kx * cg.dil_x;
-            const int pc = c64 + lh * 16; // this lane's 16 bytes within the pixel
+            const int ds = ((ky * cg.dil_y * Wp + kx * cg.dil_x) << lc) + c64; // the tap and the block within the pixel, in bytes
 #pragma unroll
             for (int q = 0; q < QS; ++q)
                 fb[q] = *(const v4i *)(b_rd + q * 16 * PITCH + kb * 64);
 #pragma unroll
             for (int rb = 0; rb < RSX; ++rb)
             {
-                const int s = s0[rb] + ds;
-                // (C is a power of two: shifts, not a quarter-rate multiply)
-                fa[rb] = *(const v4i *)(smem + ((s << lc) + (((s << sw_l) & sw_mask) ^ pc)));
+                // x: where the piece would lie unpermuted (pixel index << lc, plus the piece's place in the pixel, which
+                // stays below the pixel size); the permutation's bits come from the pixel index. Four instructions per
+                // read. (All the addresses worked out in front of the loop, or the per-column term as the C operand of a
+                // block's first matrix instruction instead of an addition in the epilogue: both measured slower.)
+                const int x = s0[rb] + ds;
+                fa[rb]      = *(const v4i *)(smem + (x ^ ((x >> sw_r) & sw_mask)));
             }
         };
         v4i fa[2][RSX], fb[2][QS];

@@ -580,15 +580,11 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const int  qflag_u = __builtin_amdgcn_readfirstlane(par[NPAR * NARROW_BN]);
     const bool fast    = have_qp && (qflag_u & 1) == 0;
 
-    // waves that share a SIMD (w, w + 4, w + 8, w + 12) get different priorities: one at a time goes through the matrix
-    // instructions and its epilogue then runs beside the matrix instructions of the next
-    switch ((wave >> 2) & 3)
-    {
-    case 0: __builtin_amdgcn_s_setprio(3); break;
-    case 1: __builtin_amdgcn_s_setprio(2); break;
-    case 2: __builtin_amdgcn_s_setprio(1); break;
-    default: break;
-    }
+    // (Different priorities for the waves that share a SIMD - one at a time through the matrix instructions, its epilogue
+    // beside the next wave's - paid while the loop carried twice the address arithmetic; with today's loop, equal
+    // priorities measured 0.4 us faster on a 8.3 us kernel. Pinning the loop's order with scheduling barriers - all six
+    // reads of block kb + 1 in front of the matrix instructions of block kb, where the compiler puts some of the A reads
+    // right in front of their first use - measured 0.1 us slower than the compiler's own order.)
     // (One instance of what follows for every wave: a second, for a last tile of 16 pixels or fewer, measured slower -
     // the code is fetched once per workgroup, a path that one wave takes alone pays for its own instruction fetches.)
     {
@@ -645,7 +641,6 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
                     acc[rb][q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[kb & 1][q], a, acc[rb][q], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_s_setprio(0);
         MI355_BAND_PHASE(4); // matrix instructions issued
 
         const int row0 = m_base + wave * NARROW_ROWS, a_M = m_base + P; // rows of the GEMM this tile covers, and where the band ends

@@ -26,9 +26,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-# per file: the narrow-N convolution kernels' file asks for the first 2 dwords of a kernel's arguments to be preloaded into
+# per file: the narrow-N convolution kernels' file asks for the first 3 dwords of a kernel's arguments to be preloaded into
 # scalar registers when a wave is launched (see conv_halo_kernel)
-FILE_FLAGS = {"gemm_narrow.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"]}
+FILE_FLAGS = {"gemm_narrow.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=3"]}
 
 
 def _compile(src, extra=(), suffix=""):

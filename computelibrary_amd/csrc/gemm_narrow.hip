@@ -432,32 +432,74 @@ __device__ long long band_clocks[6][8];
     } while (0)
 #endif
 
-template <int EPI, bool FLIP_A, int NB>
-// (p_Bp: the panel image's address once more, in front of the argument block. This file is compiled with
-// -mllvm -amdgpu-kernarg-preload-count=2: a kernel's first two argument dwords arrive in scalar registers with the wave, so
-// the panel's transfers - more than half of all - go out while the block is still being fetched: 10 scalar loads over
-// 6 cache lines per wave, 0.25 us for the first wave of a workgroup and up to 1 us for the last.)
-__global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_halo_kernel(const int8_t *p_Bp, GemmArgs g)
+// MULTI: up to NARROW_MAX_PANELS panels of 64 columns (K <= 192, NB == 1), all of them in LDS next to the window: a wave
+// takes its 32 pixels through one panel after the other - matrix instructions, then that panel's epilogue - so that the
+// window, the arguments and the start of a workgroup are paid once for up to 256 output channels.
+// KBU: with several panels, the k blocks of 64 that hold data (K <= 64: 1, <= 128: 2, else 3 - the loop need not cover the
+// panel's zeros as it does with one panel, where K is not known when the kernel is built).
+template <int EPI, bool FLIP_A, int NB, bool MULTI = false, int KBU = NB * 3>
+// (p_Bp, p_ndma: the panel image's address and its size in KiB once more, in front of the argument block. This file is
+// compiled with -mllvm -amdgpu-kernarg-preload-count=3: a kernel's first three argument dwords arrive in scalar registers
+// with the wave, so the panel's transfers - more than half of all - go out while the block is still being fetched: 10
+// scalar loads over 6 cache lines per wave, 0.25 us for the first wave of a workgroup and up to 1 us for the last.)
+__global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_halo_kernel(const int8_t *p_Bp, int32_t p_ndma,
+                                                                                                                GemmArgs g)
 {
+    static_assert(!MULTI || NB == 1, "several panels: one batch of k blocks");
+    static_assert(KBU >= 1 && KBU <= NB * 3 && (MULTI || KBU == NB * 3), "k blocks that hold data");
     constexpr int RS = NARROW_ROWS / 16, QS = NARROW_BN / 16;
     constexpr int KBLK  = NB * 3;
     constexpr int PITCH = KBLK * 64 + NARROW_PAD_PIECES * 16;
     constexpr int NPAR  = 1 + QP_COUNT;
-    constexpr int NDMA  = KBLK * 4 + NARROW_PAD_PIECES; // transfers of 1 KiB that make up the panel
-    // LDS: B panel [64][PITCH] | par[NPAR][64] | (to the next KiB) the staged window
+    constexpr int NDMA  = KBLK * 4 + NARROW_PAD_PIECES; // transfers of 1 KiB that make up a panel
+    // LDS: B panels [npan * 64][PITCH] | par[NPAR][npan * 64], the flag word | (from the next KiB) the staged window
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 #define MI355_GLOBAL __attribute__((address_space(1)))
 #ifdef MI355_PHASE_CLOCKS
     const long long t_entry = (long long)wall_clock64(); // before the first argument is asked for
 #endif
     {
-        // ---- the B panel: linear transfers of 1 KiB, by the first HALO_DMA_WAVES waves ----
+        // ---- the B panels: linear transfers of 1 KiB, wave w of the first HALO_DMA_WAVES those at w, w + 8, ... ----
+        // Written out with scalar registers of its own choosing: the arguments are in flight here, and temporaries that
+        // the compiler places in unused parts of their destination registers make it wait for them first.
         const int      wv = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-        const uint32_t l0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
-        if (wv < HALO_DMA_WAVES)
-            for (int ins = wv; ins < NDMA; ins += HALO_DMA_WAVES)
-                narrow_dma16((const void *)((const MI355_GLOBAL int8_t *)p_Bp + ins * 1024), ((uint32_t)threadIdx.x & 63u) * 16u,
-                             l0 + (uint32_t)ins * 1024u);
+        // (The panels start at LDS address 0: this kernel has no static LDS in front of the dynamic area. The address as a
+        // value would be one more such temporary.)
+        const uint32_t v16 = ((uint32_t)threadIdx.x & 63u) * 16u;
+        const uint32_t b_lo = (uint32_t)(uintptr_t)p_Bp, b_hi = (uint32_t)((uintptr_t)p_Bp >> 32);
+        if (wv < HALO_DMA_WAVES && (!MULTI || wv < p_ndma))
+        {
+            if constexpr (MULTI)
+                asm volatile("s_lshl_b32 s92, %[wv], 10\n\t"
+                             "s_mov_b32 s93, %[wv]\n"
+                             "1:\n\t"
+                             "s_add_u32 s90, %[blo], s92\n\t"
+                             "s_addc_u32 s91, %[bhi], 0\n\t"
+                             "s_mov_b32 m0, s92\n\t"
+                             "global_load_lds_dwordx4 %[v16], s[90:91]\n\t"
+                             "s_add_u32 s93, s93, %[step]\n\t"
+                             "s_add_u32 s92, s92, %[stepb]\n\t"
+                             "s_cmp_lt_i32 s93, %[n]\n\t"
+                             "s_cbranch_scc1 1b" ::[wv] "s"(wv),
+                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "s"(p_ndma), [step] "i"(HALO_DMA_WAVES),
+                             [stepb] "i"(HALO_DMA_WAVES * 1024)
+                             : "s90", "s91", "s92", "s93", "scc", "memory");
+            else
+                asm volatile("s_lshl_b32 s92, %[wv], 10\n\t"
+                             "s_mov_b32 s93, %[wv]\n"
+                             "1:\n\t"
+                             "s_add_u32 s90, %[blo], s92\n\t"
+                             "s_addc_u32 s91, %[bhi], 0\n\t"
+                             "s_mov_b32 m0, s92\n\t"
+                             "global_load_lds_dwordx4 %[v16], s[90:91]\n\t"
+                             "s_add_u32 s93, s93, %[step]\n\t"
+                             "s_add_u32 s92, s92, %[stepb]\n\t"
+                             "s_cmp_lt_i32 s93, %[n]\n\t"
+                             "s_cbranch_scc1 1b" ::[wv] "s"(wv),
+                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "i"(NDMA), [step] "i"(HALO_DMA_WAVES),
+                             [stepb] "i"(HALO_DMA_WAVES * 1024)
+                             : "s90", "s91", "s92", "s93", "scc", "memory");
+        }
     }
     ConvGeom  cg = g.conv;
     uintptr_t u_a = (uintptr_t)g.A, u_cv = (uintptr_t)g.epi.colvec, u_qp = (uintptr_t)g.epi.qp, u_fl = (uintptr_t)g.epi.qp_flag;
@@ -470,8 +512,8 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
                    "+s"(cg.stride_y), "+s"(cg.pad_left), "+s"(cg.pad_top), "+s"(cg.dil_x), "+s"(cg.dil_y), "+s"(cg.pad_word),
                    "+s"(cg.magic_C), "+s"(cg.magic_KW), "+s"(cg.magic_OW), "+s"(a_qps), "+s"(u_a), "+s"(u_cv), "+s"(u_qp),
                    "+s"(u_fl), "+s"(wpi), "+s"(rpw));
-    int32_t *par = (int32_t *)(smem + NARROW_BN * PITCH);
-    static_assert(((NARROW_BN * PITCH + NPAR * NARROW_BN * 4) & 1023) != 0, "one more word (the flag) fits in front of the next KiB");
+    const int npan = MULTI ? __builtin_amdgcn_readfirstlane(g.nblocks) : 1, ncols = npan * NARROW_BN; // panels, their columns
+    int32_t  *par  = (int32_t *)(smem + ncols * PITCH);
     const MI355_GLOBAL int32_t *const g_colvec = (const MI355_GLOBAL int32_t *)u_cv, *const g_qp = (const MI355_GLOBAL int32_t *)u_qp;
 
     const int tid  = threadIdx.x;
@@ -510,18 +552,25 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // ((x >> sw_r) & sw_mask) - the bits of x below the pixel size land below the mask
     const int sw_mask = sw_m << 5, sw_r = lc - (5 - sw_sh);
     const uint32_t lds0    = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)smem;
-    const int      img_off = (NARROW_BN * PITCH + NPAR * NARROW_BN * 4 + 1023) & ~1023;
+    const int      img_off = (ncols * PITCH + NPAR * ncols * 4 + 4 + 1023) & ~1023; // (+ 4: the flag word)
     const int      s_img   = img_off >> lc; // LDS pixel index of the window's first pixel
 
-    // epilogue constants (one dword per thread: 6 x 64 of them), the flag word of the requantisation
-    // (fetched by the waves that start first - the threads of waves 0 to 5 hold one constant each, wave 0 the flag word -
-    // and handed on through LDS: the waves that start last then have nothing to wait for before the barrier)
-    const bool have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
-    int32_t    tp      = 0;
-    if (have_qp && tid < NPAR * NARROW_BN)
+    // epilogue constants (one dword per thread: 6 x 64 of them per panel), the flag word of the requantisation
+    // (fetched by the waves that start first - with one panel the threads of waves 0 to 5 hold one constant each, wave 0
+    // the flag word - and handed on through LDS: the waves that start last then have nothing to wait for before the barrier)
+    const bool    have_qp = EPI == EPI_FIXEDPOINT && u_qp != 0;
+    constexpr int TPN     = MULTI ? (NPAR * NARROW_BN * NARROW_MAX_PANELS + HALO_WAVES * 64 - 1) / (HALO_WAVES * 64) : 1;
+    int32_t       tp[TPN];
+#pragma unroll
+    for (int i = 0; i < TPN; ++i)
     {
-        const int v = tid / NARROW_BN, col = tid - v * NARROW_BN;
-        tp          = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
+        tp[i]         = 0;
+        const int idx = tid + i * HALO_WAVES * 64;
+        if (have_qp && idx < NPAR * ncols)
+        {
+            const int v = idx / ncols, col = idx - v * ncols;
+            tp[i]       = v == 0 ? g_colvec[col] : g_qp[(v - 1) * a_qps + col];
+        }
     }
     int qflag = 1;
     if (wave == 0 && have_qp && u_fl != 0)
@@ -532,19 +581,19 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // workgroup gets its arguments, the less it should have to do before the barrier - the barrier waits for it.) ----
     const int       nimg = ((staged << lc) + 1023) >> 10;
     const uintptr_t img  = u_a + (uintptr_t)((int64_t)n * cg.H * cg.W * cg.C);
-    for (int ins = NDMA + wave; ins < NDMA + nimg; ins += HALO_DMA_WAVES)
+    for (int ins = wave; ins < nimg; ins += HALO_DMA_WAVES)
     {
         if (wave >= HALO_DMA_WAVES)
             break;
         {
-            const int q = (ins - NDMA) * 64 + lane; // position in the window, in pieces
+            const int q = ins * 64 + lane; // position in the window, in pieces
             const int s = q >> lcpr, c = (q & (cpr - 1)) ^ ((((s + s_img) >> sw_sh) & sw_m) << 1);
             const int r = narrow_div(s, magic_wp), x = s - r * Wp;
             const int iy = iy_first + r, ix = x - cg.pad_left;
             // (lanes past the window's end fill LDS nobody looks at)
             const bool      in   = (s < staged) & ((unsigned)iy < (unsigned)cg.H) & ((unsigned)ix < (unsigned)cg.W);
             const uintptr_t from = in ? img + (uint32_t)(((iy * cg.W + ix) << lc) + c * 16) : u_fill;
-            narrow_dma16_at((const void *)from, lds0 + (uint32_t)img_off + (uint32_t)(ins - NDMA) * 1024u);
+            narrow_dma16_at((const void *)from, lds0 + (uint32_t)img_off + (uint32_t)ins * 1024u);
         }
     }
 
@@ -567,17 +616,19 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     MI355_BAND_PHASE(1); // transfers issued, addresses set up
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's transfers (and its constant)
     MI355_BAND_PHASE(2); // this wave's transfers have landed
-    if (have_qp && tid < NPAR * NARROW_BN)
-        par[tid] = tp;
+#pragma unroll
+    for (int i = 0; i < TPN; ++i)
+        if (have_qp && tid + i * HALO_WAVES * 64 < NPAR * ncols)
+            par[tid + i * HALO_WAVES * 64] = tp[i];
     if (tid == 0)
-        par[NPAR * NARROW_BN] = qflag; // (the area is padded to the next KiB: there is room)
+        par[NPAR * ncols] = qflag;
     __syncthreads();
     MI355_BAND_PHASE(3); // everybody's transfers have landed
     if (!active)
         return;
     if (wave >= HALO_DMA_WAVES)
         tile_setup();
-    const int  qflag_u = __builtin_amdgcn_readfirstlane(par[NPAR * NARROW_BN]);
+    const int  qflag_u = __builtin_amdgcn_readfirstlane(par[NPAR * ncols]);
     const bool fast    = have_qp && (qflag_u & 1) == 0;
 
     // (Different priorities for the waves that share a SIMD - one at a time through the matrix instructions, its epilogue
@@ -587,6 +638,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // right in front of their first use - measured 0.1 us slower than the compiler's own order.)
     // (One instance of what follows for every wave: a second, for a last tile of 16 pixels or fewer, measured slower -
     // the code is fetched once per workgroup, a path that one wave takes alone pays for its own instruction fetches.)
+    auto run_panel = [&](const int pc0) // pc0: the panel's first column
     {
         constexpr int RSX = RS;
         v4i acc[RSX][QS];
@@ -595,7 +647,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int j = 0; j < QS; ++j)
                 acc[i][j] = (v4i){0, 0, 0, 0};
-        const char *b_rd  = smem + lr * PITCH + lh * 16;
+        const char *b_rd  = smem + (pc0 + lr) * PITCH + lh * 16;
         const int   nkb   = (g.K + 63) >> 6; // k blocks that hold data (the panel is zero beyond)
         // operand blocks of k block kb: B from the panel, A from the staged window
         auto read_ops = [&](int kb, v4i (&fa)[RSX], v4i (&fb)[QS])
@@ -626,9 +678,9 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         // the operands of the next block before the matrix instructions of this one). K may end before the last batch of 3
         // blocks does: there the panel holds zeros.
 #pragma unroll
-        for (int kb = 0; kb < KBLK; ++kb)
+        for (int kb = 0; kb < KBU; ++kb)
         {
-            if (kb + 1 < KBLK)
+            if (kb + 1 < KBU)
                 read_ops(kb + 1, fa[(kb + 1) & 1], fb[(kb + 1) & 1]);
 #pragma unroll
             for (int rb = 0; rb < RSX; ++rb)
@@ -647,7 +699,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         if (fast && g.epi.qp_pk16 && (qflag_u & 3) == 0 && g.epi.vec_store && (g.N & 3) == 0)
         {
             // the short form of the requantisation, 4 columns at a time: lane l holds, for row rb * 16 + l % 16, the 4
-            // consecutive columns q * 16 + 4 * (l / 16) + {0..3}
+            // consecutive columns pc0 + q * 16 + 4 * (l / 16) + {0..3}
             const int16_t  o16 = (int16_t)(2 * g.epi.result_offset + 1), lo16 = (int16_t)g.epi.lo, hi16 = (int16_t)g.epi.hi;
             const pk16_t   off2p1 = {o16, o16}, lo = {lo16, lo16}, hi = {hi16, hi16};
             const int32_t *rowvec = g.epi.rowvec;
@@ -659,13 +711,13 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
             {
                 const int i = row0 + rb * 16 + lr;
                 rv[rb]      = (rowvec && i < a_M) ? rowvec[i] : 0;
-                drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + 4 * lh;
+                drow[rb]    = (char *)g.D + (int64_t)i * g.ldd + pc0 + 4 * lh;
             }
 #pragma unroll
             for (int q = 0; q < QS; ++q)
             {
-                const int c  = q * 16 + 4 * lh;
-                const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * NARROW_BN + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * NARROW_BN + c);
+                const int c  = pc0 + q * 16 + 4 * lh;
+                const v4i s2 = *(const v4i *)(par + (1 + QP_S2) * ncols + c), r1 = *(const v4i *)(par + (1 + QP_RSM1) * ncols + c);
                 const v4i cv = *(const v4i *)(par + c);
                 const int32_t s2a[4] = {s2[0], s2[1], s2[2], s2[3]}, r1a[4] = {r1[0], r1[1], r1[2], r1[3]};
 #pragma unroll
@@ -686,19 +738,41 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
             // the general forms check rows against g.M: the band's end stands in for it
             GemmArgs gl = g;
             gl.M        = a_M;
-            if (fast)
-                epilogue_store_fast<RSX, QS, NARROW_BN>(acc, gl, par, row0, 0, 0, lane, 0);
+            // (the staged constants' form is built for rows of 64 constants: several panels take the general one)
+            if constexpr (MULTI)
+                epilogue_store_t<EPI, RSX, QS>(acc, gl, row0, pc0, lane, 0);
             else
-                epilogue_store_t<EPI, RSX, QS>(acc, gl, row0, 0, lane, 0);
+            {
+                if (fast)
+                    epilogue_store_fast<RSX, QS, NARROW_BN>(acc, gl, par, row0, 0, 0, lane, 0);
+                else
+                    epilogue_store_t<EPI, RSX, QS>(acc, gl, row0, 0, lane, 0);
+            }
         }
+    };
+    // (With one panel the call stands alone: as a loop of one round - the panel count a compile-time 1 - the compiler laid
+    // the same code out differently and config 4 of the benchmark ran 0.5 us slower.)
+    if constexpr (MULTI)
+    {
+        for (int np = 0; np < npan; ++np)
+            run_panel(np * NARROW_BN);
     }
+    else
+        run_panel(0);
     MI355_BAND_PHASE(5); // stores issued
 #undef MI355_GLOBAL
 }
 
 template <int EPI, bool FLIP_A>
-static const void *halo_fn(int nb)
+static const void *halo_fn(int nb, bool multi, int K)
 {
+    if (multi)
+    {
+        if (nb != 1)
+            return nullptr;
+        return K <= 64 ? (const void *)conv_halo_kernel<EPI, FLIP_A, 1, true, 1>
+                       : (K <= 128 ? (const void *)conv_halo_kernel<EPI, FLIP_A, 1, true, 2> : (const void *)conv_halo_kernel<EPI, FLIP_A, 1, true, 3>);
+    }
     switch (nb)
     {
     case 1: return (const void *)conv_halo_kernel<EPI, FLIP_A, 1>;
@@ -712,13 +786,17 @@ static const void *halo_fn(int nb)
 }
 
 // The band form for this convolution? Fills rows-per-workgroup / workgroups-per-image / LDS bytes when it applies: more
-// tiles of 32 pixels than 4 per compute unit, C a power of two from 64 on, one panel of columns, and a band whose pixels
-// (at most 16 tiles) and input window fit one workgroup; magic_wp: the reciprocal (see ConvGeom) of the window's width.
+// tiles of 32 pixels than 4 per compute unit, C a power of two from 64 on, one panel of columns (up to NARROW_MAX_PANELS
+// with K <= 192), and a band whose pixels (at most 16 tiles) and input window fit one workgroup; magic_wp: the reciprocal
+// (see ConvGeom) of the window's width.
 static bool halo_plan(const GemmArgs &a, int epi, int cus, int &rpw, int &wpi, size_t &lds, uint32_t &magic_wp)
 {
     const ConvGeom &c = a.conv;
-    if (cus <= 0 || (epi != EPI_FIXEDPOINT && epi != EPI_F32) || a.N > NARROW_BN || c.C < 64 || (c.C & (c.C - 1)) != 0 || c.C > 1024)
+    if (cus <= 0 || (epi != EPI_FIXEDPOINT && epi != EPI_F32) || c.C < 64 || (c.C & (c.C - 1)) != 0 || c.C > 1024)
         return false;
+    if (a.N > NARROW_BN && (a.N > NARROW_MAX_PANELS * NARROW_BN || a.K > 192))
+        return false;
+    const int64_t ncols = (int64_t)((a.N + NARROW_BN - 1) / NARROW_BN) * NARROW_BN;
     const int64_t images = (int64_t)a.M / ((int64_t)c.OH * c.OW);
     if (images * c.OH * c.OW != a.M || (a.M + NARROW_ROWS - 1) / NARROW_ROWS <= (int64_t)NARROW_WAVES * cus)
         return false;
@@ -734,7 +812,7 @@ static bool halo_plan(const GemmArgs &a, int epi, int cus, int &rpw, int &wpi, s
     // the staged window: band + halo + padding (see the kernel)
     const int64_t in_rows = (int64_t)(rpw - 1) * c.stride_y + (int64_t)(c.KH - 1) * c.dil_y + 1;
     const int64_t wp      = (int64_t)(c.OW - 1) * c.stride_x + (int64_t)(c.KW - 1) * c.dil_x + 1;
-    const int64_t img_off = ((int64_t)NARROW_BN * (nb * 192 + NARROW_PAD_PIECES * 16) + (1 + QP_COUNT) * NARROW_BN * 4 + 1023) & ~(int64_t)1023;
+    const int64_t img_off = (ncols * (nb * 192 + NARROW_PAD_PIECES * 16) + (1 + QP_COUNT) * ncols * 4 + 4 + 1023) & ~(int64_t)1023;
     const int64_t bytes   = img_off + ((in_rows * wp * c.C + 1023) & ~(int64_t)1023);
     if (bytes > 160 * 1024 || images * wpi > (int64_t)INT32_MAX)
         return false;
@@ -809,12 +887,15 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
         uint32_t mwp = 0;
         if (halo_plan(args, epi, device_cus(), rpw, wpi, hl, mwp))
         {
-            const void *hf = epi == EPI_FIXEDPOINT ? (flip_a ? halo_fn<EPI_FIXEDPOINT, true>(nb) : halo_fn<EPI_FIXEDPOINT, false>(nb))
-                                                   : (flip_a ? halo_fn<EPI_F32, true>(nb) : halo_fn<EPI_F32, false>(nb));
+            const int   npan  = (args.N + NARROW_BN - 1) / NARROW_BN;
+            const bool  multi = npan > 1;
+            const int   K     = args.K;
+            const void *hf    = epi == EPI_FIXEDPOINT ? (flip_a ? halo_fn<EPI_FIXEDPOINT, true>(nb, multi, K) : halo_fn<EPI_FIXEDPOINT, false>(nb, multi, K))
+                                                      : (flip_a ? halo_fn<EPI_F32, true>(nb, multi, K) : halo_fn<EPI_F32, false>(nb, multi, K));
             if (hf == nullptr)
                 return (int)hipErrorInvalidValue;
-            static std::atomic<uint32_t> raised_h[2][2][NARROW_MAX_NB];
-            std::atomic<uint32_t>       &done = raised_h[epi == EPI_F32 ? 1 : 0][flip_a ? 1 : 0][nb - 1];
+            static std::atomic<uint32_t> raised_h[2][2][NARROW_MAX_NB + 3];
+            std::atomic<uint32_t>       &done = raised_h[epi == EPI_F32 ? 1 : 0][flip_a ? 1 : 0][multi ? NARROW_MAX_NB + (K <= 64 ? 0 : (K <= 128 ? 1 : 2)) : nb - 1];
             int                          dev  = 0;
             if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32)
                 return (int)hipErrorInvalidDevice;
@@ -826,9 +907,10 @@ int narrow_launch(int epi, bool flip_a, bool conv, const GemmArgs &args, hipStre
                 done.fetch_or(1u << dev, std::memory_order_release);
             }
             GemmArgs a = args;
-            a.tiles_m = wpi, a.tiles_n = rpw, a.magic_tiles = mwp;
+            a.tiles_m = wpi, a.tiles_n = rpw, a.magic_tiles = mwp, a.nblocks = npan;
             const int64_t images = (int64_t)args.M / ((int64_t)args.conv.OH * args.conv.OW);
-            void         *kargs[] = {&a.Bp, &a};
+            int32_t       ndma   = npan * (nb * 12 + NARROW_PAD_PIECES); // KiB of the panel image
+            void         *kargs[] = {&a.Bp, &ndma, &a};
             if (band)
                 *band = true;
             return (int)hipLaunchKernel(hf, dim3((unsigned)(images * wpi)), dim3(HALO_WAVES * 64), kargs, hl, s);

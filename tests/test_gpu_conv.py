@@ -248,6 +248,58 @@ def test_conv_few_output_channels_large_images_band_form():
     cv.close()
 
 
+def test_conv_band_form_several_column_panels():
+    """Pointwise and small-patch convolutions of large images with more than 64 output channels and K <= 192: the band form
+    keeps up to four panels of 64 columns in LDS and takes a wave's 32 pixels through one after the other. 256, 192, 130
+    and 100 output channels (a ragged last panel, a channel count that is no multiple of 4), C = 64 and 128, a 1 x 3 patch
+    with padding, stride 2, both source signs, weights with an offset, per-channel and per-tensor requantisation,
+    constants outside the short form, and the F32 destination."""
+    rng = np.random.default_rng(2560)
+    cases = [
+        # (src shape, weights shape, stride, pad, dilation, src dtype, weights dtype, weights zero point)
+        ((4, 100, 100, 64), (256, 1, 1, 64), (1, 1), (0, 0, 0, 0), (1, 1), np.int8, np.int8, 0),
+        ((2, 150, 140, 128), (192, 1, 1, 128), (1, 1), (0, 0, 0, 0), (1, 1), np.uint8, np.int8, 0),
+        ((2, 400, 300, 64), (130, 1, 1, 64), (2, 2), (0, 0, 0, 0), (1, 1), np.int8, np.int8, 0),
+        ((2, 160, 150, 64), (100, 1, 3, 64), (1, 1), (1, 1, 0, 0), (1, 1), np.uint8, np.uint8, 131),
+    ]
+    for (shape, wshape, stride, pad, dil, dt, w_dt, w_zp) in cases:
+        src = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max + 1, size=shape).astype(dt)
+        w = rng.integers(np.iinfo(w_dt).min + 1, np.iinfo(w_dt).max + 1, size=wshape).astype(w_dt)
+        bias = rng.integers(-500, 500, size=wshape[0], dtype=np.int32)
+        K = wshape[1] * wshape[2] * wshape[3]
+        zp = 5 if dt == np.int8 else 131
+        lo, hi, ozp = (-128, 127, -5) if dt == np.int8 else (0, 255, 9)
+        for per_channel in (True, False):
+            reals = rng.uniform(0.5, 2.0, wshape[0] if per_channel else 1) * 40.0 / (K ** 0.5 * 74.0 * 74.0)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            if per_channel and shape[0] == 2:
+                mult[70], shift[70] = 1 << 29, -1   # a multiplier below 2^30 and a left shift: not the short form
+            want = oracle.conv_nhwc_direct(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert 0.1 < ((want > lo) & (want < hi)).mean()
+            announce("conv band form, several panels", shape, wshape, stride, pad, dil, dt.__name__, w_dt.__name__, w_zp, "per_channel", per_channel)
+            got, name = run_conv(src, w, bias, zp, w_zp, mult, shift, ozp, lo, hi, stride, pad, dil)
+            assert name == "implicit_band_32x64", name
+            np.testing.assert_array_equal(got, want)
+    # F32 destination, 160 channels
+    import torch
+    src = rng.integers(-128, 128, size=(2, 140, 130, 64), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(160, 1, 1, 64), dtype=np.int8)
+    bias_f = rng.normal(0.0, 2.0, size=160).astype(np.float32)
+    scale = float(np.float32(0.02) * np.float32(0.005))
+    cols = oracle.im2col_nhwc(src, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 4)
+    want = oracle.gemmlowp_f32(cols, oracle.weights_reshape(w), bias_f, -4, 0, scale, 0.0, 6.0, act_twice=False)
+    cv = capi.Conv(capi.conv_desc(2, 140, 130, 64, 160, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), capi.S8, capi.S8, capi.F32, -4, 0, 4,
+                                  scale=scale, act=(0.0, 6.0)))
+    sd, wd, od, bd = to_dev(src), to_dev(w), to_dev(np.zeros((2, 140, 130, 160), np.float32)), to_dev(bias_f)
+    cv.prepare(wd, bd)
+    announce("conv band form, several panels, F32 destination", cv.kernel_name)
+    cv.run(sd, od)
+    torch.cuda.synchronize()
+    assert cv.kernel_name == "implicit_band_32x64", cv.kernel_name
+    assert np.array_equal(od.cpu().numpy().reshape(-1, 160).view(np.uint32), want.view(np.uint32))
+    cv.close()
+
+
 def test_conv_deep_patches_under_few_tiles_run_as_k_slices():
     """Few output tiles under a deep patch (the last 3 x 3 layers of a classifier: 14 x 14 or 7 x 7 pixels, 512 channels):
     the K range of the on-the-fly loader runs as slices along the grid of one S32 launch and a second kernel sums the

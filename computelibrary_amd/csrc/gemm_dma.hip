@@ -709,7 +709,9 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g_in)
         int kt = 0;
         if (inside)
         {
-            const int n_lean = g.K / BK - NS + 1; // steps kt whose stage kt+NS-1 is a whole K step
+            // A last K step that K ends in goes the same way where GemmArgs::lean_tail_bz allows it
+            const bool tail_lean = g.lean_tail_bz >= 0 && g.K % BK != 0 && !(bz == g.lean_tail_bz && m0 + BM >= g.M);
+            const int  n_lean    = (tail_lean ? nk : g.K / BK) - NS + 1; // steps kt whose stage kt+NS-1 needs no decisions
             for (; kt < n_lean; ++kt)
             {
                 prod.issue_inside(kt + NS - 1, (kt + NS - 1) % NS);
@@ -1013,6 +1015,12 @@ int dma_launch(int cfg_idx, int epi, bool flip_a, bool conv, const GemmArgs &arg
     a.magic_tiles = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_tiles) + 1u : 0u;
     a.magic_group = a.tile_magic_ok ? (uint32_t)((((uint64_t)1) << 32) / (uint64_t)d_group) + 1u : 0u;
     a.nblocks     = (int32_t)nblocks;
+    // (rows and batch entries at least a K step apart: what a whole last step reads beyond K then lies in the next row or
+    // entry, in front of a_end; not when the kernel sums the rows of A from the same tiles)
+    a.lean_tail_bz = (!conv && args.K % c.cfg.BK != 0 && args.epi.rowsum_mul == 0 && args.lda >= c.cfg.BK &&
+                      (batch == 1 || args.a_batch_stride >= c.cfg.BK))
+                         ? batch - 1
+                         : -1;
     void    *kargs[] = {&a};
     dim3     grid(args.tiles_m * args.tiles_n * batch, 1, 1), block((fn_slot == 0 && c.threads_dense) ? c.threads_dense : c.threads);
     return (int)hipLaunchKernel(fn, grid, block, kargs, c.lds_bytes, s);

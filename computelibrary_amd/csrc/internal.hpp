@@ -54,6 +54,10 @@ struct GemmArgs
     // implicit convolution whose K range runs as slices (the batch entries of one launch): K values per slice, a whole
     // number of K steps; entry z covers k in [z * k_slice, (z + 1) * k_slice) of the patch and K holds k_slice. 0: no slices
     int32_t  k_slice;
+    // dense A whose K ends inside the last K step, set by dma_launch: the batch entry in whose last row tile a 16-byte
+    // column of that step could reach beyond a_end. Every other tile may fetch the step whole - the columns at and
+    // beyond K then hold whatever follows in memory and meet the zero rows of the packed B. -1: no tile may.
+    int32_t  lean_tail_bz;
 };
 
 struct MfmaConfig

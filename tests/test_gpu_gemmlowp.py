@@ -256,6 +256,41 @@ def test_every_pipelined_configuration(cfg):
         np.testing.assert_array_equal(got.view(np.uint32), oracle.gemmlowp_f32(A, B, None, ao, bo, 3e-4).view(np.uint32))
 
 
+@pytest.mark.parametrize("K,lda", [(1000, 1000), (1096, 1120), (130, 136), (1104, 1104)])
+def test_k_tail_of_tiles_inside_the_matrix_on_the_256x128_tile(K, lda):
+    """A K that ends inside the last K step, on the 4 + 4 wave form: row tiles inside the matrix fetch that step whole -
+    the columns at and beyond K hold the next row's (or the next batch entry's) bytes and meet zero rows of B - except the
+    last row tile of the last batch entry, whose reads may not pass the end of A; a ragged last row tile takes the
+    general loader either way. One product and a batch of 3 (shared and per-entry B), rows that end where the next
+    begins and rows with a gap, signed and unsigned A, a B offset (row sums from a pass of their own, or inside the
+    kernel when K is a multiple of 16 - then the step is not fetched whole), all three epilogues."""
+    rng = np.random.default_rng(zlib.crc32(repr((K, lda)).encode()))
+    tile = capi.PATH_TILE + 0
+    N = 200
+    for (batch, M, a_dt, bo) in [(1, 768, np.int8, 0), (1, 700, np.uint8, -9), (3, 512, np.int8, 0), (3, 256, np.uint8, 4)]:
+        A = rng.integers(np.iinfo(a_dt).min, np.iinfo(a_dt).max + 1, size=(batch, M, K)).astype(a_dt)
+        for b_batched in ((False, True) if batch > 1 else (False,)):
+            B = rng.integers(-128, 128, size=((batch, K, N) if b_batched else (K, N)), dtype=np.int8)
+            ao = int(rng.integers(-20, 20))
+            Aa = A if batch > 1 else A[0]
+            B3 = B if b_batched else np.broadcast_to(B, (batch, K, N))
+            announce("k tail, 256x128 tile", (batch, M, N, K), "lda", lda, a_dt.__name__, "b_offset", bo, "b batched", b_batched)
+            got, name = run_gemm(Aa, B, capi.EPI_S32, np.int32, ao, bo, path=tile, device=True, lda=lda)
+            assert name == "pp_256x128x128_s3", name
+            want = np.stack([oracle.gemmlowp_s32(A[z], B3[z], ao, bo) for z in range(batch)])
+            np.testing.assert_array_equal(got if batch > 1 else got[None], want)
+            bias = rng.integers(-3000, 3000, size=N, dtype=np.int32)
+            reals = np.exp(rng.uniform(np.log(2e-5), np.log(2e-3), size=N)) * 128.0 / np.sqrt(K)
+            mult, shift = oracle.calculate_quantized_multipliers(1.0, reals, 1.0)
+            got, _ = run_gemm(Aa, B, capi.EPI_FIXEDPOINT, np.int8, ao, bo, bias, mult, shift, -7, -128, 127, path=tile, device=True, lda=lda)
+            want = np.stack([oracle.gemmlowp_fixedpoint(A[z], B3[z], bias, ao, bo, mult, shift, -7, -128, 127, np.int8) for z in range(batch)])
+            np.testing.assert_array_equal(got if batch > 1 else got[None], want)
+            if a_dt == np.int8:
+                got, _ = run_gemm(Aa, B, capi.EPI_F32, np.float32, ao, bo, scale=3e-4, path=tile, device=True, lda=lda)
+                want = np.stack([oracle.gemmlowp_f32(A[z], B3[z], None, ao, bo, 3e-4) for z in range(batch)])
+                np.testing.assert_array_equal((got if batch > 1 else got[None]).view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("cfg", range(len(PIPELINED_CONFIGS)))
 def test_row_sums_taken_inside_the_pipelined_kernels(cfg):
     """A non-zero B offset (or an unsigned B) needs b_offset * rowsum(A): with dword-aligned rows and K a multiple of 16

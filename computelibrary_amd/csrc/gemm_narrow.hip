@@ -412,7 +412,10 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) __attribute__((amdgpu_waves_per_
 // the matrix cores or LDS: 700 issue slots per wave, a third of them in the k loop.)
 // Needs C a power of two >= 64 (a 64-byte k block then lies inside one tap and one pixel), N <= 64, K <= 1152.
 constexpr int HALO_WAVES = 16;
-constexpr int HALO_DMA_WAVES = 8; // waves that issue the transfers
+constexpr int HALO_DMA_WAVES = 8; // waves that issue the window's transfers
+// ... and the panel's: every wave - these go out in front of the argument fetch, which the last waves wait for longest
+// (0.1 us faster than from the first 8 waves only)
+constexpr int HALO_PANEL_WAVES = HALO_WAVES;
 
 // Measurement build only (-DMI355_PHASE_CLOCKS, a library of its own that the product never loads): the first lane of
 // wave 0 and of wave 12 of the first, the middle and the last workgroup leaves the 100 MHz real-time counter at the ends
@@ -459,7 +462,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const long long t_entry = (long long)wall_clock64(); // before the first argument is asked for
 #endif
     {
-        // ---- the B panels: linear transfers of 1 KiB, wave w of the first HALO_DMA_WAVES those at w, w + 8, ... ----
+        // ---- the B panels: linear transfers of 1 KiB, wave w those at w, w + HALO_PANEL_WAVES, ... ----
         // Written out with scalar registers of its own choosing: the arguments are in flight here, and temporaries that
         // the compiler places in unused parts of their destination registers make it wait for them first.
         const int      wv = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
@@ -467,7 +470,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         // value would be one more such temporary.)
         const uint32_t v16 = ((uint32_t)threadIdx.x & 63u) * 16u;
         const uint32_t b_lo = (uint32_t)(uintptr_t)p_Bp, b_hi = (uint32_t)((uintptr_t)p_Bp >> 32);
-        if (wv < HALO_DMA_WAVES && (!MULTI || wv < p_ndma))
+        if (wv < HALO_PANEL_WAVES && wv < (MULTI ? p_ndma : NDMA)) // (the loop below makes its first round unasked)
         {
             if constexpr (MULTI)
                 asm volatile("s_lshl_b32 s92, %[wv], 10\n\t"
@@ -481,8 +484,8 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
                              "s_add_u32 s92, s92, %[stepb]\n\t"
                              "s_cmp_lt_i32 s93, %[n]\n\t"
                              "s_cbranch_scc1 1b" ::[wv] "s"(wv),
-                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "s"(p_ndma), [step] "i"(HALO_DMA_WAVES),
-                             [stepb] "i"(HALO_DMA_WAVES * 1024)
+                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "s"(p_ndma),  [step] "i"(HALO_PANEL_WAVES),
+                             [stepb] "i"(HALO_PANEL_WAVES * 1024)
                              : "s90", "s91", "s92", "s93", "scc", "memory");
             else
                 asm volatile("s_lshl_b32 s92, %[wv], 10\n\t"
@@ -496,8 +499,8 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
                              "s_add_u32 s92, s92, %[stepb]\n\t"
                              "s_cmp_lt_i32 s93, %[n]\n\t"
                              "s_cbranch_scc1 1b" ::[wv] "s"(wv),
-                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "i"(NDMA), [step] "i"(HALO_DMA_WAVES),
-                             [stepb] "i"(HALO_DMA_WAVES * 1024)
+                             [blo] "s"(b_lo), [bhi] "s"(b_hi), [v16] "v"(v16), [n] "i"(NDMA),  [step] "i"(HALO_PANEL_WAVES),
+                             [stepb] "i"(HALO_PANEL_WAVES * 1024)
                              : "s90", "s91", "s92", "s93", "scc", "memory");
         }
     }

@@ -79,10 +79,20 @@ def time_launches(torch, fn, steps, warmup):
     return wall, ev0.elapsed_time(ev1) * 1e-3
 
 
+# A kernel's duration is a steady-state figure: measured over at least this many graph-replayed launches behind at least
+# GRAPH_WARM_LAUNCHES untimed ones, whatever --steps and --warmup are (with 20 launches behind one replay the clocks have
+# not settled and the first launches run from cold caches: 5-10 % longer). `value`, `ms_per_step` and `eager_us` are over
+# exactly --steps launches behind --warmup.
+GRAPH_MIN_LAUNCHES = 1000
+GRAPH_WARM_LAUNCHES = 300
+
+
 def time_graph(torch, fns, launches):
     """The kernels' own duration with no host work inside the timed region: fns (called round-robin with the capture
-    stream) are captured into one HIP graph of about 200 launches, which is replayed until `launches` launches have
-    run, after one untimed replay. Returns seconds per launch."""
+    stream) are captured into one HIP graph of about 200 launches, which is replayed until max(launches,
+    GRAPH_MIN_LAUNCHES) launches have run, after untimed replays of GRAPH_WARM_LAUNCHES launches (at least one replay).
+    Returns seconds per launch."""
+    launches = max(launches, GRAPH_MIN_LAUNCHES)
     per_graph = max(len(fns), min(launches, 200) // len(fns) * len(fns))
     replays = (launches + per_graph - 1) // per_graph
     side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
@@ -90,7 +100,8 @@ def time_graph(torch, fns, launches):
         cs = torch.cuda.current_stream().cuda_stream
         for i in range(per_graph):
             fns[i % len(fns)](cs)
-    graph.replay()
+    for _ in range(max(1, (GRAPH_WARM_LAUNCHES + per_graph - 1) // per_graph)):
+        graph.replay()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     ev0.record()

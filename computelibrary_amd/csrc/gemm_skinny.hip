@@ -406,7 +406,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmArgs g)
 // blockIdx.x, blockIdx.x + gridDim.x, ... (at most ONCE_MAX_GROUPS of them); wave w owns the k blocks
 // [w * PER, (w + 1) * PER) of every group and copies its slice of A into LDS once for all groups. With one workgroup per
 // group, A (which never leaves the L2) crosses the compute unit's vector-memory path once per group and takes a third
-// of its requests; here it crosses once per compute unit. Two groups of B loads are in flight per wave. Partial sums
+// of its requests; here it crosses once per compute unit. One group of B loads is in flight per wave, refilled half by half (see ONE_SLOT). Partial sums
 // meet in double-buffered LDS (one barrier per group) and 8 x 16 threads finish one output each, so the only work
 // behind the last byte of B is one short chain; their per-column constants are fetched before the stream starts.
 constexpr int ONCE_WAVES      = 16;
@@ -558,10 +558,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_once_kernel(OnceArgs g
             ta[i] = *(const MI355_GLOBAL v4i *)(gA + (int64_t)min(i * RPL + a_sr, g.M - 1) * g.lda + (int64_t)min(kb0, KB - 1) * 64 + col);
     }
     const MI355_GLOBAL int8_t *bp = gB + ((int64_t)min(kb0, KB - 1) * 64 + lane) * 16; // (waves without k blocks re-read the last one)
-    // B operand blocks: two groups' worth in flight per wave - or, with 64 rows (half the registers hold A), one group's
-    // worth, refilled half by half as the matrix instructions release them
+    // B operand blocks: one group's worth in flight per wave, refilled half by half as the matrix instructions release
+    // them; two groups' worth only with a single k block per wave. (Two groups' worth of 4 k blocks fit the registers and
+    // were the first design - 128 loads of 1 KiB on offer per compute unit, which admits about 44 - and measured slower:
+    // M = 8, N = 11008, K = 4096 9.15 against 8.81 us; M = 16 9.73 / 9.25; M = 32 10.95 / 10.72; N = 32000 22.2 / 21.6;
+    // K = 2048 6.17 / 5.95; only K = 1024, one block per wave, prefers two: 4.59 against 4.68 us.)
     constexpr int  H0       = PER / 2;               // k blocks of the first half
-    constexpr bool ONE_SLOT = A_GLOBAL || PER == 8; // (8 k blocks per wave: two groups' worth would not fit the registers)
+    constexpr bool ONE_SLOT = A_GLOBAL || PER >= 2;
     v4i            fb[ONE_SLOT ? 1 : 2][PER];
     auto load_b_part = [&](int slot, int gi, auto u0c, auto u1c)
     {

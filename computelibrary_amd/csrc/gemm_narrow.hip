@@ -470,7 +470,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
         // value would be one more such temporary.)
         const uint32_t v16 = ((uint32_t)threadIdx.x & 63u) * 16u;
         const uint32_t b_lo = (uint32_t)(uintptr_t)p_Bp, b_hi = (uint32_t)((uintptr_t)p_Bp >> 32);
-        if (wv < HALO_PANEL_WAVES && wv < (MULTI ? p_ndma : NDMA)) // (the loop below makes its first round unasked)
+        if (wv < HALO_PANEL_WAVES && wv < (MULTI ? p_ndma : NDMA)) // (the loop below makes its first pass unasked)
         {
             if constexpr (MULTI)
                 asm volatile("s_lshl_b32 s92, %[wv], 10\n\t"
@@ -753,7 +753,7 @@ __global__ __launch_bounds__(HALO_WAVES * 64) __attribute__((amdgpu_waves_per_eu
             }
         }
     };
-    // (With one panel the call stands alone: as a loop of one round - the panel count a compile-time 1 - the compiler laid
+    // (With one panel the call stands alone: as a loop of one iteration - the panel count a compile-time 1 - the compiler laid
     // the same code out differently and config 4 of the benchmark ran 0.5 us slower.)
     if constexpr (MULTI)
     {
